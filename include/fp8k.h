@@ -1,0 +1,107 @@
+/*
+ * fp8k - C ABI of the MI355X (gfx950) W8A8 FP8 linear kernels.
+ *
+ * Every entry point takes raw device pointers, int64 sizes / element strides, small enums
+ * and a hipStream_t passed as void*.  Nothing here allocates, frees, synchronises or reads
+ * device memory from the host, so all calls are legal under HIP graph capture.  A call
+ * returns 0 on success; otherwise a non-zero fp8k_status and a message retrievable with
+ * fp8k_last_error() (thread-local).  Arguments are validated on the host before any launch.
+ *
+ * Each function cites the reference interface it stands in for (paths relative to the
+ * SGLang checkout).
+ */
+#ifndef FP8K_H
+#define FP8K_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+  FP8K_OK = 0,
+  FP8K_ERR_INVALID = 1,     /* bad argument: shape, stride, dtype, alignment, null pointer */
+  FP8K_ERR_UNSUPPORTED = 2, /* valid in the reference API but not built here */
+  FP8K_ERR_LAUNCH = 3,      /* HIP runtime error at launch */
+  FP8K_ERR_WORKSPACE = 4    /* workspace missing or too small */
+} fp8k_status;
+
+typedef enum { FP8K_F32 = 0, FP8K_F16 = 1, FP8K_BF16 = 2 } fp8k_dtype;
+
+typedef enum {
+  FP8K_SCALE_F32 = 0,         /* one float per group, addressed by (stride_m, stride_g) */
+  FP8K_SCALE_UE8M0_PACKED = 1 /* int32 words, 4 exponent bytes each, word (g/4) byte (g%4) */
+} fp8k_scale_kind;
+
+/* Message of the last failed call on this thread ("" if none). */
+const char* fp8k_last_error(void);
+/* ABI version: bumped when a signature changes. */
+int fp8k_abi_version(void);
+
+/*
+ * Per-token-group FP8 (OCP e4m3fn) quantisation.
+ * Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_8bit
+ *   (sgl-kernel/python/sgl_kernel/gemm.py:100-136, sgl-kernel/csrc/gemm/per_token_group_quant_8bit.cu:116-217);
+ *   arithmetic of native_per_token_group_quant_fp8 (python/sglang/test/test_block_fp8.py:23-48).
+ * x [M,K] contiguous of in_dtype; q [M,K] bytes; group_size in {16,32,64,128,256,512}, K % group_size == 0.
+ * scale_kind F32: s[m*s_stride_m + g*s_stride_g] (elements), any of row-major / column-major /
+ *   column-major padded.  UE8M0_PACKED: int32 word at s[(g/4)*s_stride_g + m*s_stride_m], byte g%4;
+ *   every word of a touched row is written whole (unused bytes zero).
+ * eps: amax floor.  For bf16 input it is rounded to bf16 first, as the torch-native path does.
+ * fp8_min/fp8_max must be -448/448.
+ */
+int fp8k_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, int64_t group_size, float eps,
+                     float fp8_min, float fp8_max, int in_dtype, int64_t s_stride_m, int64_t s_stride_g,
+                     int scale_kind, void* stream);
+
+/*
+ * Per-token (row) dynamic FP8 quantisation: s[m] = rowamax/448, q = clamp(x * (1/s)).
+ * Replaces torch.ops.sgl_kernel.sgl_per_token_quant_fp8
+ *   (sgl-kernel/python/sgl_kernel/gemm.py:155-160, sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-236).
+ * x [M,K] contiguous, K % 8 == 0; q [M,K]; s float [M].
+ */
+int fp8k_token_quant(const void* x, void* q, float* s, int64_t M, int64_t K, int in_dtype, void* stream);
+
+/*
+ * Per-tensor FP8 quantisation.  is_static=0: *s must be zero on entry and receives absmax/448
+ * (atomic max), then q = clamp(x * (1/ *s)).  is_static=1: *s is read only.
+ * Replaces torch.ops.sgl_kernel.sgl_per_tensor_quant_fp8
+ *   (sgl-kernel/python/sgl_kernel/gemm.py:144-152, sgl-kernel/csrc/gemm/per_tensor_quant_fp8.cu:96-118).
+ */
+int fp8k_tensor_quant(const void* x, void* q, float* s, int64_t numel, int in_dtype, int is_static, void* stream);
+
+/*
+ * Block-scaled FP8 GEMM:  C[m,n] = sum_kb ( A[m,kb] . B[n,kb] ) * As[m,kb] * Bs[n/128,kb],  fp32 accumulate.
+ * Replaces torch.ops.sgl_kernel.fp8_blockwise_scaled_mm
+ *   (sgl-kernel/python/sgl_kernel/gemm.py:25-32, sgl-kernel/csrc/gemm/fp8_blockwise_gemm_kernel.cu:368-465)
+ *   and w8a8_block_fp8_matmul (python/sglang/srt/layers/quantization/fp8_kernel.py:1072-1168).
+ * A e4m3fn [M,K] row-major (lda elements between rows); B e4m3fn [N,K] row-major (ldb) - the same memory
+ * as the reference's column-major mat_b [K,N]; scale block is 128 x 128.
+ * As float, element (m,kb) at As[m*as_stride_m + kb*as_stride_k]; Bs float, element (nb,kb) at
+ * Bs[nb*bs_stride_n + kb*bs_stride_k].  C [M,N] of out_dtype (F16/BF16), ldc elements between rows.
+ * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, ldc*2 % 16 == 0.
+ * workspace: device scratch of at least fp8k_block_gemm_workspace_bytes(M,N,K) bytes (may be 0 -> NULL ok).
+ */
+int fp8k_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M, int64_t N,
+                    int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
+                    int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
+                    int64_t workspace_bytes, void* stream);
+int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+/*
+ * Per-token x per-channel FP8 GEMM:  C = (A . B^T) * sa[m] * sb[n] (+ bias[n]), fp32 accumulate.
+ * Replaces torch.ops.sgl_kernel.fp8_scaled_mm
+ *   (sgl-kernel/python/sgl_kernel/gemm.py:35-43, sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532).
+ * Layouts as fp8k_block_gemm; sa float [M], sb float [N]; bias NULL or [N] of bias_dtype (F32/F16/BF16),
+ * added in float32 before the output cast.
+ */
+int fp8k_scaled_mm(const void* A, const void* B, const float* sa, const float* sb, const void* bias, void* C,
+                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int out_dtype,
+                   int bias_dtype, void* workspace, int64_t workspace_bytes, void* stream);
+int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP8K_H */

@@ -1,0 +1,98 @@
+// Shared host/device helpers of the fp8k library (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/fp8k.h"
+
+namespace fp8k {
+
+// ---------------------------------------------------------------- host: errors
+int fail(int code, const char* fmt, ...);
+void clear_error();
+
+#define FP8K_REQUIRE(cond, ...)                                   \
+  do {                                                            \
+    if (!(cond)) return ::fp8k::fail(FP8K_ERR_INVALID, __VA_ARGS__); \
+  } while (0)
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(FP8K_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return FP8K_OK;
+}
+
+inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// ---------------------------------------------------------------- device: types
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v8i __attribute__((ext_vector_type(8)));
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+typedef unsigned short u16;
+
+constexpr float kFp8Max = 448.0f;
+
+// ---------------------------------------------------------------- device: conversions
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+
+// float -> bf16 bits, round to nearest even (NaN kept quiet)
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+  return (f != f) ? 0x7fc0u : r;
+}
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+}
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+  _Float16 h = (_Float16)f;
+  return (uint32_t) __builtin_bit_cast(unsigned short, h);
+}
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+  return (float)__builtin_bit_cast(_Float16, (unsigned short)b);
+}
+
+// two floats -> two OCP e4m3fn bytes in the low / high half of a dword (v_cvt_pk_fp8_f32, RNE)
+__device__ __forceinline__ uint32_t cvt_pk_fp8_lo(float a, float b, uint32_t old) {
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, false);
+}
+__device__ __forceinline__ uint32_t cvt_pk_fp8_hi(float a, float b, uint32_t old) {
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, (int)old, true);
+}
+__device__ __forceinline__ uint32_t cvt4_fp8(float a, float b, float c, float d) {
+  // the low-half convert keeps the upper 16 bits of `old`, which the high-half convert overwrites
+  return cvt_pk_fp8_hi(c, d, cvt_pk_fp8_lo(a, b, __float_as_uint(a)));
+}
+
+// ---------------------------------------------------------------- device: DPP lane exchange
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float,
+                            __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each 16
+
+// max over aligned groups of LANES consecutive lanes; every lane of the group gets the result
+template <int LANES>
+__device__ __forceinline__ float group_max(float v) {
+  if (LANES >= 2) v = fmaxf(v, dpp_f<kDppXor1>(v));
+  if (LANES >= 4) v = fmaxf(v, dpp_f<kDppXor2>(v));
+  if (LANES >= 8) v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+  if (LANES >= 16) v = fmaxf(v, dpp_f<kDppMirror>(v));
+  if (LANES >= 32) v = fmaxf(v, __shfl_xor(v, 16));
+  if (LANES >= 64) v = fmaxf(v, __shfl_xor(v, 32));
+  return v;
+}
+
+}  // namespace fp8k

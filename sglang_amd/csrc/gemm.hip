@@ -1,0 +1,147 @@
+// Host side of the FP8 GEMM entry points: argument checks mirrored from the reference ops, kernel
+// choice, launch.  No allocation, no synchronisation.
+#include "gemm_kernels.h"
+
+namespace fp8k {
+
+struct Plan {
+  int kind;    // 0 = generic, 1 = tile256
+  int splits;  // >1: split-K through the float workspace
+  int kb_per_split;
+};
+
+static Plan make_plan(int64_t M, int64_t N, int64_t K) {
+  Plan pl{0, 1, 0};
+  if (K % kTileK != 0 || N % 4 != 0) return pl;
+  pl.kind = 1;
+  const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
+  const int kb = (int)(K / kTileK);
+  int splits = 1;
+  // fewer tiles than compute units: cut K so that every CU has work, keeping >= 4 K-blocks per run
+  if (tiles < 160) {
+    splits = (int)((256 + tiles - 1) / tiles);
+    if (splits > kb / 4) splits = kb / 4;
+    if (splits < 1) splits = 1;
+  }
+  pl.kb_per_split = (kb + splits - 1) / splits;
+  pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
+  return pl;
+}
+
+static int64_t workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0) return 0;
+  Plan pl = make_plan(M, N, K);
+  return pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+}
+
+template <int MODE, int OUT_DT, int BIAS_DT>
+static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
+  GemmArgs a = a0;
+  if (pl.kind == 0) {
+    dim3 grid((unsigned)((a.N + 63) / 64), (unsigned)((a.M + 3) / 4));
+    hipLaunchKernelGGL((gemm_generic_kernel<MODE, OUT_DT, BIAS_DT>), grid, dim3(256), 0, st, a);
+    return check_launch("gemm_generic");
+  }
+  a.tiles_m = (a.M + kTileM - 1) / kTileM;
+  a.tiles_n = (a.N + kTileN - 1) / kTileN;
+  a.splits = pl.splits;
+  a.kb_per_split = pl.kb_per_split;
+  const int ntiles = a.tiles_m * a.tiles_n;
+  const unsigned nwg = (unsigned)(((ntiles + 7) / 8) * 8 * pl.splits);
+  if (pl.splits == 1) {
+    hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT, false>), dim3(nwg), dim3(512), 0, st, a);
+    return check_launch("gemm_tile256");
+  }
+  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT, true>), dim3(nwg), dim3(512), 0, st, a);
+  int rc = check_launch("gemm_tile256_splitk");
+  if (rc) return rc;
+  const int64_t quads = (int64_t)a.M * (a.N / 4);
+  hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0,
+                     st, a);
+  return check_launch("splitk_reduce");
+}
+
+static int common_checks(const char* op, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
+                         int64_t lda, int64_t ldb, int64_t ldc, int out_dtype) {
+  FP8K_REQUIRE(M >= 0 && N >= 0 && K >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(M <= 0x7fffffffLL && N <= 0x7fffffffLL && K <= 0x7fffffffLL, "%s: shape too large", op);
+  FP8K_REQUIRE(out_dtype == FP8K_F16 || out_dtype == FP8K_BF16, "%s: out_dtype must be Half or BFloat16", op);
+  FP8K_REQUIRE(K % 16 == 0, "%s: mat_a must be multiple of 16 bytes for memory alignment", op);
+  FP8K_REQUIRE((N * 2) % 16 == 0, "%s: out must be multiple of 16 bytes for memory alignment", op);
+  FP8K_REQUIRE(lda >= K && ldb >= K && ldc >= N, "%s: leading dimension smaller than the row length", op);
+  FP8K_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && (ldc * 2) % 8 == 0, "%s: rows must be 16-byte aligned", op);
+  if (M == 0 || N == 0) return FP8K_OK;
+  FP8K_REQUIRE(A && B && C, "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(A, 16) && aligned(B, 16) && aligned(C, 8), "%s: operands must be 16-byte aligned", op);
+  return FP8K_OK;
+}
+
+}  // namespace fp8k
+
+using namespace fp8k;
+
+extern "C" int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return workspace_bytes(M, N, K); }
+extern "C" int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return workspace_bytes(M, N, K); }
+
+extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M,
+                               int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
+                               int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
+                               int64_t workspace_bytes_given, void* stream) {
+  clear_error();
+  int rc = common_checks("fp8_blockwise_scaled_mm", A, B, C, M, N, K, lda, ldb, ldc, out_dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return FP8K_OK;
+  FP8K_REQUIRE(K > 0, "fp8_blockwise_scaled_mm: K must be positive");
+  FP8K_REQUIRE(As && Bs, "fp8_blockwise_scaled_mm: null scale pointer");
+  FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0,
+               "fp8_blockwise_scaled_mm: negative scale stride");
+  const Plan pl = make_plan(M, N, K);
+  const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  if (need > 0 && (!workspace || workspace_bytes_given < need))
+    return fail(FP8K_ERR_WORKSPACE, "fp8_blockwise_scaled_mm: workspace of %lld bytes required, %lld given",
+                (long long)need, (long long)(workspace ? workspace_bytes_given : 0));
+  GemmArgs a{};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.sx = As; a.sw = Bs; a.bias = nullptr; a.C = C;
+  a.partial = (float*)workspace;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.sx_m = as_stride_m; a.sx_k = as_stride_k; a.sw_n = bs_stride_n; a.sw_k = bs_stride_k;
+  hipStream_t st = (hipStream_t)stream;
+  return out_dtype == FP8K_BF16 ? launch<kModeBlock, FP8K_BF16, FP8K_F32>(a, pl, st)
+                                : launch<kModeBlock, FP8K_F16, FP8K_F32>(a, pl, st);
+}
+
+extern "C" int fp8k_scaled_mm(const void* A, const void* B, const float* sa, const float* sb, const void* bias, void* C,
+                              int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int out_dtype,
+                              int bias_dtype, void* workspace, int64_t workspace_bytes_given, void* stream) {
+  clear_error();
+  int rc = common_checks("fp8_scaled_mm", A, B, C, M, N, K, lda, ldb, ldc, out_dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return FP8K_OK;
+  FP8K_REQUIRE(K > 0, "fp8_scaled_mm: K must be positive");
+  FP8K_REQUIRE(sa && sb, "fp8_scaled_mm: null scale pointer");
+  FP8K_REQUIRE(aligned(sb, 16), "fp8_scaled_mm: scales_b must be 16-byte aligned");
+  if (bias)
+    FP8K_REQUIRE(bias_dtype == FP8K_F32 || bias_dtype == FP8K_F16 || bias_dtype == FP8K_BF16,
+                 "fp8_scaled_mm: bias dtype must be float32, float16 or bfloat16");
+  const Plan pl = make_plan(M, N, K);
+  const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  if (need > 0 && (!workspace || workspace_bytes_given < need))
+    return fail(FP8K_ERR_WORKSPACE, "fp8_scaled_mm: workspace of %lld bytes required, %lld given", (long long)need,
+                (long long)(workspace ? workspace_bytes_given : 0));
+  GemmArgs a{};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.sx = sa; a.sw = sb; a.bias = bias; a.C = C;
+  a.partial = (float*)workspace;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  hipStream_t st = (hipStream_t)stream;
+  const int bd = bias ? bias_dtype : FP8K_F32;
+#define FP8K_SMM(O, B) launch<kModeRow, O, B>(a, pl, st)
+  if (out_dtype == FP8K_BF16) {
+    if (bd == FP8K_F32) return FP8K_SMM(FP8K_BF16, FP8K_F32);
+    if (bd == FP8K_BF16) return FP8K_SMM(FP8K_BF16, FP8K_BF16);
+    return FP8K_SMM(FP8K_BF16, FP8K_F16);
+  }
+  if (bd == FP8K_F32) return FP8K_SMM(FP8K_F16, FP8K_F32);
+  if (bd == FP8K_BF16) return FP8K_SMM(FP8K_F16, FP8K_BF16);
+  return FP8K_SMM(FP8K_F16, FP8K_F16);
+#undef FP8K_SMM
+}

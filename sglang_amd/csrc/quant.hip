@@ -1,0 +1,455 @@
+// FP8 (OCP e4m3fn) quantisation kernels for gfx950: per-token-group, per-token, per-tensor.
+//
+// All three are HBM-bound streaming kernels: 16-byte loads, 8/16-byte stores, one pass over the
+// input held in registers, amax by DPP lane exchange inside the wavefront.
+#include "fp8k_common.h"
+
+namespace fp8k {
+
+// ------------------------------------------------------------------------------------------------
+// loading 8 consecutive elements as float
+// ------------------------------------------------------------------------------------------------
+template <int DT>
+struct Raw8;
+template <>
+struct Raw8<FP8K_BF16> {
+  uint4 v;
+  __device__ __forceinline__ void load(const void* base, int64_t elem) { v = *reinterpret_cast<const uint4*>((const u16*)base + elem); }
+  __device__ __forceinline__ void zero() { v = make_uint4(0, 0, 0, 0); }
+  __device__ __forceinline__ void unpack(float (&a)[8]) const {
+    a[0] = bf16_lo(v.x); a[1] = bf16_hi(v.x); a[2] = bf16_lo(v.y); a[3] = bf16_hi(v.y);
+    a[4] = bf16_lo(v.z); a[5] = bf16_hi(v.z); a[6] = bf16_lo(v.w); a[7] = bf16_hi(v.w);
+  }
+};
+template <>
+struct Raw8<FP8K_F16> {
+  uint4 v;
+  __device__ __forceinline__ void load(const void* base, int64_t elem) { v = *reinterpret_cast<const uint4*>((const u16*)base + elem); }
+  __device__ __forceinline__ void zero() { v = make_uint4(0, 0, 0, 0); }
+  __device__ __forceinline__ void unpack(float (&a)[8]) const {
+    a[0] = f16_bits_to_f32(v.x & 0xffff); a[1] = f16_bits_to_f32(v.x >> 16);
+    a[2] = f16_bits_to_f32(v.y & 0xffff); a[3] = f16_bits_to_f32(v.y >> 16);
+    a[4] = f16_bits_to_f32(v.z & 0xffff); a[5] = f16_bits_to_f32(v.z >> 16);
+    a[6] = f16_bits_to_f32(v.w & 0xffff); a[7] = f16_bits_to_f32(v.w >> 16);
+  }
+};
+template <>
+struct Raw8<FP8K_F32> {
+  float4 lo, hi;
+  __device__ __forceinline__ void load(const void* base, int64_t elem) {
+    const float4* p = reinterpret_cast<const float4*>((const float*)base + elem);
+    lo = p[0];
+    hi = p[1];
+  }
+  __device__ __forceinline__ void zero() { lo = make_float4(0, 0, 0, 0); hi = lo; }
+  __device__ __forceinline__ void unpack(float (&a)[8]) const {
+    a[0] = lo.x; a[1] = lo.y; a[2] = lo.z; a[3] = lo.w; a[4] = hi.x; a[5] = hi.y; a[6] = hi.z; a[7] = hi.w;
+  }
+};
+
+__device__ __forceinline__ float absmax8(const float (&a)[8]) {
+  float m = fmaxf(fabsf(a[0]), fabsf(a[1]));
+  m = fmaxf(fmaxf(m, fabsf(a[2])), fabsf(a[3]));
+  m = fmaxf(fmaxf(m, fabsf(a[4])), fabsf(a[5]));
+  m = fmaxf(fmaxf(m, fabsf(a[6])), fabsf(a[7]));
+  return m;
+}
+
+// q = RNE_e4m3fn(clamp(a / sc)) for 8 values, bit-identical to an IEEE float32 divide followed by
+// the cast.  The divide is replaced by two multiplies with reciprocals that bracket the true
+// quotient (relative half-width 2^-20, far wider than the 2^-22 error of x * rcp(sc)); the cast
+// is monotonic, so when both ends land on the same byte the exact quotient does too.  The rare
+// lane whose bracket straddles a rounding boundary redoes its 8 values with the real divide.
+__device__ __forceinline__ uint2 quant8_div(const float (&a)[8], float sc) {
+  const float r = __builtin_amdgcn_rcpf(sc);  // 1 ulp
+  const float r_lo = r * (1.0f - 0x1p-20f);
+  const float r_hi = r * (1.0f + 0x1p-20f);
+  uint32_t l0 = cvt4_fp8(a[0] * r_lo, a[1] * r_lo, a[2] * r_lo, a[3] * r_lo);
+  uint32_t l1 = cvt4_fp8(a[4] * r_lo, a[5] * r_lo, a[6] * r_lo, a[7] * r_lo);
+  uint32_t h0 = cvt4_fp8(a[0] * r_hi, a[1] * r_hi, a[2] * r_hi, a[3] * r_hi);
+  uint32_t h1 = cvt4_fp8(a[4] * r_hi, a[5] * r_hi, a[6] * r_hi, a[7] * r_hi);
+  // sc outside [2^-100, 2^100] (only reachable with a non-default eps or non-finite data): no bracket
+  const bool safe = (__float_as_uint(sc) - 0x0D800000u) < (0x71800000u - 0x0D800000u);
+  if (__builtin_expect((l0 != h0) | (l1 != h1) | !safe, 0)) {
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float t = a[i] / sc;  // IEEE correctly rounded (no fast-math in this build)
+      t = t < -kFp8Max ? -kFp8Max : t;  // NaN falls through, as torch.clamp does
+      t = t > kFp8Max ? kFp8Max : t;
+      y[i] = t;
+    }
+    l0 = cvt4_fp8(y[0], y[1], y[2], y[3]);
+    l1 = cvt4_fp8(y[4], y[5], y[6], y[7]);
+  }
+  return make_uint2(l0, l1);
+}
+
+// amax / 448, correctly rounded.  FAST: q0 = a*y, r = a - 448*q0 (exact in one fma), q1 = q0 + r*y with
+// y = RN(1/448) - the classic reciprocal-refinement quotient, which is correctly rounded for this
+// divisor; it is used where amax is a 16-bit float (every possible operand is covered by a test
+// that walks all of them), float32 inputs take the full IEEE divide.
+template <bool FAST>
+__device__ __forceinline__ float div448(float a) {
+  if (!FAST) return a / kFp8Max;
+  constexpr float y = 1.0f / 448.0f;
+  const float q0 = a * y;
+  const float r = __builtin_fmaf(-q0, kFp8Max, a);
+  return __builtin_fmaf(r, y, q0);
+}
+
+// ------------------------------------------------------------------------------------------------
+// per-token-group quant
+//
+// One wavefront owns a strip of 32 rows x (64*8 = 512) columns, i.e. 32 rows of GPW = 512/GROUP
+// groups.  Each lane holds 8 consecutive elements of a row (one 16-byte load for bf16/f16),
+// LPG = GROUP/8 adjacent lanes form a group.  Rows are walked top to bottom, UNROLL rows of loads
+// in flight.  Scales are kept in registers while the strip is walked (lane i of a group keeps the
+// rows r with r % LPG == i) and written once at the end, so a column-major scale tensor receives
+// LPG consecutive floats per store instead of one 4-byte write per cache line.
+// ------------------------------------------------------------------------------------------------
+constexpr int kStripRows = 32;
+
+template <int DT, int GROUP, int KIND>
+__global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
+                                                          void* __restrict__ s, int M, int G, int64_t K,
+                                                          int nquads, float eps, int64_t sm, int64_t sg) {
+  constexpr int LPG = GROUP / 8;
+  constexpr int GPW = 64 / LPG;
+  constexpr int NK = (kStripRows + LPG - 1) / LPG;
+  constexpr int UNROLL = 4;
+  static_assert(KIND == FP8K_SCALE_F32 || GROUP == 128, "packed UE8M0 scales need 128-element groups");
+
+  const int lane = threadIdx.x & 63;
+  // wave-uniform task coordinates (kept in scalar registers)
+  const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
+  const int rt = wave / nquads;
+  const int qd = wave - rt * nquads;
+  const int r0 = rt * kStripRows;
+  if (r0 >= M) return;
+  const int nrows = min(kStripRows, M - r0);
+  const int lg = lane / LPG, li = lane % LPG;
+  const int g = qd * GPW + lg;
+  const bool valid = g < G;
+  // lanes past the last group of the row read the last group again and store nothing
+  const int64_t col = (int64_t)(valid ? g : G - 1) * GROUP + li * 8;
+  const int64_t base = (int64_t)r0 * K + col;
+
+  float keep[NK];
+#pragma unroll
+  for (int k = 0; k < NK; ++k) keep[k] = 0.f;
+  uint32_t keepw = 0;
+
+  auto process = [&](const Raw8<DT>& raw, int row) {
+    float a[8];
+    raw.unpack(a);
+    float amax = fmaxf(group_max<LPG>(absmax8(a)), eps);
+    float sc = div448<DT != FP8K_F32>(amax);
+    uint2 out;
+    if (KIND == FP8K_SCALE_UE8M0_PACKED) {
+      // round the scale up to a power of two; x / 2^e == x * 2^-e exactly
+      uint32_t b = __float_as_uint(fmaxf(sc, 1e-10f));
+      uint32_t e = (b >> 23) + ((b & 0x7fffffu) != 0u);
+      float rinv = __uint_as_float((254u - e) << 23);
+      out.x = cvt4_fp8(a[0] * rinv, a[1] * rinv, a[2] * rinv, a[3] * rinv);
+      out.y = cvt4_fp8(a[4] * rinv, a[5] * rinv, a[6] * rinv, a[7] * rinv);
+      uint32_t eb = valid ? e : 0u;
+      uint32_t w = (uint32_t)__builtin_amdgcn_readlane((int)eb, 0) |
+                   ((uint32_t)__builtin_amdgcn_readlane((int)eb, 16) << 8) |
+                   ((uint32_t)__builtin_amdgcn_readlane((int)eb, 32) << 16) |
+                   ((uint32_t)__builtin_amdgcn_readlane((int)eb, 48) << 24);
+      keepw = (lane == row) ? w : keepw;
+    } else {
+      out = quant8_div(a, sc);
+#pragma unroll
+      for (int k = 0; k < NK; ++k) keep[k] = (row == k * LPG + li) ? sc : keep[k];
+    }
+    if (valid) *reinterpret_cast<uint2*>(q + base + (int64_t)row * K) = out;
+  };
+
+  // full chunks of UNROLL rows, the next chunk's loads in flight while this one is processed
+  const int nfull = nrows / UNROLL;
+  Raw8<DT> cur[UNROLL], nxt[UNROLL];
+  if (nfull > 0) {
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) cur[j].load(x, base + (int64_t)j * K);
+  }
+  for (int c = 0; c < nfull; ++c) {
+    if (c + 1 < nfull) {
+#pragma unroll
+      for (int j = 0; j < UNROLL; ++j) nxt[j].load(x, base + (int64_t)((c + 1) * UNROLL + j) * K);
+    }
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) process(cur[j], c * UNROLL + j);
+#pragma unroll
+    for (int j = 0; j < UNROLL; ++j) cur[j] = nxt[j];
+  }
+  for (int row = nfull * UNROLL; row < nrows; ++row) {
+    Raw8<DT> t;
+    t.load(x, base + (int64_t)row * K);
+    process(t, row);
+  }
+
+  if (KIND == FP8K_SCALE_UE8M0_PACKED) {
+    if (lane < nrows) reinterpret_cast<uint32_t*>(s)[(int64_t)qd * sg + (int64_t)(r0 + lane) * sm] = keepw;
+  } else {
+#pragma unroll
+    for (int k = 0; k < NK; ++k) {
+      const int row = k * LPG + li;
+      if (valid && row < nrows) reinterpret_cast<float*>(s)[(int64_t)(r0 + row) * sm + (int64_t)g * sg] = keep[k];
+    }
+  }
+}
+
+template <int DT, int GROUP, int KIND>
+static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, float eps, int64_t sm, int64_t sg,
+                              hipStream_t st) {
+  constexpr int GPW = 64 / (GROUP / 8);
+  const int G = (int)(K / GROUP);
+  const int nquads = (G + GPW - 1) / GPW;
+  const int64_t nstrips = (M + kStripRows - 1) / kStripRows;
+  const int64_t waves = nstrips * nquads;
+  const int64_t blocks = (waves + 3) / 4;
+  if (waves > 0x7fffffffLL) return fail(FP8K_ERR_INVALID, "group_quant: input too large for one launch");
+  hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND>), dim3((unsigned)blocks), dim3(256), 0, st, x, (uint8_t*)q, s,
+                     (int)M, G, K, nquads, eps, sm, sg);
+  return check_launch("group_quant");
+}
+
+template <int DT, int KIND>
+static int dispatch_group(const void* x, void* q, void* s, int64_t M, int64_t K, int64_t group, float eps, int64_t sm,
+                          int64_t sg, hipStream_t st) {
+  if (KIND == FP8K_SCALE_UE8M0_PACKED) {
+    if (group != 128) return fail(FP8K_ERR_INVALID, "group_quant: packed UE8M0 scales require group_size 128");
+    return launch_group_quant<DT, 128, KIND>(x, q, s, M, K, eps, sm, sg, st);
+  }
+  switch (group) {
+    case 16: return launch_group_quant<DT, 16, FP8K_SCALE_F32>(x, q, s, M, K, eps, sm, sg, st);
+    case 32: return launch_group_quant<DT, 32, FP8K_SCALE_F32>(x, q, s, M, K, eps, sm, sg, st);
+    case 64: return launch_group_quant<DT, 64, FP8K_SCALE_F32>(x, q, s, M, K, eps, sm, sg, st);
+    case 128: return launch_group_quant<DT, 128, FP8K_SCALE_F32>(x, q, s, M, K, eps, sm, sg, st);
+    case 256: return launch_group_quant<DT, 256, FP8K_SCALE_F32>(x, q, s, M, K, eps, sm, sg, st);
+    case 512: return launch_group_quant<DT, 512, FP8K_SCALE_F32>(x, q, s, M, K, eps, sm, sg, st);
+  }
+  return fail(FP8K_ERR_INVALID, "group_quant: group_size %lld not in {16,32,64,128,256,512}", (long long)group);
+}
+
+// ------------------------------------------------------------------------------------------------
+// per-token quant: one workgroup per row, row held in registers between the amax and the cast
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float block_max_256(float v, float* red) {
+  v = group_max<64>(v);
+  const int w = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[w] = v;
+  __syncthreads();
+  v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+  __syncthreads();
+  return v;
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void token_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
+                                                          float* __restrict__ s, int64_t K) {
+  constexpr int HOLD = 8;  // 8 chunks x 256 threads x 8 elements = 16384 columns stay in registers
+  __shared__ float red[4];
+  const int64_t row = blockIdx.x;
+  const int nchunk = (int)(K / 8);
+  Raw8<DT> raw[HOLD];
+  float m = 0.f;
+#pragma unroll
+  for (int c = 0; c < HOLD; ++c) {
+    const int ch = c * 256 + threadIdx.x;
+    if (ch < nchunk) {
+      raw[c].load(x, row * K + (int64_t)ch * 8);
+      float a[8];
+      raw[c].unpack(a);
+      m = fmaxf(m, absmax8(a));
+    }
+  }
+  for (int ch = HOLD * 256 + threadIdx.x; ch < nchunk; ch += 256) {
+    Raw8<DT> t;
+    t.load(x, row * K + (int64_t)ch * 8);
+    float a[8];
+    t.unpack(a);
+    m = fmaxf(m, absmax8(a));
+  }
+  m = block_max_256(m, red);
+  const float sc = m / kFp8Max;
+  if (threadIdx.x == 0) s[row] = sc;
+  const float inv = (sc == 0.f) ? 0.f : 1.0f / sc;
+  auto emit = [&](const float(&a)[8], int ch) {
+    float y[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = fmaxf(fminf(a[i] * inv, kFp8Max), -kFp8Max);
+    uint2 o;
+    o.x = cvt4_fp8(y[0], y[1], y[2], y[3]);
+    o.y = cvt4_fp8(y[4], y[5], y[6], y[7]);
+    *reinterpret_cast<uint2*>(q + row * K + (int64_t)ch * 8) = o;
+  };
+#pragma unroll
+  for (int c = 0; c < HOLD; ++c) {
+    const int ch = c * 256 + threadIdx.x;
+    if (ch < nchunk) {
+      float a[8];
+      raw[c].unpack(a);
+      emit(a, ch);
+    }
+  }
+  for (int ch = HOLD * 256 + threadIdx.x; ch < nchunk; ch += 256) {
+    Raw8<DT> t;
+    t.load(x, row * K + (int64_t)ch * 8);
+    float a[8];
+    t.unpack(a);
+    emit(a, ch);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// per-tensor quant: grid-stride absmax with one atomic max per workgroup, then the cast
+// ------------------------------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ float load1(const void* x, int64_t i) {
+  if (DT == FP8K_F32) return ((const float*)x)[i];
+  if (DT == FP8K_BF16) return __uint_as_float((uint32_t)((const u16*)x)[i] << 16);
+  return f16_bits_to_f32(((const u16*)x)[i]);
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void tensor_absmax_kernel(const void* __restrict__ x, float* __restrict__ s,
+                                                            int64_t numel) {
+  __shared__ float red[4];
+  const int64_t nchunk = numel / 8;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  float m = 0.f;
+  for (int64_t ch = (int64_t)blockIdx.x * 256 + threadIdx.x; ch < nchunk; ch += stride) {
+    Raw8<DT> t;
+    t.load(x, ch * 8);
+    float a[8];
+    t.unpack(a);
+    m = fmaxf(m, absmax8(a));
+  }
+  for (int64_t i = nchunk * 8 + (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride)
+    m = fmaxf(m, fabsf(load1<DT>(x, i)));
+  m = block_max_256(m, red);
+  // non-negative floats order like their bit patterns
+  if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned int*>(s), __float_as_uint(m / kFp8Max));
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void tensor_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
+                                                           const float* __restrict__ s, int64_t numel) {
+  const float inv = 1.0f / s[0];
+  const int64_t nchunk = numel / 8;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t ch = (int64_t)blockIdx.x * 256 + threadIdx.x; ch < nchunk; ch += stride) {
+    Raw8<DT> t;
+    t.load(x, ch * 8);
+    float a[8], y[8];
+    t.unpack(a);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) y[i] = fmaxf(fminf(a[i] * inv, kFp8Max), -kFp8Max);
+    uint2 o;
+    o.x = cvt4_fp8(y[0], y[1], y[2], y[3]);
+    o.y = cvt4_fp8(y[4], y[5], y[6], y[7]);
+    *reinterpret_cast<uint2*>(q + ch * 8) = o;
+  }
+  for (int64_t i = nchunk * 8 + (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
+    float y = fmaxf(fminf(load1<DT>(x, i) * inv, kFp8Max), -kFp8Max);
+    q[i] = (uint8_t)(cvt_pk_fp8_lo(y, 0.f, 0) & 0xff);
+  }
+}
+
+}  // namespace fp8k
+
+using namespace fp8k;
+
+extern "C" int fp8k_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, int64_t group_size, float eps,
+                                float fp8_min, float fp8_max, int in_dtype, int64_t s_stride_m, int64_t s_stride_g,
+                                int scale_kind, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(M >= 0 && K >= 0, "group_quant: negative shape");
+  FP8K_REQUIRE(group_size > 0 && K % group_size == 0,
+               "group_quant: the last dimension of `x` (%lld) cannot be divisible by `group_size` (%lld)", (long long)K,
+               (long long)group_size);
+  FP8K_REQUIRE(fp8_max == 448.0f && fp8_min == -448.0f, "group_quant: fp8_min/fp8_max must be -448/448 (OCP e4m3fn)");
+  FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "group_quant: bad input dtype %d",
+               in_dtype);
+  FP8K_REQUIRE(scale_kind == FP8K_SCALE_F32 || scale_kind == FP8K_SCALE_UE8M0_PACKED, "group_quant: bad scale kind %d",
+               scale_kind);
+  FP8K_REQUIRE(M <= 0x7fffffffLL && K / group_size <= 0x7fffffffLL, "group_quant: shape too large");
+  if (M == 0 || K == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && q && s, "group_quant: null pointer");
+  FP8K_REQUIRE(aligned(x, 16) && aligned(q, 8) && aligned(s, 4), "group_quant: x must be 16-byte, q 8-byte aligned");
+  const int64_t G = K / group_size;
+  if (scale_kind == FP8K_SCALE_F32) {
+    FP8K_REQUIRE(s_stride_m >= 0 && s_stride_g >= 0 && (M == 1 || s_stride_m > 0) && (G == 1 || s_stride_g > 0),
+                 "group_quant: scale strides must be positive");
+  } else {
+    FP8K_REQUIRE(s_stride_m > 0 && ((G + 3) / 4 == 1 || s_stride_g > 0), "group_quant: packed scale strides must be positive");
+  }
+  // the torch-native formula clamps amax in the input dtype: bf16 sees eps rounded to bf16
+  float eps_eff = eps;
+  if (in_dtype == FP8K_BF16) {
+    uint32_t u;
+    memcpy(&u, &eps, 4);
+    u = ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16) << 16;
+    memcpy(&eps_eff, &u, 4);
+  }
+  hipStream_t st = (hipStream_t)stream;
+#define FP8K_GQ(DT)                                                                                               \
+  (scale_kind == FP8K_SCALE_F32                                                                                   \
+       ? dispatch_group<DT, FP8K_SCALE_F32>(x, q, s, M, K, group_size, eps_eff, s_stride_m, s_stride_g, st)       \
+       : dispatch_group<DT, FP8K_SCALE_UE8M0_PACKED>(x, q, s, M, K, group_size, eps_eff, s_stride_m, s_stride_g, st))
+  switch (in_dtype) {
+    case FP8K_BF16: return FP8K_GQ(FP8K_BF16);
+    case FP8K_F16: return FP8K_GQ(FP8K_F16);
+    default: return FP8K_GQ(FP8K_F32);
+  }
+#undef FP8K_GQ
+}
+
+extern "C" int fp8k_token_quant(const void* x, void* q, float* s, int64_t M, int64_t K, int in_dtype, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(M >= 0 && K >= 0, "token_quant: negative shape");
+  FP8K_REQUIRE(K % 8 == 0, "token_quant: hidden dimension (%lld) must be divisible by 8", (long long)K);
+  FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "token_quant: bad input dtype %d",
+               in_dtype);
+  FP8K_REQUIRE(M <= 0x7fffffffLL, "token_quant: too many rows");
+  if (M == 0 || K == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && q && s, "token_quant: null pointer");
+  FP8K_REQUIRE(aligned(x, 16) && aligned(q, 8), "token_quant: x must be 16-byte, q 8-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)M), block(256);
+  switch (in_dtype) {
+    case FP8K_BF16: hipLaunchKernelGGL(token_quant_kernel<FP8K_BF16>, grid, block, 0, st, x, (uint8_t*)q, s, K); break;
+    case FP8K_F16: hipLaunchKernelGGL(token_quant_kernel<FP8K_F16>, grid, block, 0, st, x, (uint8_t*)q, s, K); break;
+    default: hipLaunchKernelGGL(token_quant_kernel<FP8K_F32>, grid, block, 0, st, x, (uint8_t*)q, s, K); break;
+  }
+  return check_launch("token_quant");
+}
+
+extern "C" int fp8k_tensor_quant(const void* x, void* q, float* s, int64_t numel, int in_dtype, int is_static,
+                                 void* stream) {
+  clear_error();
+  FP8K_REQUIRE(numel >= 0, "tensor_quant: negative size");
+  FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "tensor_quant: bad input dtype %d",
+               in_dtype);
+  if (numel == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && q && s, "tensor_quant: null pointer");
+  FP8K_REQUIRE(aligned(x, 16) && aligned(q, 8), "tensor_quant: x must be 16-byte, q 8-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t want = (numel / 8 + 255) / 256;
+  dim3 grid((unsigned)(want < 1 ? 1 : (want > 2048 ? 2048 : want))), block(256);
+#define FP8K_TQ(DT)                                                                                     \
+  do {                                                                                                  \
+    if (!is_static) hipLaunchKernelGGL(tensor_absmax_kernel<DT>, grid, block, 0, st, x, s, numel);      \
+    hipLaunchKernelGGL(tensor_quant_kernel<DT>, grid, block, 0, st, x, (uint8_t*)q, (const float*)s, numel); \
+  } while (0)
+  switch (in_dtype) {
+    case FP8K_BF16: FP8K_TQ(FP8K_BF16); break;
+    case FP8K_F16: FP8K_TQ(FP8K_F16); break;
+    default: FP8K_TQ(FP8K_F32); break;
+  }
+#undef FP8K_TQ
+  return check_launch("tensor_quant");
+}

@@ -1,0 +1,166 @@
+"""Entry points of ``sglang.srt.layers.quantization.fp8_kernel`` on this path.
+
+gfx950 is OCP FP8: fp8_dtype is float8_e4m3fn and fp8_max is 448 (the reference's fnuz branch,
+fp8_kernel.py:81-95, applies to gfx94x only and is not reproduced).
+"""
+from __future__ import annotations
+
+from typing import List, Optional, Tuple
+
+import torch
+
+from . import sgl_kernel as _ops
+
+fp8_dtype = torch.float8_e4m3fn
+fp8_max = 448.0
+fp8_min = -448.0
+
+
+def ceil_align(x: int, y: int) -> int:
+    return (x + y - 1) // y * y
+
+
+def create_per_token_group_quant_fp8_output_scale(
+    x_shape, device, group_size: int, column_major_scales: bool, scale_tma_aligned: bool, scale_ue8m0: bool
+) -> torch.Tensor:
+    """Reference: fp8_kernel.py:437-478 - the four scale layouts, returned as strided views."""
+    if scale_ue8m0:
+        assert column_major_scales and scale_tma_aligned
+        *x_batch, x_q_mn, x_q_k = x_shape
+        x_s_mn, x_s_k = x_q_mn, x_q_k // 128
+        aligned_mn = ceil_align(x_s_mn, 4)
+        aligned_k = ceil_align(x_s_k, 4)
+        return torch.empty((*x_batch, aligned_k // 4, aligned_mn), device=device, dtype=torch.int).transpose(-1, -2)[
+            ..., :x_s_mn, :
+        ]
+    if column_major_scales:
+        if scale_tma_aligned:
+            aligned_size = (x_shape[-2] + 3) // 4 * 4
+            return torch.empty(
+                tuple(x_shape[:-2]) + (x_shape[-1] // group_size, aligned_size), device=device, dtype=torch.float32
+            ).transpose(-1, -2)[: x_shape[-2], :]
+        return torch.empty(
+            (x_shape[-1] // group_size,) + tuple(x_shape[:-1]), device=device, dtype=torch.float32
+        ).permute(-1, -2)
+    return torch.empty(tuple(x_shape[:-1]) + (x_shape[-1] // group_size,), device=device, dtype=torch.float32)
+
+
+def sglang_per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    column_major_scales: bool = False,
+    scale_tma_aligned: bool = False,
+    scale_ue8m0: bool = False,
+    fuse_silu_and_mul: bool = False,
+    masked_m: Optional[torch.Tensor] = None,
+    enable_v2: Optional[bool] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:481-531."""
+    assert x.shape[-1] % group_size == 0, "the last dimension of `x` cannot be divisible by `group_size`"
+    assert x.is_contiguous(), "`x` is not contiguous"
+    out_shape = (*x.shape[:-1], x.shape[-1] // (2 if fuse_silu_and_mul else 1))
+    x_q = torch.empty(out_shape, device=x.device, dtype=fp8_dtype)
+    x_s = create_per_token_group_quant_fp8_output_scale(
+        x_shape=out_shape,
+        device=x.device,
+        group_size=group_size,
+        column_major_scales=column_major_scales,
+        scale_tma_aligned=scale_tma_aligned,
+        scale_ue8m0=scale_ue8m0,
+    )
+    if x.shape[0] > 0:
+        s2 = x_s if x_s.dim() == 2 else x_s.reshape(-1, x_s.shape[-1]) if not (column_major_scales or scale_ue8m0) else x_s
+        if s2.dim() != 2:
+            raise RuntimeError("column-major scale layouts need a 2-D input")
+        _ops.sgl_per_token_group_quant_8bit(
+            x, x_q, s2, group_size, eps, fp8_min, fp8_max, scale_ue8m0, fuse_silu_and_mul, masked_m, enable_v2=enable_v2
+        )
+    return x_q, x_s
+
+
+def per_token_group_quant_fp8(
+    x: torch.Tensor,
+    group_size: int,
+    eps: float = 1e-10,
+    dtype: torch.dtype = fp8_dtype,
+    column_major_scales: bool = False,
+    scale_tma_aligned: bool = False,
+    scale_ue8m0: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:219-327 (the Triton entry point); same kernel as the sgl-kernel one here."""
+    if dtype != fp8_dtype:
+        raise RuntimeError("per_token_group_quant_fp8: only float8_e4m3fn is built on gfx950")
+    return sglang_per_token_group_quant_fp8(
+        x, group_size, eps, column_major_scales=column_major_scales, scale_tma_aligned=scale_tma_aligned,
+        scale_ue8m0=scale_ue8m0,
+    )
+
+
+def sglang_per_token_quant_fp8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype):
+    """Reference: fp8_kernel.py:577-593 - dynamic per-token quant, scales [M,1] float32."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    x_q = torch.empty_like(x, device=x.device, dtype=dtype)
+    x_s = torch.empty(x.shape[0], 1, device=x.device, dtype=torch.float32)
+    _ops.sgl_per_token_quant_fp8(x, x_q, x_s)
+    return x_q, x_s
+
+
+def scaled_fp8_quant(
+    input: torch.Tensor,
+    scale: Optional[torch.Tensor] = None,
+    num_token_padding: Optional[int] = None,
+    use_per_token_if_dynamic: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:1431-1468 (sgl-kernel branch): static per-tensor when `scale` is given,
+    else dynamic per-token or per-tensor."""
+    assert input.ndim == 2, f"Expected 2D input tensor, got {input.ndim}D"
+    shape = input.shape
+    if num_token_padding:
+        shape = (max(num_token_padding, input.shape[0]), shape[1])
+    output = torch.empty(shape, device=input.device, dtype=fp8_dtype)
+    if scale is None:
+        if use_per_token_if_dynamic:
+            scale = torch.empty((shape[0], 1), device=input.device, dtype=torch.float32)
+            _ops.sgl_per_token_quant_fp8(input, output[: input.shape[0]], scale[: input.shape[0]])
+        else:
+            scale = torch.zeros(1, device=input.device, dtype=torch.float32)
+            _ops.sgl_per_tensor_quant_fp8(input, output[: input.shape[0]], scale, is_static=False)
+    else:
+        assert scale.numel() == 1, f"Expected scalar scale, got numel={scale.numel()}"
+        _ops.sgl_per_tensor_quant_fp8(input, output[: input.shape[0]], scale, is_static=True)
+    return output, scale
+
+
+def w8a8_block_fp8_matmul(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    As: torch.Tensor,
+    Bs: torch.Tensor,
+    block_size: List[int],
+    output_dtype: torch.dtype = torch.float16,
+) -> torch.Tensor:
+    """Reference: fp8_kernel.py:1153-1168, checks :1003-1048.
+
+    A e4m3fn [..., K]; B e4m3fn [N, K] contiguous; As float32 [..., ceil(K/bk)]; Bs float32
+    [ceil(N/bn), ceil(K/bk)]; block_size must be [128, 128] on this path.
+    """
+    assert len(block_size) == 2
+    block_n, block_k = block_size
+    if block_n != 128 or block_k != 128:
+        raise RuntimeError("w8a8_block_fp8_matmul: only block_size [128, 128] is built on this path")
+    assert A.shape[-1] == B.shape[-1]
+    assert A.shape[:-1] == As.shape[:-1] and A.is_contiguous()
+    assert (A.shape[-1] + block_k - 1) // block_k == As.shape[-1]
+    assert B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
+    N, K = B.shape
+    assert (N + block_n - 1) // block_n == Bs.shape[0]
+    assert (K + block_k - 1) // block_k == Bs.shape[1]
+    M = A.numel() // A.shape[-1]
+    C_shape = A.shape[:-1] + (N,)
+    A2 = A.reshape(M, K)
+    As2 = As.reshape(M, As.shape[-1])
+    if As2.dtype != torch.float32 or Bs.dtype != torch.float32:
+        raise RuntimeError("w8a8_block_fp8_matmul: packed UE8M0 GEMM scales are not built on this path")
+    out = _ops._block_gemm_nk(A2, B, As2, Bs, output_dtype)
+    return out.reshape(C_shape)

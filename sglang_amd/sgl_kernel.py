@@ -1,0 +1,287 @@
+"""The ops SGLang reaches through ``sgl_kernel`` on this path, backed by libfp8k.so.
+
+Signatures, argument meaning and error behaviour follow sgl-kernel/python/sgl_kernel/gemm.py,
+moe.py and elementwise.py of the reference; the native side is the C ABI in include/fp8k.h.
+Quant ops write into caller-allocated outputs; GEMM ops return a fresh tensor.  Every launch goes
+on the current torch stream of the tensor's device and never synchronises.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+from ._lib import check, dtype_code, lib, require_cuda, stream_ptr
+
+FP8_DTYPE = torch.float8_e4m3fn
+FP8_MAX = 448.0
+FP8_MIN = -448.0
+
+_workspaces: dict = {}
+
+
+def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
+    """Per-(device, stream) split-K scratch, grown on demand and reused (never freed mid-graph)."""
+    if nbytes <= 0:
+        return None
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _workspaces.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = buf
+    return buf
+
+
+# --------------------------------------------------------------------------------------------
+# quantisation
+# --------------------------------------------------------------------------------------------
+
+
+def sgl_per_token_group_quant_8bit(
+    input: torch.Tensor,
+    output_q: torch.Tensor,
+    output_s: torch.Tensor,
+    group_size: int,
+    eps: float,
+    fp8_min: float,
+    fp8_max: float,
+    scale_ue8m0: bool = False,
+    fuse_silu_and_mul: bool = False,
+    masked_m: Optional[torch.Tensor] = None,
+    enable_v2: Optional[bool] = None,
+) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:100-136 (op schema common_extension.cc:128-152).
+
+    output_s selects the scale layout by its strides and dtype: float32 [M, K/g] in any of row-major,
+    column-major, column-major padded; int32 [M, ceil(K/g/4)] (column-major, M padded to 4) when
+    scale_ue8m0.  `enable_v2` is accepted for signature compatibility: there is one kernel.
+    """
+    if fuse_silu_and_mul or masked_m is not None:
+        raise RuntimeError("sgl_per_token_group_quant_8bit: fuse_silu_and_mul / masked_m are not built on this path")
+    require_cuda(input, output_q, output_s)
+    if not input.is_contiguous():
+        raise RuntimeError("input must be contiguous")
+    if not output_q.is_contiguous():
+        raise RuntimeError("output_q must be contiguous")
+    if output_q.dtype != FP8_DTYPE:
+        raise RuntimeError("output_q must be float8_e4m3fn (int8 destination is not built on this path)")
+    if input.numel() % group_size != 0:
+        raise RuntimeError("input.numel() %% group_size != 0 (%d, %d)" % (input.numel(), group_size))
+    if output_s.dim() != 2:
+        raise RuntimeError("output_s.dim() must be 2")
+    K = input.shape[-1]
+    if K % group_size != 0:
+        raise RuntimeError("the last dimension of `x` cannot be divisible by `group_size`")
+    M = input.numel() // K if K else 0
+    G = K // group_size
+    if output_q.numel() != input.numel():
+        raise RuntimeError("output_q has the wrong number of elements")
+    if scale_ue8m0:
+        if output_s.dtype != torch.int32:
+            raise RuntimeError("scale_ue8m0 needs an int32 packed output_s")
+        if output_s.shape[0] != M or output_s.shape[1] != (G + 3) // 4:
+            raise RuntimeError("packed output_s must be [M, ceil(K/group/4)]")
+        kind = _lib.SCALE_UE8M0_PACKED
+    else:
+        if output_s.dtype != torch.float32:
+            raise RuntimeError("output_s must be float32")
+        if output_s.shape[0] != M or output_s.shape[1] != G:
+            raise RuntimeError("output_s must be [M, K/group_size]")
+        kind = _lib.SCALE_F32
+    check(
+        lib.fp8k_group_quant(
+            input.data_ptr(), output_q.data_ptr(), output_s.data_ptr(), M, K, group_size, float(eps), float(fp8_min),
+            float(fp8_max), dtype_code(input.dtype), output_s.stride(0), output_s.stride(1), kind,
+            stream_ptr(input.device),
+        )
+    )
+
+
+# legacy alias, as in the reference (gemm.py:139-141)
+sgl_per_token_group_quant_fp8 = sgl_per_token_group_quant_8bit
+
+
+def sgl_per_token_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:155-160; csrc/gemm/per_token_quant_fp8.cu:166-236."""
+    require_cuda(input, output_q, output_s)
+    if not (input.is_contiguous() and output_q.is_contiguous() and output_s.is_contiguous()):
+        raise RuntimeError("input, output_q and output_s must be contiguous")
+    if input.dim() != 2:
+        raise RuntimeError("input must be 2-D [num_tokens, hidden_dim]")
+    if output_q.dtype != FP8_DTYPE or output_s.dtype != torch.float32:
+        raise RuntimeError("output_q must be float8_e4m3fn and output_s float32")
+    M, K = input.shape
+    if K % 8 != 0:
+        raise RuntimeError("Hidden dimension must be divisible by 8, but got %d" % K)
+    if output_s.numel() != M or output_q.shape != input.shape:
+        raise RuntimeError("output shapes do not match the input")
+    check(lib.fp8k_token_quant(input.data_ptr(), output_q.data_ptr(), output_s.data_ptr(), M, K, dtype_code(input.dtype),
+                               stream_ptr(input.device)))
+
+
+def sgl_per_tensor_quant_fp8(input: torch.Tensor, output_q: torch.Tensor, output_s: torch.Tensor, is_static: bool) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:144-152; csrc/gemm/per_tensor_quant_fp8.cu:96-118.
+    Dynamic mode accumulates with an atomic max, so output_s must be zero on entry (as the caller does)."""
+    require_cuda(input, output_q, output_s)
+    if not (input.is_contiguous() and output_q.is_contiguous() and output_s.is_contiguous()):
+        raise RuntimeError("input, output_q and output_s must be contiguous")
+    if output_q.dtype != FP8_DTYPE or output_s.dtype != torch.float32 or output_s.numel() != 1:
+        raise RuntimeError("output_q must be float8_e4m3fn and output_s a float32 scalar")
+    check(lib.fp8k_tensor_quant(input.data_ptr(), output_q.data_ptr(), output_s.data_ptr(), input.numel(),
+                                dtype_code(input.dtype), 1 if is_static else 0, stream_ptr(input.device)))
+
+
+# --------------------------------------------------------------------------------------------
+# GEMMs
+# --------------------------------------------------------------------------------------------
+
+
+def _out_code(out_dtype: torch.dtype) -> int:
+    if out_dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("out_dtype must be Half or BFloat16")
+    return dtype_code(out_dtype)
+
+
+def _check_ab(mat_a: torch.Tensor, mat_b: torch.Tensor) -> None:
+    require_cuda(mat_a, mat_b)
+    if mat_a.dim() != 2:
+        raise RuntimeError("mat_a must be a 2D tensor")
+    if mat_b.dim() != 2:
+        raise RuntimeError("mat_b must be a 2D tensor")
+    if mat_a.shape[1] > 1 and mat_a.stride(1) != 1:
+        raise RuntimeError("mat_a must be a row major tensor")
+    if mat_b.shape[0] > 1 and mat_b.stride(0) != 1:
+        raise RuntimeError("mat_b must be a column major tensor")
+    if mat_a.shape[1] != mat_b.shape[0]:
+        raise RuntimeError("mat_a and mat_b shapes cannot be multiplied")
+    if mat_a.shape[1] % 16 != 0:
+        raise RuntimeError("mat_a must be multiple of 16 bytes for memory alignment")
+    if mat_a.dtype != FP8_DTYPE:
+        raise RuntimeError("mat_a must be Float8_e4m3fn")
+    if mat_b.dtype != FP8_DTYPE:
+        raise RuntimeError("mat_b must be Float8_e4m3fn")
+
+
+def fp8_blockwise_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype):
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:25-32; checks fp8_blockwise_gemm_kernel.cu:368-406.
+
+    mat_a e4m3fn [M,K] row-major; mat_b e4m3fn [K,N] column-major (a [N,K] weight transposed);
+    scales_a float32 [M, K/128] (M-major or contiguous vector); scales_b float32 [K/128, N/128]
+    (K-major or contiguous vector).  Both scale tensors are addressed by stride, so other
+    memory orders work too.  Returns [M,N] of out_dtype.
+    """
+    _check_ab(mat_a, mat_b)
+    require_cuda(scales_a, scales_b)
+    out_code = _out_code(out_dtype)
+    M, K = mat_a.shape
+    N = mat_b.shape[1]
+    if K % 128 != 0 or N % 128 != 0:
+        raise RuntimeError("fp8_blockwise_scaled_mm needs N and K to be multiples of 128")
+    if scales_a.dim() != 2 or scales_a.shape[0] != M or scales_a.shape[1] != K // 128:
+        raise RuntimeError("size of scales_a is not matched")
+    if scales_b.dim() != 2 or scales_b.shape[0] != K // 128 or scales_b.shape[1] != N // 128:
+        raise RuntimeError("size of scales_b is not matched")
+    if scales_a.dtype != torch.float32:
+        raise RuntimeError("scales_a must be Float32")
+    if scales_b.dtype != torch.float32:
+        raise RuntimeError("scales_b must be Float32")
+    if (N * 2) % 16 != 0:
+        raise RuntimeError("out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((M, N), dtype=out_dtype, device=mat_a.device)
+    if M == 0:
+        return out
+    ws_bytes = lib.fp8k_block_gemm_workspace_bytes(M, N, K)
+    ws = _workspace(mat_a.device, ws_bytes)
+    check(
+        lib.fp8k_block_gemm(
+            mat_a.data_ptr(), mat_b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(), out.data_ptr(), M, N, K,
+            mat_a.stride(0) if M > 1 else K, mat_b.stride(1) if N > 1 else K,
+            scales_a.stride(0), scales_a.stride(1), scales_b.stride(1), scales_b.stride(0), out.stride(0), out_code,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, stream_ptr(mat_a.device),
+        )
+    )
+    return out
+
+
+def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:35-43; checks fp8_gemm_kernel.cu:1450-1487.
+
+    C = (mat_a @ mat_b) * scales_a[m] * scales_b[n] (+ bias[n]).  bias may be out_dtype (the
+    device op's rule) or float32 (the CPU twin's rule, csrc/cpu/gemm_fp8.cpp:523); it is added in
+    float32 before the output cast.
+    """
+    _check_ab(mat_a, mat_b)
+    require_cuda(scales_a, scales_b, bias)
+    out_code = _out_code(out_dtype)
+    M, K = mat_a.shape
+    N = mat_b.shape[1]
+    if scales_a.numel() != M:
+        raise RuntimeError("size of scales_a is not matched")
+    if scales_b.numel() != N:
+        raise RuntimeError("size of scales_b is not matched")
+    if not scales_a.is_contiguous():
+        raise RuntimeError("scales_a must be contiguous")
+    if not scales_b.is_contiguous():
+        raise RuntimeError("scales_b msut be contiguous")
+    if scales_a.dtype != torch.float32:
+        raise RuntimeError("scales_a must be Float32")
+    if scales_b.dtype != torch.float32:
+        raise RuntimeError("scales_b must be Float32")
+    bias_code = _lib.F32
+    if bias is not None:
+        if bias.numel() != N:
+            raise RuntimeError("size of bias is not matched")
+        if not bias.is_contiguous():
+            raise RuntimeError("bias must be contiguous")
+        if bias.dtype != out_dtype and bias.dtype != torch.float32:
+            raise RuntimeError("bias dtype must match output dtype")
+        bias_code = dtype_code(bias.dtype)
+    if (N * 2) % 16 != 0:
+        raise RuntimeError("out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((M, N), dtype=out_dtype, device=mat_a.device)
+    if M == 0:
+        return out
+    ws_bytes = lib.fp8k_scaled_mm_workspace_bytes(M, N, K)
+    ws = _workspace(mat_a.device, ws_bytes)
+    check(
+        lib.fp8k_scaled_mm(
+            mat_a.data_ptr(), mat_b.data_ptr(), scales_a.data_ptr(), scales_b.data_ptr(),
+            bias.data_ptr() if bias is not None else None, out.data_ptr(), M, N, K,
+            mat_a.stride(0) if M > 1 else K, mat_b.stride(1) if N > 1 else K, out.stride(0), out_code, bias_code,
+            ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, stream_ptr(mat_a.device),
+        )
+    )
+    return out
+
+
+def _block_gemm_nk(A, B, As, Bs, out_dtype):
+    """Block GEMM on the Triton-side layout: B [N,K] row-major, Bs [ceil(N/128), ceil(K/128)].
+
+    Used by w8a8_block_fp8_matmul; unlike fp8_blockwise_scaled_mm it admits N, K that are not
+    multiples of 128 (python/sglang/srt/layers/quantization/fp8_kernel.py:1072-1149 uses cdiv + masks).
+    """
+    require_cuda(A, B, As, Bs)
+    if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
+        raise RuntimeError("A and B must be Float8_e4m3fn")
+    out_code = _out_code(out_dtype)
+    M, K = A.shape
+    N = B.shape[0]
+    if K % 16 != 0:
+        raise RuntimeError("mat_a must be multiple of 16 bytes for memory alignment")
+    if (N * 2) % 16 != 0:
+        raise RuntimeError("out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((M, N), dtype=out_dtype, device=A.device)
+    if M == 0:
+        return out
+    ws_bytes = lib.fp8k_block_gemm_workspace_bytes(M, N, K)
+    ws = _workspace(A.device, ws_bytes)
+    check(
+        lib.fp8k_block_gemm(
+            A.data_ptr(), B.data_ptr(), As.data_ptr(), Bs.data_ptr(), out.data_ptr(), M, N, K,
+            A.stride(0) if M > 1 else K, B.stride(0) if N > 1 else K, As.stride(0), As.stride(1), Bs.stride(0),
+            Bs.stride(1), out.stride(0), out_code, ws.data_ptr() if ws is not None else None,
+            ws.numel() if ws is not None else 0, stream_ptr(A.device),
+        )
+    )
+    return out

@@ -1,0 +1,201 @@
+"""GPU parity of the FP8 GEMMs against the CPU oracle.
+
+Tolerance (stated by the task): max relative error <= 1e-2 on bf16 output with fp32 accumulation,
+measured as max|C - C_ref| / max|C_ref| against the float64 oracle; integer-valued inputs with
+power-of-two scales must be reproduced exactly.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from tests.conftest import fp8_tensor
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _quantised_problem(M, N, K, seed):
+    x = O.make_activation(M, K, seed)
+    w = O.make_weight(N, K, seed)
+    xq, xs = O.per_token_group_quant_fp8(x, 128)
+    wq, ws = O.block_quant_weight(w)
+    return xq, xs, wq, ws
+
+
+def _rel_err(c, ref):
+    return float(np.abs(c.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def _run_block(xq, xs, wq, ws, dev, out_dtype=torch.bfloat16, col_major_as=False, api="triton"):
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm
+
+    A = fp8_tensor(xq, dev)
+    B = fp8_tensor(wq, dev)
+    As = torch.from_numpy(xs).to(dev)
+    Bs = torch.from_numpy(ws).to(dev)
+    if col_major_as:
+        As = As.t().contiguous().t()
+    if api == "triton":
+        C = w8a8_block_fp8_matmul(A, B, As, Bs, [128, 128], out_dtype)
+    else:
+        C = fp8_blockwise_scaled_mm(A, B.t(), As.t().contiguous().t(), Bs.t(), out_dtype)
+    torch.cuda.synchronize()
+    return C.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [1, 5, 32, 127, 128, 256, 300, 1024])
+@pytest.mark.parametrize("N,K", [(512, 512), (4608, 1024), (1536, 2304)])
+def test_block_gemm_vs_oracle(dev, M, N, K):
+    xq, xs, wq, ws = _quantised_problem(M, N, K, seed=M + N)
+    ref = O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="f32", acc=np.float64)
+    for api in ("triton", "sgl"):
+        c = _run_block(xq, xs, wq, ws, dev, api=api)
+        assert _rel_err(c, ref) <= REL_TOL, (api, _rel_err(c, ref))
+
+
+def test_block_gemm_config1(dev):
+    """BASELINE config 1: x [32,4096] with outliers, W [4096,4096], seed 0, through the linear entry point."""
+    from sglang_amd.fp8_utils import dispatch_w8a8_block_fp8_linear
+    from tests.conftest import bf16_tensor
+
+    x = O.make_activation(32, 4096, 0)
+    w = O.make_weight(4096, 4096, 0)
+    wq, ws = O.block_quant_weight(w)
+    ref = O.block_fp8_linear(x, wq, ws)
+    fn = dispatch_w8a8_block_fp8_linear()
+    out = fn(bf16_tensor(x, dev), fp8_tensor(wq, dev), [128, 128], torch.from_numpy(ws).to(dev))
+    torch.cuda.synchronize()
+    assert out.dtype == torch.bfloat16 and out.shape == (32, 4096)
+    assert _rel_err(out.float().cpu().numpy(), ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("M", [16, 1024])
+@pytest.mark.parametrize("N,K", [(24576, 1536), (32768, 512), (7168, 16384), (4608, 7168), (7168, 2304)])
+def test_block_gemm_deepseek_shapes(dev, M, N, K):
+    """DeepSeek-V3 projection shapes; checked on a sample of output rows/columns against the oracle."""
+    rng = np.random.default_rng(N + K + M)
+    xq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((M, K)).astype(np.float32) * 100, -448, 448))
+    wq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((N, K)).astype(np.float32) * 100, -448, 448))
+    xs = rng.uniform(0.5, 2.0, (M, K // 128)).astype(np.float32) * 1e-2
+    ws = rng.uniform(0.5, 2.0, (N // 128, K // 128)).astype(np.float32) * 1e-3
+    c = _run_block(xq, xs, wq, ws, dev)
+    rows = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 6)]))
+    cols = np.unique(np.concatenate([np.arange(0, 130), np.arange(N - 130, N), rng.integers(0, N, 300)]))
+    ws_cols = ws[cols // 128]
+    a = O.e4m3fn_to_f32(xq[rows]).astype(np.float64)
+    b = O.e4m3fn_to_f32(wq[cols]).astype(np.float64)
+    ref = np.zeros((rows.size, cols.size))
+    for kb in range(K // 128):
+        sl = slice(kb * 128, (kb + 1) * 128)
+        ref += (a[:, sl] @ b[:, sl].T) * xs[rows, kb][:, None] * ws_cols[:, kb][None, :]
+    got = c[np.ix_(rows, cols)]
+    assert _rel_err(got, ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("M,N,K", [(64, 256, 256), (256, 512, 1024), (1024, 256, 4096), (3, 384, 128)])
+def test_block_gemm_exact_on_integers(dev, M, N, K):
+    """Small integers and power-of-two scales: every partial sum is exactly representable."""
+    rng = np.random.default_rng(K)
+    xv = rng.integers(-4, 5, (M, K)).astype(np.float32)
+    wv = rng.integers(-4, 5, (N, K)).astype(np.float32)
+    xq, wq = O.f32_to_e4m3fn(xv), O.f32_to_e4m3fn(wv)
+    xs = (2.0 ** rng.integers(-3, 3, (M, K // 128))).astype(np.float32)
+    ws = (2.0 ** rng.integers(-3, 3, (N // 128, K // 128))).astype(np.float32)
+    ref = O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="bf16", acc=np.float64)
+    c = _run_block(xq, xs, wq, ws, dev)
+    np.testing.assert_array_equal(c, ref)
+    c16 = _run_block(xq, xs, wq, ws, dev, out_dtype=torch.float16)
+    np.testing.assert_array_equal(c16, O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="f16", acc=np.float64))
+
+
+def test_block_gemm_scale_layouts_agree(dev):
+    xq, xs, wq, ws = _quantised_problem(200, 512, 1024, 9)
+    a = _run_block(xq, xs, wq, ws, dev, col_major_as=False)
+    b = _run_block(xq, xs, wq, ws, dev, col_major_as=True)
+    c = _run_block(xq, xs, wq, ws, dev, api="sgl")
+    np.testing.assert_array_equal(a, b)
+    np.testing.assert_array_equal(a, c)
+
+
+@pytest.mark.parametrize("N,K", [(1088, 512), (136, 272), (512, 144)])
+def test_block_gemm_unaligned_shapes(dev, N, K):
+    """N or K not multiples of 128 (the reference's Triton path admits them)."""
+    M = 37
+    rng = np.random.default_rng(N)
+    xq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((M, K)).astype(np.float32) * 50, -448, 448))
+    wq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((N, K)).astype(np.float32) * 50, -448, 448))
+    kt, nt = (K + 127) // 128, (N + 127) // 128
+    xs = rng.uniform(0.5, 2, (M, kt)).astype(np.float32)
+    ws = rng.uniform(0.5, 2, (nt, kt)).astype(np.float32)
+    ref = O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="f32", acc=np.float64)
+    c = _run_block(xq, xs, wq, ws, dev)
+    assert _rel_err(c, ref) <= REL_TOL
+
+
+def _run_scaled_mm(aq, bq, sa, sb, dev, out_dtype=torch.bfloat16, bias=None):
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    A = fp8_tensor(aq, dev)
+    B = fp8_tensor(bq, dev).t()
+    C = fp8_scaled_mm(A, B, torch.from_numpy(sa).to(dev), torch.from_numpy(sb).to(dev), out_dtype,
+                      None if bias is None else bias.to(dev))
+    torch.cuda.synchronize()
+    return C.float().cpu().numpy()
+
+
+@pytest.mark.parametrize("M", [1, 8, 64, 512, 2048])
+@pytest.mark.parametrize("N,K", [(6144, 4096), (4096, 14336)])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_scaled_mm_llama_shapes(dev, M, N, K, with_bias):
+    if M == 2048 and K == 14336 and with_bias:
+        pytest.skip("covered without bias; keeps the CPU oracle time down")
+    rng = np.random.default_rng(M + N)
+    x = O.make_activation(M, K, M)
+    aq, sa = O.per_token_quant_fp8(x)
+    w = O.make_weight(N, K, N)
+    bq, sbt = O.per_tensor_quant_fp8(w)
+    sb = np.full((N,), sbt[0], dtype=np.float32)
+    bias = torch.from_numpy(O.to_bf16(rng.standard_normal(N).astype(np.float32))).to(torch.bfloat16) if with_bias else None
+    ref = O.fp8_scaled_mm(aq, bq, sa.reshape(-1), sb, "f32", None if bias is None else bias.float().numpy())
+    c = _run_scaled_mm(aq, bq, sa, sb, dev, bias=bias)
+    assert _rel_err(c, ref) <= REL_TOL
+    if with_bias:
+        c32 = _run_scaled_mm(aq, bq, sa, sb, dev, bias=bias.float())
+        np.testing.assert_array_equal(c, c32)
+
+
+def test_scaled_mm_exact_and_fp16(dev):
+    rng = np.random.default_rng(1)
+    M, N, K = 130, 512, 1024
+    aq = O.f32_to_e4m3fn(rng.integers(-3, 4, (M, K)).astype(np.float32))
+    bq = O.f32_to_e4m3fn(rng.integers(-3, 4, (N, K)).astype(np.float32))
+    sa = (2.0 ** rng.integers(-2, 3, M)).astype(np.float32)
+    sb = (2.0 ** rng.integers(-2, 3, N)).astype(np.float32)
+    for dt, name in ((torch.bfloat16, "bf16"), (torch.float16, "f16")):
+        c = _run_scaled_mm(aq, bq, sa, sb, dev, out_dtype=dt)
+        np.testing.assert_array_equal(c, O.fp8_scaled_mm(aq, bq, sa, sb, name))
+
+
+def test_gemm_errors(dev):
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_mm, fp8_scaled_mm
+
+    a = torch.zeros((4, 256), dtype=torch.float8_e4m3fn, device=dev)
+    b = torch.zeros((256, 256), dtype=torch.float8_e4m3fn, device=dev)
+    sa = torch.ones((4, 2), device=dev).t().contiguous().t()
+    sb = torch.ones((2, 2), device=dev)
+    with pytest.raises(RuntimeError, match="column major"):
+        fp8_blockwise_scaled_mm(a, b, sa, sb, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Half or BFloat16"):
+        fp8_blockwise_scaled_mm(a, b.t(), sa, sb, torch.float32)
+    with pytest.raises(RuntimeError, match="scales_a"):
+        fp8_blockwise_scaled_mm(a, b.t(), sa[:, :1], sb, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="Float8_e4m3fn"):
+        fp8_blockwise_scaled_mm(a.view(torch.uint8), b.t(), sa, sb, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="bias"):
+        fp8_scaled_mm(a, b.t(), torch.ones(4, device=dev), torch.ones(256, device=dev), torch.bfloat16,
+                      torch.ones(255, device=dev))
+    out = fp8_blockwise_scaled_mm(a[:0], b.t(), sa[:0], sb, torch.bfloat16)
+    assert out.shape == (0, 256)

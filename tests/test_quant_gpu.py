@@ -1,0 +1,203 @@
+"""GPU parity of the quantisation kernels against the CPU oracle: bytes and scales bit-exact."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from tests.conftest import bf16_tensor, u8
+
+pytestmark = pytest.mark.gpu
+
+
+def _layouts():
+    # (column_major, tma_aligned, ue8m0)
+    return [(False, False, False), (True, False, False), (True, True, False), (True, True, True)]
+
+
+def _run_group_quant(x_np, dev, group, layout, dtype=torch.bfloat16, eps=1e-10):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    cm, al, ue = layout
+    x = torch.from_numpy(x_np).to(dtype).to(dev)
+    q, s = sglang_per_token_group_quant_fp8(x, group, eps=eps, column_major_scales=cm, scale_tma_aligned=al, scale_ue8m0=ue)
+    torch.cuda.synchronize()
+    return q, s
+
+
+def _check(x_np, dev, group, layout, in_dtype="bf16", dtype=torch.bfloat16, eps=1e-10):
+    cm, al, ue = layout
+    q, s = _run_group_quant(x_np, dev, group, layout, dtype, eps)
+    q_ref, s_ref = O.per_token_group_quant_fp8(x_np, group, eps=eps, in_dtype=in_dtype, scale_ue8m0=ue)
+    M, K = x_np.shape
+    assert q.shape == (M, K) and q.dtype == torch.float8_e4m3fn
+    np.testing.assert_array_equal(u8(q), q_ref)
+    G = K // group
+    if ue:
+        assert s.dtype == torch.int32 and s.shape == (M, (G + 3) // 4)
+        assert s.stride(0) == 1 and s.stride(1) == (M + 3) // 4 * 4
+        np.testing.assert_array_equal(s.cpu().numpy(), O.pack_ue8m0_scales(s_ref))
+    else:
+        assert s.dtype == torch.float32 and s.shape == (M, G)
+        if cm:
+            assert s.stride(0) == 1 and s.stride(1) == ((M + 3) // 4 * 4 if al else M)
+        else:
+            assert s.is_contiguous()
+        np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("layout", _layouts())
+@pytest.mark.parametrize("M", [1, 3, 31, 32, 33, 64, 257, 512])
+def test_group_quant_config_shapes_small(dev, M, layout):
+    x = O.make_activation(M, 7168, seed=M)
+    _check(x, dev, 128, layout)
+
+
+@pytest.mark.parametrize("layout", _layouts())
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4])
+def test_group_quant_sweep_4096(dev, seed, layout):
+    x = O.make_activation(4096, 7168, seed=seed)
+    _check(x, dev, 128, layout)
+
+
+def test_group_quant_16384_row_major(dev):
+    x = O.make_activation(16384, 7168, seed=0)
+    _check(x, dev, 128, (False, False, False))
+
+
+@pytest.mark.parametrize("group", [16, 32, 64, 128, 256, 512])
+@pytest.mark.parametrize("K", [512, 1536, 4096])
+def test_group_sizes(dev, group, K):
+    x = O.make_activation(83, K, seed=group + K)
+    _check(x, dev, group, (False, False, False))
+    _check(x, dev, group, (True, False, False))
+
+
+@pytest.mark.parametrize("K", [128, 256, 384, 640, 2304])
+def test_ragged_group_counts(dev, K):
+    # K/128 not a multiple of 4: the last wave strip is partly empty, packed words have zero bytes
+    x = O.make_activation(45, K, seed=K)
+    for layout in _layouts():
+        _check(x, dev, 128, layout)
+
+
+def test_every_bf16_amax(dev):
+    """Scale table over every positive finite bf16 amax (32 639 values) and the eps floor."""
+    bits = np.arange(1, 0x7F80, dtype=np.uint32)
+    amax = (bits << 16).view(np.float32)
+    M = amax.size
+    rng = np.random.default_rng(5)
+    x = (rng.uniform(-1, 1, (M, 128)).astype(np.float32) * amax[:, None]).astype(np.float32)
+    x = O.to_bf16(x)
+    x[:, 7] = amax  # the group amax is exactly the table value
+    x = np.clip(x, -amax[:, None], amax[:, None])
+    for layout in _layouts():
+        _check(x, dev, 128, layout)
+
+
+def test_zero_groups_and_closed_form(dev):
+    # all-zero groups: q = 0, scale = bf16(eps)/448; amax = 448 -> scale 1, bytes = encode(x)
+    x = np.zeros((8, 256), dtype=np.float32)
+    x[1, :128] = O.to_bf16(np.linspace(-448, 448, 128).astype(np.float32))
+    x[1, 0] = 448.0
+    x[2, 128:] = -0.0
+    q, s = _run_group_quant(x, dev, 128, (False, False, False))
+    s = s.cpu().numpy()
+    assert s[1, 0] == 1.0
+    np.testing.assert_array_equal(u8(q)[1, :128], O.f32_to_e4m3fn(x[1, :128]))
+    assert s[0, 0] == np.float32(O.clamp_eps(1e-10, "bf16")) / np.float32(448)
+    assert (u8(q)[0] == 0).all() and (u8(q)[2, 128:] == 0x80).all()
+    for layout in _layouts():
+        _check(x, dev, 128, layout)
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.float16, "f16"), (torch.float32, "f32")])
+def test_other_input_dtypes(dev, dtype, name):
+    rng = np.random.default_rng(11)
+    x = rng.standard_normal((130, 1024)).astype(np.float32) * 3
+    if name == "f16":
+        x = x.astype(np.float16).astype(np.float32)
+    x[5, :128] = 0
+    for layout in _layouts():
+        _check(x, dev, 128, layout, in_dtype=name, dtype=dtype)
+
+
+def test_every_f16_amax(dev):
+    bits = np.arange(1, 0x7C00, dtype=np.uint16)
+    amax = bits.view(np.float16).astype(np.float32)
+    x = np.zeros((amax.size, 128), dtype=np.float32)
+    x[:, 3] = -amax
+    x[:, 9] = (amax.astype(np.float16) * np.float16(0.37)).astype(np.float32)
+    _check(x, dev, 128, (False, False, False), in_dtype="f16", dtype=torch.float16)
+
+
+def test_quant_leaves_neighbours_untouched(dev):
+    """Poisoned output buffers: only the declared elements are written (padded column-major rows too)."""
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_8bit
+
+    M, K = 45, 640
+    x = bf16_tensor(O.make_activation(M, K, 3), dev)
+    qbuf = torch.full((M + 2, K), 0x55, dtype=torch.uint8, device=dev)
+    sbuf = torch.full((K // 128 + 2, 48), -7.0, dtype=torch.float32, device=dev)
+    q = qbuf[1 : M + 1].view(torch.float8_e4m3fn)
+    s = sbuf[1 : 1 + K // 128].t()[:M]
+    sgl_per_token_group_quant_8bit(x, q, s, 128, 1e-10, -448.0, 448.0)
+    torch.cuda.synchronize()
+    assert (qbuf[0] == 0x55).all() and (qbuf[-1] == 0x55).all()
+    assert (sbuf[0] == -7).all() and (sbuf[-1] == -7).all() and (sbuf[:, M:] == -7).all()
+    q_ref, s_ref = O.per_token_group_quant_fp8(x.float().cpu().numpy(), 128)
+    np.testing.assert_array_equal(u8(q), q_ref)
+    np.testing.assert_array_equal(s.cpu().numpy(), s_ref)
+
+
+def test_empty_and_errors(dev):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_8bit
+
+    q, s = sglang_per_token_group_quant_fp8(torch.empty((0, 256), dtype=torch.bfloat16, device=dev), 128)
+    assert q.shape == (0, 256) and s.shape == (0, 2)
+    x = torch.zeros((4, 256), dtype=torch.bfloat16, device=dev)
+    qo = torch.empty((4, 256), dtype=torch.float8_e4m3fn, device=dev)
+    with pytest.raises(RuntimeError):
+        sgl_per_token_group_quant_8bit(x, qo, torch.empty((4, 2), device=dev), 96, 1e-10, -448.0, 448.0)
+    with pytest.raises(RuntimeError):
+        sgl_per_token_group_quant_8bit(x, qo, torch.empty((8,), device=dev), 128, 1e-10, -448.0, 448.0)
+    with pytest.raises(RuntimeError):
+        sgl_per_token_group_quant_8bit(x, qo, torch.empty((4, 2), device=dev), 128, 1e-10, -224.0, 224.0)
+    with pytest.raises(RuntimeError):
+        sgl_per_token_group_quant_8bit(x.t(), qo, torch.empty((4, 2), device=dev), 128, 1e-10, -448.0, 448.0)
+    with pytest.raises(AssertionError):
+        sglang_per_token_group_quant_fp8(x, 100)
+
+
+@pytest.mark.parametrize("M,K", [(1, 4096), (7, 4096), (512, 14336), (2048, 4096), (33, 24576)])
+def test_per_token_quant(dev, M, K):
+    from sglang_amd.fp8_kernel import sglang_per_token_quant_fp8
+
+    x = O.make_activation(M, K, seed=M + K)
+    if M > 3:
+        x[3] = 0
+    q, s = sglang_per_token_quant_fp8(bf16_tensor(x, dev))
+    torch.cuda.synchronize()
+    q_ref, s_ref = O.per_token_quant_fp8(x)
+    assert s.shape == (M, 1)
+    np.testing.assert_array_equal(s.cpu().numpy(), s_ref)
+    np.testing.assert_array_equal(u8(q), q_ref)
+
+
+@pytest.mark.parametrize("numel", [8, 1000, 4096 * 7168 + 5])
+def test_per_tensor_quant(dev, numel):
+    from sglang_amd.fp8_kernel import scaled_fp8_quant
+
+    rng = np.random.default_rng(numel)
+    cols = 8 if numel % 8 == 0 else 1
+    x = O.to_bf16(rng.standard_normal(numel).astype(np.float32) * 4).reshape(-1, cols)
+    xt = bf16_tensor(x, dev)
+    q, s = scaled_fp8_quant(xt)
+    torch.cuda.synchronize()
+    q_ref, s_ref = O.per_tensor_quant_fp8(x)
+    np.testing.assert_array_equal(s.cpu().numpy(), s_ref)
+    np.testing.assert_array_equal(u8(q), q_ref)
+    st = torch.tensor([0.05], dtype=torch.float32, device=dev)
+    q2, s2 = scaled_fp8_quant(xt, st)
+    q2_ref, _ = O.per_tensor_quant_fp8(x, 0.05)
+    np.testing.assert_array_equal(u8(q2), q2_ref)
