@@ -83,16 +83,23 @@ constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
 constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8
 constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each 16
 
-// max over aligned groups of LANES consecutive lanes; every lane of the group gets the result
+// max of NON-NEGATIVE floats over aligned groups of LANES consecutive lanes; every lane of the group
+// gets the result.  Non-negative floats order like their bit patterns, so the exchange uses integer
+// max, which folds into one DPP instruction per step (no NaN canonicalisation in between).
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_umax(uint32_t v) {
+  return max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, CTRL, 0xf, 0xf, false));
+}
 template <int LANES>
-__device__ __forceinline__ float group_max(float v) {
-  if (LANES >= 2) v = fmaxf(v, dpp_f<kDppXor1>(v));
-  if (LANES >= 4) v = fmaxf(v, dpp_f<kDppXor2>(v));
-  if (LANES >= 8) v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
-  if (LANES >= 16) v = fmaxf(v, dpp_f<kDppMirror>(v));
-  if (LANES >= 32) v = fmaxf(v, __shfl_xor(v, 16));
-  if (LANES >= 64) v = fmaxf(v, __shfl_xor(v, 32));
-  return v;
+__device__ __forceinline__ float group_max(float f) {
+  uint32_t v = __float_as_uint(f);
+  if (LANES >= 2) v = dpp_umax<kDppXor1>(v);
+  if (LANES >= 4) v = dpp_umax<kDppXor2>(v);
+  if (LANES >= 8) v = dpp_umax<kDppHalfMirror>(v);
+  if (LANES >= 16) v = dpp_umax<kDppMirror>(v);
+  if (LANES >= 32) v = max(v, (uint32_t)__shfl_xor((int)v, 16));
+  if (LANES >= 64) v = max(v, (uint32_t)__shfl_xor((int)v, 32));
+  return __uint_as_float(v);
 }
 
 }  // namespace fp8k

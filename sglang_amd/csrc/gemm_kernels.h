@@ -30,12 +30,6 @@ struct GemmArgs {
 enum { kModeBlock = 0, kModeRow = 1 };
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
-typedef const __attribute__((address_space(1))) void* gbl_ptr_t;
-
-// 16 bytes per lane straight from global memory into LDS at lds_base + lane*16 (lds_base wave-uniform)
-__device__ __forceinline__ void load16_to_lds(const uint8_t* g, uint8_t* lds_base) {
-  __builtin_amdgcn_global_load_lds((gbl_ptr_t)g, (lds_ptr_t)lds_base, 16, 0, 0);
-}
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
 
 __device__ __forceinline__ v16f mfma_32x32x64(v8i a, v8i b, v16f c) {
@@ -68,18 +62,39 @@ __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
 // 128(n) x 64(m) = 4 x 2 MFMA tiles of 32x32, K step 128 = two v_mfma_f32_32x32x64_f8f6f4.
 //
 // LDS: two stages of [W 256 rows x 128 B | X 256 rows x 128 B] = 2 x 64 KB, filled by
-// global_load_lds_dwordx4 (no register staging).  A 1 KB wave-load covers 8 rows; the 16-byte
-// chunk c of row r is stored at chunk position c ^ ((r >> 1) & 7), which makes both the linear
-// LDS-DMA writes and the ds_read_b128 operand fetches (32 rows, same logical chunk) bank-conflict
-// free.  One barrier per K step: loads for step kb+1 are issued right after the barrier that
-// publishes step kb, and run under its 16 MFMAs per wave.
+// buffer_load_dwordx4 ... lds (no register staging; rows past the matrix edge are out of the
+// descriptor's range and arrive as zeros).  A 1 KB wave-load covers 8 rows; the 16-byte chunk c of
+// row r is stored at chunk position c ^ ((r >> 1) & 7), which makes both the linear LDS-DMA writes
+// and the ds_read_b128 operand fetches (32 rows, same logical chunk) bank-conflict free.
 //
-// Block mode keeps a second, short-lived accumulator: t = W.X over one K block, then
-// acc += t * (as[m,kb] * bs[nb,kb]); row mode accumulates in place and scales in the epilogue.
+// Pipeline.  One loop iteration is one barrier interval, and the barrier sits BEFORE the last
+// quarter of a K block: by then a wave has every operand of the block in registers, so after the
+// barrier (a) the stage it just left can be refilled with block it+2 at once and (b) the first
+// operands of block it+1 are fetched while the last four MFMAs of block it still run.  Operand
+// fetches are issued two MFMA groups ahead of their use; the eight 1 KB global loads of a wave are
+// spread over the first half of the interval, two per group, because the texture-address path
+// moves 64 B/clk per CU and a burst would stall the issuing wave.  The loop body is branch-free
+// (loads past the last K block are out of range or unread), which keeps the compiler from sinking
+// the scale FMAs to the loop latch.
+//
+// Block mode keeps two short-lived accumulators: t = W.X over one K block, then
+// acc += t * (as[m,kb] * bs[nb,kb]), with the 16 FMAs of group g-1 split around the two MFMAs of
+// group g; row mode accumulates in place and scales in the epilogue.
 // ------------------------------------------------------------------------------------------------
 constexpr int kTileN = 256, kTileM = 256, kTileK = 128;
 constexpr int kStageBytes = (kTileN + kTileM) * kTileK;  // 64 KB
 constexpr int kXOff = kTileN * kTileK;                   // X tile offset inside a stage
+
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// raw buffer descriptor: base pointer + byte range; loads past the range return zero
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc((void*)p, 0, (int)bytes, 0x00020000);
+}
+// 16 bytes per lane from buffer + voff (per lane) + soff (uniform) straight into LDS at lds_base + lane*16
+__device__ __forceinline__ void buf_load16_to_lds(rsrc_t r, uint32_t voff, uint32_t soff, uint8_t* lds_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)lds_base, 16, (int)voff, (int)soff, 0, 0);
+}
+__device__ __forceinline__ void wait_vm0_lgkm0() { __builtin_amdgcn_s_waitcnt(0x0070); }  // vmcnt(0) lgkmcnt(0)
 
 template <int MODE, int OUT_DT, int BIAS_DT, bool SPLIT>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
@@ -89,15 +104,11 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int wn = w & 1, wm = w >> 1;
 
-  // ---- tile coordinates: contiguous chunk of tiles per XCD, groups of 4 m-tiles inside
   const int ntiles = p.tiles_m * p.tiles_n;
   const int per_xcd = (ntiles + 7) >> 3;
   int bid = blockIdx.x;
   int split = 0;
-  if (SPLIT) {
-    split = bid % p.splits;
-    bid /= p.splits;
-  }
+  if (SPLIT) { split = bid % p.splits; bid /= p.splits; }
   const int t = (bid & 7) * per_xcd + (bid >> 3);
   if (t >= ntiles) return;
   constexpr int GM = 4;
@@ -111,29 +122,24 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 
   const int kb_begin = SPLIT ? split * p.kb_per_split : 0;
   const int kb_end = SPLIT ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
+  const int nkb = kb_end - kb_begin;
 
-  // ---- global -> LDS: this wave fills row groups i = 4w..4w+3 (8 rows each) of W and of X
+  // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the
+  // matrix edge are out of range and read as zero
+  const int rowsW = min(kTileN, p.N - n0), rowsX = min(kTileM, p.M - m0);
+  const int kbytes = p.K - kb_begin * kTileK;
+  const rsrc_t rW = make_rsrc(p.W + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
+  const rsrc_t rX = make_rsrc(p.X + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
   const int rl = lane >> 3, cp = lane & 7;
-  const uint8_t* gW[4];
-  const uint8_t* gX[4];
+  uint32_t voW[2], voX[2];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const int i = w * 4 + j;
-    const int row = i * 8 + rl;
-    const int c = cp ^ (((i & 1) << 2) + (rl >> 1));  // data chunk stored at chunk position cp
-    const int nrow = min(n0 + row, p.N - 1);        // rows past the edge re-read the last row; never stored
-    const int mrow = min(m0 + row, p.M - 1);
-    gW[j] = p.W + (int64_t)nrow * p.ldw + c * 16 + (int64_t)kb_begin * kTileK;
-    gX[j] = p.X + (int64_t)mrow * p.ldx + c * 16 + (int64_t)kb_begin * kTileK;
+  for (int par = 0; par < 2; ++par) {
+    const int c = cp ^ ((par << 2) + (rl >> 1));
+    voW[par] = (uint32_t)(rl * p.ldw + c * 16);
+    voX[par] = (uint32_t)(rl * p.ldx + c * 16);
   }
-  auto issue_loads = [&](int stage, int kstep) {
-    uint8_t* base = smem + stage * kStageBytes + w * 4096;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) load16_to_lds(gW[j] + (int64_t)kstep * kTileK, base + j * 1024);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) load16_to_lds(gX[j] + (int64_t)kstep * kTileK, base + kXOff + j * 1024);
-  };
-
+  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = (uint32_t)(w * 32 * p.ldx);
+  const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = (uint32_t)(8 * p.ldx);
   // ---- LDS -> MFMA operands
   const int lr = lane & 31, h = lane >> 5;
   const int swz = (lr >> 1) & 7;
@@ -156,10 +162,10 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   // ---- scales (block mode)
   const int mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
   const int mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
-  const float* sx0 = p.sx + (int64_t)mrow0 * p.sx_m;
-  const float* sx1 = p.sx + (int64_t)mrow1 * p.sx_m;
+  const float* sx0 = p.sx + (int64_t)mrow0 * p.sx_m + (int64_t)kb_begin * p.sx_k;
+  const float* sx1 = p.sx + (int64_t)mrow1 * p.sx_m + (int64_t)kb_begin * p.sx_k;
   const int nb = min(n0 + wn * 128, p.N - 1) >> 7;
-  const float* swp = p.sw + (int64_t)nb * p.sw_n;
+  const float* swp = p.sw + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
 
   v16f acc[4][2];
 #pragma unroll
@@ -169,60 +175,125 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
 
-  float sc_next[2] = {0.f, 0.f};
-  if (kb_begin < kb_end) {
-    issue_loads(0, 0);
+  v8i X[2][2], WA[2], WB[2];   // [.][ks]
+  v16f tq[2];
+  float sc[2] = {0.f, 0.f}, scn[2] = {0.f, 0.f};
+  float s0n = 0.f, s1n = 0.f, sbn = 0.f;
+  int cur_stage = 0, cur_kstep = 0;
+
+#define SB() __builtin_amdgcn_sched_barrier(0)
+  auto L = [&](int idx) {  // one 1 KB global->LDS load: idx 0..3 W slices, 4..7 X slices
+    uint8_t* base = smem + cur_stage * kStageBytes + w * 4096;
+    const uint32_t ko = (uint32_t)cur_kstep * kTileK;
+    const int j = idx & 3;
+    if (idx < 4) buf_load16_to_lds(rW, voW[j & 1], soW + j * stepW + ko, base + j * 1024);
+    else buf_load16_to_lds(rX, voX[j & 1], soX + j * stepX + ko, base + kXOff + j * 1024);
+  };
+  auto RW = [&](v8i(&dst)[2], const uint8_t* st, int ns) {
+    dst[0] = frag(st, rdW + ns * 32 * kTileK, 0);
+    dst[1] = frag(st, rdW + ns * 32 * kTileK, 1);
+  };
+  auto RX = [&](const uint8_t* st, int ms) {
+    X[ms][0] = frag(st, rdX + ms * 32 * kTileK, 0);
+    X[ms][1] = frag(st, rdX + ms * 32 * kTileK, 1);
+  };
+  // one group = the two K-halves of one 32x32 tile
+  auto G = [&](const v8i(&W)[2], int ms, v16f& a, v16f& tt) {
     if (MODE == kModeBlock) {
-      const float sb = swp[(int64_t)kb_begin * p.sw_k];
-      sc_next[0] = sx0[(int64_t)kb_begin * p.sx_k] * sb;
-      sc_next[1] = sx1[(int64_t)kb_begin * p.sx_k] * sb;
+      v16f z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      tt = mfma_32x32x64(W[0], X[ms][0], z);
+      tt = mfma_32x32x64(W[1], X[ms][1], tt);
+    } else {
+      a = mfma_32x32x64(W[0], X[ms][0], a);
+      a = mfma_32x32x64(W[1], X[ms][1], a);
     }
-  }
+  };
+  // group g's two MFMAs with the previous group's 16 scale-FMAs split around them
+  auto GF = [&](const v8i(&W)[2], int ms, v16f& a, v16f& tt, v16f& ap, const v16f& tp, float s) {
+    if (MODE == kModeBlock) {
+      v16f z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      tt = mfma_32x32x64(W[0], X[ms][0], z);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < 8; ++r) ap[r] = __builtin_fmaf(tp[r], s, ap[r]);
+      __builtin_amdgcn_sched_barrier(0);
+      tt = mfma_32x32x64(W[1], X[ms][1], tt);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 8; r < 16; ++r) ap[r] = __builtin_fmaf(tp[r], s, ap[r]);
+    } else {
+      a = mfma_32x32x64(W[0], X[ms][0], a);
+      a = mfma_32x32x64(W[1], X[ms][1], a);
+    }
+  };
+  auto F = [&](v16f& a, const v16f& tt, float s) {
+    if (MODE == kModeBlock) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) a[r] = __builtin_fmaf(tt[r], s, a[r]);
+    }
+  };
 
-  for (int kb = kb_begin; kb < kb_end; ++kb) {
-    const int it = kb - kb_begin;
+  if (nkb <= 0) return;
+  // ---- prologue: block 0 into stage 0, block 1 into stage 1, groups (0,0)..(2,1) of block 0
+  cur_stage = 0; cur_kstep = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) L(i);
+  if (MODE == kModeBlock) { sc[0] = sx0[0]; sc[1] = sx1[0]; const float sb = swp[0]; sc[0] *= sb; sc[1] *= sb; }
+  wait_vm0();
+  __syncthreads();
+  cur_stage = 1; cur_kstep = 1;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) L(i);
+  if (MODE == kModeBlock) { const int kn = min(1, nkb - 1); s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k]; }
+  RX(smem, 0); RX(smem, 1); RW(WA, smem, 0); RW(WB, smem, 1);
+  SB();
+  G(WA, 0, acc[0][0], tq[0]); SB();
+  GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();
+  RW(WA, smem, 2); SB();
+  GF(WB, 0, acc[1][0], tq[0], acc[0][1], tq[1], sc[1]); SB();
+  GF(WB, 1, acc[1][1], tq[1], acc[1][0], tq[0], sc[0]); SB();
+  RW(WB, smem, 3); SB();
+  GF(WA, 0, acc[2][0], tq[0], acc[1][1], tq[1], sc[1]); SB();
+  GF(WA, 1, acc[2][1], tq[1], acc[2][0], tq[0], sc[0]); SB();
+  // pending: F(acc[2][1], tq[1], sc[1])
+
+  for (int it = 0; it < nkb - 1; ++it) {
     const int stage = it & 1;
-    wait_vm0();
+    const uint8_t* stn = smem + (stage ^ 1) * kStageBytes;  // block it+1
+    wait_vm0_lgkm0();
     __syncthreads();
-    float sc[2] = {sc_next[0], sc_next[1]};
-    if (kb + 1 < kb_end) {
-      issue_loads(stage ^ 1, it + 1);
-      if (MODE == kModeBlock) {
-        const float sb = swp[(int64_t)(kb + 1) * p.sw_k];
-        sc_next[0] = sx0[(int64_t)(kb + 1) * p.sx_k] * sb;
-        sc_next[1] = sx1[(int64_t)(kb + 1) * p.sx_k] * sb;
-      }
+    SB();
+    cur_stage = stage; cur_kstep = it + 2;
+    RW(WA, stn, 0); SB();
+    GF(WB, 0, acc[3][0], tq[0], acc[2][1], tq[1], sc[1]); SB();
+    RX(stn, 0); L(0); L(1); SB();
+    GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]); SB();
+    RX(stn, 1); RW(WB, stn, 1); L(2); L(3); SB();
+    if (MODE == kModeBlock) { scn[0] = s0n * sbn; scn[1] = s1n * sbn; }
+    GF(WA, 0, acc[0][0], tq[0], acc[3][1], tq[1], sc[1]); SB();
+    if (MODE == kModeBlock) {
+      sc[0] = scn[0]; sc[1] = scn[1];
+      const int kn = min(it + 2, nkb - 1);
+      s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
     }
-    const uint8_t* st = smem + stage * kStageBytes;
-    v8i xf[2][2];
-#pragma unroll
-    for (int ms = 0; ms < 2; ++ms)
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) xf[ms][ks] = frag(st, rdX + ms * 32 * kTileK, ks);
-#pragma unroll
-    for (int ns = 0; ns < 4; ++ns) {
-      v8i wf[2];
-#pragma unroll
-      for (int ks = 0; ks < 2; ++ks) wf[ks] = frag(st, rdW + ns * 32 * kTileK, ks);
-#pragma unroll
-      for (int ms = 0; ms < 2; ++ms) {
-        if (MODE == kModeBlock) {
-          v16f z;
-#pragma unroll
-          for (int r = 0; r < 16; ++r) z[r] = 0.f;
-          v16f tq = mfma_32x32x64(wf[0], xf[ms][0], z);
-          tq = mfma_32x32x64(wf[1], xf[ms][1], tq);
-#pragma unroll
-          for (int r = 0; r < 16; ++r) acc[ns][ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ns][ms][r]);
-        } else {
-          acc[ns][ms] = mfma_32x32x64(wf[0], xf[ms][0], acc[ns][ms]);
-          acc[ns][ms] = mfma_32x32x64(wf[1], xf[ms][1], acc[ns][ms]);
-        }
-      }
-    }
+    L(4); L(5); SB();
+    GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();
+    RW(WA, stn, 2); L(6); L(7); SB();
+    GF(WB, 0, acc[1][0], tq[0], acc[0][1], tq[1], sc[1]); SB();
+    GF(WB, 1, acc[1][1], tq[1], acc[1][0], tq[0], sc[0]); SB();
+    RW(WB, stn, 3); SB();
+    GF(WA, 0, acc[2][0], tq[0], acc[1][1], tq[1], sc[1]); SB();
+    GF(WA, 1, acc[2][1], tq[1], acc[2][0], tq[0], sc[0]); SB();
   }
+  // ---- last block's tail
+  GF(WB, 0, acc[3][0], tq[0], acc[2][1], tq[1], sc[1]);
+  GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]);
+  F(acc[3][1], tq[1], sc[1]);
 
-  // ---- epilogue: lane holds C[m][n..n+3] for 4 n-runs per 32x32 tile
 #pragma unroll
   for (int ms = 0; ms < 2; ++ms) {
     const int m = m0 + wm * 64 + ms * 32 + lr;

@@ -101,102 +101,97 @@ __device__ __forceinline__ float div448(float a) {
 // ------------------------------------------------------------------------------------------------
 // per-token-group quant
 //
-// One wavefront owns a strip of 32 rows x (64*8 = 512) columns, i.e. 32 rows of GPW = 512/GROUP
-// groups.  Each lane holds 8 consecutive elements of a row (one 16-byte load for bf16/f16),
-// LPG = GROUP/8 adjacent lanes form a group.  Rows are walked top to bottom, UNROLL rows of loads
-// in flight.  Scales are kept in registers while the strip is walked (lane i of a group keeps the
-// rows r with r % LPG == i) and written once at the end, so a column-major scale tensor receives
-// LPG consecutive floats per store instead of one 4-byte write per cache line.
+// The input is walked as a flat sequence of 1 KB "segments" (64 lanes x 8 elements = 512 columns of
+// one row, i.e. GPW = 512/GROUP groups; LPG = GROUP/8 adjacent lanes form a group).  A wavefront
+// owns SEG consecutive segments - contiguous memory whenever K is a multiple of 512 - loads them
+// all with 16-byte nontemporal loads before touching the first, and writes each back as one 8-byte
+// store per lane.  Both streams are used once, so they bypass cache retention.
 // ------------------------------------------------------------------------------------------------
-constexpr int kStripRows = 32;
+__device__ __forceinline__ uint4 load16_stream(const void* p) {
+  const v4i v = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
+  return make_uint4((uint32_t)v[0], (uint32_t)v[1], (uint32_t)v[2], (uint32_t)v[3]);
+}
+__device__ __forceinline__ void store8_stream(void* p, uint2 o) {
+  v2i v;
+  v[0] = (int)o.x;
+  v[1] = (int)o.y;
+  __builtin_nontemporal_store(v, reinterpret_cast<v2i*>(p));
+}
 
-template <int DT, int GROUP, int KIND>
+template <int DT>
+__device__ __forceinline__ void load_stream(Raw8<DT>& r, const void* base, int64_t elem) {
+  if constexpr (DT == FP8K_F32) {
+    const float* p = (const float*)base + elem;
+    const uint4 a = load16_stream(p), b = load16_stream(p + 4);
+    r.lo = make_float4(__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z), __uint_as_float(a.w));
+    r.hi = make_float4(__uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w));
+  } else {
+    r.v = load16_stream((const u16*)base + elem);
+  }
+}
+
+template <int DT, int GROUP, int KIND, int SEG>
 __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
                                                           void* __restrict__ s, int M, int G, int64_t K,
-                                                          int nquads, float eps, int64_t sm, int64_t sg) {
+                                                          int nseg_row, float eps, int64_t sm, int64_t sg) {
   constexpr int LPG = GROUP / 8;
   constexpr int GPW = 64 / LPG;
-  constexpr int NK = (kStripRows + LPG - 1) / LPG;
-  constexpr int UNROLL = 4;
   static_assert(KIND == FP8K_SCALE_F32 || GROUP == 128, "packed UE8M0 scales need 128-element groups");
 
   const int lane = threadIdx.x & 63;
-  // wave-uniform task coordinates (kept in scalar registers)
-  const int wave = __builtin_amdgcn_readfirstlane((int)(blockIdx.x * 4 + (threadIdx.x >> 6)));
-  const int rt = wave / nquads;
-  const int qd = wave - rt * nquads;
-  const int r0 = rt * kStripRows;
-  if (r0 >= M) return;
-  const int nrows = min(kStripRows, M - r0);
   const int lg = lane / LPG, li = lane % LPG;
-  const int g = qd * GPW + lg;
-  const bool valid = g < G;
-  // lanes past the last group of the row read the last group again and store nothing
-  const int64_t col = (int64_t)(valid ? g : G - 1) * GROUP + li * 8;
-  const int64_t base = (int64_t)r0 * K + col;
+  // wave-uniform task range [t0, t0 + SEG) over (row, segment-in-row) pairs
+  const unsigned total = (unsigned)M * (unsigned)nseg_row;
+  const unsigned t0 = (blockIdx.x * 4u + (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * SEG;
+  if (t0 >= total) return;
+  int row = (int)(t0 / (unsigned)nseg_row);
+  int sr = (int)(t0 - (unsigned)row * (unsigned)nseg_row);
 
-  float keep[NK];
+  Raw8<DT> raw[SEG];
+  int rows[SEG], segs[SEG];
 #pragma unroll
-  for (int k = 0; k < NK; ++k) keep[k] = 0.f;
-  uint32_t keepw = 0;
-
-  auto process = [&](const Raw8<DT>& raw, int row) {
-    float a[8];
-    raw.unpack(a);
-    float amax = fmaxf(group_max<LPG>(absmax8(a)), eps);
-    float sc = div448<DT != FP8K_F32>(amax);
-    uint2 out;
-    if (KIND == FP8K_SCALE_UE8M0_PACKED) {
-      // round the scale up to a power of two; x / 2^e == x * 2^-e exactly
-      uint32_t b = __float_as_uint(fmaxf(sc, 1e-10f));
-      uint32_t e = (b >> 23) + ((b & 0x7fffffu) != 0u);
-      float rinv = __uint_as_float((254u - e) << 23);
-      out.x = cvt4_fp8(a[0] * rinv, a[1] * rinv, a[2] * rinv, a[3] * rinv);
-      out.y = cvt4_fp8(a[4] * rinv, a[5] * rinv, a[6] * rinv, a[7] * rinv);
-      uint32_t eb = valid ? e : 0u;
-      uint32_t w = (uint32_t)__builtin_amdgcn_readlane((int)eb, 0) |
-                   ((uint32_t)__builtin_amdgcn_readlane((int)eb, 16) << 8) |
-                   ((uint32_t)__builtin_amdgcn_readlane((int)eb, 32) << 16) |
-                   ((uint32_t)__builtin_amdgcn_readlane((int)eb, 48) << 24);
-      keepw = (lane == row) ? w : keepw;
-    } else {
-      out = quant8_div(a, sc);
-#pragma unroll
-      for (int k = 0; k < NK; ++k) keep[k] = (row == k * LPG + li) ? sc : keep[k];
+  for (int j = 0; j < SEG; ++j) {
+    rows[j] = row;
+    segs[j] = sr;
+    if (t0 + j < total) {
+      const int g = sr * GPW + lg;
+      // lanes past the last group of the row re-read the last group and store nothing
+      const int64_t col = (int64_t)(g < G ? g : G - 1) * GROUP + li * 8;
+      load_stream<DT>(raw[j], x, (int64_t)row * K + col);
     }
-    if (valid) *reinterpret_cast<uint2*>(q + base + (int64_t)row * K) = out;
-  };
-
-  // full chunks of UNROLL rows, the next chunk's loads in flight while this one is processed
-  const int nfull = nrows / UNROLL;
-  Raw8<DT> cur[UNROLL], nxt[UNROLL];
-  if (nfull > 0) {
-#pragma unroll
-    for (int j = 0; j < UNROLL; ++j) cur[j].load(x, base + (int64_t)j * K);
-  }
-  for (int c = 0; c < nfull; ++c) {
-    if (c + 1 < nfull) {
-#pragma unroll
-      for (int j = 0; j < UNROLL; ++j) nxt[j].load(x, base + (int64_t)((c + 1) * UNROLL + j) * K);
+    if (++sr == nseg_row) {
+      sr = 0;
+      ++row;
     }
-#pragma unroll
-    for (int j = 0; j < UNROLL; ++j) process(cur[j], c * UNROLL + j);
-#pragma unroll
-    for (int j = 0; j < UNROLL; ++j) cur[j] = nxt[j];
   }
-  for (int row = nfull * UNROLL; row < nrows; ++row) {
-    Raw8<DT> t;
-    t.load(x, base + (int64_t)row * K);
-    process(t, row);
-  }
-
-  if (KIND == FP8K_SCALE_UE8M0_PACKED) {
-    if (lane < nrows) reinterpret_cast<uint32_t*>(s)[(int64_t)qd * sg + (int64_t)(r0 + lane) * sm] = keepw;
-  } else {
 #pragma unroll
-    for (int k = 0; k < NK; ++k) {
-      const int row = k * LPG + li;
-      if (valid && row < nrows) reinterpret_cast<float*>(s)[(int64_t)(r0 + row) * sm + (int64_t)g * sg] = keep[k];
+  for (int j = 0; j < SEG; ++j) {
+    if (t0 + j < total) {  // wave-uniform
+      const int g = segs[j] * GPW + lg;
+      const bool valid = g < G;
+      float a[8];
+      raw[j].unpack(a);
+      const float amax = fmaxf(group_max<LPG>(absmax8(a)), eps);
+      const float sc = div448<DT != FP8K_F32>(amax);
+      uint2 out;
+      if (KIND == FP8K_SCALE_UE8M0_PACKED) {
+        // round the scale up to a power of two; x / 2^e == x * 2^-e exactly
+        const uint32_t b = __float_as_uint(fmaxf(sc, 1e-10f));
+        const uint32_t e = (b >> 23) + ((b & 0x7fffffu) != 0u);
+        const float rinv = __uint_as_float((254u - e) << 23);
+        out.x = cvt4_fp8(a[0] * rinv, a[1] * rinv, a[2] * rinv, a[3] * rinv);
+        out.y = cvt4_fp8(a[4] * rinv, a[5] * rinv, a[6] * rinv, a[7] * rinv);
+        const uint32_t eb = valid ? e : 0u;  // bytes of groups past the row end stay zero
+        const uint32_t w = (uint32_t)__builtin_amdgcn_readlane((int)eb, 0) |
+                           ((uint32_t)__builtin_amdgcn_readlane((int)eb, 16) << 8) |
+                           ((uint32_t)__builtin_amdgcn_readlane((int)eb, 32) << 16) |
+                           ((uint32_t)__builtin_amdgcn_readlane((int)eb, 48) << 24);
+        if (lane == 0) reinterpret_cast<uint32_t*>(s)[(int64_t)segs[j] * sg + (int64_t)rows[j] * sm] = w;
+      } else {
+        out = quant8_div(a, sc);
+        if (valid && li == 0) reinterpret_cast<float*>(s)[(int64_t)rows[j] * sm + (int64_t)g * sg] = sc;
+      }
+      if (valid) store8_stream(q + (int64_t)rows[j] * K + (int64_t)g * GROUP + li * 8, out);
     }
   }
 }
@@ -205,14 +200,14 @@ template <int DT, int GROUP, int KIND>
 static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, float eps, int64_t sm, int64_t sg,
                               hipStream_t st) {
   constexpr int GPW = 64 / (GROUP / 8);
+  constexpr int SEG = 4;
   const int G = (int)(K / GROUP);
-  const int nquads = (G + GPW - 1) / GPW;
-  const int64_t nstrips = (M + kStripRows - 1) / kStripRows;
-  const int64_t waves = nstrips * nquads;
-  const int64_t blocks = (waves + 3) / 4;
-  if (waves > 0x7fffffffLL) return fail(FP8K_ERR_INVALID, "group_quant: input too large for one launch");
-  hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND>), dim3((unsigned)blocks), dim3(256), 0, st, x, (uint8_t*)q, s,
-                     (int)M, G, K, nquads, eps, sm, sg);
+  const int nseg_row = (G + GPW - 1) / GPW;
+  const int64_t total = M * nseg_row;
+  if (total > 0x7fffffffLL) return fail(FP8K_ERR_INVALID, "group_quant: input too large for one launch");
+  const int64_t waves = (total + SEG - 1) / SEG;
+  hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st, x,
+                     (uint8_t*)q, s, (int)M, G, K, nseg_row, eps, sm, sg);
   return check_launch("group_quant");
 }
 
