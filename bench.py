@@ -1,0 +1,297 @@
+#!/usr/bin/env python3
+"""Benchmark of the W8A8 block-FP8 linear hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--table PATH]
+
+One step = one pass of the hot path over one batch of synthetic input: per-token-group FP8
+quantisation of the activation (bf16 [M,K], groups of 128, column-major scales) followed by the
+block-scaled FP8 GEMM against a 128x128-block-quantised weight, bf16 out - what
+Fp8LinearMethod.apply runs for one projection.  The headline workload is a DeepSeek-V3 projection
+from BASELINE.json configs[2] at M=4096.  Inputs are generated on the GPU before the timed region
+and rotated over enough buffers that weights and activations come from HBM, not from the 256 MB
+last-level cache.
+
+Prints ONE JSON line.  `value` is the whole step in TFLOP/s (2*M*N*K per step); `roofline`
+prices the dominant kernel (the GEMM) against the published dense-FP8 MFMA peak, with its
+duration measured by HIP events around the GEMM launches only; `roofline_quant` does the same for
+the group-quant kernel at the largest configs[1] size against the HBM peak; `cpu_baseline` times
+the C restatement of the reference arithmetic (oracle/, OpenMP) on a bounded sample of the same
+workload on this machine's host cores.
+
+--table PATH additionally writes a per-shape report (configs[1], [2] and [3]) as markdown.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0  # MI355X published dense FP8 MFMA peak
+PEAK_HBM_GBS = 8000.0  # MI355X published HBM3E peak
+
+METRIC = "FP8 block GEMM TFLOPS (% MFMA peak) + group-quant GB/s at DeepSeek-V3 shapes"
+HEADLINE = dict(M=4096, N=18432, K=7168, name="DeepSeek-V3 gate_up (TP2) projection")
+QUANT_SHAPE = dict(M=16384, K=7168)
+
+DSV3_NK = [(24576, 1536), (32768, 512), (7168, 16384), (4608, 7168), (7168, 2304), (18432, 7168), (7168, 18432)]
+LLAMA_NK = [(6144, 4096), (4096, 4096), (28672, 4096), (4096, 14336)]
+
+
+def _activation(torch, M, K, seed, dev):
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed)
+    x = torch.randn((M, K), generator=g, device=dev, dtype=torch.float32)
+    mask = torch.rand((M, K), generator=g, device=dev) < 1e-3
+    return torch.where(mask, x * 50.0, x).to(torch.bfloat16)
+
+
+def _block_quant_weight(torch, N, K, seed, dev):
+    """N(0,0.02) bf16 weight -> e4m3fn + float32 scale per 128x128 block (scale = blockamax/448)."""
+    g = torch.Generator(device=dev)
+    g.manual_seed(seed + 1000003)
+    w = (torch.randn((N, K), generator=g, device=dev, dtype=torch.float32) * 0.02).to(torch.bfloat16).float()
+    nt, kt = (N + 127) // 128, (K + 127) // 128
+    wp = torch.zeros((nt * 128, kt * 128), device=dev)
+    wp[:N, :K] = w
+    blk = wp.view(nt, 128, kt, 128)
+    s = blk.abs().amax(dim=(1, 3)) / 448.0
+    s = torch.where(s == 0, torch.ones_like(s), s)
+    q = (blk / s[:, None, :, None]).clamp(-448.0, 448.0).view(nt * 128, kt * 128)[:N, :K]
+    return q.contiguous().to(torch.float8_e4m3fn), s.contiguous()
+
+
+def _events(torch, n):
+    return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
+
+
+def _time_calls(torch, fn, iters, warm=3):
+    """Average device time of fn(i) in microseconds, HIP events on the current stream."""
+    for i in range(warm):
+        fn(i)
+    torch.cuda.synchronize()
+    a, b = _events(torch, 2)
+    a.record()
+    for i in range(iters):
+        fn(i)
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / iters
+
+
+def quant_bytes(M, K, ue8m0=False):
+    return M * K * 3 + (M * K // 128) * (1 if ue8m0 else 4)
+
+
+def gemm_bytes(M, N, K):
+    return M * K + N * K + 2 * M * N + 4 * (M * K // 128 + (N // 128) * (K // 128))
+
+
+def run_headline(torch, dev, steps, warmup):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    M, N, K = HEADLINE["M"], HEADLINE["N"], HEADLINE["K"]
+    nbuf = 3
+    xs = [_activation(torch, M, K, s, dev) for s in range(nbuf)]
+    ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
+
+    def step(i):
+        x = xs[i % nbuf]
+        wq, wsc = ws[i % nbuf]
+        q, s = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+        return w8a8_block_fp8_matmul(q, wq, s, wsc, [128, 128], torch.bfloat16)
+
+    for i in range(warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        step(i)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    ms_per_step = (t1 - t0) * 1e3 / steps
+
+    # dominant kernel alone: events bracket only the GEMM launches (same stream), quantised inputs prepared before
+    qs = [sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True) for x in xs]
+    torch.cuda.synchronize()
+    gemm_us = _time_calls(
+        torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1], ws[i % nbuf][1],
+                                               [128, 128], torch.bfloat16), max(steps, 10))
+    return ms_per_step, gemm_us
+
+
+def run_quant_roofline(torch, dev, iters=30):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    M, K = QUANT_SHAPE["M"], QUANT_SHAPE["K"]
+    nbuf = 3  # 3 x (235 + 117 MB) > last-level cache
+    xs = [_activation(torch, M, K, s, dev) for s in range(nbuf)]
+    out = {}
+    for name, kw in (("row_major_f32", {}), ("col_major_f32", dict(column_major_scales=True)),
+                     ("ue8m0_packed", dict(column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True))):
+        us = _time_calls(torch, lambda i: sglang_per_token_group_quant_fp8(xs[i % nbuf], 128, **kw), iters)
+        out[name] = (us, quant_bytes(M, K, name == "ue8m0_packed") / us / 1e3)
+    return out
+
+
+def run_cpu_baseline(seconds_target=12.0):
+    """C restatement of quant + block GEMM (oracle/, OpenMP) on M_cpu rows of the headline workload."""
+    import numpy as np
+
+    from oracle import c_oracle, fp8_oracle as O
+
+    lib = c_oracle.load()
+    cores = lib.oracle_num_threads()
+    N, K = HEADLINE["N"], HEADLINE["K"]
+    rng = np.random.default_rng(0)
+    wq = rng.integers(0, 0x77, (N, K), dtype=np.uint8) | (rng.integers(0, 2, (N, K), dtype=np.uint8) << 7)
+    wsc = rng.uniform(1e-4, 2e-4, (N // 128, K // 128)).astype(np.float32)
+    eps = float(O.clamp_eps(1e-10, "bf16"))
+
+    def once(M):
+        x = O.bf16_bits(O.make_activation(M, K, 0))
+        t0 = time.perf_counter()
+        q, s = c_oracle.group_quant_bf16(lib, x, 128, eps)
+        c_oracle.block_gemm(lib, q, wq, s, wsc)
+        return time.perf_counter() - t0
+
+    t_probe = once(16)
+    M = int(min(1024, max(16, 16 * seconds_target / max(t_probe, 1e-3))))
+    M = max(16, M // 16 * 16)
+    dt = once(M)
+    return dict(value=2.0 * M * N * K / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                sample="C/OpenMP restatement of per-token-group quant + block-FP8 matmul on M=%d rows of the "
+                       "headline workload (N=%d, K=%d), %.1f s" % (M, N, K, dt))
+
+
+def write_table(torch, dev, path):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    lines = ["# Per-shape report (one MI355X, synthetic data, HIP-event device time, rotating buffers)", ""]
+    lines += ["## configs[1] per-token-group quant, K=7168, group 128", "",
+              "| M | layout | us | GB/s | % of 8 TB/s |", "|---|---|---|---|---|"]
+    for M in (1, 64, 512, 4096, 16384):
+        nbuf = 3 if M >= 4096 else 8
+        xs = [_activation(torch, M, 7168, s, dev) for s in range(nbuf)]
+        for name, kw in (("row", {}), ("col", dict(column_major_scales=True)),
+                         ("ue8m0", dict(column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True))):
+            us = _time_calls(torch, lambda i: sglang_per_token_group_quant_fp8(xs[i % nbuf], 128, **kw), 30)
+            gbs = quant_bytes(M, 7168, name == "ue8m0") / us / 1e3
+            lines.append("| %d | %s | %.1f | %.0f | %.1f |" % (M, name, us, gbs, gbs / PEAK_HBM_GBS * 100))
+        del xs
+    lines += ["", "## configs[2] block-FP8 GEMM, DeepSeek-V3 shapes", "",
+              "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s | GB/s (algorithmic) |", "|---|---|---|---|---|---|---|"]
+    for (N, K) in DSV3_NK:
+        nbuf = 3
+        ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
+        for M in (1, 16, 128, 1024, 4096):
+            qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True)
+                  for s in range(nbuf)]
+            us = _time_calls(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
+                                                                    ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
+            tf = 2.0 * M * N * K / us / 1e6
+            lines.append("| %d | %d | %d | %.1f | %.1f | %.1f | %.0f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100,
+                                                                          gemm_bytes(M, N, K) / us / 1e3))
+        del ws
+    lines += ["", "## configs[3] per-token fp8_scaled_mm, Llama-3-8B shapes", "",
+              "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s |", "|---|---|---|---|---|---|"]
+    for (N, K) in LLAMA_NK:
+        nbuf = 3
+        bs = [(torch.randn((N, K), device=dev) * 50).clamp(-448, 448).to(torch.float8_e4m3fn) for _ in range(nbuf)]
+        sb = torch.rand(N, device=dev) * 1e-3
+        for M in (1, 8, 64, 512, 2048, 8192):
+            a = [(torch.randn((M, K), device=dev) * 50).clamp(-448, 448).to(torch.float8_e4m3fn) for _ in range(nbuf)]
+            sa = torch.rand(M, device=dev)
+            us = _time_calls(torch, lambda i: fp8_scaled_mm(a[i % nbuf], bs[i % nbuf].t(), sa, sb, torch.bfloat16), 20)
+            tf = 2.0 * M * N * K / us / 1e6
+            lines.append("| %d | %d | %d | %.1f | %.1f | %.1f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100))
+        del bs
+    os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--table", type=str, default=None, help="also write the per-shape markdown report here")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (the path has no cross-GPU step); --gpus %d is not "
+              "supported" % args.gpus, file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the hot path has no CPU fallback", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    ms_per_step, gemm_us = run_headline(torch, dev, args.steps, args.warmup)
+    M, N, K = HEADLINE["M"], HEADLINE["N"], HEADLINE["K"]
+    flops = 2.0 * M * N * K
+    value = flops / (ms_per_step * 1e-3) / 1e12
+    gemm_tf = flops / gemm_us / 1e6
+    quant = run_quant_roofline(torch, dev)
+    q_us, q_gbs = quant["row_major_f32"]
+    if args.table:
+        write_table(torch, dev, args.table)
+    cpu = None if args.no_cpu else run_cpu_baseline()
+
+    out = {
+        "metric": METRIC,
+        "value": round(value, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "fp8_e4m3fn x fp8_e4m3fn -> f32 accumulate, bf16 out",
+        "data": "synthetic",
+        "config": {
+            "workload": "w8a8 block-FP8 linear = per-token-group quant (bf16 [%d,%d], group 128) + block-scaled FP8 "
+                        "GEMM vs 128x128-block weight [%d,%d]; %s, BASELINE configs[2]" % (M, K, N, K, HEADLINE["name"]),
+            "M": M, "N": N, "K": K, "weight_buffers_rotated": 3,
+        },
+        "roofline": {
+            "kernel": "gemm_tile256_kernel (block-scaled FP8 MFMA GEMM)",
+            "bound": "mfma",
+            "achieved": round(gemm_tf, 2),
+            "peak": PEAK_FP8_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(gemm_tf / PEAK_FP8_TFLOPS, 4),
+            "traffic": None,
+            "avg_launch_us": round(gemm_us, 2),
+        },
+        "roofline_quant": {
+            "kernel": "group_quant_kernel, bf16 [%d,%d], row-major f32 scales" % (QUANT_SHAPE["M"], QUANT_SHAPE["K"]),
+            "bound": "hbm",
+            "achieved": round(q_gbs, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(q_gbs / PEAK_HBM_GBS, 4),
+            "traffic": None,
+            "avg_launch_us": round(q_us, 2),
+            "other_layouts_GBps": {k: round(v[1], 1) for k, v in quant.items()},
+        },
+        "cpu_baseline": cpu,
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -26,6 +26,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
     "-Wno-unknown-warning-option",
+    "-Wno-pass-failed",
 ]
 
 

@@ -5,17 +5,30 @@
 namespace fp8k {
 
 struct Plan {
-  int kind;    // 0 = generic, 1 = tile256
+  int kind;    // 0 = generic, 1 = tile256, 2 = weight-streaming (few rows)
   int splits;  // >1: split-K through the float workspace
   int kb_per_split;
+  int tm;      // rows per block of the streaming kernel
 };
 
 static Plan make_plan(int64_t M, int64_t N, int64_t K) {
-  Plan pl{0, 1, 0};
+  Plan pl{0, 1, 0, 0};
   if (K % kTileK != 0 || N % 4 != 0) return pl;
+  const int kb = (int)(K / kTileK);
+  if (M <= 128 && M * K < (1LL << 31)) {
+    // decode-sized: stream the weights once, every CU takes a K slice of one 256-row weight tile
+    pl.kind = 2;
+    pl.tm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
+    const int64_t tiles_n = (N + kTileN - 1) / kTileN;
+    int splits = (int)(256 / tiles_n);
+    if (splits > kb / 4) splits = kb / 4;
+    if (splits < 1) splits = 1;
+    pl.kb_per_split = (kb + splits - 1) / splits;
+    pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
+    return pl;
+  }
   pl.kind = 1;
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
-  const int kb = (int)(K / kTileK);
   int splits = 1;
   // fewer tiles than compute units: cut K so that every CU has work, keeping >= 4 K-blocks per run
   if (tiles < 160) {
@@ -46,6 +59,29 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   a.tiles_n = (a.N + kTileN - 1) / kTileN;
   a.splits = pl.splits;
   a.kb_per_split = pl.kb_per_split;
+  if (pl.kind == 2) {
+    a.m_blocks = 1;
+    const unsigned nwg = (unsigned)(((a.tiles_n + 7) / 8) * 8 * pl.splits);
+#define FP8K_STREAM(TM, NST)                                                                                          \
+  do {                                                                                                                \
+    if (pl.splits == 1)                                                                                               \
+      hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, MODE, OUT_DT, BIAS_DT, false, false>), dim3(nwg), dim3(512), 0, \
+                         st, a);                                                                                      \
+    else                                                                                                              \
+      hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, MODE, OUT_DT, BIAS_DT, true, false>), dim3(nwg), dim3(512), 0,  \
+                         st, a);                                                                                      \
+  } while (0)
+    if (pl.tm == 32) FP8K_STREAM(32, 4);
+    else if (pl.tm == 64) FP8K_STREAM(64, 3);
+    else FP8K_STREAM(128, 3);
+#undef FP8K_STREAM
+    int rc = check_launch("gemm_stream");
+    if (rc || pl.splits == 1) return rc;
+    const int64_t quads = (int64_t)a.M * (a.N / 4);
+    hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256),
+                       0, st, a);
+    return check_launch("splitk_reduce");
+  }
   const int ntiles = a.tiles_m * a.tiles_n;
   const unsigned nwg = (unsigned)(((ntiles + 7) / 8) * 8 * pl.splits);
   if (pl.splits == 1) {

@@ -25,6 +25,16 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int splits;         // K is cut into `splits` runs of kb_per_split K-blocks
   int kb_per_split;
+  // grouped (MoE) form of the streaming kernel; all null / zero for a dense GEMM
+  const int32_t* sorted_ids;    // [m_blocks * TM] token slots, padded with values >= num_valid
+  const int32_t* expert_ids;    // [m_blocks] expert of each block of TM slots, -1 = not on this rank
+  const int32_t* num_post_pad;  // device scalar: slots in use (multiple of TM)
+  const float* topk_w;          // routed weight per slot, or null
+  int top_k;                    // X row of a slot = slot / top_k
+  int num_valid;                // number of real slots (topk_ids.numel())
+  int m_blocks;                 // blocks of TM rows
+  int64_t w_expert_stride;      // bytes between experts in W
+  int64_t sw_expert_stride;     // floats between experts in sw
 };
 
 enum { kModeBlock = 0, kModeRow = 1 };
@@ -323,6 +333,228 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
           }
           store4<OUT_DT>(p.C, (int64_t)m * p.ldc + n, v[0], v[1], v[2], v[3]);
         }
+      }
+    }
+  }
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// Weight-streaming kernel for few rows: 256(n) x TM(m) x 128(k) tile, TM in {32, 64, 128}, 8 waves each
+// owning 32 weight rows x all TM activation rows.  Used for decode-sized dense GEMMs (with split-K
+// through a float workspace so that every CU streams a share of the weights) and for the grouped
+// MoE GEMM, where a block of TM token slots belongs to one expert and activation / output rows go
+// through sorted_token_ids.  These shapes are HBM-bound (2*TM FLOP per weight byte), so the design
+// point is bytes in flight, not MFMA occupancy: NSTAGE LDS stages of [W 32 KB | X TM*128 B] are kept
+// full with partial vmcnt waits; a wave reads its 32 weight rows from LDS exactly once.
+// ------------------------------------------------------------------------------------------------
+template <int TM, int NSTAGE, int MODE, int OUT_DT, int BIAS_DT, bool SPLIT, bool MOE>
+__global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
+  constexpr int MS = TM / 32;                    // 32-row activation sub-tiles
+  constexpr int XL = (TM + 63) / 64;             // X wave-loads per wave per stage
+  constexpr int LPW = 4 + XL;                    // LDS-DMA loads per wave per stage
+  constexpr int WBYTES = kTileN * kTileK;
+  constexpr int STAGE = WBYTES + TM * kTileK;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * STAGE + 1024];
+  uint8_t* const dummy = smem + NSTAGE * STAGE;  // landing zone of padding loads
+
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+
+  // ---- work item: consecutive ids walk the m blocks of one n tile (they share weight rows in L2)
+  const int nitems = p.tiles_n * p.m_blocks;
+  const int per_xcd = (nitems + 7) >> 3;
+  int bid = blockIdx.x;
+  int split = 0;
+  if (SPLIT) { split = bid % p.splits; bid /= p.splits; }
+  const int t = (bid & 7) * per_xcd + (bid >> 3);
+  if (t >= nitems) return;
+  const int mb = t % p.m_blocks;
+  const int tile_n = t / p.m_blocks;
+  const int n0 = tile_n * kTileN;
+  const int slot0 = mb * TM;
+  int expert = 0;
+  if (MOE) {
+    if (slot0 >= p.num_post_pad[0]) return;
+    expert = p.expert_ids[mb];
+  }
+  const int nrows = MOE ? p.num_valid : p.M;  // exclusive bound of a valid slot
+
+  const int kb_begin = SPLIT ? split * p.kb_per_split : 0;
+  const int kb_end = SPLIT ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
+  const int nkb = kb_end - kb_begin;
+
+  // ---- output rows of this lane (m = ms*32 + lane%32)
+  const int lr = lane & 31, h = lane >> 5;
+  int out_slot[MS];
+  bool out_ok[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int s = slot0 + ms * 32 + lr;
+    out_slot[ms] = MOE ? p.sorted_ids[s] : s;
+    out_ok[ms] = out_slot[ms] < nrows;
+  }
+
+  if (MOE && expert < 0) {  // expert lives on another rank: the reference writes zeros
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) {
+      if (!out_ok[ms]) continue;
+      for (int j = 0; j < 4; ++j) {
+        const int n = n0 + w * 32 + h * 16 + j * 4;
+        if (n < p.N) store4<OUT_DT>(p.C, (int64_t)out_slot[ms] * p.ldc + n, 0.f, 0.f, 0.f, 0.f);
+      }
+    }
+    return;
+  }
+
+  // ---- global -> LDS
+  const uint8_t* Wb = p.W + (MOE ? (int64_t)expert * p.w_expert_stride : 0);
+  const int rowsW = min(kTileN, p.N - n0);
+  const int kbytes = p.K - kb_begin * kTileK;
+  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
+  // activations: one descriptor over every row; a padded slot points past the range and reads zeros
+  const int64_t xrows = MOE ? (int64_t)((p.num_valid + p.top_k - 1) / p.top_k) : (int64_t)p.M;
+  const rsrc_t rX = make_rsrc(p.X + (int64_t)kb_begin * kTileK, (uint32_t)((xrows - 1) * p.ldx + kbytes));
+  const int rl = lane >> 3, cp = lane & 7;
+  uint32_t voW[2];
+#pragma unroll
+  for (int par = 0; par < 2; ++par) voW[par] = (uint32_t)(rl * p.ldw + ((cp ^ ((par << 2) + (rl >> 1))) * 16));
+  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), stepW = (uint32_t)(8 * p.ldw);
+  uint32_t voX[XL];
+  bool xload[XL];
+#pragma unroll
+  for (int j = 0; j < XL; ++j) {
+    const int grp = w * XL + j;             // 8-row group of the X tile
+    xload[j] = grp * 8 < TM;                // wave-uniform
+    const int row = grp * 8 + rl;
+    const int c = cp ^ (((grp & 1) << 2) + (rl >> 1));
+    int s = nrows;
+    if (xload[j]) s = MOE ? p.sorted_ids[slot0 + row] : slot0 + row;
+    const bool ok = s < nrows;
+    const int64_t xr = MOE ? s / p.top_k : s;
+    voX[j] = ok ? (uint32_t)(xr * p.ldx + c * 16) : 0xF0000000u;
+  }
+  auto issue = [&](int kstep) {
+    uint8_t* base = smem + (kstep % NSTAGE) * STAGE;
+    const uint32_t ko = (uint32_t)kstep * kTileK;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) buf_load16_to_lds(rW, voW[j & 1], soW + j * stepW + ko, base + w * 4096 + j * 1024);
+#pragma unroll
+    for (int j = 0; j < XL; ++j)
+      buf_load16_to_lds(rX, voX[j], ko, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
+  };
+
+  // ---- LDS -> MFMA operands
+  const int swz = (lr >> 1) & 7;
+  uint32_t co[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) co[ks][j] = (uint32_t)(((ks * 4 + h * 2 + j) ^ swz) << 4);
+  const uint32_t rdW = (uint32_t)((w * 32 + lr) * kTileK);
+  const uint32_t rdX = (uint32_t)(WBYTES + lr * kTileK);
+  auto frag = [&](const uint8_t* st, uint32_t rowoff, int ks) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][0]);
+    const v4i hi = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][1]);
+    v8i r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+  };
+
+  // ---- scales (block mode): activation scale rows follow the activation rows
+  const float* sxp[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int64_t xr = out_ok[ms] ? (MOE ? out_slot[ms] / p.top_k : out_slot[ms]) : 0;
+    sxp[ms] = p.sx + xr * p.sx_m + (int64_t)kb_begin * p.sx_k;
+  }
+  const int nb = min(n0 + w * 32, p.N - 1) >> 7;
+  const float* swp = p.sw + (MOE ? (int64_t)expert * p.sw_expert_stride : 0) + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
+
+  v16f acc[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[ms][r] = 0.f;
+
+#pragma unroll
+  for (int s = 0; s < NSTAGE - 1; ++s) issue(s);
+  float sxn[MS], sbn = 0.f;
+  if (MODE == kModeBlock && nkb > 0) {
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) sxn[ms] = sxp[ms][0];
+    sbn = swp[0];
+  }
+
+  for (int it = 0; it < nkb; ++it) {
+    // stage `it` has landed once at most NSTAGE-2 younger stages are still in flight
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (((NSTAGE - 2) * LPW) & 15) | ((((NSTAGE - 2) * LPW) >> 4) << 14));
+    __syncthreads();
+    issue(it + NSTAGE - 1);  // refills the stage every wave finished before this barrier
+    float sc[MS];
+    if (MODE == kModeBlock) {
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
+      const int kn = min(it + 1, nkb - 1);
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms) sxn[ms] = sxp[ms][(int64_t)kn * p.sx_k];
+      sbn = swp[(int64_t)kn * p.sw_k];
+    }
+    const uint8_t* st = smem + (it % NSTAGE) * STAGE;
+    v8i wf[2];
+    wf[0] = frag(st, rdW, 0);
+    wf[1] = frag(st, rdW, 1);
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) {
+      const v8i x0 = frag(st, rdX + ms * 32 * kTileK, 0);
+      const v8i x1 = frag(st, rdX + ms * 32 * kTileK, 1);
+      if (MODE == kModeBlock) {
+        v16f z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        v16f tq = mfma_32x32x64(wf[0], x0, z);
+        tq = mfma_32x32x64(wf[1], x1, tq);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ms][r]);
+      } else {
+        acc[ms] = mfma_32x32x64(wf[0], x0, acc[ms]);
+        acc[ms] = mfma_32x32x64(wf[1], x1, acc[ms]);
+      }
+    }
+  }
+  wait_vm0();  // drain the padding loads before the LDS allocation is released
+
+  // ---- epilogue
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    if (!out_ok[ms]) continue;
+    const int64_t orow = out_slot[ms];
+    float rs = 1.f;
+    if (MODE == kModeRow && !SPLIT) rs = p.sx[orow];
+    if (MOE && p.topk_w) rs = p.topk_w[orow];
+#pragma unroll
+    for (int rg = 0; rg < 4; ++rg) {
+      const int n = n0 + w * 32 + rg * 8 + h * 4;
+      if (n >= p.N) continue;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = acc[ms][rg * 4 + r];
+      if (SPLIT) {
+        *reinterpret_cast<float4*>(p.partial + ((int64_t)split * p.M + orow) * p.N + n) = make_float4(v[0], v[1], v[2], v[3]);
+      } else {
+        if (MODE == kModeRow) {
+          const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
+          v[0] = v[0] * sb.x * rs; v[1] = v[1] * sb.y * rs; v[2] = v[2] * sb.z * rs; v[3] = v[3] * sb.w * rs;
+          if (p.bias) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] += load_scalar<BIAS_DT>(p.bias, n + r);
+          }
+        } else if (MOE) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] *= rs;
+        }
+        store4<OUT_DT>(p.C, orow * p.ldc + n, v[0], v[1], v[2], v[3]);
       }
     }
   }

@@ -1,0 +1,283 @@
+"""Pins of the CPU oracle (no GPU): every oracle function is checked against something that does
+not share its formula - torch's CPU conversions, closed forms from the reference's own tests,
+exhaustive tables, float64 arithmetic, brute force on tiny inputs, or integer invariants."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import c_oracle
+from oracle import fp8_oracle as O
+
+
+# ---------------------------------------------------------------- formats
+def test_e4m3fn_encode_matches_torch_on_every_16bit_prefix():
+    hi = np.arange(1 << 16, dtype=np.uint32) << 16
+    for low in (0x0000, 0x7FFF, 0x8000, 0x8001, 0xFFFF, 0x1234):
+        x = (hi | low).view(np.float32)
+        ref = torch.from_numpy(x.copy()).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+        got = O.f32_to_e4m3fn(x)
+        ok = (ref == got) | np.isnan(x)  # NaN sign is unspecified
+        assert ok.all()
+
+
+def test_e4m3fn_known_answers():
+    # OCP table: max 448, no Inf, 0x7F NaN, subnormal step 2^-9, ties to even
+    x = np.array([448, 464, 463.9, 480, 1e9, 2**-10, 1.5 * 2**-9, 2**-9, 2**-6, 0.0, -0.0, 1.0, -1.5, 17.0, 18.0],
+                 dtype=np.float32)
+    exp = [0x7E, 0x7E, 0x7E, 0x7F, 0x7F, 0x00, 0x02, 0x01, 0x08, 0x00, 0x80, 0x38, 0xBC, 0x58, 0x59]
+    assert O.f32_to_e4m3fn(x).tolist() == exp
+    assert O.f32_to_e4m3fn(np.array([19.0], np.float32))[0] == 0x5A  # 19 is a tie between 18 and 20 -> even mantissa (20)
+
+
+def test_e4m3fn_decode_matches_torch_and_roundtrips():
+    b = np.arange(256, dtype=np.uint8)
+    t = torch.from_numpy(b).view(torch.float8_e4m3fn).float().numpy()
+    assert np.array_equal(np.nan_to_num(t, nan=-7.0), np.nan_to_num(O.E4M3FN_TABLE, nan=-7.0))
+    finite = ~np.isnan(O.E4M3FN_TABLE)
+    assert np.array_equal(O.f32_to_e4m3fn(O.E4M3FN_TABLE[finite]), b[finite])
+
+
+def test_bf16_rounding_matches_torch():
+    rng = np.random.default_rng(0)
+    y = (rng.standard_normal(200000) * rng.choice([1e-20, 1.0, 1e20], 200000)).astype(np.float32)
+    assert np.array_equal(O.to_bf16(y), torch.from_numpy(y).bfloat16().float().numpy())
+    assert np.array_equal(O.bf16_from_bits(O.bf16_bits(O.to_bf16(y))), O.to_bf16(y))
+
+
+# ---------------------------------------------------------------- group quant
+def test_eps_is_clamped_in_the_input_dtype():
+    assert O.clamp_eps(1e-10, "bf16") == torch.tensor([0.0], dtype=torch.bfloat16).clamp(min=1e-10).float().item()
+    assert O.clamp_eps(1e-10, "f32") == np.float32(1e-10)
+
+
+def test_group_quant_closed_form_amax_448():
+    """python/sglang/test/srt/quant/test_fp8_kernel.py:24-45: a group whose amax is exactly 448 has scale 1
+    and quantises to the fp8 encoding of its own values."""
+    rng = np.random.default_rng(1)
+    vals = O.E4M3FN_TABLE[rng.integers(0, 0x7F, (16, 512))] * rng.choice([-1, 1], (16, 512)).astype(np.float32)
+    vals = vals.reshape(-1, 128)
+    vals[:, 0] = 448.0
+    vals = vals.reshape(16, 512)
+    q, s = O.per_token_group_quant_fp8(vals, 128, in_dtype="f32")
+    assert (s == 1.0).all()
+    assert np.array_equal(O.e4m3fn_to_f32(q), vals)
+
+
+def test_group_quant_against_torch_library_ops():
+    """Same steps with torch CPU tensor ops (abs/max/clamp/div/to(float8)) on bf16 data."""
+    x = O.make_activation(96, 2048, 3)
+    xt = torch.from_numpy(x).bfloat16()
+    g = xt.reshape(-1, 128)
+    amax = g.abs().max(dim=-1, keepdim=True)[0].clamp(min=1e-10).to(torch.float32)
+    xs = amax / 448.0
+    xq = (g / xs).clamp(min=-448.0, max=448.0).to(torch.float8_e4m3fn)
+    q, s = O.per_token_group_quant_fp8(x, 128)
+    assert np.array_equal(q.reshape(-1, 128), xq.view(torch.uint8).numpy())
+    assert np.array_equal(s.reshape(-1, 1), xs.numpy())
+
+
+def test_scale_table_every_bf16_amax():
+    bits = np.arange(1, 0x7F80, dtype=np.uint32)
+    amax = (bits << 16).view(np.float32)
+    x = np.zeros((amax.size, 128), dtype=np.float32)
+    x[:, 5] = amax
+    _, s = O.per_token_group_quant_fp8(x, 128)
+    expect = (torch.from_numpy(amax).bfloat16().clamp(min=1e-10).float() / 448.0).numpy()
+    assert np.array_equal(s[:, 0], expect)
+
+
+def test_ue8m0_bit_form_equals_pow2_ceil_log2_for_every_bf16_amax():
+    bits = np.arange(0x0080, 0x7F80, dtype=np.uint32)  # positive normal bf16
+    amax = np.maximum((bits << 16).view(np.float32), np.float32(1e-10))
+    s = (amax / np.float32(448)).astype(np.float32)
+    s = s[(s > 1e-30) & (s < 1e30)]
+    via_log = torch.pow(2.0, torch.ceil(torch.log2(torch.from_numpy(s).double()))).float().numpy()
+    assert np.array_equal(O.ceil_to_ue8m0(s), via_log)
+    assert (O.ceil_to_ue8m0(s) >= s).all() and (O.ceil_to_ue8m0(s) < 2 * s).all()
+
+
+def test_ue8m0_pack_roundtrip_and_layout():
+    rng = np.random.default_rng(2)
+    s = (2.0 ** rng.integers(-30, 10, (7, 6))).astype(np.float32)
+    w = O.pack_ue8m0_scales(s)
+    assert w.shape == (7, 2) and w.dtype == np.int32
+    by = w.view(np.uint8).reshape(7, 8)
+    assert np.array_equal(by[:, :6], O.ue8m0_byte(s)) and (by[:, 6:] == 0).all()
+    assert np.array_equal(O.unpack_ue8m0_scales(w, 6), s)
+    assert O.ue8m0_byte(np.array([1.0], np.float32))[0] == 127
+
+
+def test_ue8m0_quant_divides_by_power_of_two():
+    x = O.make_activation(8, 512, 4)
+    q, s = O.per_token_group_quant_fp8(x, 128, scale_ue8m0=True)
+    m, e = np.frexp(s)
+    assert (m == 0.5).all()
+    _, s_plain = O.per_token_group_quant_fp8(x, 128)
+    assert (s >= s_plain).all() and (s < 2 * s_plain).all()
+
+
+# ---------------------------------------------------------------- per-token / per-tensor
+def test_per_token_and_tensor_quant_against_torch_ops():
+    x = O.make_activation(33, 1024, 5)
+    x[4] = 0
+    q, s = O.per_token_quant_fp8(x)
+    xt = torch.from_numpy(x)
+    st = xt.abs().amax(dim=-1, keepdim=True) / 448.0
+    inv = torch.where(st == 0, torch.zeros_like(st), 1.0 / st)
+    qt = (xt * inv).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert np.array_equal(q, qt) and np.array_equal(s, st.numpy())
+    assert s[4, 0] == 0 and (q[4] == 0).all()
+    q2, s2 = O.per_tensor_quant_fp8(x)
+    s2t = xt.abs().max() / 448.0
+    q2t = (xt * (1.0 / s2t)).clamp(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8).numpy()
+    assert s2[0] == s2t.item() and np.array_equal(q2, q2t)
+
+
+def test_block_quant_weight_roundtrip_error():
+    w = O.make_weight(384, 640, 1)
+    q, s = O.block_quant_weight(w)
+    assert s.shape == (3, 5)
+    deq = O.e4m3fn_to_f32(q).reshape(3, 128, 5, 128) * s[:, None, :, None]
+    err = np.abs(deq.reshape(384, 640) - w)
+    assert err.max() <= np.abs(w).max() * 2**-4  # 3 mantissa bits
+    blk = np.abs(O.e4m3fn_to_f32(q)).reshape(3, 128, 5, 128).max(axis=(1, 3))
+    assert (blk == 448).all()  # every block uses the full range
+
+
+# ---------------------------------------------------------------- matmuls
+def _brute(Aq, Bq, As, Bs):
+    A, B = O.e4m3fn_to_f32(Aq).astype(np.float64), O.e4m3fn_to_f32(Bq).astype(np.float64)
+    M, K = A.shape
+    N = B.shape[0]
+    C = np.zeros((M, N))
+    for m in range(M):
+        for n in range(N):
+            for k in range(K):
+                C[m, n] += A[m, k] * B[n, k] * As[m, k // 128] * Bs[n // 128, k // 128]
+    return C
+
+
+def test_block_matmul_vs_brute_force_triple_loop():
+    rng = np.random.default_rng(6)
+    Aq = O.f32_to_e4m3fn(rng.standard_normal((5, 256)).astype(np.float32) * 20)
+    Bq = O.f32_to_e4m3fn(rng.standard_normal((130, 256)).astype(np.float32) * 20)
+    As = rng.uniform(0.5, 2, (5, 2)).astype(np.float32)
+    Bs = rng.uniform(0.5, 2, (2, 2)).astype(np.float32)
+    ref = _brute(Aq, Bq, As, Bs)
+    got = O.w8a8_block_fp8_matmul(Aq, Bq, As, Bs, out_dtype="f32", acc=np.float64)
+    np.testing.assert_allclose(got, ref, rtol=1e-6, atol=1e-6 * np.abs(ref).max())
+    got32 = O.w8a8_block_fp8_matmul(Aq, Bq, As, Bs, out_dtype="f32", acc=np.float32)
+    np.testing.assert_allclose(got32, ref, rtol=0, atol=1e-5 * np.abs(ref).max())
+
+
+def test_block_matmul_dequantise_then_matmul_and_linearity():
+    """sgl-kernel/tests/test_fp8_blockwise_gemm.py:19-59: broadcast the scales, multiply in high precision."""
+    xq, xs = O.per_token_group_quant_fp8(O.make_activation(40, 1024, 7), 128)
+    wq, ws = O.block_quant_weight(O.make_weight(384, 1024, 7))
+    a = O.e4m3fn_to_f32(xq).astype(np.float64) * np.repeat(xs, 128, axis=1)
+    b = O.e4m3fn_to_f32(wq).astype(np.float64) * np.repeat(np.repeat(ws, 128, axis=0), 128, axis=1)
+    ref = a @ b.T
+    got = O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="f32", acc=np.float64)
+    np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-6 * np.abs(ref).max())
+    got4 = O.w8a8_block_fp8_matmul(xq, wq, (xs * 4).astype(np.float32), ws, out_dtype="f32", acc=np.float64)
+    np.testing.assert_array_equal(got4, 4 * got)
+
+
+def test_scaled_mm_vs_torch_restatement():
+    """sgl-kernel/tests/test_fp8_gemm.py:6-14."""
+    rng = np.random.default_rng(8)
+    aq = O.f32_to_e4m3fn(rng.standard_normal((9, 512)).astype(np.float32) * 10)
+    bq = O.f32_to_e4m3fn(rng.standard_normal((64, 512)).astype(np.float32) * 10)
+    sa = rng.uniform(0.1, 1, 9).astype(np.float32)
+    sb = rng.uniform(0.1, 1, 64).astype(np.float32)
+    bias = O.to_bf16(rng.standard_normal(64).astype(np.float32))
+    A = torch.from_numpy(aq).view(torch.float8_e4m3fn).to(torch.float32)
+    B = torch.from_numpy(bq).view(torch.float8_e4m3fn).to(torch.float32)
+    o = torch.matmul(A, B.t()) * torch.from_numpy(sa).view(-1, 1) * torch.from_numpy(sb).view(1, -1)
+    o = (o + torch.from_numpy(bias)).to(torch.bfloat16).float().numpy()
+    got = O.fp8_scaled_mm(aq, bq, sa, sb, "bf16", bias)
+    assert np.abs(got - o).max() <= 2**-7 * np.abs(o).max()  # one bf16 ulp from summation order
+
+
+# ---------------------------------------------------------------- C restatement == numpy restatement
+def test_c_oracle_matches_numpy_oracle():
+    lib = c_oracle.load()
+    x = O.make_activation(70, 1536, 9)
+    x[3, :128] = 0
+    eps = float(O.clamp_eps(1e-10, "bf16"))
+    for ue in (False, True):
+        q, s = O.per_token_group_quant_fp8(x, 128, scale_ue8m0=ue)
+        qc, sc = c_oracle.group_quant_bf16(lib, O.bf16_bits(x), 128, eps, ue)
+        assert np.array_equal(q, qc) and np.array_equal(s.view(np.uint32), sc.view(np.uint32))
+    q, s = O.per_token_group_quant_fp8(x, 128)
+    wq, ws = O.block_quant_weight(O.make_weight(640, 1536, 9))
+    ref = O.w8a8_block_fp8_matmul(q, wq, s, ws, out_dtype="f32", acc=np.float64)
+    c = O.bf16_from_bits(c_oracle.block_gemm(lib, q, wq, s, ws))
+    assert np.abs(c - ref).max() <= 2**-7 * np.abs(ref).max()
+    sa = np.random.default_rng(1).uniform(0.1, 1, 70).astype(np.float32)
+    sb = np.random.default_rng(2).uniform(0.1, 1, 640).astype(np.float32)
+    ref2 = O.fp8_scaled_mm(q, wq, sa, sb, "f32")
+    c2 = O.bf16_from_bits(c_oracle.scaled_mm(lib, q, wq, sa, sb))
+    assert np.abs(c2 - ref2).max() <= 2**-7 * np.abs(ref2).max()
+
+
+# ---------------------------------------------------------------- MoE helpers
+@pytest.mark.parametrize("E,topk,block", [(8, 2, 16), (64, 6, 64), (256, 8, 64), (257, 8, 128)])
+def test_moe_align_invariants(E, topk, block):
+    """sgl-kernel/tests/test_moe_align.py:210-254: counts, padding, ownership."""
+    rng = np.random.default_rng(E)
+    T = 97
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    ids[rng.random(ids.shape) < 0.05] = -1
+    sorted_ids, expert_ids, npad = O.moe_align_block_size(ids, block, E)
+    numel = ids.size
+    counts = np.bincount(ids.reshape(-1) + 1, minlength=E + 1)
+    assert npad == sum((c + block - 1) // block * block for c in counts)
+    assert sorted_ids.size == numel + (E + 1) * (block - 1)
+    used = expert_ids[: npad // block]
+    assert (np.diff(used) >= 0).all()
+    for b, e in enumerate(used):
+        blk = sorted_ids[b * block : (b + 1) * block]
+        real = blk[blk < numel]
+        assert (ids.reshape(-1)[real] == e).all()
+        assert (blk[len(real):] == numel).all()
+    real_all = sorted_ids[:npad][sorted_ids[:npad] < numel]
+    assert np.array_equal(np.sort(real_all), np.arange(numel))
+    assert (sorted_ids[npad:] == numel).all()
+
+
+def test_silu_and_mul_and_sum_reduce_against_torch_bf16():
+    rng = np.random.default_rng(10)
+    x = O.to_bf16(rng.standard_normal((37, 512)).astype(np.float32) * 3)
+    xt = torch.from_numpy(x).bfloat16()
+    d = 256
+    ref = (torch.nn.functional.silu(xt[..., :d].float()).to(torch.bfloat16) * xt[..., d:]).float().numpy()
+    assert np.array_equal(O.silu_and_mul(x), ref)
+    y = O.to_bf16(rng.standard_normal((19, 8, 128)).astype(np.float32))
+    acc = torch.zeros(19, 128)
+    for k in range(8):
+        acc = acc + torch.from_numpy(y[:, k])
+    ref2 = (acc * 2.5).to(torch.bfloat16).float().numpy()
+    assert np.array_equal(O.moe_sum_reduce(y, 2.5), ref2)
+
+
+def test_grouped_topk_properties():
+    """python/sglang/srt/layers/moe/topk.py:665-738 with the DeepSeek-V3 tuple (256 experts, 8 groups, top-4 groups, top-8)."""
+    rng = np.random.default_rng(11)
+    logits = rng.standard_normal((50, 256)).astype(np.float32)
+    bias = (rng.standard_normal(256) * 0.1).astype(np.float32)
+    w, ids = O.biased_grouped_topk(logits, bias, 8, 4, 8)
+    assert w.shape == (50, 8) and ids.shape == (50, 8)
+    np.testing.assert_allclose(w.sum(-1), 1.0, rtol=1e-5)
+    for t in range(50):
+        assert len(set(ids[t].tolist())) == 8
+        assert len(set((ids[t] // 32).tolist())) <= 4
+    # torch restatement of the same selection
+    sc = torch.sigmoid(torch.from_numpy(logits))
+    scb = sc + torch.from_numpy(bias)
+    gs = scb.view(50, 8, 32).topk(2, dim=-1)[0].sum(-1)
+    gi = gs.topk(4, dim=-1)[1]
+    gm = torch.zeros_like(gs).scatter_(1, gi, 1)
+    sm = gm.unsqueeze(-1).expand(50, 8, 32).reshape(50, 256)
+    ti = scb.masked_fill(~sm.bool(), float("-inf")).topk(8, dim=-1)[1]
+    assert np.array_equal(np.sort(ids, axis=1), np.sort(ti.numpy(), axis=1))
