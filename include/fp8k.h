@@ -101,6 +101,63 @@ int fp8k_scaled_mm(const void* A, const void* B, const float* sa, const float* s
                    int bias_dtype, void* workspace, int64_t workspace_bytes, void* stream);
 int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
+/*
+ * Token alignment for the fused-MoE grouped GEMM (integer work).
+ * Replaces torch.ops.sgl_kernel.moe_align_block_size
+ *   (sgl-kernel/python/sgl_kernel/moe.py:6-25, sgl-kernel/csrc/moe/moe_align_kernel.cu:302-366); the caller
+ *   python/sglang/srt/layers/moe/fused_moe_triton/moe_align_block_size.py:57-81 passes num_experts+1 buckets.
+ * topk_ids: numel ids (int32, or int64 when ids_are_int64), values in [-1, num_buckets-1); id e goes to bucket e+1.
+ * Outputs: sorted_token_ids - for every bucket in use, its flat id positions (order inside a bucket is
+ *   unspecified) followed, when pad_sorted_token_ids, by the value numel up to a multiple of block_size;
+ *   expert_ids[b] = bucket-1 of block b for b < post_pad/block_size; num_tokens_post_pad[0] = slots in use.
+ * cumsum_buffer: num_buckets+1 ints of scratch (start offsets; consumed), may be NULL when numel <= 65536.
+ * Capacities are checked against the worst case numel + min(numel, num_buckets)*(block_size-1).
+ */
+int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64, int64_t numel, int64_t num_buckets,
+                              int64_t block_size, int32_t* sorted_token_ids, int64_t sorted_capacity,
+                              int32_t* expert_ids, int64_t expert_capacity, int32_t* num_tokens_post_pad,
+                              int32_t* cumsum_buffer, int pad_sorted_token_ids, void* stream);
+
+/*
+ * Grouped block-scaled FP8 GEMM with expert indirection:
+ *   C[slot, n] = w(slot) * sum_kb ( A[slot / top_k, kb] . B[e, n, kb] ) * As[slot / top_k, kb] * Bs[e, n/128, kb]
+ * for every slot = sorted_token_ids[i] < num_valid_tokens, i < num_tokens_post_padded[0], with
+ * e = expert_ids[i / block_m]; blocks with e < 0 write zeros; w = topk_weights[slot] or 1 when NULL.
+ * Replaces invoke_fused_moe_kernel / fused_moe_kernel with use_fp8_w8a8 and block_shape [128,128]
+ *   (python/sglang/srt/layers/moe/fused_moe_triton/fused_moe_triton_kernels.py:307-583, 586-790).
+ * A e4m3fn [ceil(num_valid/top_k), K] (lda); B e4m3fn [E, N, K] (b_stride_e bytes between experts, ldb between
+ * rows); As float (as_stride_m, as_stride_k); Bs float [E, ceil(N/128), K/128] (bs_stride_e, bs_stride_n,
+ * bs_stride_k); C [num_valid_tokens, N] of out_dtype (ldc).  block_m in {16,32,64,128} is the block size
+ * moe_align_block_size was called with; sorted_capacity = length of sorted_token_ids.  K % 128 == 0, N % 8 == 0.
+ */
+int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
+                        const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                        const int32_t* num_tokens_post_padded, const float* topk_weights, int64_t sorted_capacity,
+                        int64_t block_m, int64_t num_valid_tokens, int64_t top_k, int64_t num_experts, int64_t N,
+                        int64_t K, int64_t lda, int64_t as_stride_m, int64_t as_stride_k, int64_t b_stride_e,
+                        int64_t ldb, int64_t bs_stride_e, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc,
+                        int out_dtype, void* stream);
+
+/*
+ * out[r, c] = silu(x[r, c]) * x[r, d + c] for c < d, computed as the reference does for 16-bit types:
+ * silu in float32, rounded to the element type, multiplied, rounded again.
+ * Replaces torch.ops.sgl_kernel.silu_and_mul
+ *   (sgl-kernel/python/sgl_kernel/elementwise.py:172-184, sgl-kernel/csrc/elementwise/activation.cu:85-105,
+ *    sgl-kernel/include/hip/hip_act_and_mul.cuh:29-56).
+ * x [rows, 2d] (ldx elements between rows), out [rows, d] (ldo); d % 8 == 0; 16-byte aligned pointers.
+ */
+int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
+                      void* stream);
+
+/*
+ * out[t, :] = scale * sum_k x[t, k, :], float32 accumulation in ascending k, one rounding.
+ * Replaces torch.ops.sgl_kernel.moe_sum_reduce
+ *   (sgl-kernel/python/sgl_kernel/moe.py:83-92, sgl-kernel/csrc/moe/moe_sum_reduce.cu:56-113,227-).
+ * Strides in elements; hidden % 8 == 0.
+ */
+int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,
+                        int64_t stride_topk, int64_t out_stride_token, float scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

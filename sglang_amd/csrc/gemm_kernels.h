@@ -32,7 +32,8 @@ struct GemmArgs {
   const float* topk_w;          // routed weight per slot, or null
   int top_k;                    // X row of a slot = slot / top_k
   int num_valid;                // number of real slots (topk_ids.numel())
-  int m_blocks;                 // blocks of TM rows
+  int m_blocks;                 // dense: blocks of TM rows; grouped: capacity of sorted_ids in blocks
+  int block_m;                  // grouped: slots per block in sorted_ids (<= TM)
   int64_t w_expert_stride;      // bytes between experts in W
   int64_t sw_expert_stride;     // floats between experts in sw
 };
@@ -361,23 +362,36 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 
-  // ---- work item: consecutive ids walk the m blocks of one n tile (they share weight rows in L2)
-  const int nitems = p.tiles_n * p.m_blocks;
-  const int per_xcd = (nitems + 7) >> 3;
+  // ---- work item.  Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each).
+  // Dense: each XCD takes a contiguous run of items, consecutive ids walk the m blocks of one n tile.
+  // Grouped: the number of blocks in use is device data; each XCD takes a contiguous run of those
+  // blocks and walks all n tiles of a block before the next one, so the tiles that run together on
+  // an XCD share the block's activation rows, and the blocks of one expert share its weights.
   int bid = blockIdx.x;
   int split = 0;
-  if (SPLIT) { split = bid % p.splits; bid /= p.splits; }
-  const int t = (bid & 7) * per_xcd + (bid >> 3);
-  if (t >= nitems) return;
-  const int mb = t % p.m_blocks;
-  const int tile_n = t / p.m_blocks;
-  const int n0 = tile_n * kTileN;
-  const int slot0 = mb * TM;
-  int expert = 0;
+  int mb, tile_n;
   if (MOE) {
-    if (slot0 >= p.num_post_pad[0]) return;
-    expert = p.expert_ids[mb];
+    const int used = p.num_post_pad[0] / p.block_m;
+    const int per_xcd = (used + 7) >> 3;
+    const int j = bid >> 3;
+    const int mbl = j / p.tiles_n;
+    if (mbl >= per_xcd) return;
+    mb = (bid & 7) * per_xcd + mbl;
+    if (mb >= used || mb >= p.m_blocks) return;
+    tile_n = j - mbl * p.tiles_n;
+  } else {
+    const int nitems = p.tiles_n * p.m_blocks;
+    const int per_xcd = (nitems + 7) >> 3;
+    if (SPLIT) { split = bid % p.splits; bid /= p.splits; }
+    const int t = (bid & 7) * per_xcd + (bid >> 3);
+    if (t >= nitems) return;
+    mb = t % p.m_blocks;
+    tile_n = t / p.m_blocks;
   }
+  const int n0 = tile_n * kTileN;
+  const int block_m = MOE ? p.block_m : TM;
+  const int slot0 = mb * block_m;
+  const int expert = MOE ? p.expert_ids[mb] : 0;
   const int nrows = MOE ? p.num_valid : p.M;  // exclusive bound of a valid slot
 
   const int kb_begin = SPLIT ? split * p.kb_per_split : 0;
@@ -390,8 +404,8 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
   bool out_ok[MS];
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
-    const int s = slot0 + ms * 32 + lr;
-    out_slot[ms] = MOE ? p.sorted_ids[s] : s;
+    const int r = ms * 32 + lr;
+    out_slot[ms] = MOE ? (r < block_m ? p.sorted_ids[slot0 + r] : nrows) : slot0 + r;
     out_ok[ms] = out_slot[ms] < nrows;
   }
 
@@ -429,7 +443,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
     const int row = grp * 8 + rl;
     const int c = cp ^ (((grp & 1) << 2) + (rl >> 1));
     int s = nrows;
-    if (xload[j]) s = MOE ? p.sorted_ids[slot0 + row] : slot0 + row;
+    if (xload[j] && row < block_m) s = MOE ? p.sorted_ids[slot0 + row] : slot0 + row;
     const bool ok = s < nrows;
     const int64_t xr = MOE ? s / p.top_k : s;
     voX[j] = ok ? (uint32_t)(xr * p.ldx + c * 16) : 0xF0000000u;

@@ -1,0 +1,354 @@
+// Block-FP8 fused-MoE building blocks for gfx950: token alignment (integer), the grouped block-scaled
+// GEMM (host side; the device code is gemm_stream_kernel in gemm_kernels.h), silu_and_mul and the
+// top-k sum.  No allocation, no synchronisation, no host reads of device data.
+#include "gemm_kernels.h"
+
+namespace fp8k {
+
+// ------------------------------------------------------------------------------------------------
+// moe_align_block_size
+//
+// One workgroup of 1024 lanes: histogram of the bucket of every id (bucket = id + 1, bucket 0 holds
+// id -1) with LDS atomics, an exclusive scan of the counts rounded up to the block size by the first
+// wavefront, then per-block expert ids by binary search, the scatter of token slots through LDS
+// cursors and the padding tail of every bucket.  Ids outside [-1, buckets-1) are ignored.
+// With SCATTER = false the kernel stops after writing the start offsets to `cumsum`, and
+// moe_scatter_kernel (many workgroups, global atomics on `cumsum`) places the slots.
+// ------------------------------------------------------------------------------------------------
+constexpr int kAlignThreads = 1024;
+constexpr int kAlignMaxBuckets = 4096;
+
+template <typename IdT>
+__device__ __forceinline__ int bucket_of(const IdT* ids, int64_t i, int nb) {
+  const int64_t b = (int64_t)ids[i] + 1;
+  return (b >= 0 && b < nb) ? (int)b : -1;
+}
+
+template <typename IdT, bool SCATTER>
+__global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const IdT* __restrict__ ids, int64_t numel, int nb,
+                                                                  int block, int32_t* __restrict__ sorted,
+                                                                  int32_t* __restrict__ expert_ids,
+                                                                  int32_t* __restrict__ post_pad,
+                                                                  int32_t* __restrict__ cumsum, int pad_ids) {
+  __shared__ int32_t counts[kAlignMaxBuckets];
+  __shared__ int32_t prefix[kAlignMaxBuckets + 1];
+  __shared__ int32_t cursor[kAlignMaxBuckets];
+  const int tid = threadIdx.x;
+  for (int b = tid; b < nb; b += kAlignThreads) counts[b] = 0;
+  __syncthreads();
+  for (int64_t i = tid; i < numel; i += kAlignThreads) {
+    const int b = bucket_of(ids, i, nb);
+    if (b >= 0) atomicAdd(&counts[b], 1);
+  }
+  __syncthreads();
+  if (tid < 64) {
+    // lane l scans buckets [l*per, (l+1)*per)
+    const int per = (nb + 63) / 64;
+    const int b0 = tid * per;
+    int sum = 0;
+    for (int b = b0; b < min(nb, b0 + per); ++b) sum += (counts[b] + block - 1) / block * block;
+    int incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off);
+      if (tid >= off) incl += v;
+    }
+    int run = incl - sum;
+    for (int b = b0; b < min(nb, b0 + per); ++b) {
+      prefix[b] = run;
+      run += (counts[b] + block - 1) / block * block;
+    }
+    if (tid == 63) prefix[nb] = incl;
+  }
+  __syncthreads();
+  const int total = prefix[nb];
+  if (tid == 0) post_pad[0] = total;
+  for (int b = tid; b <= nb; b += kAlignThreads) {
+    if (cumsum) cumsum[b] = prefix[b];
+    if (b < nb) cursor[b] = prefix[b];
+  }
+  // expert of every block in use: the bucket whose [prefix[b], prefix[b+1]) range holds the block start
+  const int nblocks = total / block;
+  for (int i = tid; i < nblocks; i += kAlignThreads) {
+    const int start = i * block;
+    int lo = 0, hi = nb;  // first bucket with prefix[b+1] > start
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (prefix[mid + 1] <= start) lo = mid + 1;
+      else hi = mid;
+    }
+    expert_ids[i] = lo - 1;
+  }
+  if (pad_ids) {
+    for (int b = tid; b < nb; b += kAlignThreads)
+      for (int j = prefix[b] + counts[b]; j < prefix[b + 1]; ++j) sorted[j] = (int32_t)numel;
+  }
+  if (SCATTER) {
+    __syncthreads();
+    for (int64_t i = tid; i < numel; i += kAlignThreads) {
+      const int b = bucket_of(ids, i, nb);
+      if (b >= 0) sorted[atomicAdd(&cursor[b], 1)] = (int32_t)i;
+    }
+  }
+}
+
+template <typename IdT>
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const IdT* __restrict__ ids, int64_t numel, int nb,
+                                                          int32_t* __restrict__ sorted, int32_t* __restrict__ cumsum) {
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
+    const int b = bucket_of(ids, i, nb);
+    if (b >= 0) sorted[atomicAdd(&cumsum[b], 1)] = (int32_t)i;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// silu_and_mul: out[r, c] = T( T(silu_f32(x[r, c])) * x[r, d + c] ), T = bf16 / f16 (two roundings, as
+// the reference kernel computes Activation(x) * y on 16-bit values); float32 input has one rounding.
+// One lane handles 8 columns: two 16-byte loads, one 16-byte store.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+
+template <int DT>
+__device__ __forceinline__ float round_to(float v) {
+  if (DT == FP8K_BF16) return __uint_as_float(f32_to_bf16_bits(v) << 16);
+  if (DT == FP8K_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+  return v;
+}
+
+template <int DT>
+__device__ __forceinline__ void load8(const void* base, int64_t elem, float (&a)[8]) {
+  if (DT == FP8K_F32) {
+    const float4* p = reinterpret_cast<const float4*>((const float*)base + elem);
+    const float4 lo = p[0], hi = p[1];
+    a[0] = lo.x; a[1] = lo.y; a[2] = lo.z; a[3] = lo.w; a[4] = hi.x; a[5] = hi.y; a[6] = hi.z; a[7] = hi.w;
+  } else {
+    const uint4 v = *reinterpret_cast<const uint4*>((const u16*)base + elem);
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (DT == FP8K_BF16) { a[2 * i] = bf16_lo(w[i]); a[2 * i + 1] = bf16_hi(w[i]); }
+      else { a[2 * i] = f16_bits_to_f32(w[i] & 0xffff); a[2 * i + 1] = f16_bits_to_f32(w[i] >> 16); }
+    }
+  }
+}
+
+template <int DT>
+__device__ __forceinline__ void store8(void* base, int64_t elem, const float (&a)[8]) {
+  if (DT == FP8K_F32) {
+    float4* p = reinterpret_cast<float4*>((float*)base + elem);
+    p[0] = make_float4(a[0], a[1], a[2], a[3]);
+    p[1] = make_float4(a[4], a[5], a[6], a[7]);
+  } else {
+    uint32_t w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (DT == FP8K_BF16) w[i] = pack_bf16x2(a[2 * i], a[2 * i + 1]);
+      else w[i] = f32_to_f16_bits(a[2 * i]) | (f32_to_f16_bits(a[2 * i + 1]) << 16);
+    }
+    *reinterpret_cast<uint4*>((u16*)base + elem) = make_uint4(w[0], w[1], w[2], w[3]);
+  }
+}
+
+template <int DT>
+__global__ __launch_bounds__(256) void silu_and_mul_kernel(const void* __restrict__ x, void* __restrict__ out,
+                                                           int64_t rows, int d, int64_t ldx, int64_t ldo) {
+  const int chunks = d / 8;
+  const int64_t total = rows * chunks;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / chunks;
+    const int c = (int)(i - r * chunks) * 8;
+    float g[8], u[8], o[8];
+    load8<DT>(x, r * ldx + c, g);
+    load8<DT>(x, r * ldx + d + c, u);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) o[k] = round_to<DT>(silu_f32(g[k])) * u[k];
+    store8<DT>(out, r * ldo + c, o);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------
+// moe_sum_reduce: out[t, :] = T( scale * sum_k float(x[t, k, :]) ), k ascending, float32 accumulate
+// ------------------------------------------------------------------------------------------------
+template <int DT>
+__global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const void* __restrict__ x, void* __restrict__ out,
+                                                             int64_t tokens, int topk, int hidden, int64_t stride_t,
+                                                             int64_t stride_k, int64_t out_stride_t, float scale) {
+  const int chunks = hidden / 8;
+  const int64_t total = tokens * chunks;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const int64_t t = i / chunks;
+    const int c = (int)(i - t * chunks) * 8;
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+    for (int k = 0; k < topk; ++k) {
+      float v[8];
+      load8<DT>(x, t * stride_t + (int64_t)k * stride_k + c, v);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] += v[j];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] *= scale;
+    store8<DT>(out, t * out_stride_t + c, acc);
+  }
+}
+
+static unsigned stream_grid(int64_t work_items) {
+  const int64_t want = (work_items + 255) / 256;
+  return (unsigned)(want < 1 ? 1 : (want > 256 * 16 ? 256 * 16 : want));
+}
+
+}  // namespace fp8k
+
+using namespace fp8k;
+
+extern "C" int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64, int64_t numel, int64_t num_buckets,
+                                         int64_t block_size, int32_t* sorted_token_ids, int64_t sorted_capacity,
+                                         int32_t* expert_ids, int64_t expert_capacity, int32_t* num_tokens_post_pad,
+                                         int32_t* cumsum_buffer, int pad_sorted_token_ids, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(numel >= 0 && numel < 0x7fffffffLL, "moe_align_block_size: bad number of ids (%lld)", (long long)numel);
+  FP8K_REQUIRE(num_buckets >= 1 && num_buckets <= kAlignMaxBuckets,
+               "moe_align_block_size: num_experts must be in [1, %d] (got %lld)", kAlignMaxBuckets, (long long)num_buckets);
+  FP8K_REQUIRE(block_size >= 1 && block_size <= 1024, "moe_align_block_size: block_size must be in [1, 1024]");
+  // worst case: every bucket in use carries block_size-1 padding slots
+  const int64_t used_buckets = numel < num_buckets ? numel : num_buckets;
+  const int64_t worst = numel + used_buckets * (block_size - 1);
+  FP8K_REQUIRE(sorted_capacity >= worst, "moe_align_block_size: sorted_token_ids holds %lld slots, %lld may be needed",
+               (long long)sorted_capacity, (long long)worst);
+  FP8K_REQUIRE(expert_capacity >= worst / block_size,
+               "moe_align_block_size: experts_ids holds %lld blocks, %lld may be needed", (long long)expert_capacity,
+               (long long)(worst / block_size));
+  FP8K_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_pad, "moe_align_block_size: null output pointer");
+  FP8K_REQUIRE(numel == 0 || topk_ids, "moe_align_block_size: null topk_ids");
+  hipStream_t st = (hipStream_t)stream;
+  const bool fused = numel <= 65536 || !cumsum_buffer;
+#define FP8K_ALIGN(T)                                                                                                \
+  do {                                                                                                               \
+    if (fused) {                                                                                                     \
+      hipLaunchKernelGGL((moe_align_kernel<T, true>), dim3(1), dim3(kAlignThreads), 0, st, (const T*)topk_ids, numel, \
+                         (int)num_buckets, (int)block_size, sorted_token_ids, expert_ids, num_tokens_post_pad,        \
+                         cumsum_buffer, pad_sorted_token_ids);                                                        \
+    } else {                                                                                                         \
+      hipLaunchKernelGGL((moe_align_kernel<T, false>), dim3(1), dim3(kAlignThreads), 0, st, (const T*)topk_ids, numel, \
+                         (int)num_buckets, (int)block_size, sorted_token_ids, expert_ids, num_tokens_post_pad,        \
+                         cumsum_buffer, pad_sorted_token_ids);                                                        \
+      hipLaunchKernelGGL((moe_scatter_kernel<T>), dim3(stream_grid(numel)), dim3(256), 0, st, (const T*)topk_ids,     \
+                         numel, (int)num_buckets, sorted_token_ids, cumsum_buffer);                                   \
+    }                                                                                                                \
+  } while (0)
+  if (ids_are_int64) FP8K_ALIGN(int64_t);
+  else FP8K_ALIGN(int32_t);
+#undef FP8K_ALIGN
+  return check_launch("moe_align_block_size");
+}
+
+extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
+                                   const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                   const int32_t* num_tokens_post_padded, const float* topk_weights,
+                                   int64_t sorted_capacity, int64_t block_m, int64_t num_valid_tokens, int64_t top_k,
+                                   int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_m,
+                                   int64_t as_stride_k, int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e,
+                                   int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* stream) {
+  clear_error();
+  const char* op = "moe_block_gemm";
+  FP8K_REQUIRE(N > 0 && K > 0 && num_experts > 0 && top_k > 0, "%s: bad shape", op);
+  FP8K_REQUIRE(N <= 0x7fffffffLL && K <= 0x7fffffffLL && num_valid_tokens >= 0 && num_valid_tokens < 0x7fffffffLL,
+               "%s: shape too large", op);
+  FP8K_REQUIRE(out_dtype == FP8K_F16 || out_dtype == FP8K_BF16, "%s: out_dtype must be Half or BFloat16", op);
+  FP8K_REQUIRE(K % kTileK == 0, "%s: K (%lld) must be a multiple of 128", op, (long long)K);
+  FP8K_REQUIRE(N % 8 == 0, "%s: N (%lld) must be a multiple of 8", op, (long long)N);
+  FP8K_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128,
+               "%s: block_m must be 16, 32, 64 or 128 (got %lld)", op, (long long)block_m);
+  FP8K_REQUIRE(sorted_capacity >= 0 && sorted_capacity < 0x7fffffffLL, "%s: bad sorted_token_ids length", op);
+  FP8K_REQUIRE(lda >= K && ldb >= K && ldc >= N, "%s: leading dimension smaller than the row length", op);
+  FP8K_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && (ldc * 2) % 8 == 0, "%s: rows must be 16-byte aligned", op);
+  if (num_valid_tokens == 0 || sorted_capacity < block_m) return FP8K_OK;
+  FP8K_REQUIRE(A && B && As && Bs && C && sorted_token_ids && expert_ids && num_tokens_post_padded, "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(A, 16) && aligned(B, 16) && aligned(C, 8) && b_stride_e % 16 == 0,
+               "%s: operands must be 16-byte aligned", op);
+  const int64_t xrows = (num_valid_tokens + top_k - 1) / top_k;
+  FP8K_REQUIRE(xrows * lda < 0xE0000000LL, "%s: activation matrix exceeds 3.5 GiB, split the token batch", op);
+  FP8K_REQUIRE(256 * ldb + K < 0xE0000000LL, "%s: weight rows too long", op);
+  FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0 && bs_stride_e >= 0,
+               "%s: negative scale stride", op);
+
+  GemmArgs a{};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.sx = As; a.sw = Bs; a.C = C;
+  a.M = (int)num_valid_tokens; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.sx_m = as_stride_m; a.sx_k = as_stride_k; a.sw_n = bs_stride_n; a.sw_k = bs_stride_k;
+  a.tiles_m = 0; a.tiles_n = (int)((N + kTileN - 1) / kTileN);
+  a.splits = 1; a.kb_per_split = (int)(K / kTileK);
+  a.sorted_ids = sorted_token_ids; a.expert_ids = expert_ids; a.num_post_pad = num_tokens_post_padded;
+  a.topk_w = topk_weights; a.top_k = (int)top_k; a.num_valid = (int)num_valid_tokens;
+  a.m_blocks = (int)(sorted_capacity / block_m);
+  a.block_m = (int)block_m;
+  a.w_expert_stride = b_stride_e; a.sw_expert_stride = bs_stride_e;
+  const int64_t per_xcd = (a.m_blocks + 7) / 8;
+  const int64_t nwg = per_xcd * 8 * a.tiles_n;
+  FP8K_REQUIRE(nwg < 0x7fffffffLL, "%s: grid too large", op);
+  hipStream_t st = (hipStream_t)stream;
+#define FP8K_MOE(TM, NST, O) \
+  hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, kModeBlock, O, FP8K_F32, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a)
+  if (out_dtype == FP8K_BF16) {
+    if (block_m <= 32) FP8K_MOE(32, 4, FP8K_BF16);
+    else if (block_m == 64) FP8K_MOE(64, 3, FP8K_BF16);
+    else FP8K_MOE(128, 3, FP8K_BF16);
+  } else {
+    if (block_m <= 32) FP8K_MOE(32, 4, FP8K_F16);
+    else if (block_m == 64) FP8K_MOE(64, 3, FP8K_F16);
+    else FP8K_MOE(128, 3, FP8K_F16);
+  }
+#undef FP8K_MOE
+  return check_launch(op);
+}
+
+extern "C" int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
+                                 void* stream) {
+  clear_error();
+  FP8K_REQUIRE(rows >= 0 && d >= 0, "silu_and_mul: negative shape");
+  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "silu_and_mul: bad dtype %d", dtype);
+  FP8K_REQUIRE(d % 8 == 0 && d <= 0x7fffffffLL, "silu_and_mul: the output width (%lld) must be a multiple of 8", (long long)d);
+  FP8K_REQUIRE(ldx >= 2 * d && ldo >= d && ldx % 8 == 0 && ldo % 8 == 0, "silu_and_mul: bad row strides");
+  if (rows == 0 || d == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && out, "silu_and_mul: null pointer");
+  FP8K_REQUIRE(aligned(x, 16) && aligned(out, 16), "silu_and_mul: The pointers must be multiple of 16 bytes.");
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(stream_grid(rows * (d / 8))), block(256);
+  switch (dtype) {
+    case FP8K_BF16: hipLaunchKernelGGL(silu_and_mul_kernel<FP8K_BF16>, grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
+    case FP8K_F16: hipLaunchKernelGGL(silu_and_mul_kernel<FP8K_F16>, grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
+    default: hipLaunchKernelGGL(silu_and_mul_kernel<FP8K_F32>, grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
+  }
+  return check_launch("silu_and_mul");
+}
+
+extern "C" int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden,
+                                   int64_t stride_token, int64_t stride_topk, int64_t out_stride_token, float scale,
+                                   int dtype, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(tokens >= 0 && topk >= 0 && hidden >= 0, "moe_sum_reduce: negative shape");
+  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "moe_sum_reduce: bad dtype %d", dtype);
+  FP8K_REQUIRE(hidden % 8 == 0 && hidden <= 0x7fffffffLL && topk <= 0x7fffffffLL,
+               "moe_sum_reduce: hidden size (%lld) must be a multiple of 8", (long long)hidden);
+  FP8K_REQUIRE(stride_token % 8 == 0 && stride_topk % 8 == 0 && out_stride_token % 8 == 0 && stride_topk >= hidden &&
+                   out_stride_token >= hidden,
+               "moe_sum_reduce: strides must be multiples of 8 elements and cover a row");
+  if (tokens == 0 || hidden == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && out, "moe_sum_reduce: null pointer");
+  FP8K_REQUIRE(aligned(x, 16) && aligned(out, 16), "moe_sum_reduce: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(stream_grid(tokens * (hidden / 8))), block(256);
+#define FP8K_SR(DT) \
+  hipLaunchKernelGGL(moe_sum_reduce_kernel<DT>, grid, block, 0, st, x, out, tokens, (int)topk, (int)hidden, stride_token, stride_topk, out_stride_token, scale)
+  switch (dtype) {
+    case FP8K_BF16: FP8K_SR(FP8K_BF16); break;
+    case FP8K_F16: FP8K_SR(FP8K_F16); break;
+    default: FP8K_SR(FP8K_F32); break;
+  }
+#undef FP8K_SR
+  return check_launch("moe_sum_reduce");
+}

@@ -1,0 +1,248 @@
+"""Block-FP8 fused-experts pipeline behind the reference's Python interface.
+
+Mirrors ``sglang.srt.layers.moe.fused_moe_triton`` for the one configuration this path builds:
+``use_fp8_w8a8=True`` with ``block_shape=[128, 128]`` (DeepSeek-V3 style experts).  Sequence, as in
+fused_moe.py:498-639 of the reference:
+
+    moe_align_block_size -> quant + grouped GEMM (w13) -> silu_and_mul -> quant + grouped GEMM (w2,
+    times the routed weight) -> sum over top-k (times routed_scaling_factor)
+
+Every stage is a call into libfp8k.so; intermediates are torch tensors on the current stream.
+"""
+from __future__ import annotations
+
+from typing import Any, Dict, List, Optional, Tuple
+
+import torch
+
+from . import sgl_kernel as _ops
+from .fp8_kernel import sglang_per_token_group_quant_fp8
+
+CHUNK_SIZE = 64 * 1024  # tokens per pass, as in the reference (fused_moe.py:423)
+
+
+def moe_align_block_size(
+    topk_ids: torch.Tensor, block_size: int, num_experts: int
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Reference: python/sglang/srt/layers/moe/fused_moe_triton/moe_align_block_size.py:17-82.
+
+    Returns (sorted_token_ids [numel + (E+1)(B-1)], expert_ids [ceil(that/B)], num_tokens_post_padded [1]).
+    Padding slots hold topk_ids.numel(); expert -1 (not on this rank) gets its own leading blocks.
+    """
+    max_num_tokens_padded = topk_ids.numel() + (num_experts + 1) * (block_size - 1)
+    sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=topk_ids.device)
+    max_num_m_blocks = (max_num_tokens_padded + block_size - 1) // block_size
+    expert_ids = torch.empty((max_num_m_blocks,), dtype=torch.int32, device=topk_ids.device)
+    num_tokens_post_pad = torch.empty((1,), dtype=torch.int32, device=topk_ids.device)
+    cumsum_buffer = torch.empty((num_experts + 2,), dtype=torch.int32, device=topk_ids.device)
+    _ops.moe_align_block_size(
+        topk_ids, num_experts + 1, block_size, sorted_ids, expert_ids, num_tokens_post_pad, cumsum_buffer, True
+    )
+    return sorted_ids, expert_ids, num_tokens_post_pad
+
+
+def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
+    """Rows per block of the grouped GEMM (the reference's BLOCK_SIZE_M, fused_moe_triton_config.py).
+
+    The grouped kernel streams a 256-row weight tile once per block of rows, so the block should hold
+    all rows an expert is expected to receive, up to the kernel's 128-row limit.
+    """
+    per_expert = (M * topk + E - 1) // max(E, 1)
+    if per_expert <= 32:
+        bm = 32
+    elif per_expert <= 64:
+        bm = 64
+    else:
+        bm = 128
+    return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}
+
+
+def invoke_fused_moe_kernel(
+    A: torch.Tensor,
+    B: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    C: torch.Tensor,
+    A_scale: Optional[torch.Tensor],
+    B_scale: Optional[torch.Tensor],
+    B_zp: Optional[torch.Tensor],
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    sorted_token_ids: torch.Tensor,
+    expert_ids: torch.Tensor,
+    num_tokens_post_padded: torch.Tensor,
+    mul_routed_weight: bool,
+    top_k: int,
+    config: Dict[str, Any],
+    compute_type=None,
+    use_fp8_w8a8: bool = True,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    block_shape: Optional[List[int]] = None,
+    no_combine: bool = False,
+    a_use_tma: bool = False,
+    b_use_tma: bool = False,
+    c_sorted: bool = False,
+    filter_expert: bool = True,
+) -> None:
+    """Reference: fused_moe_triton_kernels.py:586-790.  A is bf16/fp16 and is group-quantised here
+    (as the reference does, :627-637) unless it already is e4m3fn with A_scale given."""
+    assert topk_weights.stride(1) == 1
+    assert sorted_token_ids.stride(0) == 1
+    if not use_fp8_w8a8 or use_int8_w8a8 or use_int8_w8a16 or use_int4_w4a16 or per_channel_quant:
+        raise RuntimeError("invoke_fused_moe_kernel: only use_fp8_w8a8 with block_shape [128, 128] is built on this path")
+    if block_shape is None or list(block_shape) != [128, 128]:
+        raise RuntimeError("invoke_fused_moe_kernel: block_shape must be [128, 128]")
+    if bias is not None or B_zp is not None or c_sorted or a_use_tma or b_use_tma:
+        raise RuntimeError("invoke_fused_moe_kernel: bias, zero points and the TMA layouts are not built on this path")
+    assert B_scale is not None
+    if A.dtype != torch.float8_e4m3fn:
+        assert A_scale is None
+        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1])
+    assert (A.shape[-1] + 127) // 128 == A_scale.shape[-1]
+    assert (B.shape[-2] + 127) // 128 == B_scale.shape[-2]
+    assert (B.shape[-1] + 127) // 128 == B_scale.shape[-1]
+    _ops.moe_block_gemm(
+        A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
+        mul_routed_weight, top_k, int(config["BLOCK_SIZE_M"]), topk_ids.numel(),
+    )
+
+
+def fused_experts_impl(
+    hidden_states: torch.Tensor,
+    w1: torch.Tensor,
+    w2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    b1: Optional[torch.Tensor] = None,
+    b2: Optional[torch.Tensor] = None,
+    inplace: bool = False,
+    activation: str = "silu",
+    is_gated: bool = True,
+    apply_router_weight_on_input: bool = False,
+    use_fp8_w8a8: bool = False,
+    use_int8_w8a8: bool = False,
+    use_int8_w8a16: bool = False,
+    use_int4_w4a16: bool = False,
+    per_channel_quant: bool = False,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    w1_zp: Optional[torch.Tensor] = None,
+    w2_zp: Optional[torch.Tensor] = None,
+    a1_scale: Optional[torch.Tensor] = None,
+    a2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+    no_combine: bool = False,
+    routed_scaling_factor: Optional[float] = None,
+    gemm1_alpha: Optional[float] = None,
+    gemm1_limit: Optional[float] = None,
+    filter_expert: bool = True,
+) -> torch.Tensor:
+    """Reference: fused_moe.py:369-660.  hidden_states [T,H] bf16/fp16; w1 e4m3fn [E,2I,H]; w2 e4m3fn
+    [E,H,I]; w1_scale/w2_scale float32 per 128x128 block; topk_weights float32 [T,k]; topk_ids int [T,k]
+    (-1 = expert on another rank, contributes zero)."""
+    if not use_fp8_w8a8 or block_shape is None:
+        raise RuntimeError("fused_experts_impl: only use_fp8_w8a8=True with block_shape=[128, 128] is built on this path")
+    if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None:
+        raise RuntimeError("fused_experts_impl: only the gated silu activation is built on this path")
+    if apply_router_weight_on_input or b1 is not None or b2 is not None or a1_scale is not None or a2_scale is not None:
+        raise RuntimeError("fused_experts_impl: router weight on input, biases and static activation scales are not built")
+    assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
+    assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype in [torch.float16, torch.bfloat16]
+
+    num_tokens, _ = hidden_states.shape
+    E, N, _ = w1.shape
+    topk = topk_ids.shape[1]
+    M = min(num_tokens, CHUNK_SIZE)
+    dev, dt = hidden_states.device, hidden_states.dtype
+    if topk_weights.dtype != torch.float32:
+        topk_weights = topk_weights.float()
+    topk_weights = topk_weights.contiguous()
+    topk_ids = topk_ids.contiguous()
+
+    cache1 = torch.empty((M * topk, N), device=dev, dtype=dt)
+    cache2 = torch.empty((M * topk, N // 2), device=dev, dtype=dt)
+    cache3 = torch.empty((M, topk, w2.shape[1]), device=dev, dtype=dt)
+    if no_combine:
+        assert not inplace
+        out_hidden_states = torch.empty((num_tokens, topk, w2.shape[1]), device=dev, dtype=dt)
+    elif inplace:
+        out_hidden_states = hidden_states
+    else:
+        out_hidden_states = torch.empty_like(hidden_states)
+    if routed_scaling_factor is None:
+        routed_scaling_factor = 1.0
+
+    for chunk in range((num_tokens // CHUNK_SIZE) + 1):
+        begin, end = chunk * CHUNK_SIZE, min((chunk + 1) * CHUNK_SIZE, num_tokens)
+        curr = hidden_states[begin:end]
+        tokens = curr.shape[0]
+        if tokens == 0:
+            break
+        config = get_default_config(tokens, E, topk)
+        curr_ids = topk_ids[begin:end]
+        curr_w = topk_weights[begin:end]
+        ic1 = cache1[: tokens * topk]
+        ic2 = cache2[: tokens * topk]
+        ic3 = out_hidden_states[begin:end] if no_combine else cache3[:tokens]
+
+        sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(curr_ids, config["BLOCK_SIZE_M"], E)
+        invoke_fused_moe_kernel(
+            curr, w1, None, ic1, None, w1_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
+            num_tokens_post_padded, False, topk, config, use_fp8_w8a8=True, block_shape=block_shape,
+        )
+        _ops.silu_and_mul(ic1, ic2)
+        invoke_fused_moe_kernel(
+            ic2, w2, None, ic3, None, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
+            num_tokens_post_padded, True, 1, config, use_fp8_w8a8=True, block_shape=block_shape,
+        )
+        if not no_combine:
+            _ops.moe_sum_reduce(ic3, out_hidden_states[begin:end], routed_scaling_factor)
+    return out_hidden_states
+
+
+def fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, **kwargs) -> torch.Tensor:
+    """Out-of-place fused experts (the reference's outplace_fused_experts, fused_moe.py:180-245)."""
+    kwargs.pop("inplace", None)
+    return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, **kwargs)
+
+
+def biased_grouped_topk_impl(
+    hidden_states: torch.Tensor,
+    gating_output: torch.Tensor,
+    correction_bias: torch.Tensor,
+    topk: int,
+    renormalize: bool,
+    num_expert_group: Optional[int] = None,
+    topk_group: Optional[int] = None,
+    routed_scaling_factor: Optional[float] = None,
+    apply_routed_scaling_factor_on_output: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Routing harness in plain torch (reference: python/sglang/srt/layers/moe/topk.py:665-738): sigmoid
+    scores, group score = sum of the two best biased scores, keep topk_group groups, top-k experts
+    among them, weights = un-biased scores, renormalised.  Not a kernel of this path."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    scores = gating_output.sigmoid()
+    num_token = scores.shape[0]
+    scores_for_choice = scores.view(num_token, -1) + correction_bias.unsqueeze(0)
+    group_scores = scores_for_choice.view(num_token, num_expert_group, -1).topk(2, dim=-1)[0].sum(dim=-1)
+    group_idx = torch.topk(group_scores, k=topk_group, dim=-1, sorted=False)[1]
+    group_mask = torch.zeros_like(group_scores)
+    group_mask.scatter_(1, group_idx, 1)
+    score_mask = (
+        group_mask.unsqueeze(-1).expand(num_token, num_expert_group, scores.shape[-1] // num_expert_group)
+        .reshape(num_token, -1)
+    )
+    tmp_scores = scores_for_choice.masked_fill(~score_mask.bool(), float("-inf"))
+    _, topk_ids = torch.topk(tmp_scores, k=topk, dim=-1, sorted=False)
+    topk_weights = scores.gather(1, topk_ids)
+    if renormalize:
+        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+        if apply_routed_scaling_factor_on_output:
+            topk_weights = topk_weights * routed_scaling_factor
+    return topk_weights.to(torch.float32), topk_ids.to(torch.int32)

@@ -285,3 +285,129 @@ def _block_gemm_nk(A, B, As, Bs, out_dtype):
         )
     )
     return out
+
+
+# --------------------------------------------------------------------------------------------
+# fused-MoE helpers
+# --------------------------------------------------------------------------------------------
+
+
+def moe_align_block_size(
+    topk_ids: torch.Tensor,
+    num_experts: int,
+    block_size: int,
+    sorted_token_ids: torch.Tensor,
+    experts_ids: torch.Tensor,
+    num_tokens_post_pad: torch.Tensor,
+    cumsum_buffer: Optional[torch.Tensor],
+    pad_sorted_token_ids: bool = False,
+) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:6-25; csrc/moe/moe_align_kernel.cu:302-366.
+
+    `num_experts` is the number of buckets: the Python caller passes E+1 so that id -1 (an expert
+    on another rank) lands in bucket 0 and expert e in bucket e+1.  All outputs are caller-allocated.
+    """
+    require_cuda(topk_ids, sorted_token_ids, experts_ids, num_tokens_post_pad, cumsum_buffer)
+    if topk_ids.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("topk_ids must be int32 or int64")
+    if not topk_ids.is_contiguous():
+        raise RuntimeError("topk_ids must be contiguous")
+    for t, name in ((sorted_token_ids, "sorted_token_ids"), (experts_ids, "experts_ids"),
+                    (num_tokens_post_pad, "num_tokens_post_pad")):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("%s must be a contiguous int32 tensor" % name)
+    if cumsum_buffer is not None:
+        if cumsum_buffer.dtype != torch.int32 or cumsum_buffer.numel() < num_experts + 1:
+            raise RuntimeError("cumsum_buffer must be int32 with at least num_experts + 1 entries")
+    check(
+        lib.fp8k_moe_align_block_size(
+            topk_ids.data_ptr(), 1 if topk_ids.dtype == torch.int64 else 0, topk_ids.numel(), num_experts, block_size,
+            sorted_token_ids.data_ptr(), sorted_token_ids.numel(), experts_ids.data_ptr(), experts_ids.numel(),
+            num_tokens_post_pad.data_ptr(), cumsum_buffer.data_ptr() if cumsum_buffer is not None else None,
+            1 if pad_sorted_token_ids else 0, stream_ptr(topk_ids.device),
+        )
+    )
+
+
+def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Reference: sgl-kernel/python/sgl_kernel/elementwise.py:172-184."""
+    if input.shape[-1] * input.dtype.itemsize % 16 != 0:
+        raise ValueError("The pointers must be multiple of 16 bytes.")
+    if out is not None:
+        assert input.ndim == out.ndim, f"{input.ndim} != {out.ndim}"
+        assert input.shape[:-1] == out.shape[:-1], f"{input.shape[:-1]} != {out.shape[:-1]}"
+        assert input.shape[-1] == 2 * out.shape[-1], f"{input.shape[-1]} != {2 * out.shape[-1]}"
+    else:
+        out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
+    require_cuda(input, out)
+    if out.dtype != input.dtype:
+        raise RuntimeError("silu_and_mul: out must have the dtype of input")
+    if not (input.is_contiguous() and out.is_contiguous()):
+        raise RuntimeError("silu_and_mul: input and out must be contiguous")
+    d = out.shape[-1]
+    rows = out.numel() // d if d else 0
+    check(lib.fp8k_silu_and_mul(input.data_ptr(), out.data_ptr(), rows, d, 2 * d, d, dtype_code(input.dtype),
+                                stream_ptr(input.device)))
+    return out
+
+
+def moe_sum_reduce(input_tensor: torch.Tensor, output_tensor: torch.Tensor, routed_scaling_factor: float = 0) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:83-92; csrc/moe/moe_sum_reduce.cu:227-.
+    input [tokens, topk, hidden] (hidden contiguous), output [tokens, hidden]."""
+    require_cuda(input_tensor, output_tensor)
+    if input_tensor.dim() != 3 or output_tensor.dim() != 2:
+        raise RuntimeError("moe_sum_reduce: input must be [tokens, topk, hidden] and output [tokens, hidden]")
+    T, topk, H = input_tensor.shape
+    if output_tensor.shape[0] != T or output_tensor.shape[1] != H:
+        raise RuntimeError("moe_sum_reduce: output shape does not match the input")
+    if input_tensor.dtype != output_tensor.dtype:
+        raise RuntimeError("moe_sum_reduce: input and output dtypes differ")
+    if (H > 1 and input_tensor.stride(2) != 1) or (H > 1 and output_tensor.stride(1) != 1):
+        raise RuntimeError("moe_sum_reduce: the hidden dimension must be contiguous")
+    check(lib.fp8k_moe_sum_reduce(input_tensor.data_ptr(), output_tensor.data_ptr(), T, topk, H, input_tensor.stride(0),
+                                  input_tensor.stride(1), output_tensor.stride(0), float(routed_scaling_factor),
+                                  dtype_code(input_tensor.dtype), stream_ptr(input_tensor.device)))
+
+
+def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                   mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int) -> None:
+    """Grouped block-FP8 GEMM behind invoke_fused_moe_kernel (see include/fp8k.h: fp8k_moe_block_gemm).
+    A e4m3fn [rows, K]; B e4m3fn [E, N, K]; A_scale float32 [rows, K/128]; B_scale float32 [E, N/128, K/128];
+    C [num_valid_tokens, N] (any leading shape, flattened) bf16/fp16, written in place."""
+    require_cuda(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
+        raise RuntimeError("moe_block_gemm: A and B must be Float8_e4m3fn")
+    if A_scale.dtype != torch.float32 or B_scale.dtype != torch.float32:
+        raise RuntimeError("moe_block_gemm: scales must be Float32")
+    if B.dim() != 3 or B_scale.dim() != 3 or A.dim() != 2 or A_scale.dim() != 2:
+        raise RuntimeError("moe_block_gemm: A [rows,K], B [E,N,K], A_scale [rows,K/128], B_scale [E,N/128,K/128]")
+    E, N, K = B.shape
+    if A.shape[1] != K or (K > 1 and (A.stride(1) != 1 or B.stride(2) != 1)):
+        raise RuntimeError("moe_block_gemm: K must be the contiguous dimension of A and B")
+    if A_scale.shape[0] != A.shape[0] or A_scale.shape[1] != (K + 127) // 128:
+        raise RuntimeError("moe_block_gemm: A_scale shape does not match A")
+    if B_scale.shape[0] != E or B_scale.shape[1] != (N + 127) // 128 or B_scale.shape[2] != (K + 127) // 128:
+        raise RuntimeError("moe_block_gemm: B_scale shape does not match B")
+    C2 = C.view(-1, C.shape[-1])
+    if C2.shape[1] != N or C2.shape[0] < num_valid_tokens or C2.stride(1) != 1:
+        raise RuntimeError("moe_block_gemm: C must be [num_valid_tokens, N] with N contiguous")
+    if A.shape[0] * top_k < num_valid_tokens:
+        raise RuntimeError("moe_block_gemm: A has too few rows for num_valid_tokens / top_k")
+    if mul_routed_weight:
+        if topk_weights.dtype != torch.float32 or not topk_weights.is_contiguous() or topk_weights.numel() < num_valid_tokens:
+            raise RuntimeError("moe_block_gemm: topk_weights must be contiguous Float32 with one entry per slot")
+    for t in (sorted_token_ids, expert_ids, num_tokens_post_padded):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("moe_block_gemm: index tensors must be contiguous int32")
+    if expert_ids.numel() * block_m < sorted_token_ids.numel() - (sorted_token_ids.numel() % block_m):
+        raise RuntimeError("moe_block_gemm: expert_ids is shorter than sorted_token_ids / block_m")
+    check(
+        lib.fp8k_moe_block_gemm(
+            A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C2.data_ptr(),
+            sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(),
+            topk_weights.data_ptr() if mul_routed_weight else None, sorted_token_ids.numel(), block_m,
+            num_valid_tokens, top_k, E, N, K, A.stride(0), A_scale.stride(0), A_scale.stride(1), B.stride(0),
+            B.stride(1), B_scale.stride(0), B_scale.stride(1), B_scale.stride(2), C2.stride(0), _out_code(C.dtype),
+            stream_ptr(A.device),
+        )
+    )

@@ -1,0 +1,319 @@
+"""GPU parity of the fused-MoE stages against the CPU oracle.
+
+Integer stage (moe_align_block_size): exact, compared through the invariants the reference's own test
+uses (sgl-kernel/tests/test_moe_align.py:210-254) because the order inside an expert is unspecified.
+Floating-point stages: silu_and_mul within one bf16 ulp of the oracle (device expf vs numpy exp),
+moe_sum_reduce exact (same float32 summation order), grouped GEMM and the whole layer within the
+path's 1e-2 max-relative-error bound.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from tests.conftest import bf16_tensor, fp8_tensor
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _rel_err(c, ref):
+    return float(np.abs(c.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def _random_ids(rng, T, E, topk, frac_minus1=0.0):
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    if frac_minus1:
+        ids[rng.random(ids.shape) < frac_minus1] = -1
+    return ids
+
+
+def _check_align(ids, E, block, sorted_ids, expert_ids, npad):
+    numel = ids.size
+    flat = ids.reshape(-1)
+    counts = np.bincount(flat + 1, minlength=E + 1)
+    assert npad == sum((c + block - 1) // block * block for c in counts)
+    ref_sorted, ref_experts, ref_npad = O.moe_align_block_size(ids, block, E)
+    assert npad == ref_npad
+    used = expert_ids[: npad // block]
+    np.testing.assert_array_equal(used, ref_experts[: npad // block])
+    for b in range(npad // block):
+        blk = sorted_ids[b * block : (b + 1) * block]
+        ref_blk = ref_sorted[b * block : (b + 1) * block]
+        # same members, real slots first then padding
+        nreal = int((ref_blk < numel).sum())
+        assert (blk[nreal:] == numel).all()
+        assert (blk[:nreal] < numel).all()
+    # every slot appears exactly once; per-expert ranges hold exactly that expert's slots (as sets)
+    real = sorted_ids[:npad][sorted_ids[:npad] < numel]
+    np.testing.assert_array_equal(np.sort(real), np.arange(numel))
+    start = 0
+    for bkt in range(E + 1):
+        c = counts[bkt]
+        padded = (c + block - 1) // block * block
+        seg = sorted_ids[start : start + padded]
+        np.testing.assert_array_equal(np.sort(seg[:c]), np.nonzero(flat + 1 == bkt)[0])
+        assert (seg[c:] == numel).all()
+        start += padded
+
+
+@pytest.mark.parametrize("T,E,topk,block", [(1, 256, 8, 32), (7, 8, 2, 16), (97, 64, 6, 64), (4096, 256, 8, 128),
+                                           (333, 257, 8, 64), (9000, 256, 8, 64), (33, 16, 1, 128)])
+@pytest.mark.parametrize("id_dtype", [torch.int32, torch.int64])
+def test_moe_align_block_size(dev, T, E, topk, block, id_dtype):
+    from sglang_amd.fused_moe import moe_align_block_size
+
+    rng = np.random.default_rng(T + E)
+    ids = _random_ids(rng, T, E, topk, 0.05 if T > 1 else 0.0)
+    t_ids = torch.from_numpy(ids).to(dev).to(id_dtype)
+    sorted_ids, expert_ids, npad = moe_align_block_size(t_ids, block, E)
+    torch.cuda.synchronize()
+    assert sorted_ids.numel() == ids.size + (E + 1) * (block - 1)
+    assert expert_ids.numel() == (sorted_ids.numel() + block - 1) // block
+    _check_align(ids, E, block, sorted_ids.cpu().numpy(), expert_ids.cpu().numpy(), int(npad.item()))
+
+
+def test_moe_align_skewed_and_unpadded(dev):
+    """All ids on one expert; pad_sorted_token_ids=False leaves the padding slots untouched."""
+    from sglang_amd import sgl_kernel as ops
+
+    E, block = 32, 64
+    ids = np.full((500, 4), 5, dtype=np.int32)
+    t_ids = torch.from_numpy(ids).to(dev)
+    cap = ids.size + (E + 1) * (block - 1)
+    sorted_ids = torch.full((cap,), -7, dtype=torch.int32, device=dev)
+    expert_ids = torch.full(((cap + block - 1) // block,), -9, dtype=torch.int32, device=dev)
+    npad = torch.zeros(1, dtype=torch.int32, device=dev)
+    cumsum = torch.zeros(E + 2, dtype=torch.int32, device=dev)
+    ops.moe_align_block_size(t_ids, E + 1, block, sorted_ids, expert_ids, npad, cumsum, False)
+    torch.cuda.synchronize()
+    n = int(npad.item())
+    assert n == (2000 + block - 1) // block * block
+    s = sorted_ids.cpu().numpy()
+    np.testing.assert_array_equal(np.sort(s[:2000]), np.arange(2000))
+    assert (s[2000:] == -7).all()
+    e = expert_ids.cpu().numpy()
+    assert (e[: n // block] == 5).all() and (e[n // block :] == -9).all()
+    with pytest.raises(RuntimeError, match="sorted_token_ids holds"):
+        ops.moe_align_block_size(t_ids, E + 1, block, sorted_ids[:100], expert_ids, npad, cumsum, True)
+
+
+@pytest.mark.parametrize("rows,d", [(1, 2048), (37, 256), (32768, 2048)])
+def test_silu_and_mul(dev, rows, d):
+    from sglang_amd.sgl_kernel import silu_and_mul
+
+    rng = np.random.default_rng(rows)
+    x = O.to_bf16(rng.standard_normal((rows, 2 * d)).astype(np.float32) * 4)
+    out = silu_and_mul(bf16_tensor(x, dev))
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    ref = O.silu_and_mul(x)
+    # one bf16 ulp of the silu value (2^-8 relative) carried through the product
+    tol = np.abs(ref) * 2.0**-7 + 1e-30
+    assert (np.abs(got - ref) <= tol).all()
+    assert (got != ref).mean() < 1e-3
+    # the library routine on the same device agrees with the same bound
+    xt = bf16_tensor(x, dev)
+    lib_ref = (torch.nn.functional.silu(xt[:, :d].float()).to(torch.bfloat16) * xt[:, d:]).float().cpu().numpy()
+    assert (np.abs(got - lib_ref) <= np.abs(lib_ref) * 2.0**-7 + 1e-30).all()
+
+
+def test_silu_and_mul_other_dtypes_and_errors(dev):
+    from sglang_amd.sgl_kernel import silu_and_mul
+
+    x = torch.randn(9, 64, device=dev)
+    ref = torch.nn.functional.silu(x[:, :32]) * x[:, 32:]
+    torch.testing.assert_close(silu_and_mul(x), ref, rtol=1e-5, atol=1e-6)
+    xh = x.half()
+    refh = torch.nn.functional.silu(xh[:, :32].float()).half() * xh[:, 32:]
+    torch.testing.assert_close(silu_and_mul(xh), refh, rtol=2e-3, atol=1e-6)
+    with pytest.raises(ValueError, match="multiple of 16 bytes"):
+        silu_and_mul(torch.zeros(3, 12, device=dev, dtype=torch.bfloat16))
+    assert silu_and_mul(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16)).shape == (0, 32)
+
+
+@pytest.mark.parametrize("T,topk,H,scale", [(1, 8, 7168, 2.5), (19, 8, 128, 1.0), (4096, 8, 7168, 2.5), (5, 1, 64, 0.5)])
+def test_moe_sum_reduce_exact(dev, T, topk, H, scale):
+    from sglang_amd.sgl_kernel import moe_sum_reduce
+
+    rng = np.random.default_rng(T)
+    x = O.to_bf16(rng.standard_normal((T, topk, H)).astype(np.float32))
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    moe_sum_reduce(bf16_tensor(x, dev), out, scale)
+    torch.cuda.synchronize()
+    np.testing.assert_array_equal(out.float().cpu().numpy(), O.moe_sum_reduce(x, scale))
+
+
+def _expert_weights(rng, E, N, K):
+    wq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((E, N, K)).astype(np.float32) * 100, -448, 448))
+    ws = (rng.uniform(0.5, 2.0, (E, (N + 127) // 128, K // 128)) * 1e-3).astype(np.float32)
+    return wq, ws
+
+
+@pytest.mark.parametrize("T,E,topk,N,K,block", [(5, 8, 2, 512, 256, 16), (64, 8, 2, 384, 512, 32), (300, 16, 4, 1024, 1024, 64),
+                                               (700, 4, 2, 256, 384, 128), (3, 16, 8, 1024, 7168, 32)])
+def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block):
+    """GEMM1 form (row = slot // top_k, no routed weight) and GEMM2 form (row = slot, times routed weight)."""
+    from sglang_amd.fused_moe import moe_align_block_size
+    from sglang_amd.sgl_kernel import moe_block_gemm
+
+    rng = np.random.default_rng(T * 7 + N)
+    ids = _random_ids(rng, T, E, topk, 0.1 if T > 5 else 0.0)
+    wq, ws = _expert_weights(rng, E, N, K)
+    t_ids = torch.from_numpy(ids).to(dev)
+    sorted_ids, expert_ids, npad = moe_align_block_size(t_ids, block, E)
+    tw = rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32)
+    Bq, Bs = fp8_tensor(wq, dev), torch.from_numpy(ws).to(dev)
+    for top_k, rows in ((topk, T), (1, T * topk)):
+        xq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((rows, K)).astype(np.float32) * 100, -448, 448))
+        xs = (rng.uniform(0.5, 2.0, (rows, K // 128)) * 1e-2).astype(np.float32)
+        C = torch.full((T * topk, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        mul = top_k == 1
+        moe_block_gemm(fp8_tensor(xq, dev), Bq, C, torch.from_numpy(xs).to(dev), Bs, torch.from_numpy(tw).to(dev),
+                       sorted_ids, expert_ids, npad, mul, top_k, block, ids.size)
+        torch.cuda.synchronize()
+        got = C.float().cpu().numpy()
+        assert np.isfinite(got).all(), "some output row was not written"
+        ref = np.zeros((T * topk, N), dtype=np.float64)
+        flat = ids.reshape(-1)
+        for e in range(E):
+            slots = np.nonzero(flat == e)[0]
+            if slots.size == 0:
+                continue
+            r = slots // top_k
+            part = O.w8a8_block_fp8_matmul(xq[r], wq[e], xs[r], ws[e], out_dtype="f32", acc=np.float64)
+            ref[slots] = part * (tw.reshape(-1)[slots][:, None] if mul else 1.0)
+        assert (got[flat == -1] == 0).all()
+        assert _rel_err(got, ref) <= REL_TOL
+
+
+def test_grouped_gemm_exact_on_integers(dev):
+    from sglang_amd.fused_moe import moe_align_block_size
+    from sglang_amd.sgl_kernel import moe_block_gemm
+
+    rng = np.random.default_rng(3)
+    T, E, topk, N, K, block = 90, 6, 3, 512, 512, 64
+    ids = _random_ids(rng, T, E, topk)
+    wq = O.f32_to_e4m3fn(rng.integers(-4, 5, (E, N, K)).astype(np.float32))
+    ws = (2.0 ** rng.integers(-3, 3, (E, N // 128, K // 128))).astype(np.float32)
+    xq = O.f32_to_e4m3fn(rng.integers(-4, 5, (T, K)).astype(np.float32))
+    xs = (2.0 ** rng.integers(-3, 3, (T, K // 128))).astype(np.float32)
+    sorted_ids, expert_ids, npad = moe_align_block_size(torch.from_numpy(ids).to(dev), block, E)
+    C = torch.empty((T * topk, N), dtype=torch.bfloat16, device=dev)
+    moe_block_gemm(fp8_tensor(xq, dev), fp8_tensor(wq, dev), C, torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev),
+                   torch.ones((T, topk), device=dev), sorted_ids, expert_ids, npad, False, topk, block, ids.size)
+    torch.cuda.synchronize()
+    got = C.float().cpu().numpy()
+    flat = ids.reshape(-1)
+    for e in range(E):
+        slots = np.nonzero(flat == e)[0]
+        ref = O.w8a8_block_fp8_matmul(xq[slots // topk], wq[e], xs[slots // topk], ws[e], out_dtype="bf16", acc=np.float64)
+        np.testing.assert_array_equal(got[slots], ref)
+
+
+def _moe_problem(rng, T, E, H, I, topk, grouped_routing):
+    x = O.make_activation(T, H, int(rng.integers(1 << 30)))
+    w13 = O.to_bf16(rng.standard_normal((E, 2 * I, H)).astype(np.float32) * 0.02)
+    w2 = O.to_bf16(rng.standard_normal((E, H, I)).astype(np.float32) * 0.02)
+    w13q = np.empty((E, 2 * I, H), np.uint8); w13s = np.empty((E, 2 * I // 128, H // 128), np.float32)
+    w2q = np.empty((E, H, I), np.uint8); w2s = np.empty((E, H // 128, I // 128), np.float32)
+    for e in range(E):
+        w13q[e], w13s[e] = O.block_quant_weight(w13[e])
+        w2q[e], w2s[e] = O.block_quant_weight(w2[e])
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    if grouped_routing:
+        bias = (rng.standard_normal(E) * 0.1).astype(np.float32)
+        tw, ids = O.biased_grouped_topk(logits, bias, 8, 4, topk)
+    else:
+        ids = np.argsort(-logits, axis=1)[:, :topk].astype(np.int32)
+        sc = 1 / (1 + np.exp(-np.take_along_axis(logits, ids, 1)))
+        tw = (sc / sc.sum(-1, keepdims=True)).astype(np.float32)
+    return x, w13q, w13s, w2q, w2s, tw, ids
+
+
+@pytest.mark.parametrize("T,E,H,I,topk,grouped", [(1, 8, 512, 256, 2, False), (40, 8, 512, 256, 2, False),
+                                                 (300, 32, 1024, 512, 8, True), (1000, 8, 256, 128, 4, False)])
+def test_fused_experts_vs_oracle(dev, T, E, H, I, topk, grouped):
+    from sglang_amd.fused_moe import fused_experts_impl
+
+    rng = np.random.default_rng(T + E)
+    x, w13q, w13s, w2q, w2s, tw, ids = _moe_problem(rng, T, E, H, I, topk, grouped)
+    rsf = 2.5
+    ref = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf)
+    out = fused_experts_impl(
+        bf16_tensor(x, dev), fp8_tensor(w13q, dev), fp8_tensor(w2q, dev), torch.from_numpy(tw).to(dev),
+        torch.from_numpy(ids).to(dev), use_fp8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev),
+        w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], routed_scaling_factor=rsf,
+    )
+    torch.cuda.synchronize()
+    assert out.shape == (T, H) and out.dtype == torch.bfloat16
+    got = out.float().cpu().numpy()
+    assert _rel_err(got, ref) <= REL_TOL
+    # the reference's own acceptance metric for this layer (python/sglang/test/test_block_fp8.py:519-523)
+    assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.02
+
+
+def test_fused_experts_with_absent_experts_and_no_combine(dev):
+    """ids == -1 (expert on another rank) contribute zero; no_combine returns the per-slot rows."""
+    from sglang_amd.fused_moe import fused_experts_impl
+
+    rng = np.random.default_rng(5)
+    T, E, H, I, topk = 50, 8, 256, 128, 2
+    x, w13q, w13s, w2q, w2s, tw, ids = _moe_problem(rng, T, E, H, I, topk, False)
+    ids[rng.random(ids.shape) < 0.3] = -1
+    ref = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0)
+    args = (bf16_tensor(x, dev), fp8_tensor(w13q, dev), fp8_tensor(w2q, dev), torch.from_numpy(tw).to(dev),
+            torch.from_numpy(ids).to(dev))
+    kw = dict(use_fp8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+              block_shape=[128, 128])
+    out = fused_experts_impl(*args, **kw)
+    per_slot = fused_experts_impl(*args, no_combine=True, **kw)
+    torch.cuda.synchronize()
+    assert _rel_err(out.float().cpu().numpy(), ref) <= REL_TOL
+    assert per_slot.shape == (T, topk, H)
+    assert (per_slot.float().cpu().numpy()[ids == -1] == 0).all()
+    np.testing.assert_array_equal(out.float().cpu().numpy(), O.moe_sum_reduce(per_slot.float().cpu().numpy(), 1.0))
+
+
+def test_fused_experts_deepseek_dims_few_tokens(dev):
+    """256 experts, hidden 7168, intermediate 2048, top-8 grouped-sigmoid routing; weights are generated
+    on the device (11 GB) and only the experts the tokens hit are copied back for the oracle."""
+    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl
+
+    T, E, H, I, topk = 3, 256, 7168, 2048, 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+
+    def rand_fp8(shape):
+        b = torch.randint(0, 256, shape, generator=g, device=dev, dtype=torch.uint8)
+        b = torch.where((b & 0x7F) == 0x7F, b & 0xFE, b)  # no NaN codes
+        return b.view(torch.float8_e4m3fn)
+
+    w1 = rand_fp8((E, 2 * I, H))
+    w2 = rand_fp8((E, H, I))
+    w1s = torch.rand((E, 2 * I // 128, H // 128), generator=g, device=dev) * 2e-4 + 1e-4
+    w2s = torch.rand((E, H // 128, I // 128), generator=g, device=dev) * 2e-4 + 1e-4
+    x = O.make_activation(T, H, 0)
+    logits = torch.randn((T, E), generator=g, device=dev)
+    bias = torch.randn((E,), generator=g, device=dev) * 0.1
+    xt = bf16_tensor(x, dev)
+    tw, ids = biased_grouped_topk_impl(xt, logits, bias, topk, True, 8, 4)
+    out = fused_experts_impl(xt, w1, w2, tw, ids, use_fp8_w8a8=True, w1_scale=w1s, w2_scale=w2s, block_shape=[128, 128],
+                             routed_scaling_factor=2.5)
+    torch.cuda.synchronize()
+    ids_np, tw_np = ids.cpu().numpy(), tw.cpu().numpy()
+
+    class Lazy:
+        def __init__(self, t, as_u8):
+            self.t, self.as_u8, self.shape = t, as_u8, tuple(t.shape)
+
+        def __getitem__(self, e):
+            v = self.t[e]
+            return (v.view(torch.uint8) if self.as_u8 else v).cpu().numpy()
+
+    ref = O.fused_moe_block_fp8(x, Lazy(w1, True), Lazy(w1s, False), Lazy(w2, True), Lazy(w2s, False), tw_np, ids_np, 2.5)
+    assert _rel_err(out.float().cpu().numpy(), ref) <= REL_TOL
+    # routing agrees with the numpy restatement (as sets; top-k order is unspecified)
+    w_ref, ids_ref = O.biased_grouped_topk(logits.cpu().numpy(), bias.cpu().numpy(), 8, 4, topk)
+    np.testing.assert_array_equal(np.sort(ids_np, 1), np.sort(ids_ref, 1))
