@@ -83,8 +83,46 @@ def _time_calls(torch, fn, iters, warm=3):
     return a.elapsed_time(b) * 1e3 / iters
 
 
+def _time_graph(torch, fn, iters, replays=3):
+    """Average device time of fn(i) in microseconds with the launches replayed from one HIP graph, so
+    that host-side launch cost (Python, ctypes, allocator) does not show up in small-shape timings.
+    Every entry point of the library is capture-legal (no allocation, no sync, no memset)."""
+    for i in range(2):
+        fn(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(iters):
+            fn(i)
+    g.replay()
+    torch.cuda.synchronize()
+    a, b = _events(torch, 2)
+    a.record()
+    for _ in range(replays):
+        g.replay()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) * 1e3 / (iters * replays)
+
+
 def quant_bytes(M, K, ue8m0=False):
     return M * K * 3 + (M * K // 128) * (1 if ue8m0 else 4)
+
+
+def measured_traffic(kernel):
+    """HBM bytes per launch of `kernel` on the headline workload, as derived from rocprofv3 FETCH_SIZE / WRITE_SIZE
+    counter runs of this script (the summary under profiles/ carries one `TRAFFIC_BYTES <kernel> <bytes>` line per
+    kernel); None when no such summary is present."""
+    path = os.path.join(ROOT, "profiles", "bench_headline_hbm_traffic_pmc.md")
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "TRAFFIC_BYTES" and parts[1] == kernel:
+                    return int(parts[2])
+    except OSError:
+        pass
+    return None
 
 
 def gemm_bytes(M, N, K):
@@ -133,7 +171,7 @@ def run_quant_roofline(torch, dev, iters=30):
     out = {}
     for name, kw in (("row_major_f32", {}), ("col_major_f32", dict(column_major_scales=True)),
                      ("ue8m0_packed", dict(column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True))):
-        us = _time_calls(torch, lambda i: sglang_per_token_group_quant_fp8(xs[i % nbuf], 128, **kw), iters)
+        us = _time_graph(torch, lambda i: sglang_per_token_group_quant_fp8(xs[i % nbuf], 128, **kw), iters)
         out[name] = (us, quant_bytes(M, K, name == "ue8m0_packed") / us / 1e3)
     return out
 
@@ -159,20 +197,59 @@ def run_cpu_baseline(seconds_target=12.0):
         c_oracle.block_gemm(lib, q, wq, s, wsc)
         return time.perf_counter() - t0
 
-    t_probe = once(16)
-    M = int(min(1024, max(16, 16 * seconds_target / max(t_probe, 1e-3))))
-    M = max(16, M // 16 * 16)
-    dt = once(M)
-    return dict(value=2.0 * M * N * K / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
-                sample="C/OpenMP restatement of per-token-group quant + block-FP8 matmul on M=%d rows of the "
-                       "headline workload (N=%d, K=%d), %.1f s" % (M, N, K, dt))
+    # size the sample to about `seconds_target` of CPU work: rows of the headline batch, whole batches if fast
+    t_probe = once(64)
+    rows = 64 * seconds_target / max(t_probe, 1e-3)
+    M = int(min(HEADLINE["M"], max(64, rows // 64 * 64)))
+    reps = int(max(1, min(8, rows // HEADLINE["M"])))
+    dt = sum(once(M) for _ in range(reps))
+    return dict(value=2.0 * M * reps * N * K / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                sample="C/OpenMP restatement of per-token-group quant + block-FP8 matmul, %d pass(es) over M=%d rows "
+                       "of the headline workload (N=%d, K=%d), %.1f s of CPU time on %d threads"
+                       % (reps, M, N, K, dt, cores))
+
+
+def _rand_fp8(torch, shape, gen, dev):
+    b = torch.randint(0, 256, shape, generator=gen, device=dev, dtype=torch.uint8)
+    return torch.where((b & 0x7F) == 0x7F, b & 0xFE, b).view(torch.float8_e4m3fn)  # no NaN codes
+
+
+def moe_table(torch, dev):
+    """BASELINE configs[4]: 256 experts, hidden 7168, intermediate 2048, top-8 grouped-sigmoid routing."""
+    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl
+
+    E, H, I, topk = 256, 7168, 2048, 8
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    w1 = _rand_fp8(torch, (E, 2 * I, H), g, dev)
+    w2 = _rand_fp8(torch, (E, H, I), g, dev)
+    w1s = torch.rand((E, 2 * I // 128, H // 128), generator=g, device=dev) * 2e-4 + 1e-4
+    w2s = torch.rand((E, H // 128, I // 128), generator=g, device=dev) * 2e-4 + 1e-4
+    bias = torch.randn((E,), generator=g, device=dev) * 0.1
+    lines = ["", "## configs[4] block-FP8 fused MoE layer (E=256, H=7168, I=2048, top-8 of 8 groups / top-4 groups)", "",
+             "whole layer: align + quant + grouped GEMM w13 + silu_and_mul + quant + grouped GEMM w2 + top-k sum; "
+             "bytes = fp8 weights of the experts hit (44.04 MB each)", "",
+             "| M | experts hit | us | TFLOP/s | weight GB/s | % of 8 TB/s |", "|---|---|---|---|---|---|"]
+    for M in (1, 32, 256, 4096):
+        x = _activation(torch, M, H, M, dev)
+        logits = torch.randn((M, E), generator=g, device=dev)
+        tw, ids = biased_grouped_topk_impl(x, logits, bias, topk, True, 8, 4)
+        hit = int(torch.unique(ids).numel())
+        kw = dict(use_fp8_w8a8=True, w1_scale=w1s, w2_scale=w2s, block_shape=[128, 128], routed_scaling_factor=2.5)
+        us = _time_graph(torch, lambda i: fused_experts_impl(x, w1, w2, tw, ids, **kw), 10 if M < 4096 else 5)
+        flops = 2.0 * M * topk * 3 * I * H
+        wbytes = hit * 3 * I * H
+        lines.append("| %d | %d | %.1f | %.1f | %.0f | %.1f |" % (M, hit, us, flops / us / 1e6, wbytes / us / 1e3,
+                                                                 wbytes / us / 1e3 / PEAK_HBM_GBS * 100))
+    return lines
 
 
 def write_table(torch, dev, path):
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
     from sglang_amd.sgl_kernel import fp8_scaled_mm
 
-    lines = ["# Per-shape report (one MI355X, synthetic data, HIP-event device time, rotating buffers)", ""]
+    lines = ["# Per-shape report (one MI355X, synthetic data, rotating buffers; device time by HIP events around a",
+             "# HIP graph that replays the launches back to back, so host launch cost is excluded)", ""]
     lines += ["## configs[1] per-token-group quant, K=7168, group 128", "",
               "| M | layout | us | GB/s | % of 8 TB/s |", "|---|---|---|---|---|"]
     for M in (1, 64, 512, 4096, 16384):
@@ -180,7 +257,7 @@ def write_table(torch, dev, path):
         xs = [_activation(torch, M, 7168, s, dev) for s in range(nbuf)]
         for name, kw in (("row", {}), ("col", dict(column_major_scales=True)),
                          ("ue8m0", dict(column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True))):
-            us = _time_calls(torch, lambda i: sglang_per_token_group_quant_fp8(xs[i % nbuf], 128, **kw), 30)
+            us = _time_graph(torch, lambda i: sglang_per_token_group_quant_fp8(xs[i % nbuf], 128, **kw), 30)
             gbs = quant_bytes(M, 7168, name == "ue8m0") / us / 1e3
             lines.append("| %d | %s | %.1f | %.0f | %.1f |" % (M, name, us, gbs, gbs / PEAK_HBM_GBS * 100))
         del xs
@@ -192,7 +269,7 @@ def write_table(torch, dev, path):
         for M in (1, 16, 128, 1024, 4096):
             qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True)
                   for s in range(nbuf)]
-            us = _time_calls(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
+            us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
                                                                     ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
             tf = 2.0 * M * N * K / us / 1e6
             lines.append("| %d | %d | %d | %.1f | %.1f | %.1f | %.0f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100,
@@ -207,10 +284,11 @@ def write_table(torch, dev, path):
         for M in (1, 8, 64, 512, 2048, 8192):
             a = [(torch.randn((M, K), device=dev) * 50).clamp(-448, 448).to(torch.float8_e4m3fn) for _ in range(nbuf)]
             sa = torch.rand(M, device=dev)
-            us = _time_calls(torch, lambda i: fp8_scaled_mm(a[i % nbuf], bs[i % nbuf].t(), sa, sb, torch.bfloat16), 20)
+            us = _time_graph(torch, lambda i: fp8_scaled_mm(a[i % nbuf], bs[i % nbuf].t(), sa, sb, torch.bfloat16), 20)
             tf = 2.0 * M * N * K / us / 1e6
             lines.append("| %d | %d | %d | %.1f | %.1f | %.1f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100))
         del bs
+    lines += moe_table(torch, dev)
     os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
@@ -223,6 +301,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--table", type=str, default=None, help="also write the per-shape markdown report here")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 256 MiB read + 256 MiB write elementwise kernel (reference point for "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no cross-GPU step); --gpus %d is not "
@@ -246,6 +327,13 @@ def main() -> int:
     q_us, q_gbs = quant["row_major_f32"]
     if args.table:
         write_table(torch, dev, args.table)
+    if args.copy_calibration:
+        src = torch.ones(64 << 20, dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
     cpu = None if args.no_cpu else run_cpu_baseline()
 
     out = {
@@ -273,7 +361,7 @@ def main() -> int:
             "peak": PEAK_FP8_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(gemm_tf / PEAK_FP8_TFLOPS, 4),
-            "traffic": None,
+            "traffic": measured_traffic("gemm_tile256_kernel"),
             "avg_launch_us": round(gemm_us, 2),
         },
         "roofline_quant": {
@@ -283,7 +371,7 @@ def main() -> int:
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
             "frac": round(q_gbs / PEAK_HBM_GBS, 4),
-            "traffic": None,
+            "traffic": measured_traffic("group_quant_kernel"),
             "avg_launch_us": round(q_us, 2),
             "other_layouts_GBps": {k: round(v[1], 1) for k, v in quant.items()},
         },
