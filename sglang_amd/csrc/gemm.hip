@@ -1,11 +1,13 @@
 // Host side of the FP8 GEMM entry points: argument checks mirrored from the reference ops, kernel
 // choice, launch.  No allocation, no synchronisation.
-#include "gemm_kernels.h"
+#include <algorithm>
+
+#include "gemm_direct.h"
 
 namespace fp8k {
 
 struct Plan {
-  int kind;    // 0 = generic, 1 = tile256, 2 = weight-streaming (few rows)
+  int kind;    // 0 = generic, 1 = tile256, 2 = weight-streaming through LDS (33..128 rows), 3 = direct (<= 32 rows)
   int splits;  // >1: split-K through the float workspace
   int kb_per_split;
   int tm;      // rows per block of the streaming kernel
@@ -15,6 +17,22 @@ static Plan make_plan(int64_t M, int64_t N, int64_t K) {
   Plan pl{0, 1, 0, 0};
   if (K % kTileK != 0 || N % 4 != 0) return pl;
   const int kb = (int)(K / kTileK);
+  if (M <= 32 && M * K < (1LL << 31)) {
+    // decode-sized: weights go HBM -> registers -> matrix core; K is cut so that every CU holds two workgroups,
+    // in whole 8-block chunks, as long as the float partials stay a small fraction of the weight bytes
+    pl.kind = 3;
+    pl.tm = M <= 16 ? 16 : 32;
+    const int64_t tiles_n = (N + kDirTileN - 1) / kDirTileN;
+    int64_t splits = (1024 + tiles_n - 1) / tiles_n;
+    splits = std::min<int64_t>(splits, (kb + kDirKC - 1) / kDirKC);
+    splits = std::min<int64_t>(splits, std::max<int64_t>(1, K / (64 * M)));
+    if (splits < 1) splits = 1;
+    int kbps = (int)((kb + splits - 1) / splits);
+    kbps = (kbps + kDirKC - 1) / kDirKC * kDirKC;
+    pl.kb_per_split = kbps;
+    pl.splits = (kb + kbps - 1) / kbps;
+    return pl;
+  }
   if (M <= 128 && M * K < (1LL << 31)) {
     // decode-sized: stream the weights once, every CU takes a K slice of one 256-row weight tile
     pl.kind = 2;
@@ -59,6 +77,27 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   a.tiles_n = (a.N + kTileN - 1) / kTileN;
   a.splits = pl.splits;
   a.kb_per_split = pl.kb_per_split;
+  if (pl.kind == 3) {
+    a.m_blocks = 1;
+    a.tiles_n = (a.N + kDirTileN - 1) / kDirTileN;
+    const unsigned nwg = (unsigned)(a.tiles_n * pl.splits);
+#define FP8K_DIRECT(TM)                                                                                             \
+  do {                                                                                                              \
+    if (pl.splits == 1)                                                                                             \
+      hipLaunchKernelGGL((gemm_direct_kernel<TM, MODE, OUT_DT, BIAS_DT, false, false>), dim3(nwg), dim3(512), 0, st, a); \
+    else                                                                                                            \
+      hipLaunchKernelGGL((gemm_direct_kernel<TM, MODE, OUT_DT, BIAS_DT, true, false>), dim3(nwg), dim3(512), 0, st, a);  \
+  } while (0)
+    if (pl.tm == 16) FP8K_DIRECT(16);
+    else FP8K_DIRECT(32);
+#undef FP8K_DIRECT
+    int rc = check_launch("gemm_direct");
+    if (rc || pl.splits == 1) return rc;
+    const int64_t quads = (int64_t)a.M * (a.N / 4);
+    hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256),
+                       0, st, a);
+    return check_launch("splitk_reduce");
+  }
   if (pl.kind == 2) {
     a.m_blocks = 1;
     const unsigned nwg = (unsigned)(((a.tiles_n + 7) / 8) * 8 * pl.splits);

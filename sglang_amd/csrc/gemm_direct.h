@@ -1,0 +1,219 @@
+// Weight-streaming FP8 GEMM for very few activation rows (decode and small-batch MoE), gfx950.
+//
+// With at most 32 activation rows per block the GEMM is a pure HBM stream of the weight matrix
+// (2*TM FLOP per weight byte), so the weight bytes never touch LDS: a wavefront owns 16 weight rows
+// and loads them from global memory straight into the register layout of the "A" operand of
+// v_mfma_f32_16x16x128_f8f6f4 (lane l holds 32 bytes of row l%16), eight K blocks ahead of their use.
+// The matrix core only sums over K, so the K order inside a 128-byte block is free as long as both
+// operands agree: lane (row, q = l/16) takes bytes [q*16, q*16+16) and [64+q*16, 64+q*16+16) of the
+// block, which makes each of the two 16-byte loads cover whole 64-byte runs of 16 rows.
+// No barrier, no LDS round trip and no wait other than the compiler's own register dependencies sits
+// between HBM and the matrix core for the weights.
+//
+// The activation rows (a few KB per K block, shared by the 8 waves = 128 weight rows of a workgroup)
+// are staged through LDS in chunks of 8 K blocks: registers -> ds_write one chunk ahead, one barrier
+// per chunk, rows padded by 16 bytes so the 16 rows of an operand fetch fall into different banks.
+// In block mode the chunk also carries as[m,kb]*bs[nb,kb] (a workgroup spans exactly one 128-row
+// weight scale block), zero past the K range, so the K tail needs no branch.
+#pragma once
+
+#include "gemm_kernels.h"
+
+namespace fp8k {
+
+constexpr int kDirTileN = 128;                   // 8 waves x 16 weight rows
+constexpr int kDirKC = 8;                        // K blocks per activation chunk = weight prefetch depth
+constexpr int kDirXRow = kDirKC * kTileK + 16;   // LDS row stride of a staged activation row
+constexpr uint32_t kOutOfRange = 0xF0000000u;    // buffer offset past every descriptor range: reads zero
+
+__device__ __forceinline__ v4f mfma_16x16x128(v8i a, v8i b, v4f c) {
+  return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+__device__ __forceinline__ v4i buf_load16(rsrc_t r, uint32_t voff) {
+  return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0);
+}
+__device__ __forceinline__ v8i join(v4i lo, v4i hi) {
+  v8i r;
+  r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+  r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+  return r;
+}
+
+template <int TM, int MODE, int OUT_DT, int BIAS_DT, bool SPLIT, bool MOE>
+__global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
+  static_assert(TM == 16 || TM == 32, "gemm_direct_kernel: 16 or 32 activation rows per block");
+  constexpr int MS = TM / 16;   // 16-row activation sub-tiles
+  constexpr int XPW = TM / 8;   // activation rows staged by one wave
+  __shared__ __attribute__((aligned(16))) uint8_t xs[2][TM * kDirXRow];
+  __shared__ float scs[2][kDirKC][TM];
+
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r = lane & 15, kq = lane >> 4;
+
+  // ---- work item (same walk as gemm_stream_kernel)
+  int bid = blockIdx.x;
+  int split = 0;
+  int mb, tile_n;
+  if (MOE) {
+    const int used = p.num_post_pad[0] / p.block_m;
+    const int per_xcd = (used + 7) >> 3;
+    const int j = bid >> 3;
+    const int mbl = j / p.tiles_n;
+    if (mbl >= per_xcd) return;
+    mb = (bid & 7) * per_xcd + mbl;
+    if (mb >= used || mb >= p.m_blocks) return;
+    tile_n = j - mbl * p.tiles_n;
+  } else {
+    if (SPLIT) { split = bid % p.splits; bid /= p.splits; }
+    if (bid >= p.tiles_n * p.m_blocks) return;
+    mb = bid % p.m_blocks;
+    tile_n = bid / p.m_blocks;
+  }
+  const int block_m = MOE ? p.block_m : TM;
+  const int slot0 = mb * block_m;
+  const int expert = MOE ? p.expert_ids[mb] : 0;
+  const int nrows = MOE ? p.num_valid : p.M;
+  const int n0 = tile_n * kDirTileN;
+  const int n0w = n0 + w * 16;
+
+  const int kb_begin = SPLIT ? split * p.kb_per_split : 0;
+  const int kb_end = SPLIT ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
+  // an expert that lives on another rank contributes zeros: run no K block, the epilogue stores them
+  const int nkb = (MOE && expert < 0) ? 0 : max(kb_end - kb_begin, 0);
+  const int nch = (nkb + kDirKC - 1) / kDirKC;
+  const uint32_t kbytes = (uint32_t)nkb * kTileK;   // bytes of this K range per row
+
+  auto slot_of = [&](int i) -> int {   // row slot of block row i, or nrows when the row is padding
+    if (i >= block_m) return nrows;
+    const int s = MOE ? p.sorted_ids[slot0 + i] : slot0 + i;
+    return s < nrows ? s : nrows;
+  };
+
+  // ---- weights: 16 rows of this wave, straight into MFMA operand registers
+  const uint8_t* Wb = p.W + (MOE && expert >= 0 ? (int64_t)expert * p.w_expert_stride : 0);
+  const int rowsW = min(16, p.N - n0w);
+  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0w * p.ldw + (int64_t)kb_begin * kTileK,
+                              rowsW > 0 ? (uint32_t)((rowsW - 1) * p.ldw) + kbytes : 0u);
+  const uint32_t voW = (uint32_t)(r * p.ldw + kq * 16);
+  v4i wreg[kDirKC][2];
+  auto load_w = [&](int slot, int kb) {
+    const uint32_t vo = kb < nkb ? voW + (uint32_t)kb * kTileK : kOutOfRange;
+    wreg[slot][0] = buf_load16(rW, vo);
+    wreg[slot][1] = buf_load16(rW, kb < nkb ? vo + 64 : kOutOfRange);
+  };
+
+  // ---- activations: wave w stages rows w*XPW .. w*XPW+XPW-1 of the block, 1 KB (8 K blocks) per row
+  const int64_t xrows = MOE ? (int64_t)((p.num_valid + p.top_k - 1) / p.top_k) : (int64_t)p.M;
+  const rsrc_t rX = make_rsrc(p.X + (int64_t)kb_begin * kTileK, (uint32_t)((xrows - 1) * p.ldx) + kbytes);
+  uint32_t voX[XPW];
+#pragma unroll
+  for (int j = 0; j < XPW; ++j) {
+    const int s = slot_of(w * XPW + j);
+    const int64_t xr = MOE ? s / p.top_k : s;
+    voX[j] = s < nrows ? (uint32_t)(xr * p.ldx) + lane * 16 : kOutOfRange;
+  }
+  v4i xreg[XPW];
+  // ---- block mode: lane t < TM*8 stages as[m,kb]*bs[nb,kb] of (m = t % TM, kb = chunk*8 + t / TM)
+  const int sm = threadIdx.x % TM, skb = threadIdx.x / TM;
+  const bool stager = MODE == kModeBlock && (int)threadIdx.x < TM * kDirKC;
+  const float* sxp = p.sx;
+  const float* swp = p.sw;
+  bool srow_ok = false;
+  if (stager) {
+    const int s = slot_of(sm);
+    srow_ok = s < nrows;
+    const int64_t xr = srow_ok ? (MOE ? s / p.top_k : s) : 0;
+    sxp = p.sx + xr * p.sx_m + (int64_t)kb_begin * p.sx_k;
+    swp = p.sw + (MOE && expert >= 0 ? (int64_t)expert * p.sw_expert_stride : 0) +
+          (int64_t)(min(n0, p.N - 1) >> 7) * p.sw_n + (int64_t)kb_begin * p.sw_k;
+  }
+  float sreg = 0.f;
+  auto stage_load = [&](int c) {
+    const uint32_t k0 = (uint32_t)c * (kDirKC * kTileK);
+#pragma unroll
+    for (int j = 0; j < XPW; ++j) {
+      const bool ok = voX[j] != kOutOfRange && k0 + lane * 16 < kbytes;
+      xreg[j] = buf_load16(rX, ok ? voX[j] + k0 : kOutOfRange);
+    }
+    if (MODE == kModeBlock) {
+      const int kb = c * kDirKC + skb;
+      sreg = 0.f;
+      if (stager && srow_ok && kb < nkb) sreg = sxp[(int64_t)kb * p.sx_k] * swp[(int64_t)kb * p.sw_k];
+    }
+  };
+  auto stage_store = [&](int buf) {
+#pragma unroll
+    for (int j = 0; j < XPW; ++j)
+      *reinterpret_cast<v4i*>(&xs[buf][(w * XPW + j) * kDirXRow + lane * 16]) = xreg[j];
+    if (stager) scs[buf][skb][sm] = sreg;
+  };
+
+  v4f acc[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) acc[ms] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  // ---- prologue: chunk 0 into LDS, chunk 1 in registers, weights of K blocks 0..7 in flight
+  stage_load(0);
+#pragma unroll
+  for (int d = 0; d < kDirKC; ++d) load_w(d, d);
+  stage_store(0);
+  stage_load(1);
+
+  const uint32_t xrd = (uint32_t)(r * kDirXRow + kq * 16);
+  for (int c = 0; c < nch; ++c) {
+    const int buf = c & 1;
+    __syncthreads();        // chunk c is visible; every wave is done with chunk c-1
+    stage_store(buf ^ 1);   // chunk c+1
+    stage_load(c + 2);
+#pragma unroll
+    for (int kbl = 0; kbl < kDirKC; ++kbl) {
+      const v8i wa = join(wreg[kbl][0], wreg[kbl][1]);
+      load_w(kbl, (c + 1) * kDirKC + kbl);
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms) {
+        const uint8_t* xp = &xs[buf][ms * 16 * kDirXRow + xrd + kbl * kTileK];
+        const v8i xa = join(*reinterpret_cast<const v4i*>(xp), *reinterpret_cast<const v4i*>(xp + 64));
+        if (MODE == kModeBlock) {
+          const v4f t = mfma_16x16x128(wa, xa, v4f{0.f, 0.f, 0.f, 0.f});
+          const float sc = scs[buf][kbl][ms * 16 + r];
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[ms][i] = __builtin_fmaf(t[i], sc, acc[ms][i]);
+        } else {
+          acc[ms] = mfma_16x16x128(wa, xa, acc[ms]);
+        }
+      }
+    }
+  }
+
+  // ---- epilogue: lane holds n = n0w + kq*4 .. +3 of activation row ms*16 + r
+  const int n = n0w + kq * 4;
+  if (n >= p.N) return;
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int s = slot_of(ms * 16 + r);
+    if (s >= nrows) continue;
+    const int64_t orow = s;
+    float v[4] = {acc[ms][0], acc[ms][1], acc[ms][2], acc[ms][3]};
+    if (SPLIT) {
+      *reinterpret_cast<float4*>(p.partial + ((int64_t)split * p.M + orow) * p.N + n) = make_float4(v[0], v[1], v[2], v[3]);
+      continue;
+    }
+    if (MODE == kModeRow) {
+      const float sa = p.sx[orow];
+      const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
+      v[0] = v[0] * sb.x * sa; v[1] = v[1] * sb.y * sa; v[2] = v[2] * sb.z * sa; v[3] = v[3] * sb.w * sa;
+      if (p.bias) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += load_scalar<BIAS_DT>(p.bias, n + i);
+      }
+    } else if (MOE && p.topk_w) {
+      const float tw = p.topk_w[orow];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] *= tw;
+    }
+    store4<OUT_DT>(p.C, orow * p.ldc + n, v[0], v[1], v[2], v[3]);
+  }
+}
+
+}  // namespace fp8k

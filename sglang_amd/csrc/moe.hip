@@ -1,7 +1,7 @@
 // Block-FP8 fused-MoE building blocks for gfx950: token alignment (integer), the grouped block-scaled
 // GEMM (host side; the device code is gemm_stream_kernel in gemm_kernels.h), silu_and_mul and the
 // top-k sum.  No allocation, no synchronisation, no host reads of device data.
-#include "gemm_kernels.h"
+#include "gemm_direct.h"
 
 namespace fp8k {
 
@@ -287,10 +287,25 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
   a.m_blocks = (int)(sorted_capacity / block_m);
   a.block_m = (int)block_m;
   a.w_expert_stride = b_stride_e; a.sw_expert_stride = bs_stride_e;
+  const bool direct = block_m <= 32;  // few rows per expert: weights go straight to registers, 128-row tiles
+  if (direct) a.tiles_n = (int)((N + kDirTileN - 1) / kDirTileN);
   const int64_t per_xcd = (a.m_blocks + 7) / 8;
   const int64_t nwg = per_xcd * 8 * a.tiles_n;
   FP8K_REQUIRE(nwg < 0x7fffffffLL, "%s: grid too large", op);
   hipStream_t st = (hipStream_t)stream;
+#define FP8K_MOE_DIRECT(TM, O) \
+  hipLaunchKernelGGL((gemm_direct_kernel<TM, kModeBlock, O, FP8K_F32, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a)
+  if (direct) {
+    if (out_dtype == FP8K_BF16) {
+      if (block_m == 16) FP8K_MOE_DIRECT(16, FP8K_BF16);
+      else FP8K_MOE_DIRECT(32, FP8K_BF16);
+    } else {
+      if (block_m == 16) FP8K_MOE_DIRECT(16, FP8K_F16);
+      else FP8K_MOE_DIRECT(32, FP8K_F16);
+    }
+    return check_launch(op);
+  }
+#undef FP8K_MOE_DIRECT
 #define FP8K_MOE(TM, NST, O) \
   hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, kModeBlock, O, FP8K_F32, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a)
   if (out_dtype == FP8K_BF16) {

@@ -99,7 +99,8 @@ def invoke_fused_moe_kernel(
     assert B_scale is not None
     if A.dtype != torch.float8_e4m3fn:
         assert A_scale is None
-        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1])
+        # column-major scales: one coalesced load per K block for the lanes of a wave (any layout is accepted)
+        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1], column_major_scales=True)
     assert (A.shape[-1] + 127) // 128 == A_scale.shape[-1]
     assert (B.shape[-2] + 127) // 128 == B_scale.shape[-2]
     assert (B.shape[-1] + 127) // 128 == B_scale.shape[-1]
