@@ -11,26 +11,30 @@ struct Plan {
   int splits;  // >1: split-K through the float workspace
   int kb_per_split;
   int tm;      // rows per block of the streaming kernel
+  int tail_first;   // tile256: first tile that is cut along K (== number of tiles when none is)
+  int64_t ws_bytes; // float workspace the plan needs
 };
 
+constexpr int kNumCU = 256;  // MI355X
+
 static Plan make_plan(int64_t M, int64_t N, int64_t K) {
-  Plan pl{0, 1, 0, 0};
+  Plan pl{0, 1, 0, 0, 0, 0};
   if (K % kTileK != 0 || N % 4 != 0) return pl;
   const int kb = (int)(K / kTileK);
   if (M <= 32 && M * K < (1LL << 31)) {
-    // decode-sized: weights go HBM -> registers -> matrix core; K is cut so that every CU holds two workgroups,
-    // in whole 8-block chunks, as long as the float partials stay a small fraction of the weight bytes
+    // decode-sized: weights go HBM -> registers -> matrix core.  K is cut so that about 512 workgroups (two per
+    // CU, one round) stream at once, at least 8 K blocks each, while the float partials stay a small fraction of
+    // the weight bytes
     pl.kind = 3;
     pl.tm = M <= 16 ? 16 : 32;
     const int64_t tiles_n = (N + kDirTileN - 1) / kDirTileN;
-    int64_t splits = (1024 + tiles_n - 1) / tiles_n;
-    splits = std::min<int64_t>(splits, (kb + kDirKC - 1) / kDirKC);
+    int64_t splits = std::max<int64_t>(1, 512 / tiles_n);
+    splits = std::min<int64_t>(splits, std::max<int64_t>(1, kb / kDirKC));
     splits = std::min<int64_t>(splits, std::max<int64_t>(1, K / (64 * M)));
-    if (splits < 1) splits = 1;
-    int kbps = (int)((kb + splits - 1) / splits);
-    kbps = (kbps + kDirKC - 1) / kDirKC * kDirKC;
+    const int kbps = (int)((kb + splits - 1) / splits);
     pl.kb_per_split = kbps;
     pl.splits = (kb + kbps - 1) / kbps;
+    pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
     return pl;
   }
   if (M <= 128 && M * K < (1LL << 31)) {
@@ -43,26 +47,30 @@ static Plan make_plan(int64_t M, int64_t N, int64_t K) {
     if (splits < 1) splits = 1;
     pl.kb_per_split = (kb + splits - 1) / splits;
     pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
+    pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
     return pl;
   }
   pl.kind = 1;
+  // One workgroup (one CU) per 256x256 tile.  The tiles of the last, partial round over the CUs are cut along K
+  // so that the round keeps every CU busy for 1/splits of a tile time (>= 4 K blocks per piece).
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
-  int splits = 1;
-  // fewer tiles than compute units: cut K so that every CU has work, keeping >= 4 K-blocks per run
-  if (tiles < 160) {
-    splits = (int)((256 + tiles - 1) / tiles);
-    if (splits > kb / 4) splits = kb / 4;
-    if (splits < 1) splits = 1;
-  }
+  const int64_t rest = tiles % kNumCU;
+  int splits = rest ? (int)(kNumCU / rest) : 1;
+  if (splits > kb / 4) splits = kb / 4;
+  if (splits < 1) splits = 1;
+  // With at least one full round before it, the cut only pays when the tile time it saves (about 2 us per K block)
+  // outweighs writing and re-reading the float partials (256 KB per piece): measured break-even.
+  if (tiles > kNumCU && kb * (splits - 1) * 8 <= rest * splits * splits) splits = 1;
   pl.kb_per_split = (kb + splits - 1) / splits;
   pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
+  pl.tail_first = (int)(pl.splits > 1 ? tiles - rest : tiles);
+  pl.ws_bytes = pl.splits > 1 ? rest * pl.splits * (int64_t)(kTileM * kTileN) * 4 : 0;
   return pl;
 }
 
 static int64_t workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
-  Plan pl = make_plan(M, N, K);
-  return pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  return make_plan(M, N, K).ws_bytes;
 }
 
 template <int MODE, int OUT_DT, int BIAS_DT>
@@ -122,18 +130,14 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
     return check_launch("splitk_reduce");
   }
   const int ntiles = a.tiles_m * a.tiles_n;
-  const unsigned nwg = (unsigned)(((ntiles + 7) / 8) * 8 * pl.splits);
-  if (pl.splits == 1) {
-    hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT, false>), dim3(nwg), dim3(512), 0, st, a);
-    return check_launch("gemm_tile256");
-  }
-  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT, true>), dim3(nwg), dim3(512), 0, st, a);
-  int rc = check_launch("gemm_tile256_splitk");
-  if (rc) return rc;
-  const int64_t quads = (int64_t)a.M * (a.N / 4);
-  hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256), 0,
-                     st, a);
-  return check_launch("splitk_reduce");
+  a.tail_first = pl.tail_first;
+  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
+  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
+  int rc = check_launch("gemm_tile256");
+  if (rc || pl.tail_first == ntiles) return rc;
+  hipLaunchKernelGGL((tile_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((ntiles - pl.tail_first) * 64)), dim3(256),
+                     0, st, a);
+  return check_launch("tile_reduce");
 }
 
 static int common_checks(const char* op, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
@@ -145,6 +149,7 @@ static int common_checks(const char* op, const void* A, const void* B, void* C, 
   FP8K_REQUIRE((N * 2) % 16 == 0, "%s: out must be multiple of 16 bytes for memory alignment", op);
   FP8K_REQUIRE(lda >= K && ldb >= K && ldc >= N, "%s: leading dimension smaller than the row length", op);
   FP8K_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && (ldc * 2) % 8 == 0, "%s: rows must be 16-byte aligned", op);
+  FP8K_REQUIRE(lda < (1LL << 23) && ldb < (1LL << 23) && K < (1LL << 23), "%s: rows longer than 8 MiB are not supported", op);
   if (M == 0 || N == 0) return FP8K_OK;
   FP8K_REQUIRE(A && B && C, "%s: null pointer", op);
   FP8K_REQUIRE(aligned(A, 16) && aligned(B, 16) && aligned(C, 8), "%s: operands must be 16-byte aligned", op);
@@ -171,7 +176,7 @@ extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, co
   FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0,
                "fp8_blockwise_scaled_mm: negative scale stride");
   const Plan pl = make_plan(M, N, K);
-  const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  const int64_t need = pl.ws_bytes;
   if (need > 0 && (!workspace || workspace_bytes_given < need))
     return fail(FP8K_ERR_WORKSPACE, "fp8_blockwise_scaled_mm: workspace of %lld bytes required, %lld given",
                 (long long)need, (long long)(workspace ? workspace_bytes_given : 0));
@@ -199,7 +204,7 @@ extern "C" int fp8k_scaled_mm(const void* A, const void* B, const float* sa, con
     FP8K_REQUIRE(bias_dtype == FP8K_F32 || bias_dtype == FP8K_F16 || bias_dtype == FP8K_BF16,
                  "fp8_scaled_mm: bias dtype must be float32, float16 or bfloat16");
   const Plan pl = make_plan(M, N, K);
-  const int64_t need = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  const int64_t need = pl.ws_bytes;
   if (need > 0 && (!workspace || workspace_bytes_given < need))
     return fail(FP8K_ERR_WORKSPACE, "fp8_scaled_mm: workspace of %lld bytes required, %lld given", (long long)need,
                 (long long)(workspace ? workspace_bytes_given : 0));

@@ -25,6 +25,7 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int splits;         // K is cut into `splits` runs of kb_per_split K-blocks
   int kb_per_split;
+  int tail_first;     // tile256 only: tiles [tail_first, tiles) are the ones cut along K
   // grouped (MoE) form of the streaming kernel; all null / zero for a dense GEMM
   const int32_t* sorted_ids;    // [m_blocks * TM] token slots, padded with values >= num_valid
   const int32_t* expert_ids;    // [m_blocks] expert of each block of TM slots, -1 = not on this rank
@@ -74,7 +75,8 @@ __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
 //
 // LDS: two stages of [W 256 rows x 128 B | X 256 rows x 128 B] = 2 x 64 KB, filled by
 // buffer_load_dwordx4 ... lds (no register staging; rows past the matrix edge are out of the
-// descriptor's range and arrive as zeros).  A 1 KB wave-load covers 8 rows; the 16-byte chunk c of
+// descriptor's range - the complete offset is in the range-checked per-lane operand - and arrive
+// as zeros without touching memory).  A 1 KB wave-load covers 8 rows; the 16-byte chunk c of
 // row r is stored at chunk position c ^ ((r >> 1) & 7), which makes both the linear LDS-DMA writes
 // and the ds_read_b128 operand fetches (32 rows, same logical chunk) bank-conflict free.
 //
@@ -107,7 +109,24 @@ __device__ __forceinline__ void buf_load16_to_lds(rsrc_t r, uint32_t voff, uint3
 }
 __device__ __forceinline__ void wait_vm0_lgkm0() { __builtin_amdgcn_s_waitcnt(0x0070); }  // vmcnt(0) lgkmcnt(0)
 
-template <int MODE, int OUT_DT, int BIAS_DT, bool SPLIT>
+// tile index -> (tile_m, tile_n): tiles are numbered in groups of 4 m-tiles, m fastest inside a group, so that
+// the tiles that run together on one XCD cover 4 activation tiles x a run of weight tiles
+__device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
+  constexpr int GM = 4;
+  const int group = t / (GM * tiles_n);
+  const int first_m = group * GM;
+  const int gsz = min(tiles_m - first_m, GM);
+  const int tin = t - group * GM * tiles_n;
+  tile_m = first_m + tin % gsz;
+  tile_n = tin / gsz;
+}
+
+// Tiles [0, tail_first) are computed whole, one per workgroup, each XCD walking a contiguous run of them.
+// Tiles [tail_first, tiles) - the last, partial round over the chip's CUs - are cut into `splits` K ranges, one
+// workgroup each, so that the round takes 1/splits of a tile time; they leave float partials in the workspace
+// ([tile - tail_first][split][256 m][256 n]) for tile_reduce_kernel.  Their workgroup ids come last, so they are
+// dispatched when the whole tiles drain.
+template <int MODE, int OUT_DT, int BIAS_DT>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kStageBytes];
 
@@ -116,23 +135,25 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   const int wn = w & 1, wm = w >> 1;
 
   const int ntiles = p.tiles_m * p.tiles_n;
-  const int per_xcd = (ntiles + 7) >> 3;
-  int bid = blockIdx.x;
-  int split = 0;
-  if (SPLIT) { split = bid % p.splits; bid /= p.splits; }
-  const int t = (bid & 7) * per_xcd + (bid >> 3);
-  if (t >= ntiles) return;
-  constexpr int GM = 4;
-  const int group = t / (GM * p.tiles_n);
-  const int first_m = group * GM;
-  const int gsz = min(p.tiles_m - first_m, GM);
-  const int tin = t - group * GM * p.tiles_n;
-  const int tile_m = first_m + tin % gsz;
-  const int tile_n = tin / gsz;
+  const int per_xcd = (p.tail_first + 7) >> 3;
+  const int bid = blockIdx.x;
+  int t, split = 0;
+  const bool is_split = bid >= per_xcd * 8;
+  if (!is_split) {
+    t = (bid & 7) * per_xcd + (bid >> 3);
+    if (t >= p.tail_first) return;
+  } else {
+    const int b2 = bid - per_xcd * 8;
+    t = p.tail_first + b2 / p.splits;
+    split = b2 % p.splits;
+    if (t >= ntiles) return;
+  }
+  int tile_m, tile_n;
+  tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
   const int m0 = tile_m * kTileM, n0 = tile_n * kTileN;
 
-  const int kb_begin = SPLIT ? split * p.kb_per_split : 0;
-  const int kb_end = SPLIT ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
+  const int kb_begin = is_split ? split * p.kb_per_split : 0;
+  const int kb_end = is_split ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
   const int nkb = kb_end - kb_begin;
 
   // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the
@@ -197,8 +218,10 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     uint8_t* base = smem + cur_stage * kStageBytes + w * 4096;
     const uint32_t ko = (uint32_t)cur_kstep * kTileK;
     const int j = idx & 3;
-    if (idx < 4) buf_load16_to_lds(rW, voW[j & 1], soW + j * stepW + ko, base + j * 1024);
-    else buf_load16_to_lds(rX, voX[j & 1], soX + j * stepX + ko, base + kXOff + j * 1024);
+    // the whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt from the
+    // range check, and rows past the matrix edge must read as zero, not touch memory)
+    if (idx < 4) buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + ko), 0, base + j * 1024);
+    else buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + ko), 0, base + kXOff + j * 1024);
   };
   auto RW = [&](v8i(&dst)[2], const uint8_t* st, int ns) {
     dst[0] = frag(st, rdW + ns * 32 * kTileK, 0);
@@ -310,7 +333,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     const int m = m0 + wm * 64 + ms * 32 + lr;
     if (m >= p.M) continue;
     float sa = 1.f;
-    if (MODE == kModeRow && !SPLIT) sa = p.sx[m];
+    if (MODE == kModeRow && !is_split) sa = p.sx[m];
 #pragma unroll
     for (int ns = 0; ns < 4; ++ns) {
 #pragma unroll
@@ -320,9 +343,9 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
         float v[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) v[r] = acc[ns][ms][rg * 4 + r];
-        if (SPLIT) {
-          float4 o = make_float4(v[0], v[1], v[2], v[3]);
-          *reinterpret_cast<float4*>(p.partial + ((int64_t)split * p.M + m) * p.N + n) = o;
+        if (is_split) {
+          float* tile_part = p.partial + ((int64_t)(t - p.tail_first) * p.splits + split) * (kTileM * kTileN);
+          *reinterpret_cast<float4*>(tile_part + (m - m0) * kTileN + (n - n0)) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
           if (MODE == kModeRow) {
             const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
@@ -452,10 +475,11 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
     uint8_t* base = smem + (kstep % NSTAGE) * STAGE;
     const uint32_t ko = (uint32_t)kstep * kTileK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) buf_load16_to_lds(rW, voW[j & 1], soW + j * stepW + ko, base + w * 4096 + j * 1024);
+    for (int j = 0; j < 4; ++j)
+      buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + ko), 0, base + w * 4096 + j * 1024);
 #pragma unroll
     for (int j = 0; j < XL; ++j)
-      buf_load16_to_lds(rX, voX[j], ko, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
+      buf_load16_to_lds(rX, voX[j] + ko, 0, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
   };
 
   // ---- LDS -> MFMA operands
@@ -587,6 +611,36 @@ __global__ __launch_bounds__(256) void splitk_reduce_kernel(const GemmArgs p) {
   float4 s = make_float4(0, 0, 0, 0);
   for (int k = 0; k < p.splits; ++k) {
     const float4 v = *reinterpret_cast<const float4*>(p.partial + ((int64_t)k * p.M + m) * p.N + n);
+    s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+  }
+  if (MODE == kModeRow) {
+    const float sa = p.sx[m];
+    const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
+    s.x = s.x * sb.x * sa; s.y = s.y * sb.y * sa; s.z = s.z * sb.z * sa; s.w = s.w * sb.w * sa;
+    if (p.bias) {
+      s.x += load_scalar<BIAS_DT>(p.bias, n); s.y += load_scalar<BIAS_DT>(p.bias, n + 1);
+      s.z += load_scalar<BIAS_DT>(p.bias, n + 2); s.w += load_scalar<BIAS_DT>(p.bias, n + 3);
+    }
+  }
+  store4<OUT_DT>(p.C, (int64_t)m * p.ldc + n, s.x, s.y, s.z, s.w);
+}
+
+// ------------------------------------------------------------------------------------------------
+// reduction of the K-cut tiles of gemm_tile256_kernel: 64 workgroups per tile, one float4 of 4 n per lane
+// ------------------------------------------------------------------------------------------------
+template <int MODE, int OUT_DT, int BIAS_DT>
+__global__ __launch_bounds__(256) void tile_reduce_kernel(const GemmArgs p) {
+  const int tl = blockIdx.x >> 6;
+  int tile_m, tile_n;
+  tile_coords(p.tail_first + tl, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  const int q = ((blockIdx.x & 63) << 8) + threadIdx.x;  // quad index inside the tile
+  const int ml = q >> 6, nl = (q & 63) << 2;
+  const int m = tile_m * kTileM + ml, n = tile_n * kTileN + nl;
+  if (m >= p.M || n >= p.N) return;
+  const float* src = p.partial + (int64_t)tl * p.splits * (kTileM * kTileN) + ml * kTileN + nl;
+  float4 s = make_float4(0, 0, 0, 0);
+  for (int k = 0; k < p.splits; ++k) {
+    const float4 v = *reinterpret_cast<const float4*>(src + (int64_t)k * (kTileM * kTileN));
     s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
   }
   if (MODE == kModeRow) {
