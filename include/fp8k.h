@@ -127,7 +127,7 @@ int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64, int64_t n
  *   (python/sglang/srt/layers/moe/fused_moe_triton/fused_moe_triton_kernels.py:307-583, 586-790).
  * A e4m3fn [ceil(num_valid/top_k), K] (lda); B e4m3fn [E, N, K] (b_stride_e bytes between experts, ldb between
  * rows); As float (as_stride_m, as_stride_k); Bs float [E, ceil(N/128), K/128] (bs_stride_e, bs_stride_n,
- * bs_stride_k); C [num_valid_tokens, N] of out_dtype (ldc).  block_m in {16,32,64,128} is the block size
+ * bs_stride_k); C [num_valid_tokens, N] of out_dtype (ldc).  block_m in {16,32,64,128,256} is the block size
  * moe_align_block_size was called with; sorted_capacity = length of sorted_token_ids.  K % 128 == 0, N % 8 == 0.
  */
 int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,

@@ -29,7 +29,7 @@ static Plan make_plan(int64_t M, int64_t N, int64_t K) {
     pl.tm = M <= 16 ? 16 : 32;
     const int64_t tiles_n = (N + kDirTileN - 1) / kDirTileN;
     int64_t splits = std::max<int64_t>(1, 512 / tiles_n);
-    splits = std::min<int64_t>(splits, std::max<int64_t>(1, kb / kDirKC));
+    splits = std::min<int64_t>(splits, std::max<int64_t>(1, kb / kDirDepth));
     splits = std::min<int64_t>(splits, std::max<int64_t>(1, K / (64 * M)));
     const int kbps = (int)((kb + splits - 1) / splits);
     pl.kb_per_split = kbps;
@@ -132,7 +132,7 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   const int ntiles = a.tiles_m * a.tiles_n;
   a.tail_first = pl.tail_first;
   const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
-  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
+  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT, false>), dim3(nwg), dim3(512), 0, st, a);
   int rc = check_launch("gemm_tile256");
   if (rc || pl.tail_first == ntiles) return rc;
   hipLaunchKernelGGL((tile_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((ntiles - pl.tail_first) * 64)), dim3(256),

@@ -1,21 +1,21 @@
-// Weight-streaming FP8 GEMM for very few activation rows (decode and small-batch MoE), gfx950.
+// Weight-streaming FP8 GEMM for at most 32 activation rows per block (decode and small-batch MoE), gfx950.
 //
-// With at most 32 activation rows per block the GEMM is a pure HBM stream of the weight matrix
-// (2*TM FLOP per weight byte), so the weight bytes never touch LDS: a wavefront owns 16 weight rows
-// and loads them from global memory straight into the register layout of the "A" operand of
-// v_mfma_f32_16x16x128_f8f6f4 (lane l holds 32 bytes of row l%16), eight K blocks ahead of their use.
-// The matrix core only sums over K, so the K order inside a 128-byte block is free as long as both
-// operands agree: lane (row, q = l/16) takes bytes [q*16, q*16+16) and [64+q*16, 64+q*16+16) of the
-// block, which makes each of the two 16-byte loads cover whole 64-byte runs of 16 rows (cached loads:
-// the two halves of a 128-byte line meet in the vector cache; marked non-temporal they measured 10 % slower).
-// No barrier, no LDS round trip and no wait other than the compiler's own register dependencies sits
-// between HBM and the matrix core for the weights.
+// With so few activation rows the GEMM is an HBM stream of the weight matrix (2*TM FLOP per weight byte, under the
+// chip's ridge), so the weight bytes never touch LDS: a wavefront owns 16 weight rows and loads them from global
+// memory straight into the register layout of the "A" operand of v_mfma_f32_16x16x128_f8f6f4 (lane l holds 32
+// bytes of row l%16), eight K blocks ahead of their use.  The matrix core only sums over K, so the K order inside
+// a 128-byte block is free as long as both operands agree: lane (row, q = l/16) takes bytes [q*16, q*16+16) and
+// [64+q*16, 64+q*16+16) of the block, which makes each of the two 16-byte loads cover whole 64-byte runs of 16
+// rows (cached loads: the two halves of a 128-byte line meet in the vector cache; marked non-temporal they
+// measured 10 % slower).  No barrier, no LDS round trip and no wait other than the compiler's own register
+// dependencies sits between HBM and the matrix core for the weights.
 //
-// The activation rows (a few KB per K block, shared by the 8 waves = 128 weight rows of a workgroup)
-// are staged through LDS in chunks of 8 K blocks: registers -> ds_write one chunk ahead, one barrier
-// per chunk, rows padded by 16 bytes so the 16 rows of an operand fetch fall into different banks.
-// In block mode the chunk also carries as[m,kb]*bs[nb,kb] (a workgroup spans exactly one 128-row
-// weight scale block), zero past the K range, so the K tail needs no branch.
+// The activation rows (shared by the 8 waves = 128 weight rows of a workgroup) are staged through LDS in chunks
+// of 8 K blocks: registers -> ds_write one chunk ahead, one barrier per chunk, rows padded by 16 bytes so the
+// 16 rows of an operand fetch fall into different banks.  (Every wave re-reads all activation rows of the block
+// from LDS, which is why blocks of 64 and 128 rows measured slower here than through gemm_stream_kernel.)  In block mode the chunk also
+// carries as[m,kb]*bs[nb,kb] (a workgroup spans exactly one 128-row weight scale block), zero past the K range,
+// so the K tail needs no branch.
 #pragma once
 
 #include "gemm_kernels.h"
@@ -23,8 +23,7 @@
 namespace fp8k {
 
 constexpr int kDirTileN = 128;                   // 8 waves x 16 weight rows
-constexpr int kDirKC = 8;                        // K blocks per activation chunk = weight prefetch depth
-constexpr int kDirXRow = kDirKC * kTileK + 16;   // LDS row stride of a staged activation row
+constexpr int kDirDepth = 8;                     // weight prefetch depth in K blocks = K blocks per activation chunk
 constexpr uint32_t kOutOfRange = 0xF0000000u;    // buffer offset past every descriptor range: reads zero
 
 __device__ __forceinline__ v4f mfma_16x16x128(v8i a, v8i b, v4f c) {
@@ -33,7 +32,6 @@ __device__ __forceinline__ v4f mfma_16x16x128(v8i a, v8i b, v4f c) {
 __device__ __forceinline__ v4i buf_load16(rsrc_t r, uint32_t voff) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0);
 }
-
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
@@ -43,11 +41,19 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
 
 template <int TM, int MODE, int OUT_DT, int BIAS_DT, bool SPLIT, bool MOE>
 __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
-  static_assert(TM == 16 || TM == 32, "gemm_direct_kernel: 16 or 32 activation rows per block");
-  constexpr int MS = TM / 16;   // 16-row activation sub-tiles
-  constexpr int XPW = TM / 8;   // activation rows staged by one wave
-  __shared__ __attribute__((aligned(16))) uint8_t xs[2][TM * kDirXRow];
-  __shared__ float scs[2][kDirKC][TM];
+  static_assert(TM == 16 || TM == 32, "gemm_direct_kernel: 16 or 32 rows per block (more rows are LDS-read bound here)");
+  constexpr int MS = TM / 16;                 // 16-row activation sub-tiles
+  constexpr int KC = kDirDepth;               // K blocks per activation chunk
+  constexpr int DEPTH = kDirDepth;
+  constexpr int U = DEPTH / KC;               // chunks per trip of the unrolled loop
+  constexpr int RB = KC * kTileK;             // bytes of one activation row in a chunk
+  constexpr int XROW = RB + 16;               // LDS row stride
+  constexpr int LPR = RB / 16;                // lanes per staged row
+  constexpr int RPI = 64 / LPR;               // rows per staging load
+  constexpr int XI = TM / 8 / RPI;            // staging loads per wave per chunk
+  static_assert(TM * KC <= 512, "one scale product per lane and chunk");
+  __shared__ __attribute__((aligned(16))) uint8_t xs[2][TM * XROW];
+  __shared__ float scs[2][KC][TM];
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -83,7 +89,7 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
   const int kb_end = SPLIT ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
   // an expert that lives on another rank contributes zeros: run no K block, the epilogue stores them
   const int nkb = (MOE && expert < 0) ? 0 : max(kb_end - kb_begin, 0);
-  const int nch = (nkb + kDirKC - 1) / kDirKC;
+  const int nch = (nkb + KC - 1) / KC;
   const uint32_t kbytes = (uint32_t)nkb * kTileK;   // bytes of this K range per row
 
   auto slot_of = [&](int i) -> int {   // row slot of block row i, or nrows when the row is padding
@@ -98,27 +104,29 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
   const rsrc_t rW = make_rsrc(Wb + (int64_t)n0w * p.ldw + (int64_t)kb_begin * kTileK,
                               rowsW > 0 ? (uint32_t)((rowsW - 1) * p.ldw) + kbytes : 0u);
   const uint32_t voW = (uint32_t)(r * p.ldw + kq * 16);
-  v4i wreg[kDirKC][2];
+  v4i wreg[DEPTH][2];
   auto load_w = [&](int slot, int kb) {
     const uint32_t vo = kb < nkb ? voW + (uint32_t)kb * kTileK : kOutOfRange;
     wreg[slot][0] = buf_load16(rW, vo);
     wreg[slot][1] = buf_load16(rW, kb < nkb ? vo + 64 : kOutOfRange);
   };
 
-  // ---- activations: wave w stages rows w*XPW .. w*XPW+XPW-1 of the block, 1 KB (8 K blocks) per row
+  // ---- activations: wave w stages rows w*TM/8 .. of the block, RB bytes per row and chunk;
+  // staging load j of a lane covers row w*TM/8 + j*RPI + lane/LPR, bytes (lane%LPR)*16 ..
   const int64_t xrows = MOE ? (int64_t)((p.num_valid + p.top_k - 1) / p.top_k) : (int64_t)p.M;
   const rsrc_t rX = make_rsrc(p.X + (int64_t)kb_begin * kTileK, (uint32_t)((xrows - 1) * p.ldx) + kbytes);
-  uint32_t voX[XPW];
+  const int xcol = (lane % LPR) * 16;
+  uint32_t voX[XI];
 #pragma unroll
-  for (int j = 0; j < XPW; ++j) {
-    const int s = slot_of(w * XPW + j);
+  for (int j = 0; j < XI; ++j) {
+    const int s = slot_of(w * (TM / 8) + j * RPI + lane / LPR);
     const int64_t xr = MOE ? s / p.top_k : s;
-    voX[j] = s < nrows ? (uint32_t)(xr * p.ldx) + lane * 16 : kOutOfRange;
+    voX[j] = s < nrows ? (uint32_t)(xr * p.ldx) + xcol : kOutOfRange;
   }
-  v4i xreg[XPW];
-  // ---- block mode: lane t < TM*8 stages as[m,kb]*bs[nb,kb] of (m = t % TM, kb = chunk*8 + t / TM)
+  v4i xreg[XI];
+  // ---- block mode: lane t < TM*KC stages as[m,kb]*bs[nb,kb] of (m = t % TM, kb = chunk*KC + t / TM)
   const int sm = threadIdx.x % TM, skb = threadIdx.x / TM;
-  const bool stager = MODE == kModeBlock && (int)threadIdx.x < TM * kDirKC;
+  const bool stager = MODE == kModeBlock && (int)threadIdx.x < TM * KC;
   const float* sxp = p.sx;
   const float* swp = p.sw;
   bool srow_ok = false;
@@ -132,22 +140,22 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
   }
   float sreg = 0.f;
   auto stage_load = [&](int c) {
-    const uint32_t k0 = (uint32_t)c * (kDirKC * kTileK);
+    const uint32_t k0 = (uint32_t)c * RB;
 #pragma unroll
-    for (int j = 0; j < XPW; ++j) {
-      const bool ok = voX[j] != kOutOfRange && k0 + lane * 16 < kbytes;
+    for (int j = 0; j < XI; ++j) {
+      const bool ok = voX[j] != kOutOfRange && k0 + xcol < kbytes;
       xreg[j] = buf_load16(rX, ok ? voX[j] + k0 : kOutOfRange);
     }
     if (MODE == kModeBlock) {
-      const int kb = c * kDirKC + skb;
+      const int kb = c * KC + skb;
       sreg = 0.f;
       if (stager && srow_ok && kb < nkb) sreg = sxp[(int64_t)kb * p.sx_k] * swp[(int64_t)kb * p.sw_k];
     }
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
-    for (int j = 0; j < XPW; ++j)
-      *reinterpret_cast<v4i*>(&xs[buf][(w * XPW + j) * kDirXRow + lane * 16]) = xreg[j];
+    for (int j = 0; j < XI; ++j)
+      *reinterpret_cast<v4i*>(&xs[buf][(w * (TM / 8) + j * RPI + lane / LPR) * XROW + xcol]) = xreg[j];
     if (stager) scs[buf][skb][sm] = sreg;
   };
 
@@ -158,36 +166,40 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
   // ---- prologue: chunk 0 into LDS, chunk 1 in registers, weights of K blocks 0..7 in flight
   stage_load(0);
 #pragma unroll
-  for (int d = 0; d < kDirKC; ++d) load_w(d, d);
+  for (int d = 0; d < DEPTH; ++d) load_w(d, d);
   stage_store(0);
   stage_load(1);
 
-  const uint32_t xrd = (uint32_t)(r * kDirXRow + kq * 16);
-  for (int c = 0; c < nch; ++c) {
-    const int buf = c & 1;
-    __syncthreads();        // chunk c is visible; every wave is done with chunk c-1
-    stage_store(buf ^ 1);   // chunk c+1
-    stage_load(c + 2);
+  const uint32_t xrd = (uint32_t)(r * XROW + kq * 16);
+  for (int c0 = 0; c0 < nch; c0 += U) {
 #pragma unroll
-    for (int kbl = 0; kbl < kDirKC; ++kbl) {
-      const v8i wa = join(wreg[kbl][0], wreg[kbl][1]);
-      load_w(kbl, (c + 1) * kDirKC + kbl);
+    for (int u = 0; u < U; ++u) {
+      const int c = c0 + u;         // a chunk past the K range holds zeros and zero scales
+      const int buf = c & 1;
+      __syncthreads();              // chunk c is visible; every wave is done with chunk c-1
+      stage_store(buf ^ 1);         // chunk c+1
+      stage_load(c + 2);
 #pragma unroll
-      for (int ms = 0; ms < MS; ++ms) {
-        const uint8_t* xp = &xs[buf][ms * 16 * kDirXRow + xrd + kbl * kTileK];
-        const v8i xa = join(*reinterpret_cast<const v4i*>(xp), *reinterpret_cast<const v4i*>(xp + 64));
-        if (MODE == kModeBlock) {
-          const v4f t = mfma_16x16x128(wa, xa, v4f{0.f, 0.f, 0.f, 0.f});
-          const float sc = scs[buf][kbl][ms * 16 + r];
+      for (int kbl = 0; kbl < KC; ++kbl) {
+        const int slot = u * KC + kbl;
+        const v8i wa = join(wreg[slot][0], wreg[slot][1]);
+        load_w(slot, c * KC + kbl + DEPTH);
 #pragma unroll
-          for (int i = 0; i < 4; ++i) acc[ms][i] = __builtin_fmaf(t[i], sc, acc[ms][i]);
-        } else {
-          acc[ms] = mfma_16x16x128(wa, xa, acc[ms]);
+        for (int ms = 0; ms < MS; ++ms) {
+          const uint8_t* xp = &xs[buf][ms * 16 * XROW + xrd + kbl * kTileK];
+          const v8i xa = join(*reinterpret_cast<const v4i*>(xp), *reinterpret_cast<const v4i*>(xp + 64));
+          if (MODE == kModeBlock) {
+            const v4f t = mfma_16x16x128(wa, xa, v4f{0.f, 0.f, 0.f, 0.f});
+            const float sc = scs[buf][kbl][ms * 16 + r];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[ms][i] = __builtin_fmaf(t[i], sc, acc[ms][i]);
+          } else {
+            acc[ms] = mfma_16x16x128(wa, xa, acc[ms]);
+          }
         }
       }
     }
   }
-
   // ---- epilogue: lane holds n = n0w + kq*4 .. +3 of activation row ms*16 + r
   const int n = n0w + kq * 4;
   if (n >= p.N) return;

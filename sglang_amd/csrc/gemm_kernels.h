@@ -126,41 +126,82 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // workgroup each, so that the round takes 1/splits of a tile time; they leave float partials in the workspace
 // ([tile - tail_first][split][256 m][256 n]) for tile_reduce_kernel.  Their workgroup ids come last, so they are
 // dispatched when the whole tiles drain.
-template <int MODE, int OUT_DT, int BIAS_DT>
+//
+// MOE: grouped form.  A "tile" is (block of up to 256 token slots of one expert) x (256 weight rows of that
+// expert); activation rows are gathered and output rows scattered through sorted_token_ids, whose slot ids sit
+// in an LDS table.  Each XCD walks a contiguous run of the blocks in use and all n tiles of a block in turn.
+template <int MODE, int OUT_DT, int BIAS_DT, bool MOE>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kStageBytes];
+  __shared__ int32_t slot_tab[MOE ? kTileM : 1];
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int wn = w & 1, wm = w >> 1;
 
-  const int ntiles = p.tiles_m * p.tiles_n;
-  const int per_xcd = (p.tail_first + 7) >> 3;
   const int bid = blockIdx.x;
-  int t, split = 0;
-  const bool is_split = bid >= per_xcd * 8;
-  if (!is_split) {
-    t = (bid & 7) * per_xcd + (bid >> 3);
-    if (t >= p.tail_first) return;
-  } else {
-    const int b2 = bid - per_xcd * 8;
-    t = p.tail_first + b2 / p.splits;
-    split = b2 % p.splits;
-    if (t >= ntiles) return;
-  }
+  int t = 0, split = 0;
+  bool is_split = false;
   int tile_m, tile_n;
-  tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
-  const int m0 = tile_m * kTileM, n0 = tile_n * kTileN;
+  int expert = 0;
+  if (MOE) {
+    const int used = p.num_post_pad[0] / p.block_m;
+    const int per_xcd = (used + 7) >> 3;
+    const int j = bid >> 3;
+    const int mbl = j / p.tiles_n;
+    if (mbl >= per_xcd) return;
+    tile_m = (bid & 7) * per_xcd + mbl;
+    if (tile_m >= used || tile_m >= p.m_blocks) return;
+    tile_n = j - mbl * p.tiles_n;
+    expert = p.expert_ids[tile_m];
+  } else {
+    const int ntiles = p.tiles_m * p.tiles_n;
+    const int per_xcd = (p.tail_first + 7) >> 3;
+    is_split = bid >= per_xcd * 8;
+    if (!is_split) {
+      t = (bid & 7) * per_xcd + (bid >> 3);
+      if (t >= p.tail_first) return;
+    } else {
+      const int b2 = bid - per_xcd * 8;
+      t = p.tail_first + b2 / p.splits;
+      split = b2 % p.splits;
+      if (t >= ntiles) return;
+    }
+    tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
+  }
+  const int m0 = MOE ? 0 : tile_m * kTileM, n0 = tile_n * kTileN;
+  const int nrows = MOE ? p.num_valid : p.M;   // exclusive bound of a valid output row
 
   const int kb_begin = is_split ? split * p.kb_per_split : 0;
   const int kb_end = is_split ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
   const int nkb = kb_end - kb_begin;
 
+  // grouped: slot id of every row of the block (nrows = padding), then the rows this lane loads and scales
+  auto slot_at = [&](int i) -> int { return MOE ? slot_tab[i] : m0 + i; };
+  if (MOE) {
+    if (threadIdx.x < kTileM) {
+      const int i = threadIdx.x;
+      int s = nrows;
+      if (i < p.block_m) s = min(p.sorted_ids[tile_m * p.block_m + i], nrows);
+      slot_tab[i] = s;
+    }
+    __syncthreads();
+    if (expert < 0) {  // expert on another rank: the reference writes zeros
+      for (int i = threadIdx.x; i < kTileM * (kTileN / 4); i += 512) {
+        const int s = slot_tab[i / (kTileN / 4)];
+        const int n = n0 + (i % (kTileN / 4)) * 4;
+        if (s < nrows && n < p.N) store4<OUT_DT>(p.C, (int64_t)s * p.ldc + n, 0.f, 0.f, 0.f, 0.f);
+      }
+      return;
+    }
+  }
+
   // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the
   // matrix edge are out of range and read as zero
-  const int rowsW = min(kTileN, p.N - n0), rowsX = min(kTileM, p.M - m0);
+  const uint8_t* Wb = p.W + (MOE ? (int64_t)expert * p.w_expert_stride : 0);
+  const int rowsW = min(kTileN, p.N - n0), rowsX = MOE ? (nrows + p.top_k - 1) / p.top_k : min(kTileM, p.M - m0);
   const int kbytes = p.K - kb_begin * kTileK;
-  const rsrc_t rW = make_rsrc(p.W + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
+  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
   const rsrc_t rX = make_rsrc(p.X + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
   const int rl = lane >> 3, cp = lane & 7;
   uint32_t voW[2], voX[2];
@@ -168,10 +209,18 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   for (int par = 0; par < 2; ++par) {
     const int c = cp ^ ((par << 2) + (rl >> 1));
     voW[par] = (uint32_t)(rl * p.ldw + c * 16);
-    voX[par] = (uint32_t)(rl * p.ldx + c * 16);
+    voX[par] = (uint32_t)((MOE ? 0 : rl * p.ldx) + c * 16);
   }
-  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = (uint32_t)(w * 32 * p.ldx);
-  const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = (uint32_t)(8 * p.ldx);
+  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = MOE ? 0u : (uint32_t)(w * 32 * p.ldx);
+  const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = MOE ? 0u : (uint32_t)(8 * p.ldx);
+  uint32_t xgather[MOE ? 4 : 1];  // grouped: byte offset of the activation row behind each of this lane's 4 loads
+  if (MOE) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int s = slot_tab[w * 32 + j * 8 + rl];
+      xgather[j] = s < nrows ? (uint32_t)(s / p.top_k) * (uint32_t)p.ldx : 0xF0000000u;
+    }
+  }
   // ---- LDS -> MFMA operands
   const int lr = lane & 31, h = lane >> 5;
   const int swz = (lr >> 1) & 7;
@@ -192,12 +241,19 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   };
 
   // ---- scales (block mode)
-  const int mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
-  const int mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
+  int mrow0, mrow1;  // activation rows whose scales this lane applies (any valid row for padding lanes)
+  if (MOE) {
+    const int s0 = slot_tab[wm * 64 + lr], s1 = slot_tab[wm * 64 + 32 + lr];
+    mrow0 = s0 < nrows ? s0 / p.top_k : 0;
+    mrow1 = s1 < nrows ? s1 / p.top_k : 0;
+  } else {
+    mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
+    mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
+  }
   const float* sx0 = p.sx + (int64_t)mrow0 * p.sx_m + (int64_t)kb_begin * p.sx_k;
   const float* sx1 = p.sx + (int64_t)mrow1 * p.sx_m + (int64_t)kb_begin * p.sx_k;
   const int nb = min(n0 + wn * 128, p.N - 1) >> 7;
-  const float* swp = p.sw + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
+  const float* swp = p.sw + (MOE ? (int64_t)expert * p.sw_expert_stride : 0) + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
 
   v16f acc[4][2];
 #pragma unroll
@@ -221,7 +277,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     // the whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt from the
     // range check, and rows past the matrix edge must read as zero, not touch memory)
     if (idx < 4) buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + ko), 0, base + j * 1024);
-    else buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + ko), 0, base + kXOff + j * 1024);
+    else buf_load16_to_lds(rX, voX[j & 1] + (MOE ? xgather[j] + ko : soX + j * stepX + ko), 0, base + kXOff + j * 1024);
   };
   auto RW = [&](v8i(&dst)[2], const uint8_t* st, int ns) {
     dst[0] = frag(st, rdW + ns * 32 * kTileK, 0);
@@ -330,10 +386,12 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 
 #pragma unroll
   for (int ms = 0; ms < 2; ++ms) {
-    const int m = m0 + wm * 64 + ms * 32 + lr;
-    if (m >= p.M) continue;
+    const int ml = wm * 64 + ms * 32 + lr;  // row inside the tile
+    const int m = slot_at(ml);               // output row
+    if (m >= nrows) continue;
     float sa = 1.f;
     if (MODE == kModeRow && !is_split) sa = p.sx[m];
+    if (MOE && p.topk_w) sa = p.topk_w[m];
 #pragma unroll
     for (int ns = 0; ns < 4; ++ns) {
 #pragma unroll
@@ -345,7 +403,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
         for (int r = 0; r < 4; ++r) v[r] = acc[ns][ms][rg * 4 + r];
         if (is_split) {
           float* tile_part = p.partial + ((int64_t)(t - p.tail_first) * p.splits + split) * (kTileM * kTileN);
-          *reinterpret_cast<float4*>(tile_part + (m - m0) * kTileN + (n - n0)) = make_float4(v[0], v[1], v[2], v[3]);
+          *reinterpret_cast<float4*>(tile_part + ml * kTileN + (n - n0)) = make_float4(v[0], v[1], v[2], v[3]);
         } else {
           if (MODE == kModeRow) {
             const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
@@ -354,6 +412,9 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] += load_scalar<BIAS_DT>(p.bias, n + r);
             }
+          } else if (MOE) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] *= sa;
           }
           store4<OUT_DT>(p.C, (int64_t)m * p.ldc + n, v[0], v[1], v[2], v[3]);
         }

@@ -261,8 +261,8 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
   FP8K_REQUIRE(out_dtype == FP8K_F16 || out_dtype == FP8K_BF16, "%s: out_dtype must be Half or BFloat16", op);
   FP8K_REQUIRE(K % kTileK == 0, "%s: K (%lld) must be a multiple of 128", op, (long long)K);
   FP8K_REQUIRE(N % 8 == 0, "%s: N (%lld) must be a multiple of 8", op, (long long)N);
-  FP8K_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128,
-               "%s: block_m must be 16, 32, 64 or 128 (got %lld)", op, (long long)block_m);
+  FP8K_REQUIRE(block_m == 16 || block_m == 32 || block_m == 64 || block_m == 128 || block_m == 256,
+               "%s: block_m must be 16, 32, 64, 128 or 256 (got %lld)", op, (long long)block_m);
   FP8K_REQUIRE(sorted_capacity >= 0 && sorted_capacity < 0x7fffffffLL, "%s: bad sorted_token_ids length", op);
   FP8K_REQUIRE(lda >= K && ldb >= K && ldc >= N, "%s: leading dimension smaller than the row length", op);
   FP8K_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && (ldc * 2) % 8 == 0, "%s: rows must be 16-byte aligned", op);
@@ -272,7 +272,7 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
                "%s: operands must be 16-byte aligned", op);
   const int64_t xrows = (num_valid_tokens + top_k - 1) / top_k;
   FP8K_REQUIRE(xrows * lda < 0xE0000000LL, "%s: activation matrix exceeds 3.5 GiB, split the token batch", op);
-  FP8K_REQUIRE(256 * ldb + K < 0xE0000000LL, "%s: weight rows too long", op);
+  FP8K_REQUIRE(ldb < (1LL << 23) && lda < (1LL << 23), "%s: rows longer than 8 MiB are not supported", op);
   FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0 && bs_stride_e >= 0,
                "%s: negative scale stride", op);
 
@@ -306,6 +306,13 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
     return check_launch(op);
   }
 #undef FP8K_MOE_DIRECT
+  if (block_m == 256) {  // many rows per expert: the MFMA-bound 256x256 tile kernel, one block of slots per tile
+    if (out_dtype == FP8K_BF16)
+      hipLaunchKernelGGL((gemm_tile256_kernel<kModeBlock, FP8K_BF16, FP8K_F32, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+    else
+      hipLaunchKernelGGL((gemm_tile256_kernel<kModeBlock, FP8K_F16, FP8K_F32, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+    return check_launch(op);
+  }
 #define FP8K_MOE(TM, NST, O) \
   hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, kModeBlock, O, FP8K_F32, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a)
   if (out_dtype == FP8K_BF16) {

@@ -44,16 +44,17 @@ def moe_align_block_size(
 def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     """Rows per block of the grouped GEMM (the reference's BLOCK_SIZE_M, fused_moe_triton_config.py).
 
-    The grouped kernel streams a 256-row weight tile once per block of rows, so the block should hold
-    all rows an expert is expected to receive, up to the kernel's 128-row limit.
+    Measured on MI355X with 256 experts: up to about 8 rows per expert the register-streaming kernel with
+    32-row blocks wins; beyond that 128-row blocks (one weight pass per expert) through the LDS-staged
+    streaming kernel; with several hundred rows per expert the 256x256 MFMA tile kernel.
     """
     per_expert = (M * topk + E - 1) // max(E, 1)
-    if per_expert <= 32:
+    if per_expert <= 8:
         bm = 32
-    elif per_expert <= 64:
-        bm = 64
-    else:
+    elif per_expert <= 384:
         bm = 128
+    else:
+        bm = 256
     return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}
 
 

@@ -152,7 +152,8 @@ def _expert_weights(rng, E, N, K):
 
 
 @pytest.mark.parametrize("T,E,topk,N,K,block", [(5, 8, 2, 512, 256, 16), (64, 8, 2, 384, 512, 32), (300, 16, 4, 1024, 1024, 64),
-                                               (700, 4, 2, 256, 384, 128), (3, 16, 8, 1024, 7168, 32)])
+                                               (700, 4, 2, 256, 384, 128), (3, 16, 8, 1024, 7168, 32),
+                                               (700, 4, 2, 512, 384, 256), (300, 16, 4, 1024, 1024, 256)])
 def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block):
     """GEMM1 form (row = slot // top_k, no routed weight) and GEMM2 form (row = slot, times routed weight)."""
     from sglang_amd.fused_moe import moe_align_block_size
