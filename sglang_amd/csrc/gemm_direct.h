@@ -1,21 +1,23 @@
 // Weight-streaming FP8 GEMM for at most 32 activation rows per block (decode and small-batch MoE), gfx950.
 //
-// With so few activation rows the GEMM is an HBM stream of the weight matrix (2*TM FLOP per weight byte, under the
-// chip's ridge), so the weight bytes never touch LDS: a wavefront owns 16 weight rows and loads them from global
-// memory straight into the register layout of the "A" operand of v_mfma_f32_16x16x128_f8f6f4 (lane l holds 32
-// bytes of row l%16), eight K blocks ahead of their use.  The matrix core only sums over K, so the K order inside
-// a 128-byte block is free as long as both operands agree: lane (row, q = l/16) takes bytes [q*16, q*16+16) and
-// [64+q*16, 64+q*16+16) of the block, which makes each of the two 16-byte loads cover whole 64-byte runs of 16
-// rows (cached loads: the two halves of a 128-byte line meet in the vector cache; marked non-temporal they
-// measured 10 % slower).  No barrier, no LDS round trip and no wait other than the compiler's own register
-// dependencies sits between HBM and the matrix core for the weights.
+// With so few activation rows the GEMM is an HBM stream of the weight matrix (2*TM FLOP per weight byte, far under
+// the chip's ridge), so everything is arranged around the weight loads.  A wavefront owns 16 weight rows and keeps
+// eight K blocks (16 KB) of them in flight in registers: two non-temporal 16-byte loads per lane and K block, each
+// instruction covering 8 whole 128-byte lines (lane l: row l/8, 16-byte chunk l%8) - whole-line requests measured
+// 25 % more HBM bandwidth here than the half-line requests that loading straight into the matrix-core operand
+// layout would make.  The move into that layout (operand "A" of v_mfma_f32_16x16x128_f8f6f4: lane l holds 32 bytes
+// of row l%16) is a round trip through a 2 KB LDS slot private to the wave: LDS operations of one wave execute in
+// order, so it needs no barrier and no wait beyond the register dependency.  The matrix core only sums over K, so
+// the K order inside a 128-byte block is free as long as both operands agree: lane (row, q = l/16) takes chunks
+// q and 4+q of the block.
 //
 // The activation rows (shared by the 8 waves = 128 weight rows of a workgroup) are staged through LDS in chunks
-// of 8 K blocks: registers -> ds_write one chunk ahead, one barrier per chunk, rows padded by 16 bytes so the
-// 16 rows of an operand fetch fall into different banks.  (Every wave re-reads all activation rows of the block
-// from LDS, which is why blocks of 64 and 128 rows measured slower here than through gemm_stream_kernel.)  In block mode the chunk also
-// carries as[m,kb]*bs[nb,kb] (a workgroup spans exactly one 128-row weight scale block), zero past the K range,
-// so the K tail needs no branch.
+// of 8 K blocks: registers -> ds_write one chunk ahead, one barrier per chunk (an LDS-only barrier: the weight
+// loads stay in flight across it), rows padded by 16 bytes so the 16 rows of an operand fetch fall into different
+// banks.  In block mode the chunk also carries as[m,kb]*bs[nb,kb] (a workgroup spans exactly one 128-row weight
+// scale block), zero past the K range, so the K tail needs no branch.  (Every wave re-reads all activation rows
+// of the block from LDS, which is why blocks of 64 and 128 rows measured slower here than through
+// gemm_stream_kernel.)
 #pragma once
 
 #include "gemm_kernels.h"
@@ -32,6 +34,9 @@ __device__ __forceinline__ v4f mfma_16x16x128(v8i a, v8i b, v4f c) {
 __device__ __forceinline__ v4i buf_load16(rsrc_t r, uint32_t voff) {
   return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 0);
 }
+__device__ __forceinline__ v4i buf_load16_stream(rsrc_t r, uint32_t voff) {  // non-temporal: used once
+  return __builtin_amdgcn_raw_buffer_load_b128(r, voff, 0, 2);
+}
 __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
   v8i r;
   r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
@@ -40,7 +45,7 @@ __device__ __forceinline__ v8i join(v4i lo, v4i hi) {
 }
 
 template <int TM, int MODE, int OUT_DT, int BIAS_DT, bool SPLIT, bool MOE>
-__global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
+__global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const GemmArgs p) {
   static_assert(TM == 16 || TM == 32, "gemm_direct_kernel: 16 or 32 rows per block (more rows are LDS-read bound here)");
   constexpr int MS = TM / 16;                 // 16-row activation sub-tiles
   constexpr int KC = kDirDepth;               // K blocks per activation chunk
@@ -54,6 +59,7 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
   static_assert(TM * KC <= 512, "one scale product per lane and chunk");
   __shared__ __attribute__((aligned(16))) uint8_t xs[2][TM * XROW];
   __shared__ float scs[2][KC][TM];
+  __shared__ __attribute__((aligned(16))) uint8_t wl[8][16 * kTileK];  // per wave: one K block of its 16 weight rows
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -103,12 +109,25 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
   const int rowsW = min(16, p.N - n0w);
   const rsrc_t rW = make_rsrc(Wb + (int64_t)n0w * p.ldw + (int64_t)kb_begin * kTileK,
                               rowsW > 0 ? (uint32_t)((rowsW - 1) * p.ldw) + kbytes : 0u);
-  const uint32_t voW = (uint32_t)(r * p.ldw + kq * 16);
+  // load j of a K block: row j*8 + lane/8, chunk lane%8; in LDS chunk c of row i sits at position c ^ ((i>>1)&7),
+  // which keeps both the line-shaped writes and the operand-shaped reads free of bank conflicts
+  const int wrow = lane >> 3, wc = lane & 7;
+  const uint32_t voW0 = (uint32_t)(wrow * p.ldw + wc * 16), voW1 = (uint32_t)((wrow + 8) * p.ldw + wc * 16);
+  uint8_t* const wslot = wl[w];
+  const uint32_t wst0 = (uint32_t)(wrow * kTileK + ((wc ^ ((wrow >> 1) & 7)) << 4));
+  const uint32_t wst1 = (uint32_t)((wrow + 8) * kTileK + ((wc ^ (((wrow + 8) >> 1) & 7)) << 4));
+  const uint32_t wrd0 = (uint32_t)(r * kTileK + ((kq ^ ((r >> 1) & 7)) << 4));
+  const uint32_t wrd1 = (uint32_t)(r * kTileK + (((4 + kq) ^ ((r >> 1) & 7)) << 4));
   v4i wreg[DEPTH][2];
   auto load_w = [&](int slot, int kb) {
-    const uint32_t vo = kb < nkb ? voW + (uint32_t)kb * kTileK : kOutOfRange;
-    wreg[slot][0] = buf_load16(rW, vo);
-    wreg[slot][1] = buf_load16(rW, kb < nkb ? vo + 64 : kOutOfRange);
+    const bool ok = kb < nkb;
+    wreg[slot][0] = buf_load16_stream(rW, ok ? voW0 + (uint32_t)kb * kTileK : kOutOfRange);
+    wreg[slot][1] = buf_load16_stream(rW, ok ? voW1 + (uint32_t)kb * kTileK : kOutOfRange);
+  };
+  auto weight_operand = [&](int slot) -> v8i {  // registers (line layout) -> LDS -> registers (operand layout)
+    *reinterpret_cast<v4i*>(wslot + wst0) = wreg[slot][0];
+    *reinterpret_cast<v4i*>(wslot + wst1) = wreg[slot][1];
+    return join(*reinterpret_cast<const v4i*>(wslot + wrd0), *reinterpret_cast<const v4i*>(wslot + wrd1));
   };
 
   // ---- activations: wave w stages rows w*TM/8 .. of the block, RB bytes per row and chunk;
@@ -138,7 +157,7 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
     swp = p.sw + (MOE && expert >= 0 ? (int64_t)expert * p.sw_expert_stride : 0) +
           (int64_t)(min(n0, p.N - 1) >> 7) * p.sw_n + (int64_t)kb_begin * p.sw_k;
   }
-  float sreg = 0.f;
+  float sreg_x = 0.f, sreg_w = 0.f;  // multiplied at store time: using them here would wait for every load in flight
   auto stage_load = [&](int c) {
     const uint32_t k0 = (uint32_t)c * RB;
 #pragma unroll
@@ -148,27 +167,42 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
     }
     if (MODE == kModeBlock) {
       const int kb = c * KC + skb;
-      sreg = 0.f;
-      if (stager && srow_ok && kb < nkb) sreg = sxp[(int64_t)kb * p.sx_k] * swp[(int64_t)kb * p.sw_k];
+      sreg_x = 0.f;
+      sreg_w = 0.f;
+      if (stager && srow_ok && kb < nkb) {
+        sreg_x = sxp[(int64_t)kb * p.sx_k];
+        sreg_w = swp[(int64_t)kb * p.sw_k];
+      }
     }
   };
   auto stage_store = [&](int buf) {
 #pragma unroll
     for (int j = 0; j < XI; ++j)
       *reinterpret_cast<v4i*>(&xs[buf][(w * (TM / 8) + j * RPI + lane / LPR) * XROW + xcol]) = xreg[j];
-    if (stager) scs[buf][skb][sm] = sreg;
+    if (stager) scs[buf][skb][sm] = sreg_x * sreg_w;
   };
 
   v4f acc[MS];
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) acc[ms] = v4f{0.f, 0.f, 0.f, 0.f};
 
-  // ---- prologue: chunk 0 into LDS, chunk 1 in registers, weights of K blocks 0..7 in flight
+  // ---- prologue: chunks 0 and 1 requested, then the weights of K blocks 0..7, then chunk 0 into LDS.  The loop
+  // keeps the same age order (staging loads older than the weight loads issued after them), so that the wait
+  // for a staged chunk never has to drain the weight prefetch.
   stage_load(0);
+  v4i xreg0[XI];
+#pragma unroll
+  for (int j = 0; j < XI; ++j) xreg0[j] = xreg[j];
+  const float s0x = sreg_x, s0w = sreg_w;
+  stage_load(1);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int d = 0; d < DEPTH; ++d) load_w(d, d);
-  stage_store(0);
-  stage_load(1);
+  __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+  for (int j = 0; j < XI; ++j)
+    *reinterpret_cast<v4i*>(&xs[0][(w * (TM / 8) + j * RPI + lane / LPR) * XROW + xcol]) = xreg0[j];
+  if (stager) scs[0][skb][sm] = s0x * s0w;
 
   const uint32_t xrd = (uint32_t)(r * XROW + kq * 16);
   for (int c0 = 0; c0 < nch; c0 += U) {
@@ -176,13 +210,16 @@ __global__ __launch_bounds__(512, 4) void gemm_direct_kernel(const GemmArgs p) {
     for (int u = 0; u < U; ++u) {
       const int c = c0 + u;         // a chunk past the K range holds zeros and zero scales
       const int buf = c & 1;
-      __syncthreads();              // chunk c is visible; every wave is done with chunk c-1
+      lds_barrier();                // chunk c is visible; every wave is done with chunk c-1 (weight loads stay in flight)
       stage_store(buf ^ 1);         // chunk c+1
       stage_load(c + 2);
+      // memory operations retire in order: the staging loads must stay OLDER than this trip's weight loads, or
+      // the wait for them at the next barrier would drain the weight prefetch
+      __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int kbl = 0; kbl < KC; ++kbl) {
         const int slot = u * KC + kbl;
-        const v8i wa = join(wreg[slot][0], wreg[slot][1]);
+        const v8i wa = weight_operand(slot);
         load_w(slot, c * KC + kbl + DEPTH);
 #pragma unroll
         for (int ms = 0; ms < MS; ++ms) {

@@ -109,6 +109,19 @@ __device__ __forceinline__ void buf_load16_to_lds(rsrc_t r, uint32_t voff, uint3
 }
 __device__ __forceinline__ void wait_vm0_lgkm0() { __builtin_amdgcn_s_waitcnt(0x0070); }  // vmcnt(0) lgkmcnt(0)
 
+// Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a release fence, and on this family
+// stores and loads share vmcnt, so it drains every outstanding global load of the wave - which would empty a
+// multi-stage prefetch pipeline at each barrier.  Here a wave waits for its own LDS operations (and for all but
+// `vm_in_flight` of its vector-memory operations, 63 = no wait), then joins the barrier.
+template <int VM_IN_FLIGHT = 63>
+__device__ __forceinline__ void lds_barrier() {
+  static_assert(VM_IN_FLIGHT >= 0 && VM_IN_FLIGHT < 64, "vmcnt is a 6-bit counter");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0070 | (VM_IN_FLIGHT & 15) | ((VM_IN_FLIGHT >> 4) << 14));  // lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // tile index -> (tile_m, tile_n): tiles are numbered in groups of 4 m-tiles, m fastest inside a group, so that
 // the tiles that run together on one XCD cover 4 activation tiles x a run of weight tiles
 __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int& tile_m, int& tile_n) {
@@ -579,27 +592,35 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
 
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s) issue(s);
-  float sxn[MS], sbn = 0.f;
-  if (MODE == kModeBlock && nkb > 0) {
+  // Scales travel two K blocks ahead, and the loads of block it+2 are issued BEFORE the stage loads of the same
+  // trip: memory operations retire in order, so a scale that is younger than a stage load could only be waited
+  // for by draining that stage load too, which would serialise the whole pipeline on HBM latency.
+  constexpr int SL = MODE == kModeBlock ? MS + 1 : 0;  // scale loads per trip
+  float sxa[MS], sxb[MS], sba = 0.f, sbb = 0.f;         // scales of the even / odd K blocks in flight
+  auto load_scales = [&](float (&sx)[MS], float& sb, int kb) {
+    const int kn = min(kb, nkb - 1);
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) sxn[ms] = sxp[ms][0];
-    sbn = swp[0];
+    for (int ms = 0; ms < MS; ++ms) sx[ms] = sxp[ms][(int64_t)kn * p.sx_k];
+    sb = swp[(int64_t)kn * p.sw_k];
+  };
+  if (MODE == kModeBlock && nkb > 0) {
+    load_scales(sxa, sba, 0);
+    load_scales(sxb, sbb, 1);
   }
 
-  for (int it = 0; it < nkb; ++it) {
-    // stage `it` has landed once at most NSTAGE-2 younger stages are still in flight
-    __builtin_amdgcn_s_waitcnt(0x0F70 | (((NSTAGE - 2) * LPW) & 15) | ((((NSTAGE - 2) * LPW) >> 4) << 14));
-    __syncthreads();
-    issue(it + NSTAGE - 1);  // refills the stage every wave finished before this barrier
+  // one K block; (sx, sb) hold its scales on entry and are reloaded with those of block it+2
+  auto trip = [&](int it, float (&sx)[MS], float& sb) {
+    // stage `it` has landed once at most NSTAGE-2 younger trips (stage + scale loads each) are still in flight
+    constexpr int kInFlight = (NSTAGE - 2) * (LPW + SL);
+    lds_barrier<kInFlight>();
     float sc[MS];
     if (MODE == kModeBlock) {
 #pragma unroll
-      for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
-      const int kn = min(it + 1, nkb - 1);
-#pragma unroll
-      for (int ms = 0; ms < MS; ++ms) sxn[ms] = sxp[ms][(int64_t)kn * p.sx_k];
-      sbn = swp[(int64_t)kn * p.sw_k];
+      for (int ms = 0; ms < MS; ++ms) sc[ms] = sx[ms] * sb;
+      load_scales(sx, sb, it + 2);
+      __builtin_amdgcn_sched_barrier(0);  // keep the scale loads ahead of the stage loads
     }
+    issue(it + NSTAGE - 1);  // refills the stage every wave finished before this barrier
     const uint8_t* st = smem + (it % NSTAGE) * STAGE;
     v8i wf[2];
     wf[0] = frag(st, rdW, 0);
@@ -621,7 +642,13 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
         acc[ms] = mfma_32x32x64(wf[1], x1, acc[ms]);
       }
     }
+  };
+  int it = 0;
+  for (; it + 1 < nkb; it += 2) {
+    trip(it, sxa, sba);
+    trip(it + 1, sxb, sbb);
   }
+  if (it < nkb) trip(it, sxa, sba);
   wait_vm0();  // drain the padding loads before the LDS allocation is released
 
   // ---- epilogue

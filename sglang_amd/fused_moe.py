@@ -45,11 +45,13 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     """Rows per block of the grouped GEMM (the reference's BLOCK_SIZE_M, fused_moe_triton_config.py).
 
     Measured on MI355X with 256 experts: up to about 8 rows per expert the register-streaming kernel with
-    32-row blocks wins; beyond that 128-row blocks (one weight pass per expert) through the LDS-staged
+    16- or 32-row blocks wins; beyond that 128-row blocks (one weight pass per expert) through the LDS-staged
     streaming kernel; with several hundred rows per expert the 256x256 MFMA tile kernel.
     """
     per_expert = (M * topk + E - 1) // max(E, 1)
-    if per_expert <= 8:
+    if per_expert <= 1:
+        bm = 16
+    elif per_expert <= 8:
         bm = 32
     elif per_expert <= 384:
         bm = 128
