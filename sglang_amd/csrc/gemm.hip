@@ -40,7 +40,7 @@ static Plan make_plan(int64_t M, int64_t N, int64_t K) {
   if (M <= 128 && M * K < (1LL << 31)) {
     // decode-sized: stream the weights once, every CU takes a K slice of one 256-row weight tile
     pl.kind = 2;
-    pl.tm = M <= 32 ? 32 : (M <= 64 ? 64 : 128);
+    pl.tm = M <= 64 ? 64 : 128;
     const int64_t tiles_n = (N + kTileN - 1) / kTileN;
     int splits = (int)(256 / tiles_n);
     if (splits > kb / 4) splits = kb / 4;
@@ -109,18 +109,17 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   if (pl.kind == 2) {
     a.m_blocks = 1;
     const unsigned nwg = (unsigned)(((a.tiles_n + 7) / 8) * 8 * pl.splits);
-#define FP8K_STREAM(TM, NST)                                                                                          \
+#define FP8K_STREAM(TM, NST, NW)                                                                                      \
   do {                                                                                                                \
     if (pl.splits == 1)                                                                                               \
-      hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, MODE, OUT_DT, BIAS_DT, false, false>), dim3(nwg), dim3(512), 0, \
-                         st, a);                                                                                      \
+      hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, NW, MODE, OUT_DT, BIAS_DT, false, false>), dim3(nwg),           \
+                         dim3(NW * 64), 0, st, a);                                                                    \
     else                                                                                                              \
-      hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, MODE, OUT_DT, BIAS_DT, true, false>), dim3(nwg), dim3(512), 0,  \
-                         st, a);                                                                                      \
+      hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, NW, MODE, OUT_DT, BIAS_DT, true, false>), dim3(nwg),            \
+                         dim3(NW * 64), 0, st, a);                                                                    \
   } while (0)
-    if (pl.tm == 32) FP8K_STREAM(32, 4);
-    else if (pl.tm == 64) FP8K_STREAM(64, 3);
-    else FP8K_STREAM(128, 3);
+    if (pl.tm == 64) FP8K_STREAM(64, 3, 8);
+    else FP8K_STREAM(128, 3, 8);
 #undef FP8K_STREAM
     int rc = check_launch("gemm_stream");
     if (rc || pl.splits == 1) return rc;

@@ -438,19 +438,25 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 
 
 // ------------------------------------------------------------------------------------------------
-// Weight-streaming kernel for few rows: 256(n) x TM(m) x 128(k) tile, TM in {32, 64, 128}, 8 waves each
-// owning 32 weight rows x all TM activation rows.  Used for decode-sized dense GEMMs (with split-K
-// through a float workspace so that every CU streams a share of the weights) and for the grouped
-// MoE GEMM, where a block of TM token slots belongs to one expert and activation / output rows go
-// through sorted_token_ids.  These shapes are HBM-bound (2*TM FLOP per weight byte), so the design
-// point is bytes in flight, not MFMA occupancy: NSTAGE LDS stages of [W 32 KB | X TM*128 B] are kept
-// full with partial vmcnt waits; a wave reads its 32 weight rows from LDS exactly once.
+// Weight-streaming kernel for 33..128 activation rows: 256(n) x TM(m) x 128(k) tile, TM in {64, 128}.
+// Used for small dense batches (with split-K through a float workspace so that every CU streams a share
+// of the weights) and for the grouped MoE GEMM, where a block of up to TM token slots belongs to one
+// expert and activation / output rows go through sorted_token_ids.  These shapes sit under the chip's
+// ridge (2*TM FLOP per weight byte), so the design point is bytes in flight, not MFMA occupancy:
+// NSTAGE LDS stages of [W 32 KB | X TM*128 B] are kept full with partial vmcnt waits and an LDS-only
+// barrier per K block.  NW = 8 waves: each owns 32 weight rows x all TM rows (the form in use).  NW = 16
+// waves: 8 along n x 2 along m, each 32 weight rows x TM/2 rows; it measured 5-8 % slower on the MoE shapes
+// (more LDS operand traffic per MFMA) and is kept as a tuning option.
 // ------------------------------------------------------------------------------------------------
-template <int TM, int NSTAGE, int MODE, int OUT_DT, int BIAS_DT, bool SPLIT, bool MOE>
-__global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
-  constexpr int MS = TM / 32;                    // 32-row activation sub-tiles
-  constexpr int XL = (TM + 63) / 64;             // X wave-loads per wave per stage
-  constexpr int LPW = 4 + XL;                    // LDS-DMA loads per wave per stage
+template <int TM, int NSTAGE, int NW, int MODE, int OUT_DT, int BIAS_DT, bool SPLIT, bool MOE>
+__global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs p) {
+  static_assert((TM == 64 || TM == 128) && (NW == 8 || NW == 16), "gemm_stream_kernel: unsupported shape");
+  constexpr int MH = NW / 8;                     // waves along m
+  constexpr int MS = TM / 32 / MH;               // 32-row activation sub-tiles per wave
+  constexpr int WL = 32 / NW;                    // W wave-loads (8 rows each) per wave per stage
+  constexpr int XG = TM / 8;                     // 8-row groups of the X tile
+  constexpr int XL = (XG + NW - 1) / NW;         // X wave-loads per wave per stage
+  constexpr int LPW = WL + XL;                   // LDS-DMA loads per wave per stage
   constexpr int WBYTES = kTileN * kTileK;
   constexpr int STAGE = WBYTES + TM * kTileK;
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * STAGE + 1024];
@@ -458,6 +464,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int wn = w & 7, wm = w >> 3;             // wave position: 32 weight rows, half of the m rows
 
   // ---- work item.  Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each).
   // Dense: each XCD takes a contiguous run of items, consecutive ids walk the m blocks of one n tile.
@@ -495,13 +502,14 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
   const int kb_end = SPLIT ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
   const int nkb = kb_end - kb_begin;
 
-  // ---- output rows of this lane (m = ms*32 + lane%32)
+  // ---- output rows of this lane (block row = wm*TM/2 + ms*32 + lane%32)
   const int lr = lane & 31, h = lane >> 5;
+  const int mrow0 = wm * (TM / MH);
   int out_slot[MS];
   bool out_ok[MS];
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
-    const int r = ms * 32 + lr;
+    const int r = mrow0 + ms * 32 + lr;
     out_slot[ms] = MOE ? (r < block_m ? p.sorted_ids[slot0 + r] : nrows) : slot0 + r;
     out_ok[ms] = out_slot[ms] < nrows;
   }
@@ -511,14 +519,15 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
     for (int ms = 0; ms < MS; ++ms) {
       if (!out_ok[ms]) continue;
       for (int j = 0; j < 4; ++j) {
-        const int n = n0 + w * 32 + h * 16 + j * 4;
+        const int n = n0 + wn * 32 + h * 16 + j * 4;
         if (n < p.N) store4<OUT_DT>(p.C, (int64_t)out_slot[ms] * p.ldc + n, 0.f, 0.f, 0.f, 0.f);
       }
     }
     return;
   }
 
-  // ---- global -> LDS
+  // ---- global -> LDS: wave load g of W covers rows g*8 .. g*8+7 (lane: row lane/8, chunk lane%8, stored at
+  // chunk position c ^ ((row>>1)&7)); the whole offset travels in the bounds-checked per-lane operand
   const uint8_t* Wb = p.W + (MOE ? (int64_t)expert * p.w_expert_stride : 0);
   const int rowsW = min(kTileN, p.N - n0);
   const int kbytes = p.K - kb_begin * kTileK;
@@ -527,16 +536,18 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
   const int64_t xrows = MOE ? (int64_t)((p.num_valid + p.top_k - 1) / p.top_k) : (int64_t)p.M;
   const rsrc_t rX = make_rsrc(p.X + (int64_t)kb_begin * kTileK, (uint32_t)((xrows - 1) * p.ldx + kbytes));
   const int rl = lane >> 3, cp = lane & 7;
-  uint32_t voW[2];
+  uint32_t voW[WL];
 #pragma unroll
-  for (int par = 0; par < 2; ++par) voW[par] = (uint32_t)(rl * p.ldw + ((cp ^ ((par << 2) + (rl >> 1))) * 16));
-  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), stepW = (uint32_t)(8 * p.ldw);
+  for (int j = 0; j < WL; ++j) {
+    const int g = w * WL + j;
+    voW[j] = (uint32_t)((g * 8 + rl) * p.ldw + ((cp ^ (((g & 1) << 2) + (rl >> 1))) * 16));
+  }
   uint32_t voX[XL];
   bool xload[XL];
 #pragma unroll
   for (int j = 0; j < XL; ++j) {
     const int grp = w * XL + j;             // 8-row group of the X tile
-    xload[j] = grp * 8 < TM;                // wave-uniform
+    xload[j] = grp < XG;                    // wave-uniform
     const int row = grp * 8 + rl;
     const int c = cp ^ (((grp & 1) << 2) + (rl >> 1));
     int s = nrows;
@@ -549,8 +560,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
     uint8_t* base = smem + (kstep % NSTAGE) * STAGE;
     const uint32_t ko = (uint32_t)kstep * kTileK;
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + ko), 0, base + w * 4096 + j * 1024);
+    for (int j = 0; j < WL; ++j) buf_load16_to_lds(rW, voW[j] + ko, 0, base + (w * WL + j) * 1024);
 #pragma unroll
     for (int j = 0; j < XL; ++j)
       buf_load16_to_lds(rX, voX[j] + ko, 0, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
@@ -563,8 +573,8 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
   for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
     for (int j = 0; j < 2; ++j) co[ks][j] = (uint32_t)(((ks * 4 + h * 2 + j) ^ swz) << 4);
-  const uint32_t rdW = (uint32_t)((w * 32 + lr) * kTileK);
-  const uint32_t rdX = (uint32_t)(WBYTES + lr * kTileK);
+  const uint32_t rdW = (uint32_t)((wn * 32 + lr) * kTileK);
+  const uint32_t rdX = (uint32_t)(WBYTES + (mrow0 + lr) * kTileK);
   auto frag = [&](const uint8_t* st, uint32_t rowoff, int ks) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][0]);
     const v4i hi = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][1]);
@@ -581,7 +591,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
     const int64_t xr = out_ok[ms] ? (MOE ? out_slot[ms] / p.top_k : out_slot[ms]) : 0;
     sxp[ms] = p.sx + xr * p.sx_m + (int64_t)kb_begin * p.sx_k;
   }
-  const int nb = min(n0 + w * 32, p.N - 1) >> 7;
+  const int nb = min(n0 + wn * 32, p.N - 1) >> 7;
   const float* swp = p.sw + (MOE ? (int64_t)expert * p.sw_expert_stride : 0) + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
 
   v16f acc[MS];
@@ -661,7 +671,7 @@ __global__ __launch_bounds__(512, 1) void gemm_stream_kernel(const GemmArgs p) {
     if (MOE && p.topk_w) rs = p.topk_w[orow];
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
-      const int n = n0 + w * 32 + rg * 8 + h * 4;
+      const int n = n0 + wn * 32 + rg * 8 + h * 4;
       if (n >= p.N) continue;
       float v[4];
 #pragma unroll

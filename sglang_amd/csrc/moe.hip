@@ -313,16 +313,14 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
       hipLaunchKernelGGL((gemm_tile256_kernel<kModeBlock, FP8K_F16, FP8K_F32, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
     return check_launch(op);
   }
-#define FP8K_MOE(TM, NST, O) \
-  hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, kModeBlock, O, FP8K_F32, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a)
+#define FP8K_MOE(TM, NST, NW, O) \
+  hipLaunchKernelGGL((gemm_stream_kernel<TM, NST, NW, kModeBlock, O, FP8K_F32, false, true>), dim3((unsigned)nwg), dim3(NW * 64), 0, st, a)
   if (out_dtype == FP8K_BF16) {
-    if (block_m <= 32) FP8K_MOE(32, 4, FP8K_BF16);
-    else if (block_m == 64) FP8K_MOE(64, 3, FP8K_BF16);
-    else FP8K_MOE(128, 3, FP8K_BF16);
+    if (block_m == 64) FP8K_MOE(64, 3, 8, FP8K_BF16);
+    else FP8K_MOE(128, 3, 8, FP8K_BF16);
   } else {
-    if (block_m <= 32) FP8K_MOE(32, 4, FP8K_F16);
-    else if (block_m == 64) FP8K_MOE(64, 3, FP8K_F16);
-    else FP8K_MOE(128, 3, FP8K_F16);
+    if (block_m == 64) FP8K_MOE(64, 3, 8, FP8K_F16);
+    else FP8K_MOE(128, 3, 8, FP8K_F16);
   }
 #undef FP8K_MOE
   return check_launch(op);
