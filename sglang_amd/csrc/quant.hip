@@ -55,34 +55,61 @@ __device__ __forceinline__ float absmax8(const float (&a)[8]) {
   return m;
 }
 
-// q = RNE_e4m3fn(clamp(a / sc)) for 8 values, bit-identical to an IEEE float32 divide followed by
-// the cast.  The divide is replaced by two multiplies with reciprocals that bracket the true
-// quotient (relative half-width 2^-20, far wider than the 2^-22 error of x * rcp(sc)); the cast
-// is monotonic, so when both ends land on the same byte the exact quotient does too.  The rare
-// lane whose bracket straddles a rounding boundary redoes its 8 values with the real divide.
-__device__ __forceinline__ uint2 quant8_div(const float (&a)[8], float sc) {
+// q = RNE_e4m3fn(clamp(RN32(a / sc))) for 8 values - bit-identical to an IEEE float32 divide followed by the
+// cast - without a divide and without a branch.  The quotient is bracketed by two multiplies with reciprocals
+// (relative half-width 2^-20, far wider than the 2^-22 error of x * rcp(sc)); the cast is monotonic, so where
+// both ends give the same byte the exact quotient does too.  Where they differ, for 16-bit inputs the answer
+// follows from number theory instead of a divide.  Let amax = ma * 2^ea and x = mx * 2^ex with integer
+// mantissas below 2^11, and Q0 = 448 x / amax, the quotient by the UNROUNDED scale.  Q0 is a rational with
+// denominator ma, so it is either exactly a rounding boundary m = (2t+1) * 2^i of the cast or at least 2^-16
+// (relative) away from every boundary; the bracket (2^-19) plus the rounding of the scale (2^-24) cannot
+// bridge that, hence a differing byte means Q0 == m, a structural tie (0.3 % of real activations).  What the
+// reference then produces depends only on how the scale was rounded, e = sc * 448 - amax (exact in one fma):
+//   * e == 0 (ma is a multiple of 7, one group in seven): the quotient is m itself, round-half-to-even picks
+//     the code with a clear low bit;
+//   * e != 0: 7 does not divide ma, so 7 divides 2t+1, and the cast's boundaries only offer 2t+1 = 21 (normal
+//     range, lower code even) and 7 (subnormal range, upper code even).  The float32 quotient m / (1 + e/amax)
+//     rounds to m unless |e/amax| exceeds half an ulp at m, 2^-20/21 resp. 2^-22/7; equality would need
+//     7 | ma.  So: scale rounded up by more than 2^-22/7 -> always the lower code; rounded down by more than
+//     2^-20/21 -> always the upper code; otherwise the tie goes to the even code.
+// All three cases are lane-group uniform selects and three bit operations per word.  Scales outside
+// [2^-100, 2^100] (reachable only with a non-default eps or non-finite data) and float32 inputs, whose
+// mantissas are too long for the argument, set `redo`: the caller recomputes those lanes with the real divide.
+template <bool SHORT_MANTISSA>
+__device__ __forceinline__ uint2 quant8_bracket(const float (&a)[8], float sc, float amax, bool& redo) {
   const float r = __builtin_amdgcn_rcpf(sc);  // 1 ulp
   const float r_lo = r * (1.0f - 0x1p-20f);
   const float r_hi = r * (1.0f + 0x1p-20f);
-  uint32_t l0 = cvt4_fp8(a[0] * r_lo, a[1] * r_lo, a[2] * r_lo, a[3] * r_lo);
-  uint32_t l1 = cvt4_fp8(a[4] * r_lo, a[5] * r_lo, a[6] * r_lo, a[7] * r_lo);
-  uint32_t h0 = cvt4_fp8(a[0] * r_hi, a[1] * r_hi, a[2] * r_hi, a[3] * r_hi);
-  uint32_t h1 = cvt4_fp8(a[4] * r_hi, a[5] * r_hi, a[6] * r_hi, a[7] * r_hi);
-  // sc outside [2^-100, 2^100] (only reachable with a non-default eps or non-finite data): no bracket
+  const uint32_t l0 = cvt4_fp8(a[0] * r_lo, a[1] * r_lo, a[2] * r_lo, a[3] * r_lo);
+  const uint32_t l1 = cvt4_fp8(a[4] * r_lo, a[5] * r_lo, a[6] * r_lo, a[7] * r_lo);
+  const uint32_t h0 = cvt4_fp8(a[0] * r_hi, a[1] * r_hi, a[2] * r_hi, a[3] * r_hi);
+  const uint32_t h1 = cvt4_fp8(a[4] * r_hi, a[5] * r_hi, a[6] * r_hi, a[7] * r_hi);
   const bool safe = (__float_as_uint(sc) - 0x0D800000u) < (0x71800000u - 0x0D800000u);
-  if (__builtin_expect((l0 != h0) | (l1 != h1) | !safe, 0)) {
-    float y[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      float t = a[i] / sc;  // IEEE correctly rounded (no fast-math in this build)
-      t = t < -kFp8Max ? -kFp8Max : t;  // NaN falls through, as torch.clamp does
-      t = t > kFp8Max ? kFp8Max : t;
-      y[i] = t;
-    }
-    l0 = cvt4_fp8(y[0], y[1], y[2], y[3]);
-    l1 = cvt4_fp8(y[4], y[5], y[6], y[7]);
+  if (!SHORT_MANTISSA) {
+    redo = !safe | (l0 != h0) | (l1 != h1);
+    return make_uint2(l0, l1);
   }
-  return make_uint2(l0, l1);
+  redo = !safe;
+  const float e = __builtin_fmaf(sc, kFp8Max, -amax);                   // exact
+  const bool take_lower = __builtin_fmaf(e, 0x1.cp24f, -amax) > 0.0f;   // e/amax >  2^-22/7   (7 * 2^22)
+  const bool take_upper = __builtin_fmaf(e, 0x1.5p24f, amax) < 0.0f;    // e/amax < -2^-20/21  (21 * 2^20)
+  // default: bytes whose low-end code is odd take the high-end code (equal bytes are unaffected)
+  const uint32_t s0 = take_lower ? 0u : (take_upper ? 0xFFFFFFFFu : (l0 & 0x01010101u) * 0xFFu);
+  const uint32_t s1 = take_lower ? 0u : (take_upper ? 0xFFFFFFFFu : (l1 & 0x01010101u) * 0xFFu);
+  return make_uint2((h0 & s0) | (l0 & ~s0), (h1 & s1) | (l1 & ~s1));
+}
+
+// the same 8 values through the IEEE divide (cold path)
+__device__ __forceinline__ uint2 quant8_divide(const float (&a)[8], float sc) {
+  float y[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float t = a[i] / sc;  // correctly rounded (no fast-math in this build)
+    t = t < -kFp8Max ? -kFp8Max : t;  // NaN falls through, as torch.clamp does
+    t = t > kFp8Max ? kFp8Max : t;
+    y[i] = t;
+  }
+  return make_uint2(cvt4_fp8(y[0], y[1], y[2], y[3]), cvt4_fp8(y[4], y[5], y[6], y[7]));
 }
 
 // amax / 448, correctly rounded.  FAST: q0 = a*y, r = a - 448*q0 (exact in one fma), q1 = q0 + r*y with
@@ -149,6 +176,8 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
 
   Raw8<DT> raw[SEG];
   int rows[SEG], segs[SEG];
+  float scv[SEG];
+  uint32_t redo_mask = 0;
 #pragma unroll
   for (int j = 0; j < SEG; ++j) {
     rows[j] = row;
@@ -188,10 +217,33 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
                            ((uint32_t)__builtin_amdgcn_readlane((int)eb, 48) << 24);
         if (lane == 0) reinterpret_cast<uint32_t*>(s)[(int64_t)segs[j] * sg + (int64_t)rows[j] * sm] = w;
       } else {
-        out = quant8_div(a, sc);
+        bool redo;
+        out = quant8_bracket<DT != FP8K_F32>(a, sc, amax, redo);
+        redo_mask |= (redo & valid) ? (1u << j) : 0u;
+        scv[j] = sc;
         if (valid && li == 0) reinterpret_cast<float*>(s)[(int64_t)rows[j] * sm + (int64_t)g * sg] = sc;
       }
       if (valid) store8_stream(q + (int64_t)rows[j] * K + (int64_t)g * GROUP + li * 8, out);
+    }
+  }
+  // cold: lanes whose bracket was inconclusive reload their 8 values (still in cache) and divide
+  if (KIND == FP8K_SCALE_F32 && __builtin_expect(redo_mask != 0, 0)) {
+#pragma unroll 1
+    for (int j = 0; j < SEG; ++j) {
+      if (redo_mask & (1u << j)) {
+        float sc = scv[0];
+#pragma unroll
+        for (int i = 1; i < SEG; ++i) sc = j == i ? scv[i] : sc;
+        int row = rows[0], seg = segs[0];
+#pragma unroll
+        for (int i = 1; i < SEG; ++i) { row = j == i ? rows[i] : row; seg = j == i ? segs[i] : seg; }
+        const int64_t at = (int64_t)row * K + (int64_t)(seg * GPW + lg) * GROUP + li * 8;
+        Raw8<DT> again;
+        again.load(x, at);
+        float a[8];
+        again.unpack(a);
+        store8_stream(q + at, quant8_divide(a, sc));
+      }
     }
   }
 }

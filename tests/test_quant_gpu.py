@@ -94,6 +94,58 @@ def test_every_bf16_amax(dev):
         _check(x, dev, 128, layout)
 
 
+@pytest.mark.parametrize("name,dtype", [("bf16", torch.bfloat16), ("f16", torch.float16)])
+def test_exact_scale_groups_are_full_of_ties(dev, name, dtype):
+    """When the amax mantissa is a multiple of 7, amax/448 is exact and x/scale lands exactly on fp8 rounding
+    ties for many x (0.5 % of real activations): every such amax, against every mantissa of x over a range
+    of exponents, must follow round-half-to-even exactly as the float32 divide + cast does."""
+    if name == "bf16":
+        mant_bits, to_dt = 7, O.to_bf16
+    else:
+        mant_bits, to_dt = 10, lambda v: v.astype(np.float16).astype(np.float32)
+    specials = [m for m in range(1 << mant_bits, 2 << mant_bits) if m % 7 == 0]
+    rows = []
+    for m in specials:
+        amax = np.float32(m) / np.float32(1 << mant_bits)  # in [1, 2)
+        xm = np.arange(1 << mant_bits, 2 << mant_bits, dtype=np.float32) / np.float32(1 << mant_bits)
+        xm = xm[:: max(1, xm.size // 128)][:128]
+        for e in range(0, 9):  # x = mantissa * 2^-e, below amax
+            g = (xm * np.float32(2.0 ** -e)).astype(np.float32)
+            g = np.where(g > amax, g / 2, g)
+            g[::2] *= -1
+            g[5] = amax
+            rows.append(to_dt(g))
+    x = np.stack(rows).astype(np.float32)
+    vals = O.e4m3fn_to_f32(np.arange(0, 0x7F, dtype=np.uint8)).astype(np.float64)
+    mids = (vals[:-1] + vals[1:]) / 2
+    y = np.abs(x.astype(np.float64)) / (np.abs(x).max(-1, keepdims=True).astype(np.float64) / 448.0)
+    ties = int(np.isin(y, mids).sum())  # exact half-way cases in this input
+    assert ties > 300
+    for layout in _layouts():
+        _check(x, dev, 128, layout, in_dtype=name, dtype=dtype)
+
+
+def test_structural_ties_for_every_bf16_amax_mantissa(dev):
+    """x = amax * t * 2^i / 448 (whenever that is a bf16 number) makes 448 x / amax exactly the rounding boundary
+    t * 2^i of the cast, for every amax mantissa - including those whose scale amax/448 is inexact, where the
+    reference's result depends on how the scale was rounded (boundaries 21 * 2^i and, among fp8 subnormals,
+    7 * 2^-10).  Both signs, three amax exponents."""
+    rows = []
+    for ma in range(128, 256):
+        for ea in (-3, 0, 5):
+            amax = np.float32(ma) * np.float32(2.0 ** (ea - 7))
+            vals = np.array([np.float64(amax) * t * 2.0**i / 448.0 for i in range(-18, 1) for t in range(1, 32, 2)])
+            vb = O.to_bf16(vals.astype(np.float32))
+            vb = vb[(vb.astype(np.float64) == vals) & (np.abs(vb) <= amax)][:127]
+            g = np.zeros(128, np.float32)
+            g[0] = amax
+            g[1 : 1 + vb.size] = vb * np.where(np.arange(vb.size) % 2 == 0, 1, -1)
+            rows.append(g)
+    x = np.stack(rows)
+    for layout in _layouts():
+        _check(x, dev, 128, layout)
+
+
 def test_zero_groups_and_closed_form(dev):
     # all-zero groups: q = 0, scale = bf16(eps)/448; amax = 448 -> scale 1, bytes = encode(x)
     x = np.zeros((8, 256), dtype=np.float32)
