@@ -157,7 +157,7 @@ __device__ __forceinline__ void load_stream(Raw8<DT>& r, const void* base, int64
   }
 }
 
-template <int DT, int GROUP, int KIND, int SEG>
+template <int DT, int GROUP, int KIND, int SEG, bool ROWFAST>
 __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
                                                           void* __restrict__ s, int M, int G, int64_t K,
                                                           int nseg_row, float eps, int64_t sm, int64_t sg) {
@@ -167,35 +167,49 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
 
   const int lane = threadIdx.x & 63;
   const int lg = lane / LPG, li = lane % LPG;
-  // wave-uniform task range [t0, t0 + SEG) over (row, segment-in-row) pairs
+  // A wave owns SEG tasks (row, segment-in-row).  Row-major scales: SEG consecutive segments, i.e. contiguous
+  // memory and SEG*GPW consecutive scales.  ROWFAST (scales whose rows are contiguous: column-major float,
+  // packed UE8M0): the same segment of SEG consecutive rows, so that the SEG scales of a group column are
+  // adjacent words that leave the wave together.
+  const unsigned wave = blockIdx.x * 4u + (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const unsigned total = (unsigned)M * (unsigned)nseg_row;
-  const unsigned t0 = (blockIdx.x * 4u + (unsigned)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6))) * SEG;
-  if (t0 >= total) return;
-  int row = (int)(t0 / (unsigned)nseg_row);
-  int sr = (int)(t0 - (unsigned)row * (unsigned)nseg_row);
+  int row, sr;
+  if (ROWFAST) {
+    row = (int)(wave / (unsigned)nseg_row) * SEG;
+    sr = (int)(wave % (unsigned)nseg_row);
+    if (row >= M) return;
+  } else {
+    if (wave * SEG >= total) return;
+    row = (int)(wave * SEG / (unsigned)nseg_row);
+    sr = (int)(wave * SEG - (unsigned)row * (unsigned)nseg_row);
+  }
 
   Raw8<DT> raw[SEG];
   int rows[SEG], segs[SEG];
+  bool act[SEG];  // wave-uniform: task j exists
   float scv[SEG];
   uint32_t redo_mask = 0;
 #pragma unroll
   for (int j = 0; j < SEG; ++j) {
     rows[j] = row;
     segs[j] = sr;
-    if (t0 + j < total) {
+    act[j] = ROWFAST ? row < M : wave * SEG + j < total;
+    if (act[j]) {
       const int g = sr * GPW + lg;
       // lanes past the last group of the row re-read the last group and store nothing
       const int64_t col = (int64_t)(g < G ? g : G - 1) * GROUP + li * 8;
       load_stream<DT>(raw[j], x, (int64_t)row * K + col);
     }
-    if (++sr == nseg_row) {
+    if (ROWFAST) {
+      ++row;
+    } else if (++sr == nseg_row) {
       sr = 0;
       ++row;
     }
   }
 #pragma unroll
   for (int j = 0; j < SEG; ++j) {
-    if (t0 + j < total) {  // wave-uniform
+    if (act[j]) {  // wave-uniform
       const int g = segs[j] * GPW + lg;
       const bool valid = g < G;
       float a[8];
@@ -256,10 +270,16 @@ static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_
   const int G = (int)(K / GROUP);
   const int nseg_row = (G + GPW - 1) / GPW;
   const int64_t total = M * nseg_row;
-  if (total > 0x7fffffffLL) return fail(FP8K_ERR_INVALID, "group_quant: input too large for one launch");
-  const int64_t waves = (total + SEG - 1) / SEG;
-  hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG>), dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, st, x,
-                     (uint8_t*)q, s, (int)M, G, K, nseg_row, eps, sm, sg);
+  if (total > 0x7fffffffLL / SEG) return fail(FP8K_ERR_INVALID, "group_quant: input too large for one launch");
+  const bool rowfast = KIND == FP8K_SCALE_UE8M0_PACKED || sm < sg;  // rows of the scale tensor are contiguous
+  const int64_t waves = rowfast ? (M + SEG - 1) / SEG * nseg_row : (total + SEG - 1) / SEG;
+  const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
+  if (rowfast)
+    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, true>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M, G,
+                       K, nseg_row, eps, sm, sg);
+  else
+    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, false>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M,
+                       G, K, nseg_row, eps, sm, sg);
   return check_launch("group_quant");
 }
 
