@@ -397,6 +397,69 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]);
   F(acc[3][1], tq[1], sc[1]);
 
+  // Finished tiles leave through LDS so that every store instruction writes whole 256-byte row segments
+  // (the accumulator layout alone gives 8 bytes per row per lane: 32 partial lines per instruction).
+  // Each wave re-lays its own 64 x 128 block out in a private 16 KB slot of the stage memory, 16-byte
+  // chunks XOR-swizzled by the row so that both the 8-byte writes and the 16-byte reads spread over all banks.
+  const bool wide = !is_split && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  if (wide) {
+    lds_barrier();  // every wave has taken its last operands out of the stages
+    uint8_t* ep = smem + w * 16384;
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms) {
+      const int r = ms * 32 + lr;
+      const int m = slot_at(wm * 64 + r);
+      float sa = 1.f;
+      if (m < nrows) {
+        if (MODE == kModeRow) sa = p.sx[m];
+        if (MOE && p.topk_w) sa = p.topk_w[m];
+      }
+#pragma unroll
+      for (int ns = 0; ns < 4; ++ns) {
+#pragma unroll
+        for (int rg = 0; rg < 4; ++rg) {
+          const int n = n0 + wn * 128 + ns * 32 + rg * 8 + h * 4;
+          float v[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] = acc[ns][ms][rg * 4 + q];
+          if (MODE == kModeRow) {
+            float4 sb = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (n < p.N) sb = *reinterpret_cast<const float4*>(p.sw + n);
+            v[0] = v[0] * sb.x * sa; v[1] = v[1] * sb.y * sa; v[2] = v[2] * sb.z * sa; v[3] = v[3] * sb.w * sa;
+            if (p.bias && n < p.N) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q) v[q] += load_scalar<BIAS_DT>(p.bias, n + q);
+            }
+          } else if (MOE) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] *= sa;
+          }
+          uint2 o;
+          if (OUT_DT == FP8K_BF16) {
+            o.x = pack_bf16x2(v[0], v[1]);
+            o.y = pack_bf16x2(v[2], v[3]);
+          } else {
+            o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+            o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+          }
+          const int chunk = (ns * 4 + rg) ^ (r & 15);
+          *reinterpret_cast<uint2*>(ep + r * 256 + chunk * 16 + h * 8) = o;
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
+    const int rr = lane >> 4, pc = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int r = i * 4 + rr;
+      const uint4 o = *reinterpret_cast<const uint4*>(ep + r * 256 + pc * 16);
+      const int m = slot_at(wm * 64 + r);
+      const int n = n0 + wn * 128 + ((pc ^ (r & 15)) << 3);
+      if (m < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)m * p.ldc + n) = o;
+    }
+    return;
+  }
+
 #pragma unroll
   for (int ms = 0; ms < 2; ++ms) {
     const int ml = wm * 64 + ms * 32 + lr;  // row inside the tile
