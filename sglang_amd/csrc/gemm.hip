@@ -131,7 +131,7 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   const int ntiles = a.tiles_m * a.tiles_n;
   a.tail_first = pl.tail_first;
   const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
-  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT, false>), dim3(nwg), dim3(512), 0, st, a);
+  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
   int rc = check_launch("gemm_tile256");
   if (rc || pl.tail_first == ntiles) return rc;
   hipLaunchKernelGGL((tile_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((ntiles - pl.tail_first) * 64)), dim3(256),

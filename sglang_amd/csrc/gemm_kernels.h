@@ -139,14 +139,9 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // workgroup each, so that the round takes 1/splits of a tile time; they leave float partials in the workspace
 // ([tile - tail_first][split][256 m][256 n]) for tile_reduce_kernel.  Their workgroup ids come last, so they are
 // dispatched when the whole tiles drain.
-//
-// MOE: grouped form.  A "tile" is (block of up to 256 token slots of one expert) x (256 weight rows of that
-// expert); activation rows are gathered and output rows scattered through sorted_token_ids, whose slot ids sit
-// in an LDS table.  Each XCD walks a contiguous run of the blocks in use and all n tiles of a block in turn.
-template <int MODE, int OUT_DT, int BIAS_DT, bool MOE>
+template <int MODE, int OUT_DT, int BIAS_DT>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
   __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kStageBytes];
-  __shared__ int32_t slot_tab[MOE ? kTileM : 1];
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -156,18 +151,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   int t = 0, split = 0;
   bool is_split = false;
   int tile_m, tile_n;
-  int expert = 0;
-  if (MOE) {
-    const int used = p.num_post_pad[0] / p.block_m;
-    const int per_xcd = (used + 7) >> 3;
-    const int j = bid >> 3;
-    const int mbl = j / p.tiles_n;
-    if (mbl >= per_xcd) return;
-    tile_m = (bid & 7) * per_xcd + mbl;
-    if (tile_m >= used || tile_m >= p.m_blocks) return;
-    tile_n = j - mbl * p.tiles_n;
-    expert = p.expert_ids[tile_m];
-  } else {
+  {
     const int ntiles = p.tiles_m * p.tiles_n;
     const int per_xcd = (p.tail_first + 7) >> 3;
     is_split = bid >= per_xcd * 8;
@@ -182,37 +166,19 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     }
     tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
   }
-  const int m0 = MOE ? 0 : tile_m * kTileM, n0 = tile_n * kTileN;
-  const int nrows = MOE ? p.num_valid : p.M;   // exclusive bound of a valid output row
+  const int m0 = tile_m * kTileM, n0 = tile_n * kTileN;
+  const int nrows = p.M;   // exclusive bound of a valid output row
 
   const int kb_begin = is_split ? split * p.kb_per_split : 0;
   const int kb_end = is_split ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
   const int nkb = kb_end - kb_begin;
 
-  // grouped: slot id of every row of the block (nrows = padding), then the rows this lane loads and scales
-  auto slot_at = [&](int i) -> int { return MOE ? slot_tab[i] : m0 + i; };
-  if (MOE) {
-    if (threadIdx.x < kTileM) {
-      const int i = threadIdx.x;
-      int s = nrows;
-      if (i < p.block_m) s = min(p.sorted_ids[tile_m * p.block_m + i], nrows);
-      slot_tab[i] = s;
-    }
-    __syncthreads();
-    if (expert < 0) {  // expert on another rank: the reference writes zeros
-      for (int i = threadIdx.x; i < kTileM * (kTileN / 4); i += 512) {
-        const int s = slot_tab[i / (kTileN / 4)];
-        const int n = n0 + (i % (kTileN / 4)) * 4;
-        if (s < nrows && n < p.N) store4<OUT_DT>(p.C, (int64_t)s * p.ldc + n, 0.f, 0.f, 0.f, 0.f);
-      }
-      return;
-    }
-  }
+  auto slot_at = [&](int i) -> int { return m0 + i; };
 
   // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the
   // matrix edge are out of range and read as zero
-  const uint8_t* Wb = p.W + (MOE ? (int64_t)expert * p.w_expert_stride : 0);
-  const int rowsW = min(kTileN, p.N - n0), rowsX = MOE ? (nrows + p.top_k - 1) / p.top_k : min(kTileM, p.M - m0);
+  const uint8_t* Wb = p.W;
+  const int rowsW = min(kTileN, p.N - n0), rowsX = min(kTileM, p.M - m0);
   const int kbytes = p.K - kb_begin * kTileK;
   const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
   const rsrc_t rX = make_rsrc(p.X + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
@@ -222,18 +188,10 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   for (int par = 0; par < 2; ++par) {
     const int c = cp ^ ((par << 2) + (rl >> 1));
     voW[par] = (uint32_t)(rl * p.ldw + c * 16);
-    voX[par] = (uint32_t)((MOE ? 0 : rl * p.ldx) + c * 16);
+    voX[par] = (uint32_t)(rl * p.ldx + c * 16);
   }
-  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = MOE ? 0u : (uint32_t)(w * 32 * p.ldx);
-  const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = MOE ? 0u : (uint32_t)(8 * p.ldx);
-  uint32_t xgather[MOE ? 4 : 1];  // grouped: byte offset of the activation row behind each of this lane's 4 loads
-  if (MOE) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int s = slot_tab[w * 32 + j * 8 + rl];
-      xgather[j] = s < nrows ? (uint32_t)(s / p.top_k) * (uint32_t)p.ldx : 0xF0000000u;
-    }
-  }
+  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = (uint32_t)(w * 32 * p.ldx);
+  const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = (uint32_t)(8 * p.ldx);
   // ---- LDS -> MFMA operands
   const int lr = lane & 31, h = lane >> 5;
   const int swz = (lr >> 1) & 7;
@@ -254,19 +212,13 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   };
 
   // ---- scales (block mode)
-  int mrow0, mrow1;  // activation rows whose scales this lane applies (any valid row for padding lanes)
-  if (MOE) {
-    const int s0 = slot_tab[wm * 64 + lr], s1 = slot_tab[wm * 64 + 32 + lr];
-    mrow0 = s0 < nrows ? s0 / p.top_k : 0;
-    mrow1 = s1 < nrows ? s1 / p.top_k : 0;
-  } else {
-    mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
-    mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
-  }
+  // activation rows whose scales this lane applies (any valid row for padding lanes)
+  const int mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
+  const int mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
   const float* sx0 = p.sx + (int64_t)mrow0 * p.sx_m + (int64_t)kb_begin * p.sx_k;
   const float* sx1 = p.sx + (int64_t)mrow1 * p.sx_m + (int64_t)kb_begin * p.sx_k;
   const int nb = min(n0 + wn * 128, p.N - 1) >> 7;
-  const float* swp = p.sw + (MOE ? (int64_t)expert * p.sw_expert_stride : 0) + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
+  const float* swp = p.sw + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
 
   v16f acc[4][2];
 #pragma unroll
@@ -290,7 +242,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     // the whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt from the
     // range check, and rows past the matrix edge must read as zero, not touch memory)
     if (idx < 4) buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + ko), 0, base + j * 1024);
-    else buf_load16_to_lds(rX, voX[j & 1] + (MOE ? xgather[j] + ko : soX + j * stepX + ko), 0, base + kXOff + j * 1024);
+    else buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + ko), 0, base + kXOff + j * 1024);
   };
   auto RW = [&](v8i(&dst)[2], const uint8_t* st, int ns) {
     dst[0] = frag(st, rdW + ns * 32 * kTileK, 0);
@@ -410,10 +362,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       const int r = ms * 32 + lr;
       const int m = slot_at(wm * 64 + r);
       float sa = 1.f;
-      if (m < nrows) {
-        if (MODE == kModeRow) sa = p.sx[m];
-        if (MOE && p.topk_w) sa = p.topk_w[m];
-      }
+      if (MODE == kModeRow && m < nrows) sa = p.sx[m];
 #pragma unroll
       for (int ns = 0; ns < 4; ++ns) {
 #pragma unroll
@@ -430,9 +379,6 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
               for (int q = 0; q < 4; ++q) v[q] += load_scalar<BIAS_DT>(p.bias, n + q);
             }
-          } else if (MOE) {
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] *= sa;
           }
           uint2 o;
           if (OUT_DT == FP8K_BF16) {
@@ -467,7 +413,6 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     if (m >= nrows) continue;
     float sa = 1.f;
     if (MODE == kModeRow && !is_split) sa = p.sx[m];
-    if (MOE && p.topk_w) sa = p.topk_w[m];
 #pragma unroll
     for (int ns = 0; ns < 4; ++ns) {
 #pragma unroll
@@ -488,9 +433,6 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
               for (int r = 0; r < 4; ++r) v[r] += load_scalar<BIAS_DT>(p.bias, n + r);
             }
-          } else if (MOE) {
-#pragma unroll
-            for (int r = 0; r < 4; ++r) v[r] *= sa;
           }
           store4<OUT_DT>(p.C, (int64_t)m * p.ldc + n, v[0], v[1], v[2], v[3]);
         }
@@ -538,14 +480,27 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   int split = 0;
   int mb, tile_n;
   if (MOE) {
-    const int used = p.num_post_pad[0] / p.block_m;
+    const int used = min(p.num_post_pad[0] / p.block_m, p.m_blocks);
     const int per_xcd = (used + 7) >> 3;
     const int j = bid >> 3;
     const int mbl = j / p.tiles_n;
     if (mbl >= per_xcd) return;
-    mb = (bid & 7) * per_xcd + mbl;
-    if (mb >= used || mb >= p.m_blocks) return;
-    tile_n = j - mbl * p.tiles_n;
+    const int first_blk = (bid & 7) * per_xcd, end_blk = min(first_blk + per_xcd, used);
+    mb = first_blk + mbl;
+    if (mb >= end_blk) return;
+    // Blocks of one expert that sit next to each other in the run form groups of up to kShare; inside a
+    // group consecutive workgroup ids walk the blocks first and the n tiles second, so the workgroups that
+    // stream the same weight tile are dispatched together and meet in L2 instead of fetching it once each.
+    constexpr int kShare = 4;
+    const int e = p.expert_ids[mb];
+    int idx = 0;                       // position of this block inside its run of equal expert ids
+    while (mb - idx > first_blk && p.expert_ids[mb - idx - 1] == e) ++idx;
+    const int gfirst = mb - (idx & (kShare - 1));
+    int g = (idx & (kShare - 1)) + 1;  // group size: forward to the end of the run, at most kShare
+    while (g < kShare && gfirst + g < end_blk && p.expert_ids[gfirst + g] == e) ++g;
+    const int r = j - (gfirst - first_blk) * p.tiles_n;  // slot inside the group: 0 .. g*tiles_n-1
+    tile_n = r / g;
+    mb = gfirst + (r - tile_n * g);
   } else {
     const int nitems = p.tiles_n * p.m_blocks;
     const int per_xcd = (nitems + 7) >> 3;

@@ -1,0 +1,247 @@
+// Grouped (MoE) block-FP8 GEMM for experts with 129..256 token slots: 256(n) x 256(m) x 128(k) tile,
+// 8 wavefronts, weights streamed three K blocks deep.
+//
+// With a few hundred token slots per expert the grouped GEMM is bound by streaming each expert's weights
+// from HBM exactly once.  Two 128-row blocks of one expert in two workgroups fetch the weight tile twice
+// (they drift apart by more than an L2's worth of traffic), and the 256x256 MFMA tile kernel keeps only one
+// K block of prefetch in flight, which is enough against L2 but not against HBM latency.  This kernel keeps
+// the streaming kernel's depth on the weights and pairs both 128-row halves on one weight stage:
+//   LDS = 3 weight stages (32 KB each) + 2 activation stages (32 KB each) = 160 KB, the whole CU.
+//   Activation tiles are re-read by every n tile of the block and come from L2; one stage ahead is enough.
+//   Waves: 4 along n (64 weight rows) x 2 along m (128 slots), 2 x 4 MFMA tiles of 32x32 each (24 KB of LDS
+//   operands per 16 MFMAs); a half without real slots skips its MFMAs.
+// Load order inside a K block is scales, activations, weights, so that at the next barrier only the four
+// youngest weight loads of each wave may still be in flight (memory operations retire in order).
+#pragma once
+
+#include "gemm_kernels.h"
+
+namespace fp8k {
+
+template <int OUT_DT>
+__global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p) {
+  constexpr int TM = 256, WST = 3, XST = 2, MS = 4, NS = 2, LW = 4;  // LW: wave loads per tile per stage
+  constexpr int WBYTES = kTileN * kTileK, XBYTES = TM * kTileK;
+  constexpr int XBASE = WST * WBYTES;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[WST * WBYTES + XST * XBYTES];
+
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int wn = w & 3, wm = w >> 2;
+
+  // ---- work item: each XCD takes a contiguous run of the blocks in use and walks all n tiles of a block
+  const int bid = blockIdx.x;
+  const int used = min(p.num_post_pad[0] / TM, p.m_blocks);
+  const int per_xcd = (used + 7) >> 3;
+  const int j = bid >> 3;
+  const int mbl = j / p.tiles_n;
+  if (mbl >= per_xcd) return;
+  const int first_blk = (bid & 7) * per_xcd, end_blk = min(first_blk + per_xcd, used);
+  int mb = first_blk + mbl;
+  if (mb >= end_blk) return;
+  // Blocks of one expert that sit next to each other in the run form groups of up to kShare; inside a group
+  // consecutive workgroup ids walk the blocks first and the n tiles second, so the workgroups that stream
+  // the same weight tile are dispatched together and share it in L2.
+  constexpr int kShare = 4;
+  const int expert = p.expert_ids[mb];
+  int idx = 0;  // position of this block inside its run of equal expert ids
+  while (mb - idx > first_blk && p.expert_ids[mb - idx - 1] == expert) ++idx;
+  const int gfirst = mb - (idx & (kShare - 1));
+  int g = (idx & (kShare - 1)) + 1;  // group size: forward to the end of the run, at most kShare
+  while (g < kShare && gfirst + g < end_blk && p.expert_ids[gfirst + g] == expert) ++g;
+  const int r = j - (gfirst - first_blk) * p.tiles_n;  // slot inside the group: 0 .. g*tiles_n-1
+  const int tile_n = r / g;
+  mb = gfirst + (r - tile_n * g);
+  const int n0 = tile_n * kTileN;
+  const int slot0 = mb * TM;
+  const int nrows = p.num_valid;
+
+  const int lr = lane & 31, h = lane >> 5;
+  if (expert < 0) {  // expert on another rank: the reference writes zeros
+    for (int ms = 0; ms < MS; ++ms) {
+      const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
+      if (s >= nrows) continue;
+      for (int q = 0; q < 4; ++q) {
+        for (int ns = 0; ns < NS; ++ns) {
+          const int n = n0 + wn * 64 + ns * 32 + h * 16 + q * 4;
+          if (n < p.N) store4<OUT_DT>(p.C, (int64_t)s * p.ldc + n, 0.f, 0.f, 0.f, 0.f);
+        }
+      }
+    }
+    return;
+  }
+  // real slots come first in a block: the upper half is in use iff its first slot is
+  const bool active = wm == 0 || __builtin_amdgcn_readfirstlane(p.sorted_ids[slot0 + 128]) < nrows;
+
+  // ---- global -> LDS: a wave load covers 8 rows (lane: row lane/8, 16-byte chunk lane%8, stored at chunk
+  // position c ^ ((row>>1)&7)); whole offsets travel in the bounds-checked per-lane operand
+  const uint8_t* Wb = p.W + (int64_t)expert * p.w_expert_stride;
+  const int rowsW = min(kTileN, p.N - n0);
+  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw, (uint32_t)((rowsW - 1) * p.ldw + p.K));
+  const int64_t xrows = (int64_t)((p.num_valid + p.top_k - 1) / p.top_k);
+  const rsrc_t rX = make_rsrc(p.X, (uint32_t)((xrows - 1) * p.ldx + p.K));
+  const int rl = lane >> 3, cp = lane & 7;
+  uint32_t voW[LW], voX[LW];
+#pragma unroll
+  for (int q = 0; q < LW; ++q) {
+    const int g = w * LW + q;  // 8-row group, 0..31, of both tiles
+    const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
+    voW[q] = (uint32_t)((g * 8 + rl) * p.ldw + c * 16);
+    const int s = p.sorted_ids[slot0 + g * 8 + rl];
+    voX[q] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
+  }
+  auto issue_w = [&](int kstep) {
+    uint8_t* base = smem + (kstep % WST) * WBYTES + w * (LW * 1024);
+    const uint32_t ko = (uint32_t)kstep * kTileK;
+#pragma unroll
+    for (int q = 0; q < LW; ++q) buf_load16_to_lds(rW, voW[q] + ko, 0, base + q * 1024);
+  };
+  auto issue_x = [&](int kstep) {
+    uint8_t* base = smem + XBASE + (kstep & 1) * XBYTES + w * (LW * 1024);
+    const uint32_t ko = (uint32_t)kstep * kTileK;
+#pragma unroll
+    for (int q = 0; q < LW; ++q) buf_load16_to_lds(rX, voX[q] + ko, 0, base + q * 1024);
+  };
+
+  // ---- LDS -> MFMA operands
+  const int swz = (lr >> 1) & 7;
+  uint32_t co[2][2];
+#pragma unroll
+  for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+    for (int q = 0; q < 2; ++q) co[ks][q] = (uint32_t)(((ks * 4 + h * 2 + q) ^ swz) << 4);
+  const uint32_t rdW = (uint32_t)((wn * 64 + lr) * kTileK);
+  const uint32_t rdX = (uint32_t)((wm * 128 + lr) * kTileK);
+  auto frag = [&](const uint8_t* st, uint32_t rowoff, int ks) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][0]);
+    const v4i hi = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][1]);
+    v8i r;
+    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+    return r;
+  };
+
+  // ---- scales: activation scale rows follow the activation rows
+  uint32_t sxo[MS];  // element offsets into the activation scales (the host checks they fit 32 bits)
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
+    sxo[ms] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u;
+  }
+  const int nb = min(n0 + wn * 64, p.N - 1) >> 7;  // the wave's 64 weight rows lie inside one 128-row block
+  const float* swp = p.sw + (int64_t)expert * p.sw_expert_stride + (int64_t)nb * p.sw_n;
+  const int nkb = p.K / kTileK;
+
+  v16f acc[NS][MS];
+#pragma unroll
+  for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
+
+  float sxa[MS], sxb[MS], sba = 0.f, sbb = 0.f;  // scales of the even / odd K blocks in flight
+  auto load_scales = [&](float (&sx)[MS], float& sb, int kb) {
+    const int kn = min(kb, nkb - 1);
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) sx[ms] = p.sx[sxo[ms] + (uint32_t)(kn * (int)p.sx_k)];
+    sb = swp[(int64_t)kn * p.sw_k];
+  };
+  load_scales(sxa, sba, 0);
+  load_scales(sxb, sbb, 1);
+  __builtin_amdgcn_sched_barrier(0);
+  issue_x(0);
+  issue_w(0);
+  issue_w(1);
+
+  // one K block; (sx, sb) hold its scales on entry and are reloaded with those of block it+2
+  auto trip = [&](int it, float (&sx)[MS], float& sb) {
+    lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
+    float sc[MS];
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) sc[ms] = sx[ms] * sb;
+    load_scales(sx, sb, it + 2);
+    __builtin_amdgcn_sched_barrier(0);  // scales, then activations, then weights
+    issue_x(it + 1);                    // into the stage of block it-1, which every wave has left
+    issue_w(it + 2);
+    if (!active) return;
+    const uint8_t* sw_ = smem + (it % WST) * WBYTES;
+    const uint8_t* sx_ = smem + XBASE + (it & 1) * XBYTES;
+    v8i wf[NS][2];
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns) {
+      wf[ns][0] = frag(sw_, rdW + ns * 32 * kTileK, 0);
+      wf[ns][1] = frag(sw_, rdW + ns * 32 * kTileK, 1);
+    }
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) {
+      const v8i x0 = frag(sx_, rdX + ms * 32 * kTileK, 0);
+      const v8i x1 = frag(sx_, rdX + ms * 32 * kTileK, 1);
+#pragma unroll
+      for (int ns = 0; ns < NS; ++ns) {
+        v16f z;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) z[r] = 0.f;
+        v16f tq = mfma_32x32x64(wf[ns][0], x0, z);
+        tq = mfma_32x32x64(wf[ns][1], x1, tq);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ns][ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ns][ms][r]);
+      }
+    }
+  };
+  int it = 0;
+  for (; it + 1 < nkb; it += 2) {
+    trip(it, sxa, sba);
+    trip(it + 1, sxb, sbb);
+  }
+  if (it < nkb) trip(it, sxa, sba);
+  wait_vm0();     // the loads past the last K block still target the stages
+  lds_barrier();  // every wave has left the stages: they become the output staging area
+
+  // ---- epilogue through LDS: [256 slots][256 n] 16-bit, 512 B per row, 16-byte chunks XOR-swizzled by the
+  // row so that the accumulator-shaped 8-byte writes spread over all banks; every store instruction then
+  // writes two whole 512-byte row segments
+  const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int row = wm * 128 + ms * 32 + lr;
+    const int oslot = p.sorted_ids[slot0 + row];
+    const bool ok = oslot < nrows;
+    const float rs = (p.topk_w && ok) ? p.topk_w[oslot] : 1.f;
+#pragma unroll
+    for (int nr = 0; nr < NS * 4; ++nr) {
+      const int ns = nr >> 2, rg = nr & 3;
+      float v[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) v[r] = acc[ns][ms][rg * 4 + r] * rs;
+      if (wide) {
+        uint2 o;
+        if (OUT_DT == FP8K_BF16) {
+          o.x = pack_bf16x2(v[0], v[1]);
+          o.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+          o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+        }
+        const int chunk = (wn * 8 + nr) ^ (row & 31);
+        *reinterpret_cast<uint2*>(smem + row * 512 + chunk * 16 + h * 8) = o;
+      } else {
+        const int n = n0 + wn * 64 + nr * 8 + h * 4;
+        if (ok && n < p.N) store4<OUT_DT>(p.C, (int64_t)oslot * p.ldc + n, v[0], v[1], v[2], v[3]);
+      }
+    }
+  }
+  if (!wide) return;
+  lds_barrier();
+  const int rr = lane >> 5, pc = lane & 31;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) {
+    const int row = w * 32 + i * 2 + rr;
+    const int s = p.sorted_ids[slot0 + row];
+    const int n = n0 + ((pc ^ (row & 31)) << 3);
+    const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + pc * 16);
+    if (s < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)s * p.ldc + n) = o;
+  }
+}
+
+}  // namespace fp8k

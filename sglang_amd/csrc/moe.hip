@@ -2,6 +2,7 @@
 // GEMM (host side; the device code is gemm_stream_kernel in gemm_kernels.h), silu_and_mul and the
 // top-k sum.  No allocation, no synchronisation, no host reads of device data.
 #include "gemm_direct.h"
+#include "gemm_moe256.h"
 
 namespace fp8k {
 
@@ -306,11 +307,12 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
     return check_launch(op);
   }
 #undef FP8K_MOE_DIRECT
-  if (block_m == 256) {  // many rows per expert: the MFMA-bound 256x256 tile kernel, one block of slots per tile
+  FP8K_REQUIRE(xrows * as_stride_m + (K / kTileK) * as_stride_k < 0xffffffffLL, "%s: activation scale tensor too large", op);
+  if (block_m == 256) {  // 129..256 and more slots per expert: both 128-row halves on one weight stage
     if (out_dtype == FP8K_BF16)
-      hipLaunchKernelGGL((gemm_tile256_kernel<kModeBlock, FP8K_BF16, FP8K_F32, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+      hipLaunchKernelGGL((moe_stream256_kernel<FP8K_BF16>), dim3((unsigned)nwg), dim3(512), 0, st, a);
     else
-      hipLaunchKernelGGL((gemm_tile256_kernel<kModeBlock, FP8K_F16, FP8K_F32, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+      hipLaunchKernelGGL((moe_stream256_kernel<FP8K_F16>), dim3((unsigned)nwg), dim3(512), 0, st, a);
     return check_launch(op);
   }
 #define FP8K_MOE(TM, NST, NW, O) \

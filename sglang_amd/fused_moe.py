@@ -44,16 +44,19 @@ def moe_align_block_size(
 def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     """Rows per block of the grouped GEMM (the reference's BLOCK_SIZE_M, fused_moe_triton_config.py).
 
-    Measured on MI355X with 256 experts: up to about 8 rows per expert the register-streaming kernel with
-    16- or 32-row blocks wins; beyond that 128-row blocks (one weight pass per expert) through the LDS-staged
-    streaming kernel; with several hundred rows per expert the 256x256 MFMA tile kernel.
+    Measured on MI355X with 256 experts, top-8 and near-balanced routing: while the layer streams every expert's
+    weights for a handful of rows each, the register-streaming kernel with 16- or 32-row blocks wins; from about
+    16 rows per expert the LDS-staged streaming kernel with 64- and then 128-row blocks; from about 100 rows per
+    expert the 256-row kernel, which puts both 128-row halves of an expert on one pass over its weights.
     """
     per_expert = (M * topk + E - 1) // max(E, 1)
-    if per_expert <= 1:
+    if per_expert <= 4:
         bm = 16
-    elif per_expert <= 8:
+    elif per_expert <= 16:
         bm = 32
-    elif per_expert <= 384:
+    elif per_expert <= 40:
+        bm = 64
+    elif per_expert <= 96:
         bm = 128
     else:
         bm = 256
