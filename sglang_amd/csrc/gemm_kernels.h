@@ -398,9 +398,9 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
     for (int i = 0; i < 16; ++i) {
       const int r = i * 4 + rr;
-      const uint4 o = *reinterpret_cast<const uint4*>(ep + r * 256 + pc * 16);
+      const uint4 o = *reinterpret_cast<const uint4*>(ep + r * 256 + ((pc ^ (r & 15)) << 4));
       const int m = slot_at(wm * 64 + r);
-      const int n = n0 + wn * 128 + ((pc ^ (r & 15)) << 3);
+      const int n = n0 + wn * 128 + (pc << 3);  // consecutive lanes store consecutive 16-byte chunks
       if (m < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)m * p.ldc + n) = o;
     }
     return;
@@ -679,7 +679,61 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   if (it < nkb) trip(it, sxa, sba);
   wait_vm0();  // drain the padding loads before the LDS allocation is released
 
-  // ---- epilogue
+  // ---- epilogue.  Finished 16-bit tiles leave through LDS ([TM rows][256 n], 512 B per row, 16-byte chunks
+  // XOR-swizzled by the row) so that every store instruction writes two whole 512-byte row segments instead
+  // of 8 bytes in each of 32 rows.
+  if (!SPLIT && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0) {
+    lds_barrier();  // every wave has left the stages
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) {
+      const int row = mrow0 + ms * 32 + lr;
+      float rs = 1.f;
+      if (out_ok[ms]) {
+        if (MODE == kModeRow) rs = p.sx[out_slot[ms]];
+        if (MOE && p.topk_w) rs = p.topk_w[out_slot[ms]];
+      }
+#pragma unroll
+      for (int rg = 0; rg < 4; ++rg) {
+        const int n = n0 + wn * 32 + rg * 8 + h * 4;
+        float v[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) v[r] = acc[ms][rg * 4 + r];
+        if (MODE == kModeRow) {
+          float4 sb = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (n < p.N) sb = *reinterpret_cast<const float4*>(p.sw + n);
+          v[0] = v[0] * sb.x * rs; v[1] = v[1] * sb.y * rs; v[2] = v[2] * sb.z * rs; v[3] = v[3] * sb.w * rs;
+          if (p.bias && n < p.N) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) v[r] += load_scalar<BIAS_DT>(p.bias, n + r);
+          }
+        } else if (MOE) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] *= rs;
+        }
+        uint2 o;
+        if (OUT_DT == FP8K_BF16) {
+          o.x = pack_bf16x2(v[0], v[1]);
+          o.y = pack_bf16x2(v[2], v[3]);
+        } else {
+          o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+          o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+        }
+        *reinterpret_cast<uint2*>(smem + row * 512 + (((wn * 4 + rg) ^ (row & 31)) << 4) + h * 8) = o;
+      }
+    }
+    lds_barrier();
+    const int rr = lane >> 5, pc = lane & 31;
+#pragma unroll
+    for (int i = 0; i < TM / NW / 2; ++i) {
+      const int row = w * (TM / NW) + i * 2 + rr;
+      int slot = slot0 + row;
+      if (MOE) slot = row < block_m ? p.sorted_ids[slot0 + row] : nrows;
+      const int n = n0 + (pc << 3);
+      const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + ((pc ^ (row & 31)) << 4));
+      if (slot < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)slot * p.ldc + n) = o;
+    }
+    return;
+  }
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
     if (!out_ok[ms]) continue;

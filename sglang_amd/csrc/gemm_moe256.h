@@ -238,8 +238,8 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   for (int i = 0; i < 16; ++i) {
     const int row = w * 32 + i * 2 + rr;
     const int s = p.sorted_ids[slot0 + row];
-    const int n = n0 + ((pc ^ (row & 31)) << 3);
-    const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + pc * 16);
+    const int n = n0 + (pc << 3);  // consecutive lanes store consecutive 16-byte chunks
+    const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + ((pc ^ (row & 31)) << 4));
     if (s < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)s * p.ldc + n) = o;
   }
 }
