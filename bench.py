@@ -231,7 +231,7 @@ def _rand_fp8(torch, shape, gen, dev):
     return torch.where((b & 0x7F) == 0x7F, b & 0xFE, b).view(torch.float8_e4m3fn)  # no NaN codes
 
 
-def moe_table(torch, dev):
+def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384)):
     """BASELINE configs[4]: 256 experts, hidden 7168, intermediate 2048, top-8 grouped-sigmoid routing."""
     from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl
 
@@ -247,7 +247,7 @@ def moe_table(torch, dev):
              "whole layer: align + quant + grouped GEMM w13 + silu_and_mul + quant + grouped GEMM w2 + top-k sum; "
              "bytes = fp8 weights of the experts hit (44.04 MB each)", "",
              "| M | experts hit | us | TFLOP/s | weight GB/s | % of 8 TB/s |", "|---|---|---|---|---|---|"]
-    for M in (1, 32, 256, 1024, 4096, 16384):
+    for M in token_counts:
         x = _activation(torch, M, H, M, dev)
         logits = torch.randn((M, E), generator=g, device=dev)
         tw, ids = biased_grouped_topk_impl(x, logits, bias, topk, True, 8, 4)
@@ -320,6 +320,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB read + 256 MiB write elementwise kernel (reference point for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--moe", type=str, default=None,
+                    help="only time the fused MoE layer at these token counts (comma separated) and print its table")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no cross-GPU step); --gpus %d is not "
@@ -334,6 +336,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if args.moe:
+        print("\n".join(moe_table(torch, dev, tuple(int(t) for t in args.moe.split(",")))))
+        return 0
     ms_per_step, gemm_us = run_headline(torch, dev, args.steps, args.warmup)
     M, N, K = HEADLINE["M"], HEADLINE["N"], HEADLINE["K"]
     flops = 2.0 * M * N * K

@@ -1,6 +1,6 @@
 // Block-FP8 fused-MoE building blocks for gfx950: token alignment (integer), the grouped block-scaled
-// GEMM (host side; the device code is gemm_stream_kernel in gemm_kernels.h), silu_and_mul and the
-// top-k sum.  No allocation, no synchronisation, no host reads of device data.
+// GEMM (host side; the device code is the grouped form of gemm_direct_kernel for 16/32-slot blocks, of
+// gemm_stream_kernel for 64/128 and moe_stream256_kernel for 256), silu_and_mul and the top-k sum.  No allocation, no synchronisation, no host reads of device data.
 #include "gemm_direct.h"
 #include "gemm_moe256.h"
 

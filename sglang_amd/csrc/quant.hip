@@ -128,11 +128,13 @@ __device__ __forceinline__ float div448(float a) {
 // ------------------------------------------------------------------------------------------------
 // per-token-group quant
 //
-// The input is walked as a flat sequence of 1 KB "segments" (64 lanes x 8 elements = 512 columns of
-// one row, i.e. GPW = 512/GROUP groups; LPG = GROUP/8 adjacent lanes form a group).  A wavefront
-// owns SEG consecutive segments - contiguous memory whenever K is a multiple of 512 - loads them
-// all with 16-byte nontemporal loads before touching the first, and writes each back as one 8-byte
-// store per lane.  Both streams are used once, so they bypass cache retention.
+// The unit of work is a 1 KB "segment" (64 lanes x 8 elements = 512 columns of one row, i.e.
+// GPW = 512/GROUP groups; LPG = GROUP/8 adjacent lanes form a group).  A wavefront owns SEG segments:
+// SEG consecutive ones of the flat input (contiguous memory whenever K is a multiple of 512) for
+// row-major scales, or the same segment of SEG consecutive rows (ROWFAST) for scale layouts whose rows
+// are the contiguous direction.  It loads them all with 16-byte nontemporal loads before touching the
+// first, and writes each back as one 8-byte store per lane.  Both streams are used once, so they
+// bypass cache retention.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ uint4 load16_stream(const void* p) {
   const v4i v = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(p));
