@@ -95,6 +95,47 @@ def test_block_gemm_deepseek_shapes(dev, M, N, K):
     assert _rel_err(got, ref) <= REL_TOL
 
 
+def test_block_gemm_headline_full_size(dev):
+    """The benchmark's own shape (M=4096 against the [18432, 7168] gate_up weight): a sample of rows and columns
+    against the oracle, and two properties that need no oracle at this size - a row of the output depends on
+    nothing but its own activation row (permuting rows permutes the result bit for bit, whatever tile a row
+    lands in), and power-of-two scale factors pass through exactly."""
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
+
+    M, N, K = 4096, 18432, 7168
+    rng = np.random.default_rng(4096)
+
+    def codes(shape):  # random e4m3fn bytes of moderate magnitude, no NaN codes
+        b = rng.integers(0, 0x60, shape, dtype=np.uint8) | (rng.integers(0, 2, shape, dtype=np.uint8) << 7)
+        return b
+
+    xq, wq = codes((M, K)), codes((N, K))
+    xs = (rng.uniform(0.5, 2.0, (M, K // 128)) * 1e-2).astype(np.float32)
+    ws = (rng.uniform(0.5, 2.0, (N // 128, K // 128)) * 1e-3).astype(np.float32)
+    A, B = fp8_tensor(xq, dev), fp8_tensor(wq, dev)
+    As, Bs = torch.from_numpy(xs).to(dev).t().contiguous().t(), torch.from_numpy(ws).to(dev)
+    C = w8a8_block_fp8_matmul(A, B, As, Bs, [128, 128], torch.bfloat16)
+
+    rows = np.unique(np.concatenate([[0, 255, 256, M - 1], rng.integers(0, M, 6)]))
+    cols = np.unique(np.concatenate([np.arange(0, 130), np.arange(N - 130, N), rng.integers(0, N, 300)]))
+    a = O.e4m3fn_to_f32(xq[rows]).astype(np.float64)
+    b = O.e4m3fn_to_f32(wq[cols]).astype(np.float64)
+    ws_cols = ws[cols // 128]
+    ref = np.zeros((rows.size, cols.size))
+    for kb in range(K // 128):
+        sl = slice(kb * 128, (kb + 1) * 128)
+        ref += (a[:, sl] @ b[:, sl].T) * xs[rows, kb][:, None] * ws_cols[:, kb][None, :]
+    got = C[torch.from_numpy(rows).to(dev)][:, torch.from_numpy(cols).to(dev)].float().cpu().numpy()
+    assert _rel_err(got, ref) <= REL_TOL
+
+    perm = torch.from_numpy(rng.permutation(M)).to(dev)
+    Ap = A.view(torch.uint8)[perm].contiguous().view(torch.float8_e4m3fn)
+    Cp = w8a8_block_fp8_matmul(Ap, B, As[perm].t().contiguous().t(), Bs, [128, 128], torch.bfloat16)
+    assert torch.equal(Cp, C[perm])
+    C4 = w8a8_block_fp8_matmul(A, B, As * 0.5, Bs * 8.0, [128, 128], torch.bfloat16)
+    assert torch.equal(C4, C * 4.0)
+
+
 @pytest.mark.parametrize("M,N,K", [(64, 256, 256), (256, 512, 1024), (1024, 256, 4096), (3, 384, 128)])
 def test_block_gemm_exact_on_integers(dev, M, N, K):
     """Small integers and power-of-two scales: every partial sum is exactly representable."""
