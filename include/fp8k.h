@@ -56,6 +56,18 @@ int fp8k_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, int6
                      int scale_kind, void* stream);
 
 /*
+ * silu_and_mul fused into the per-token-group quantisation: quantises T(T(silu(x[m,c])) * x[m,K+c]) for c < K.
+ * Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_8bit_v2 with fuse_silu_and_mul = true and no masked_m
+ *   (sgl-kernel/python/sgl_kernel/gemm.py:100-136, sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:336-341;
+ *   wrapper python/sglang/srt/layers/quantization/fp8_kernel.py:481-531).
+ * x [M,2K] contiguous of in_dtype (gate columns first, then up); q [M,K] bytes; group_size must be 128.
+ * The result is bit-identical to fp8k_silu_and_mul followed by fp8k_group_quant; scales as in fp8k_group_quant.
+ */
+int fp8k_silu_mul_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, int64_t group_size, float eps,
+                              float fp8_min, float fp8_max, int in_dtype, int64_t s_stride_m, int64_t s_stride_g,
+                              int scale_kind, void* stream);
+
+/*
  * Per-token (row) dynamic FP8 quantisation: s[m] = rowamax/448, q = clamp(x * (1/s)).
  * Replaces torch.ops.sgl_kernel.sgl_per_token_quant_fp8
  *   (sgl-kernel/python/sgl_kernel/gemm.py:155-160, sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-236).

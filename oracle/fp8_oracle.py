@@ -358,6 +358,13 @@ def silu_and_mul(x):
     return to_bf16((silu * u).astype(np.float32))
 
 
+def silu_mul_per_token_group_quant_fp8(x, group_size=128, eps=1e-10, scale_ue8m0=False):
+    """Reference: sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:336-341 (FUSE_SILU_AND_MUL: the value that
+    is quantised is T(T(silu(gate))) * up in the input type T) - i.e. silu_and_mul followed by the group quant.
+    x float32-of-bf16 [M, 2K] -> (q [M, K], scales)."""
+    return per_token_group_quant_fp8(silu_and_mul(x), group_size, eps=eps, scale_ue8m0=scale_ue8m0)
+
+
 def moe_sum_reduce(x, routed_scaling_factor=1.0):
     """Reference: sgl-kernel/csrc/moe/moe_sum_reduce.cu:56-113: out[t] = bf16(rsf * sum_k f32(x[t,k])),
     k ascending, float32 accumulation."""

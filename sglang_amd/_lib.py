@@ -33,6 +33,10 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_f32, _c_f32, _c_f32, _c_int, _c_i64, _c_i64, _c_int, _c_ptr],
     ),
+    "fp8k_silu_mul_group_quant": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_f32, _c_f32, _c_f32, _c_int, _c_i64, _c_i64, _c_int, _c_ptr],
+    ),
     "fp8k_token_quant": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr]),
     "fp8k_tensor_quant": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_ptr]),
     "fp8k_block_gemm": (

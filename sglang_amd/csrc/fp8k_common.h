@@ -102,4 +102,15 @@ __device__ __forceinline__ float group_max(float f) {
   return __uint_as_float(v);
 }
 
+// silu in float32 and the rounding of a float to the element type DT (identity for float32): shared by
+// silu_and_mul and by the group quant that fuses it, so that both produce the same 16-bit values
+__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
+
+template <int DT>
+__device__ __forceinline__ float round_to(float v) {
+  if (DT == FP8K_BF16) return __uint_as_float(f32_to_bf16_bits(v) << 16);
+  if (DT == FP8K_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
+  return v;
+}
+
 }  // namespace fp8k

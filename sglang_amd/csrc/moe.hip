@@ -108,15 +108,6 @@ __global__ __launch_bounds__(256) void moe_scatter_kernel(const IdT* __restrict_
 // the reference kernel computes Activation(x) * y on 16-bit values); float32 input has one rounding.
 // One lane handles 8 columns: two 16-byte loads, one 16-byte store.
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ float silu_f32(float v) { return v / (1.0f + expf(-v)); }
-
-template <int DT>
-__device__ __forceinline__ float round_to(float v) {
-  if (DT == FP8K_BF16) return __uint_as_float(f32_to_bf16_bits(v) << 16);
-  if (DT == FP8K_F16) return f16_bits_to_f32(f32_to_f16_bits(v));
-  return v;
-}
-
 template <int DT>
 __device__ __forceinline__ void load8(const void* base, int64_t elem, float (&a)[8]) {
   if (DT == FP8K_F32) {

@@ -159,10 +159,22 @@ __device__ __forceinline__ void load_stream(Raw8<DT>& r, const void* base, int64
   }
 }
 
-template <int DT, int GROUP, int KIND, int SEG, bool ROWFAST>
+// FUSE: the value that gets quantised is T( T(silu(gate)) * up ) with gate = x[m, c], up = x[m, K + c] of an
+// input row of 2K elements - what silu_and_mul would have written to memory, bit for bit (same two roundings).
+template <int DT>
+__device__ __forceinline__ void silu_mul8(const Raw8<DT>& gate, const Raw8<DT>& up, float (&a)[8]) {
+  float g[8], u[8];
+  gate.unpack(g);
+  up.unpack(u);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = round_to<DT>(round_to<DT>(silu_f32(g[i])) * u[i]);
+}
+
+template <int DT, int GROUP, int KIND, int SEG, bool ROWFAST, bool FUSE>
 __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
                                                           void* __restrict__ s, int M, int G, int64_t K,
                                                           int nseg_row, float eps, int64_t sm, int64_t sg) {
+  const int64_t XK = FUSE ? 2 * K : K;  // elements per input row
   constexpr int LPG = GROUP / 8;
   constexpr int GPW = 64 / LPG;
   static_assert(KIND == FP8K_SCALE_F32 || GROUP == 128, "packed UE8M0 scales need 128-element groups");
@@ -186,7 +198,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
     sr = (int)(wave * SEG - (unsigned)row * (unsigned)nseg_row);
   }
 
-  Raw8<DT> raw[SEG];
+  Raw8<DT> raw[SEG], up[FUSE ? SEG : 1];
   int rows[SEG], segs[SEG];
   bool act[SEG];  // wave-uniform: task j exists
   float scv[SEG];
@@ -200,7 +212,8 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
       const int g = sr * GPW + lg;
       // lanes past the last group of the row re-read the last group and store nothing
       const int64_t col = (int64_t)(g < G ? g : G - 1) * GROUP + li * 8;
-      load_stream<DT>(raw[j], x, (int64_t)row * K + col);
+      load_stream<DT>(raw[j], x, (int64_t)row * XK + col);
+      if (FUSE) load_stream<DT>(up[j], x, (int64_t)row * XK + K + col);
     }
     if (ROWFAST) {
       ++row;
@@ -215,7 +228,8 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
       const int g = segs[j] * GPW + lg;
       const bool valid = g < G;
       float a[8];
-      raw[j].unpack(a);
+      if (FUSE) silu_mul8<DT>(raw[j], up[FUSE ? j : 0], a);
+      else raw[j].unpack(a);
       const float amax = fmaxf(group_max<LPG>(absmax8(a)), eps);
       const float sc = div448<DT != FP8K_F32>(amax);
       uint2 out;
@@ -253,18 +267,24 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
         int row = rows[0], seg = segs[0];
 #pragma unroll
         for (int i = 1; i < SEG; ++i) { row = j == i ? rows[i] : row; seg = j == i ? segs[i] : seg; }
-        const int64_t at = (int64_t)row * K + (int64_t)(seg * GPW + lg) * GROUP + li * 8;
+        const int64_t col = (int64_t)(seg * GPW + lg) * GROUP + li * 8;
         Raw8<DT> again;
-        again.load(x, at);
+        again.load(x, (int64_t)row * XK + col);
         float a[8];
-        again.unpack(a);
-        store8_stream(q + at, quant8_divide(a, sc));
+        if (FUSE) {
+          Raw8<DT> again_up;
+          again_up.load(x, (int64_t)row * XK + K + col);
+          silu_mul8<DT>(again, again_up, a);
+        } else {
+          again.unpack(a);
+        }
+        store8_stream(q + (int64_t)row * K + col, quant8_divide(a, sc));
       }
     }
   }
 }
 
-template <int DT, int GROUP, int KIND>
+template <int DT, int GROUP, int KIND, bool FUSE = false>
 static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, float eps, int64_t sm, int64_t sg,
                               hipStream_t st) {
   constexpr int GPW = 64 / (GROUP / 8);
@@ -277,10 +297,10 @@ static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_
   const int64_t waves = rowfast ? (M + SEG - 1) / SEG * nseg_row : (total + SEG - 1) / SEG;
   const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   if (rowfast)
-    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, true>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M, G,
+    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, true, FUSE>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M, G,
                        K, nseg_row, eps, sm, sg);
   else
-    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, false>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M,
+    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, false, FUSE>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M,
                        G, K, nseg_row, eps, sm, sg);
   return check_launch("group_quant");
 }
@@ -475,6 +495,49 @@ extern "C" int fp8k_group_quant(const void* x, void* q, void* s, int64_t M, int6
     default: return FP8K_GQ(FP8K_F32);
   }
 #undef FP8K_GQ
+}
+
+extern "C" int fp8k_silu_mul_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, int64_t group_size,
+                                         float eps, float fp8_min, float fp8_max, int in_dtype, int64_t s_stride_m,
+                                         int64_t s_stride_g, int scale_kind, void* stream) {
+  clear_error();
+  const char* op = "silu_mul_group_quant";
+  FP8K_REQUIRE(M >= 0 && K >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(group_size == 128, "%s: the fused form is built for group_size 128 (got %lld)", op, (long long)group_size);
+  FP8K_REQUIRE(K % group_size == 0, "%s: the output width (%lld) cannot be divisible by `group_size` (%lld)", op,
+               (long long)K, (long long)group_size);
+  FP8K_REQUIRE(fp8_max == 448.0f && fp8_min == -448.0f, "%s: fp8_min/fp8_max must be -448/448 (OCP e4m3fn)", op);
+  FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "%s: bad input dtype %d", op, in_dtype);
+  FP8K_REQUIRE(scale_kind == FP8K_SCALE_F32 || scale_kind == FP8K_SCALE_UE8M0_PACKED, "%s: bad scale kind %d", op, scale_kind);
+  FP8K_REQUIRE(M <= 0x7fffffffLL && K / group_size <= 0x3fffffffLL, "%s: shape too large", op);
+  if (M == 0 || K == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && q && s, "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(x, 16) && aligned(q, 8) && aligned(s, 4), "%s: x must be 16-byte, q 8-byte aligned", op);
+  const int64_t G = K / group_size;
+  if (scale_kind == FP8K_SCALE_F32) {
+    FP8K_REQUIRE(s_stride_m >= 0 && s_stride_g >= 0 && (M == 1 || s_stride_m > 0) && (G == 1 || s_stride_g > 0),
+                 "%s: scale strides must be positive", op);
+  } else {
+    FP8K_REQUIRE(s_stride_m > 0 && ((G + 3) / 4 == 1 || s_stride_g > 0), "%s: packed scale strides must be positive", op);
+  }
+  float eps_eff = eps;  // clamped in the input dtype, as in fp8k_group_quant
+  if (in_dtype == FP8K_BF16) {
+    uint32_t u;
+    memcpy(&u, &eps, 4);
+    u = ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16) << 16;
+    memcpy(&eps_eff, &u, 4);
+  }
+  hipStream_t st = (hipStream_t)stream;
+#define FP8K_SGQ(DT)                                                                                                 \
+  (scale_kind == FP8K_SCALE_F32                                                                                     \
+       ? launch_group_quant<DT, 128, FP8K_SCALE_F32, true>(x, q, s, M, K, eps_eff, s_stride_m, s_stride_g, st)      \
+       : launch_group_quant<DT, 128, FP8K_SCALE_UE8M0_PACKED, true>(x, q, s, M, K, eps_eff, s_stride_m, s_stride_g, st))
+  switch (in_dtype) {
+    case FP8K_BF16: return FP8K_SGQ(FP8K_BF16);
+    case FP8K_F16: return FP8K_SGQ(FP8K_F16);
+    default: return FP8K_SGQ(FP8K_F32);
+  }
+#undef FP8K_SGQ
 }
 
 extern "C" int fp8k_token_quant(const void* x, void* q, float* s, int64_t M, int64_t K, int in_dtype, void* stream) {

@@ -173,7 +173,6 @@ def fused_experts_impl(
     topk_ids = topk_ids.contiguous()
 
     cache1 = torch.empty((M * topk, N), device=dev, dtype=dt)
-    cache2 = torch.empty((M * topk, N // 2), device=dev, dtype=dt)
     cache3 = torch.empty((M, topk, w2.shape[1]), device=dev, dtype=dt)
     if no_combine:
         assert not inplace
@@ -195,7 +194,6 @@ def fused_experts_impl(
         curr_ids = topk_ids[begin:end]
         curr_w = topk_weights[begin:end]
         ic1 = cache1[: tokens * topk]
-        ic2 = cache2[: tokens * topk]
         ic3 = out_hidden_states[begin:end] if no_combine else cache3[:tokens]
 
         sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(curr_ids, config["BLOCK_SIZE_M"], E)
@@ -203,9 +201,11 @@ def fused_experts_impl(
             curr, w1, None, ic1, None, w1_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
             num_tokens_post_padded, False, topk, config, use_fp8_w8a8=True, block_shape=block_shape,
         )
-        _ops.silu_and_mul(ic1, ic2)
+        # silu_and_mul fused into the requantisation (same bytes as silu_and_mul + group quant, one pass less
+        # over the [tokens*topk, N] intermediate)
+        a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=True, fuse_silu_and_mul=True)
         invoke_fused_moe_kernel(
-            ic2, w2, None, ic3, None, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
+            a2_q, w2, None, ic3, a2_s, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
             num_tokens_post_padded, True, 1, config, use_fp8_w8a8=True, block_shape=block_shape,
         )
         if not no_combine:

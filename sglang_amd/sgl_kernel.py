@@ -56,9 +56,11 @@ def sgl_per_token_group_quant_8bit(
     output_s selects the scale layout by its strides and dtype: float32 [M, K/g] in any of row-major,
     column-major, column-major padded; int32 [M, ceil(K/g/4)] (column-major, M padded to 4) when
     scale_ue8m0.  `enable_v2` is accepted for signature compatibility: there is one kernel.
+    fuse_silu_and_mul (the v2 op, gemm.py:118-133): input is [M, 2K] (gate columns, then up), output_q [M, K];
+    what is quantised is silu_and_mul's 16-bit result, bit for bit.
     """
-    if fuse_silu_and_mul or masked_m is not None:
-        raise RuntimeError("sgl_per_token_group_quant_8bit: fuse_silu_and_mul / masked_m are not built on this path")
+    if masked_m is not None:
+        raise RuntimeError("sgl_per_token_group_quant_8bit: masked_m (the masked expert layout) is not built on this path")
     require_cuda(input, output_q, output_s)
     if not input.is_contiguous():
         raise RuntimeError("input must be contiguous")
@@ -70,12 +72,14 @@ def sgl_per_token_group_quant_8bit(
         raise RuntimeError("input.numel() %% group_size != 0 (%d, %d)" % (input.numel(), group_size))
     if output_s.dim() != 2:
         raise RuntimeError("output_s.dim() must be 2")
-    K = input.shape[-1]
+    if fuse_silu_and_mul and input.shape[-1] % 2 != 0:
+        raise RuntimeError("fuse_silu_and_mul needs an even last dimension")
+    K = input.shape[-1] // 2 if fuse_silu_and_mul else input.shape[-1]
     if K % group_size != 0:
         raise RuntimeError("the last dimension of `x` cannot be divisible by `group_size`")
-    M = input.numel() // K if K else 0
+    M = input.numel() // input.shape[-1] if K else 0
     G = K // group_size
-    if output_q.numel() != input.numel():
+    if output_q.numel() != M * K:
         raise RuntimeError("output_q has the wrong number of elements")
     if scale_ue8m0:
         if output_s.dtype != torch.int32:
@@ -89,8 +93,9 @@ def sgl_per_token_group_quant_8bit(
         if output_s.shape[0] != M or output_s.shape[1] != G:
             raise RuntimeError("output_s must be [M, K/group_size]")
         kind = _lib.SCALE_F32
+    fn = lib.fp8k_silu_mul_group_quant if fuse_silu_and_mul else lib.fp8k_group_quant
     check(
-        lib.fp8k_group_quant(
+        fn(
             input.data_ptr(), output_q.data_ptr(), output_s.data_ptr(), M, K, group_size, float(eps), float(fp8_min),
             float(fp8_max), dtype_code(input.dtype), output_s.stride(0), output_s.stride(1), kind,
             stream_ptr(input.device),

@@ -253,3 +253,50 @@ def test_per_tensor_quant(dev, numel):
     q2, s2 = scaled_fp8_quant(xt, st)
     q2_ref, _ = O.per_tensor_quant_fp8(x, 0.05)
     np.testing.assert_array_equal(u8(q2), q2_ref)
+
+
+@pytest.mark.parametrize("layout", _layouts())
+@pytest.mark.parametrize("M,K", [(1, 128), (37, 2048), (512, 2048), (4096, 2048)])
+def test_silu_mul_group_quant_equals_the_two_step_pipeline(dev, M, K, layout):
+    """fuse_silu_and_mul (reference: per_token_group_quant_8bit_v2.cu:336-341): the bytes and scales must equal
+    silu_and_mul followed by the group quant, bit for bit - against this library's two kernels, and against
+    the oracle's quant applied to the 16-bit values that silu_and_mul produced (the silu itself is compared
+    with the oracle, to one bf16 ulp because of expf, in the MoE tests)."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import silu_and_mul
+
+    cm, al, ue = layout
+    kw = dict(column_major_scales=cm, scale_tma_aligned=al, scale_ue8m0=ue)
+    x = torch.from_numpy(O.make_activation(M, 2 * K, seed=M + K)).to(dev).to(torch.bfloat16)
+    q, s = sglang_per_token_group_quant_fp8(x, 128, fuse_silu_and_mul=True, **kw)
+    mid = torch.empty((M, K), device=dev, dtype=torch.bfloat16)
+    silu_and_mul(x, mid)
+    q2, s2 = sglang_per_token_group_quant_fp8(mid, 128, **kw)
+    torch.cuda.synchronize()
+    assert q.shape == (M, K) and s.shape == s2.shape and s.stride() == s2.stride()
+    np.testing.assert_array_equal(u8(q), u8(q2))
+    if kw.get("scale_ue8m0"):
+        assert torch.equal(s, s2)
+    else:
+        assert torch.equal(s.contiguous().view(torch.int32), s2.contiguous().view(torch.int32))
+    q_ref, s_ref = O.per_token_group_quant_fp8(mid.float().cpu().numpy(), 128, scale_ue8m0=bool(kw.get("scale_ue8m0")))
+    np.testing.assert_array_equal(u8(q), q_ref)
+
+
+def test_silu_mul_group_quant_other_dtypes_and_errors(dev):
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import silu_and_mul
+
+    for dt in (torch.float16, torch.float32):
+        x = (torch.randn((65, 512), device=dev) * 3).to(dt)
+        q, s = sglang_per_token_group_quant_fp8(x, 128, fuse_silu_and_mul=True)
+        mid = torch.empty((65, 256), device=dev, dtype=dt)
+        silu_and_mul(x, mid)
+        q2, s2 = sglang_per_token_group_quant_fp8(mid, 128)
+        np.testing.assert_array_equal(u8(q), u8(q2))
+        assert torch.equal(s, s2)
+    x = torch.randn((4, 512), device=dev, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="group_size 128"):
+        sglang_per_token_group_quant_fp8(x, 64, fuse_silu_and_mul=True)
+    with pytest.raises(RuntimeError, match="masked_m"):
+        sglang_per_token_group_quant_fp8(x, 128, fuse_silu_and_mul=True, masked_m=torch.zeros(1, device=dev, dtype=torch.int32))
