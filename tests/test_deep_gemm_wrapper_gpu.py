@@ -1,0 +1,93 @@
+"""GPU parity of the DeepGEMM-shaped entry points (plain, contiguous grouped, masked grouped) against the oracle's
+block matmul applied group by group.  Tolerance as for the other GEMMs: max relative error <= 1e-2 on bf16 output;
+rows that the layout marks as skipped must stay untouched."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+from tests.conftest import fp8_tensor
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def _codes(rng, shape):
+    return rng.integers(0, 0x60, shape, dtype=np.uint8) | (rng.integers(0, 2, shape, dtype=np.uint8) << 7)
+
+
+def _rel(c, ref):
+    return float(np.abs(c.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
+
+
+def test_gemm_nt_f8f8bf16(dev):
+    from sglang_amd.deep_gemm_wrapper import gemm_nt_f8f8bf16
+
+    rng = np.random.default_rng(1)
+    M, N, K = 200, 512, 1024
+    aq, bq = _codes(rng, (M, K)), _codes(rng, (N, K))
+    a_s = rng.uniform(0.5, 2.0, (M, K // 128)).astype(np.float32) * 1e-2
+    b_s = rng.uniform(0.5, 2.0, (N // 128, K // 128)).astype(np.float32) * 1e-2
+    out = torch.empty((M, N), device=dev, dtype=torch.bfloat16)
+    gemm_nt_f8f8bf16((fp8_tensor(aq, dev), torch.from_numpy(a_s).to(dev)), (fp8_tensor(bq, dev), torch.from_numpy(b_s).to(dev)), out)
+    ref = O.w8a8_block_fp8_matmul(aq, bq, a_s, b_s, acc=np.float64)
+    assert _rel(out.float().cpu().numpy(), ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("G,rows,N,K", [(4, [128, 0, 256, 128], 512, 512), (8, [128] * 8, 256, 1024), (3, [384, 128, 640], 384, 256)])
+def test_grouped_contiguous(dev, G, rows, N, K):
+    """Rows of each group contiguous and padded to 128 (DeepGEMM's alignment); the padding rows carry -1."""
+    from sglang_amd.deep_gemm_wrapper import grouped_gemm_nt_f8f8bf16_contig
+
+    rng = np.random.default_rng(G * 1000 + N)
+    m_sum = sum(rows)
+    m_indices = np.full((m_sum,), -1, dtype=np.int32)
+    at = 0
+    for g, r in enumerate(rows):
+        real = r - (37 if r >= 128 else 0)  # the tail of every group's range is padding
+        m_indices[at:at + real] = g
+        at += r
+    aq, bq = _codes(rng, (m_sum, K)), _codes(rng, (G, N, K))
+    a_s = rng.uniform(0.5, 2.0, (m_sum, K // 128)).astype(np.float32) * 1e-2
+    b_s = rng.uniform(0.5, 2.0, (G, N // 128, K // 128)).astype(np.float32) * 1e-2
+    out = torch.full((m_sum, N), 7.0, device=dev, dtype=torch.bfloat16)
+    grouped_gemm_nt_f8f8bf16_contig((fp8_tensor(aq, dev), torch.from_numpy(a_s).to(dev)),
+                                    (fp8_tensor(bq, dev), torch.from_numpy(b_s).to(dev)), out, torch.from_numpy(m_indices).to(dev))
+    got = out.float().cpu().numpy()
+    for g in range(G):
+        sel = np.nonzero(m_indices == g)[0]
+        if sel.size:
+            ref = O.w8a8_block_fp8_matmul(aq[sel], bq[g], a_s[sel], b_s[g], acc=np.float64)
+            assert _rel(got[sel], ref) <= REL_TOL
+    assert np.all(got[m_indices < 0] == 7.0)
+
+
+@pytest.mark.parametrize("G,m_max,masked,N,K", [(4, 128, [0, 5, 128, 77], 256, 512), (6, 512, [300, 1, 512, 0, 129, 256], 512, 256)])
+def test_grouped_masked(dev, G, m_max, masked, N, K):
+    from sglang_amd.deep_gemm_wrapper import grouped_gemm_nt_f8f8bf16_masked
+
+    rng = np.random.default_rng(G * 77 + m_max)
+    aq, bq = _codes(rng, (G, m_max, K)), _codes(rng, (G, N, K))
+    a_s = rng.uniform(0.5, 2.0, (G, m_max, K // 128)).astype(np.float32) * 1e-2
+    b_s = rng.uniform(0.5, 2.0, (G, N // 128, K // 128)).astype(np.float32) * 1e-2
+    out = torch.full((G, m_max, N), -3.0, device=dev, dtype=torch.bfloat16)
+    grouped_gemm_nt_f8f8bf16_masked((fp8_tensor(aq, dev), torch.from_numpy(a_s).to(dev)),
+                                    (fp8_tensor(bq, dev), torch.from_numpy(b_s).to(dev)), out,
+                                    torch.tensor(masked, device=dev, dtype=torch.int32), max(sum(masked) // G, 1))
+    got = out.float().cpu().numpy()
+    for g in range(G):
+        m = masked[g]
+        if m:
+            ref = O.w8a8_block_fp8_matmul(aq[g, :m], bq[g], a_s[g, :m], b_s[g], acc=np.float64)
+            assert _rel(got[g, :m], ref) <= REL_TOL
+        assert np.all(got[g, m:] == -3.0)
+
+
+def test_wrapper_errors(dev):
+    from sglang_amd.deep_gemm_wrapper import gemm_nt_f8f8bf16
+
+    a = torch.zeros((4, 128), device=dev, dtype=torch.float8_e4m3fn)
+    s_packed = torch.zeros((4, 1), device=dev, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="float32"):
+        gemm_nt_f8f8bf16((a, s_packed), (a, torch.ones((1, 1), device=dev)), torch.empty((4, 4), device=dev, dtype=torch.bfloat16))
