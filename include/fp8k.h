@@ -68,6 +68,21 @@ int fp8k_silu_mul_group_quant(const void* x, void* q, void* s, int64_t M, int64_
                               int scale_kind, void* stream);
 
 /*
+ * Masked-layout form of the two calls above: x [E, m_max, K] (or [E, m_max, 2K] with fuse_silu_and_mul), q [E, m_max, K];
+ * only the first masked_m[e] rows of expert e are read and written.
+ * Replaces torch.ops.sgl_kernel.sgl_per_token_group_quant_8bit_v2 with masked_m
+ *   (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu, wrapper fp8_kernel.py:481-531) and the Triton
+ *   silu_and_mul_masked_post_quant_fwd (python/sglang/srt/layers/moe/ep_moe/kernels.py:364-429).
+ * Scales as in fp8k_group_quant with one more stride: row i of expert e, group g at
+ *   s[e*s_stride_e + i*s_stride_m + g*s_stride_g] (packed UE8M0: word g/4 at (g/4)*s_stride_g).
+ * masked_m: int32[E] on the device.  group_size must be 128.
+ */
+int fp8k_group_quant_masked(const void* x, void* q, void* s, int64_t E, int64_t m_max, int64_t K, int64_t group_size,
+                            float eps, float fp8_min, float fp8_max, int in_dtype, int64_t s_stride_e,
+                            int64_t s_stride_m, int64_t s_stride_g, int scale_kind, int fuse_silu_and_mul,
+                            const int32_t* masked_m, void* stream);
+
+/*
  * Per-token (row) dynamic FP8 quantisation: s[m] = rowamax/448, q = clamp(x * (1/s)).
  * Replaces torch.ops.sgl_kernel.sgl_per_token_quant_fp8
  *   (sgl-kernel/python/sgl_kernel/gemm.py:155-160, sgl-kernel/csrc/gemm/per_token_quant_fp8.cu:15-236).

@@ -37,6 +37,11 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_f32, _c_f32, _c_f32, _c_int, _c_i64, _c_i64, _c_int, _c_ptr],
     ),
+    "fp8k_group_quant_masked": (
+        _c_int,
+        [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_f32, _c_f32, _c_f32, _c_int, _c_i64, _c_i64, _c_i64,
+         _c_int, _c_int, _c_ptr, _c_ptr],
+    ),
     "fp8k_token_quant": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr]),
     "fp8k_tensor_quant": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_ptr]),
     "fp8k_block_gemm": (

@@ -170,11 +170,19 @@ __device__ __forceinline__ void silu_mul8(const Raw8<DT>& gate, const Raw8<DT>& 
   for (int i = 0; i < 8; ++i) a[i] = round_to<DT>(round_to<DT>(silu_f32(g[i])) * u[i]);
 }
 
-template <int DT, int GROUP, int KIND, int SEG, bool ROWFAST, bool FUSE>
+// MASKED: the M rows are E experts x m_max slots; only the first masked_m[e] slots of expert e are quantised
+// (the others are neither read nor written), and the scale of slot i of expert e sits at e*se + i*sm + g*sg.
+template <int DT, int GROUP, int KIND, int SEG, bool ROWFAST, bool FUSE, bool MASKED>
 __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
                                                           void* __restrict__ s, int M, int G, int64_t K,
-                                                          int nseg_row, float eps, int64_t sm, int64_t sg) {
+                                                          int nseg_row, float eps, int64_t sm, int64_t sg,
+                                                          const int32_t* __restrict__ masked_m, int m_max, int64_t se) {
   const int64_t XK = FUSE ? 2 * K : K;  // elements per input row
+  auto scale_row = [&](int r) -> int64_t {  // offset of the scales of row r
+    if (!MASKED) return (int64_t)r * sm;
+    const int e = r / m_max;
+    return (int64_t)e * se + (int64_t)(r - e * m_max) * sm;
+  };
   constexpr int LPG = GROUP / 8;
   constexpr int GPW = 64 / LPG;
   static_assert(KIND == FP8K_SCALE_F32 || GROUP == 128, "packed UE8M0 scales need 128-element groups");
@@ -208,6 +216,10 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
     rows[j] = row;
     segs[j] = sr;
     act[j] = ROWFAST ? row < M : wave * SEG + j < total;
+    if (MASKED && act[j]) {
+      const int e = row / m_max;
+      act[j] = row - e * m_max < masked_m[e];
+    }
     if (act[j]) {
       const int g = sr * GPW + lg;
       // lanes past the last group of the row re-read the last group and store nothing
@@ -245,13 +257,13 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
                            ((uint32_t)__builtin_amdgcn_readlane((int)eb, 16) << 8) |
                            ((uint32_t)__builtin_amdgcn_readlane((int)eb, 32) << 16) |
                            ((uint32_t)__builtin_amdgcn_readlane((int)eb, 48) << 24);
-        if (lane == 0) reinterpret_cast<uint32_t*>(s)[(int64_t)segs[j] * sg + (int64_t)rows[j] * sm] = w;
+        if (lane == 0) reinterpret_cast<uint32_t*>(s)[(int64_t)segs[j] * sg + scale_row(rows[j])] = w;
       } else {
         bool redo;
         out = quant8_bracket<DT != FP8K_F32>(a, sc, amax, redo);
         redo_mask |= (redo & valid) ? (1u << j) : 0u;
         scv[j] = sc;
-        if (valid && li == 0) reinterpret_cast<float*>(s)[(int64_t)rows[j] * sm + (int64_t)g * sg] = sc;
+        if (valid && li == 0) reinterpret_cast<float*>(s)[scale_row(rows[j]) + (int64_t)g * sg] = sc;
       }
       if (valid) store8_stream(q + (int64_t)rows[j] * K + (int64_t)g * GROUP + li * 8, out);
     }
@@ -284,9 +296,9 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
   }
 }
 
-template <int DT, int GROUP, int KIND, bool FUSE = false>
+template <int DT, int GROUP, int KIND, bool FUSE = false, bool MASKED = false>
 static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_t K, float eps, int64_t sm, int64_t sg,
-                              hipStream_t st) {
+                              hipStream_t st, const int32_t* masked_m = nullptr, int m_max = 1, int64_t se = 0) {
   constexpr int GPW = 64 / (GROUP / 8);
   constexpr int SEG = 4;
   const int G = (int)(K / GROUP);
@@ -297,11 +309,11 @@ static int launch_group_quant(const void* x, void* q, void* s, int64_t M, int64_
   const int64_t waves = rowfast ? (M + SEG - 1) / SEG * nseg_row : (total + SEG - 1) / SEG;
   const dim3 grid((unsigned)((waves + 3) / 4)), block(256);
   if (rowfast)
-    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, true, FUSE>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M, G,
-                       K, nseg_row, eps, sm, sg);
+    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, true, FUSE, MASKED>), grid, block, 0, st, x, (uint8_t*)q, s,
+                       (int)M, G, K, nseg_row, eps, sm, sg, masked_m, m_max, se);
   else
-    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, false, FUSE>), grid, block, 0, st, x, (uint8_t*)q, s, (int)M,
-                       G, K, nseg_row, eps, sm, sg);
+    hipLaunchKernelGGL((group_quant_kernel<DT, GROUP, KIND, SEG, false, FUSE, MASKED>), grid, block, 0, st, x, (uint8_t*)q, s,
+                       (int)M, G, K, nseg_row, eps, sm, sg, masked_m, m_max, se);
   return check_launch("group_quant");
 }
 
@@ -538,6 +550,47 @@ extern "C" int fp8k_silu_mul_group_quant(const void* x, void* q, void* s, int64_
     default: return FP8K_SGQ(FP8K_F32);
   }
 #undef FP8K_SGQ
+}
+
+extern "C" int fp8k_group_quant_masked(const void* x, void* q, void* s, int64_t E, int64_t m_max, int64_t K,
+                                       int64_t group_size, float eps, float fp8_min, float fp8_max, int in_dtype,
+                                       int64_t s_stride_e, int64_t s_stride_m, int64_t s_stride_g, int scale_kind,
+                                       int fuse_silu_and_mul, const int32_t* masked_m, void* stream) {
+  clear_error();
+  const char* op = "group_quant_masked";
+  FP8K_REQUIRE(E >= 0 && m_max >= 0 && K >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(group_size == 128, "%s: the masked form is built for group_size 128 (got %lld)", op, (long long)group_size);
+  FP8K_REQUIRE(K % group_size == 0, "%s: the output width (%lld) cannot be divisible by `group_size` (%lld)", op,
+               (long long)K, (long long)group_size);
+  FP8K_REQUIRE(fp8_max == 448.0f && fp8_min == -448.0f, "%s: fp8_min/fp8_max must be -448/448 (OCP e4m3fn)", op);
+  FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "%s: bad input dtype %d", op, in_dtype);
+  FP8K_REQUIRE(scale_kind == FP8K_SCALE_F32 || scale_kind == FP8K_SCALE_UE8M0_PACKED, "%s: bad scale kind %d", op, scale_kind);
+  FP8K_REQUIRE(E * m_max <= 0x7fffffffLL && m_max <= 0x7fffffffLL && K / group_size <= 0x3fffffffLL, "%s: shape too large", op);
+  if (E == 0 || m_max == 0 || K == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && q && s && masked_m, "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(x, 16) && aligned(q, 8) && aligned(s, 4) && aligned(masked_m, 4), "%s: x must be 16-byte, q 8-byte aligned", op);
+  FP8K_REQUIRE(s_stride_e >= 0 && s_stride_m >= 0 && s_stride_g >= 0, "%s: negative scale stride", op);
+  float eps_eff = eps;  // clamped in the input dtype, as in fp8k_group_quant
+  if (in_dtype == FP8K_BF16) {
+    uint32_t u;
+    memcpy(&u, &eps, 4);
+    u = ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16) << 16;
+    memcpy(&eps_eff, &u, 4);
+  }
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t M = E * m_max;
+#define FP8K_MQ3(DT, KIND, FUSE) \
+  launch_group_quant<DT, 128, KIND, FUSE, true>(x, q, s, M, K, eps_eff, s_stride_m, s_stride_g, st, masked_m, (int)m_max, s_stride_e)
+#define FP8K_MQ2(DT, KIND) (fuse_silu_and_mul ? FP8K_MQ3(DT, KIND, true) : FP8K_MQ3(DT, KIND, false))
+#define FP8K_MQ(DT) (scale_kind == FP8K_SCALE_F32 ? FP8K_MQ2(DT, FP8K_SCALE_F32) : FP8K_MQ2(DT, FP8K_SCALE_UE8M0_PACKED))
+  switch (in_dtype) {
+    case FP8K_BF16: return FP8K_MQ(FP8K_BF16);
+    case FP8K_F16: return FP8K_MQ(FP8K_F16);
+    default: return FP8K_MQ(FP8K_F32);
+  }
+#undef FP8K_MQ
+#undef FP8K_MQ2
+#undef FP8K_MQ3
 }
 
 extern "C" int fp8k_token_quant(const void* x, void* q, float* s, int64_t M, int64_t K, int in_dtype, void* stream) {

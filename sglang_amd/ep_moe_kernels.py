@@ -1,0 +1,37 @@
+"""Masked-layout MoE helpers of the DeepEP low-latency path on this library's kernels.
+
+Reference: python/sglang/srt/layers/moe/ep_moe/kernels.py:364-429 (`silu_and_mul_masked_post_quant_fwd`, a Triton
+kernel there).  Together with `deep_gemm_wrapper.grouped_gemm_nt_f8f8bf16_masked` these are the three compute steps
+of the masked expert runner (moe_runner/deep_gemm.py): grouped GEMM, silu_and_mul + requant, grouped GEMM.
+"""
+import torch
+
+from . import sgl_kernel as _ops
+from .fp8_kernel import fp8_max, fp8_min
+
+
+def silu_and_mul_masked_post_quant_fwd(
+    input: torch.Tensor,
+    output: torch.Tensor,
+    output_scale: torch.Tensor,
+    quant_group_size: int,
+    masked_m: torch.Tensor,
+    scale_ue8m0: bool = False,
+) -> None:
+    """input [expert_num, token_num_padded, 2*hidden] bf16/fp16; output [expert_num, token_num_padded, hidden]
+    float8_e4m3fn; output_scale float32 [expert_num, token_num_padded, hidden // group] in any strides; masked_m
+    int32 [expert_num].  Rows at or past masked_m[e] are left untouched.  The values quantised are
+    T(T(silu(gate)) * up) in the input type T, the scale is max(amax, 1e-10) / 448, as in the reference kernel."""
+    assert input.is_contiguous()
+    assert output.dtype == torch.float8_e4m3fn
+    assert output.is_contiguous()
+    assert len(input.shape) == 3
+    assert input.shape[0] == masked_m.shape[0]
+    assert input.shape[-1] % 2 == 0
+    assert (input.shape[-1] // 2) % quant_group_size == 0
+    if scale_ue8m0:
+        raise RuntimeError("silu_and_mul_masked_post_quant_fwd: float32-stored UE8M0 scales are not built on this path "
+                           "(use sglang_per_token_group_quant_fp8(..., scale_ue8m0=True, masked_m=...) for packed ones)")
+    _ops.sgl_per_token_group_quant_8bit(
+        input, output, output_scale, quant_group_size, 1e-10, fp8_min, fp8_max, False, True, masked_m.to(torch.int32)
+    )

@@ -69,6 +69,15 @@ def sglang_per_token_group_quant_fp8(
         scale_tma_aligned=scale_tma_aligned,
         scale_ue8m0=scale_ue8m0,
     )
+    if masked_m is not None:
+        # masked expert layout [num_experts, max_tokens, hidden]: scales keep their three strides
+        if x.dim() != 3:
+            raise RuntimeError("masked_m needs a 3-D input [num_experts, max_tokens, hidden]")
+        if x.numel() > 0:
+            _ops.sgl_per_token_group_quant_8bit(
+                x, x_q, x_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, fuse_silu_and_mul, masked_m, enable_v2=enable_v2
+            )
+        return x_q, x_s
     if x.shape[0] > 0:
         s2 = x_s if x_s.dim() == 2 else x_s.reshape(-1, x_s.shape[-1]) if not (column_major_scales or scale_ue8m0) else x_s
         if s2.dim() != 2:

@@ -59,9 +59,10 @@ def sgl_per_token_group_quant_8bit(
     fuse_silu_and_mul (the v2 op, gemm.py:118-133): input is [M, 2K] (gate columns, then up), output_q [M, K];
     what is quantised is silu_and_mul's 16-bit result, bit for bit.
     """
+    require_cuda(input, output_q, output_s, masked_m)
     if masked_m is not None:
-        raise RuntimeError("sgl_per_token_group_quant_8bit: masked_m (the masked expert layout) is not built on this path")
-    require_cuda(input, output_q, output_s)
+        return _group_quant_masked(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0,
+                                   fuse_silu_and_mul, masked_m)
     if not input.is_contiguous():
         raise RuntimeError("input must be contiguous")
     if not output_q.is_contiguous():
@@ -99,6 +100,45 @@ def sgl_per_token_group_quant_8bit(
             input.data_ptr(), output_q.data_ptr(), output_s.data_ptr(), M, K, group_size, float(eps), float(fp8_min),
             float(fp8_max), dtype_code(input.dtype), output_s.stride(0), output_s.stride(1), kind,
             stream_ptr(input.device),
+        )
+    )
+
+
+def _group_quant_masked(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, fuse_silu_and_mul,
+                        masked_m) -> None:
+    """Masked expert layout of the v2 op (gemm.py:118-133): input [E, m_max, K] (or 2K with fuse_silu_and_mul),
+    output_q [E, m_max, K], output_s [E, m_max, K/g] float32 in any strides or int32 [E, m_max, ceil(K/g/4)] packed;
+    masked_m int32 [E] - rows at or past masked_m[e] are neither read nor written."""
+    if input.dim() != 3 or output_q.dim() != 3 or output_s.dim() != 3:
+        raise RuntimeError("masked_m needs 3-D input, output_q and output_s ([num_experts, max_tokens, hidden])")
+    if not (input.is_contiguous() and output_q.is_contiguous()):
+        raise RuntimeError("input and output_q must be contiguous")
+    if output_q.dtype != FP8_DTYPE:
+        raise RuntimeError("output_q must be float8_e4m3fn (int8 destination is not built on this path)")
+    E, m_max, width = input.shape
+    if fuse_silu_and_mul and width % 2 != 0:
+        raise RuntimeError("fuse_silu_and_mul needs an even last dimension")
+    K = width // 2 if fuse_silu_and_mul else width
+    if K % group_size != 0:
+        raise RuntimeError("the last dimension of `x` cannot be divisible by `group_size`")
+    G = K // group_size
+    if tuple(output_q.shape) != (E, m_max, K):
+        raise RuntimeError("output_q must be [num_experts, max_tokens, hidden]")
+    if masked_m.dtype != torch.int32 or masked_m.numel() != E or not masked_m.is_contiguous():
+        raise RuntimeError("masked_m must be contiguous int32 [num_experts]")
+    if scale_ue8m0:
+        if output_s.dtype != torch.int32 or tuple(output_s.shape) != (E, m_max, (G + 3) // 4):
+            raise RuntimeError("packed output_s must be int32 [num_experts, max_tokens, ceil(K/group/4)]")
+        kind = _lib.SCALE_UE8M0_PACKED
+    else:
+        if output_s.dtype != torch.float32 or tuple(output_s.shape) != (E, m_max, G):
+            raise RuntimeError("output_s must be float32 [num_experts, max_tokens, K/group_size]")
+        kind = _lib.SCALE_F32
+    check(
+        lib.fp8k_group_quant_masked(
+            input.data_ptr(), output_q.data_ptr(), output_s.data_ptr(), E, m_max, K, group_size, float(eps),
+            float(fp8_min), float(fp8_max), dtype_code(input.dtype), output_s.stride(0), output_s.stride(1),
+            output_s.stride(2), kind, 1 if fuse_silu_and_mul else 0, masked_m.data_ptr(), stream_ptr(input.device),
         )
     )
 

@@ -300,3 +300,61 @@ def test_silu_mul_group_quant_other_dtypes_and_errors(dev):
         sglang_per_token_group_quant_fp8(x, 64, fuse_silu_and_mul=True)
     with pytest.raises(RuntimeError, match="masked_m"):
         sglang_per_token_group_quant_fp8(x, 128, fuse_silu_and_mul=True, masked_m=torch.zeros(1, device=dev, dtype=torch.int32))
+
+
+@pytest.mark.parametrize("fuse", [False, True])
+@pytest.mark.parametrize("layout", _layouts())
+def test_masked_group_quant(dev, layout, fuse):
+    """Masked expert layout (reference: per_token_group_quant_8bit_v2.cu with masked_m, ep_moe/kernels.py:364-429):
+    rows below masked_m[e] must equal the unmasked op on the same rows bit for bit, rows at or past it must be
+    left untouched (output and scales)."""
+    from sglang_amd.fp8_kernel import create_per_token_group_quant_fp8_output_scale, fp8_max, fp8_min, sglang_per_token_group_quant_fp8
+    from sglang_amd.sgl_kernel import sgl_per_token_group_quant_8bit
+
+    cm, al, ue = layout
+    E, m_max, K = 5, 40, 512
+    masked = [0, 40, 7, 33, 1]
+    width = 2 * K if fuse else K
+    x = torch.from_numpy(O.make_activation(E * m_max, width, seed=11)).to(dev).to(torch.bfloat16).view(E, m_max, width)
+    mm = torch.tensor(masked, device=dev, dtype=torch.int32)
+    q = torch.full((E, m_max, K), 0x55, device=dev, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    G = K // 128
+    if ue:
+        s = create_per_token_group_quant_fp8_output_scale((E, m_max, K), dev, 128, cm, al, ue)
+    elif cm:  # per-expert column-major (tokens contiguous), optionally padded to 4 tokens
+        pad = (m_max + 3) // 4 * 4 if al else m_max
+        s = torch.empty((E, G, pad), device=dev, dtype=torch.float32).transpose(-1, -2)[:, :m_max, :]
+    else:
+        s = torch.empty((E, m_max, G), device=dev, dtype=torch.float32)
+    s.fill_(7 if ue else 7.0)
+    sgl_per_token_group_quant_8bit(x, q, s, 128, 1e-10, fp8_min, fp8_max, ue, fuse, mm)
+    torch.cuda.synchronize()
+    qn, sn = u8(q).reshape(E, m_max, K), s.cpu().numpy()
+    for e in range(E):
+        m = masked[e]
+        if m:
+            q2, s2 = sglang_per_token_group_quant_fp8(x[e, :m].contiguous(), 128, fuse_silu_and_mul=fuse, column_major_scales=cm,
+                                                      scale_tma_aligned=al, scale_ue8m0=ue)
+            np.testing.assert_array_equal(qn[e, :m], u8(q2).reshape(m, K))
+            np.testing.assert_array_equal(sn[e, :m].view(np.uint32), s2.cpu().numpy().view(np.uint32))
+        assert np.all(qn[e, m:] == 0x55)
+        if not ue:
+            assert np.all(sn[e, m:] == 7.0)
+
+
+def test_silu_and_mul_masked_post_quant_fwd(dev):
+    from sglang_amd.ep_moe_kernels import silu_and_mul_masked_post_quant_fwd
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    E, m_max, K = 3, 130, 256
+    masked = torch.tensor([130, 0, 65], device=dev, dtype=torch.int32)
+    x = (torch.randn((E, m_max, 2 * K), device=dev) * 2).to(torch.bfloat16)
+    out = torch.zeros((E, m_max, K), device=dev, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    sc = torch.zeros((E, m_max, K // 128), device=dev, dtype=torch.float32)
+    silu_and_mul_masked_post_quant_fwd(x, out, sc, 128, masked)
+    for e, m in enumerate(masked.tolist()):
+        if m:
+            q2, s2 = sglang_per_token_group_quant_fp8(x[e, :m].contiguous(), 128, fuse_silu_and_mul=True)
+            np.testing.assert_array_equal(u8(out).reshape(E, m_max, K)[e, :m], u8(q2).reshape(m, K))
+            assert torch.equal(sc[e, :m], s2)
+        assert torch.all(sc[e, m:] == 0)
