@@ -185,6 +185,21 @@ int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t
 int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,
                         int64_t stride_topk, int64_t out_stride_token, float scale, int dtype, void* stream);
 
+/*
+ * Grouped top-k routing with a selection bias (DeepSeek-V3 style gate).
+ * Replaces torch.ops.sgl_kernel.moe_fused_gate (sgl-kernel/python/sgl_kernel/moe.py:105-137,
+ *   sgl-kernel/csrc/moe/moe_fused_gate.cu:52-257, schema common_extension.cc:240-244).
+ * input [num_rows, num_experts] and bias [num_experts] of `dtype`; topk_weights float32 [num_rows, topk];
+ * topk_ids int32 [num_rows, topk].  num_experts a power of two, divisible by num_expert_group,
+ * num_experts / num_expert_group <= 32, num_expert_group <= 64.  The last num_fused_shared_experts entries of a
+ * row are the shared experts (ids num_experts + i, weight sum / routed_scaling_factor); weights are renormalised
+ * to sum 1 and, if apply_routed_scaling_factor_on_output, multiplied by routed_scaling_factor.
+ */
+int fp8k_moe_fused_gate(const void* input, const void* bias, float* topk_weights, int32_t* topk_ids, int64_t num_rows,
+                        int64_t num_experts, int64_t num_expert_group, int64_t topk_group, int64_t topk,
+                        int64_t num_fused_shared_experts, double routed_scaling_factor,
+                        int apply_routed_scaling_factor_on_output, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -399,6 +399,49 @@ def biased_grouped_topk(logits, bias, num_expert_group, topk_group, topk, renorm
     return w.astype(np.float32), ids.astype(np.int32)
 
 
+def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, num_fused_shared_experts=0,
+                   routed_scaling_factor=0.0, apply_routed_scaling_factor_on_output=False, in_dtype="f32"):
+    """Reference: moe_fused_gate_impl, sgl-kernel/csrc/moe/moe_fused_gate.cu:52-257, followed step by step
+    (pure-Python loops: small cases only).  Arithmetic happens in the input type T: T(sigmoid), T(score + bias),
+    T(top1 + top2) per group; the weakest group is dropped repeatedly (ties: the higher group goes), then the best
+    remaining expert is taken repeatedly (ties: the lower expert wins).  x [rows, E] and bias [E] hold values of
+    `in_dtype` ("f32" or "bf16").  Returns (weights f32 [rows, topk], ids int32 [rows, topk])."""
+    rnd = to_bf16 if in_dtype == "bf16" else (lambda a: np.asarray(a, np.float32))
+    x = np.asarray(x, np.float32)
+    bias = np.asarray(bias, np.float32)
+    rows, E = x.shape
+    vpt = E // num_expert_group
+    take = topk - num_fused_shared_experts
+    out_w = np.zeros((rows, topk), np.float32)
+    out_i = np.zeros((rows, topk), np.int32)
+    with np.errstate(over="ignore"):
+        score = rnd((np.float32(1) / (np.float32(1) + np.exp(-x).astype(np.float32))).astype(np.float32))
+    choice_all = rnd((score + bias[None, :]).astype(np.float32))
+    for r in range(rows):
+        choice = choice_all[r].copy().reshape(num_expert_group, vpt)
+        for _ in range(num_expert_group - topk_group):
+            srt = -np.sort(-choice, axis=1)
+            sums = rnd((srt[:, 0] + srt[:, 1]).astype(np.float32)) if vpt > 1 else srt[:, 0]
+            worst = max(g for g in range(num_expert_group) if sums[g] == sums.min())
+            choice[worst, :] = np.inf
+        flat = np.where(np.isinf(choice) & (choice > 0), -np.inf, choice).reshape(-1)
+        wsum = np.float32(0)
+        for k in range(take):
+            e = int(np.argmax(flat))  # first maximum = lowest index
+            out_i[r, k] = e
+            out_w[r, k] = score[r, e]
+            wsum = np.float32(wsum + score[r, e])
+            flat[e] = -np.inf
+        for i in range(num_fused_shared_experts):
+            out_i[r, take + i] = E + i
+            out_w[r, take + i] = np.float32(np.float64(wsum) / routed_scaling_factor)
+        w = (out_w[r] / wsum).astype(np.float32)
+        if apply_routed_scaling_factor_on_output:
+            w = (w.astype(np.float64) * routed_scaling_factor).astype(np.float32)
+        out_w[r] = w
+    return out_w, out_i
+
+
 # --------------------------------------------------------------------------
 # a.8 + pipeline: block-FP8 fused MoE
 # --------------------------------------------------------------------------

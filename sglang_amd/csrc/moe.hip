@@ -365,3 +365,212 @@ extern "C" int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int
 #undef FP8K_SR
   return check_launch("moe_sum_reduce");
 }
+
+// ------------------------------------------------------------------------------------------------
+// moe_fused_gate: grouped top-k routing with a selection bias (DeepSeek-V3 style), one token per sub-group of
+// TPR = num_expert_group lanes, VPT = experts / groups values per lane (a lane holds one whole expert group).
+//   score  = T(sigmoid(x));  choice = T(score + bias)                       (arithmetic in the input type T)
+//   group weight = T(top1 + top2 of choice inside the group); the groups with the smallest weight are dropped
+//   one at a time until topk_group remain (ties: the higher group goes), then the topk best choices among the
+//   remaining groups are taken one at a time (ties: the lower expert wins).  Weights are the un-biased scores,
+//   renormalised to sum 1 (shared experts, if any, are appended with weight sum / routed_scaling_factor before
+//   the renormalisation), optionally times routed_scaling_factor.
+// ------------------------------------------------------------------------------------------------
+template <int DT>
+__device__ __forceinline__ float gate_load(const void* p, int64_t i) {
+  if (DT == FP8K_F32) return ((const float*)p)[i];
+  if (DT == FP8K_BF16) return __uint_as_float((uint32_t)((const u16*)p)[i] << 16);
+  return f16_bits_to_f32(((const u16*)p)[i]);
+}
+
+template <int DT, int VPT>
+__global__ __launch_bounds__(256) void moe_fused_gate_kernel(const void* __restrict__ input, const void* __restrict__ bias,
+                                                             float* __restrict__ out_w, int32_t* __restrict__ out_i,
+                                                             int64_t num_rows, int tpr, int topk_group, int topk,
+                                                             int num_shared, double rsf, int scale_output) {
+  const int lane_in_row = threadIdx.x % tpr;
+  const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) / tpr;
+  const bool live = row < num_rows;            // dead sub-groups run along (shuffles stay inside a sub-group)
+  const int first = lane_in_row * VPT;
+  const int experts = tpr * VPT;
+  const float kCleared = __builtin_inff();
+
+  float score[VPT], choice[VPT];
+  {
+    float xin[VPT], bin[VPT];
+    constexpr int kPer16 = DT == FP8K_F32 ? 4 : 8;  // elements per 16-byte load
+    if constexpr (VPT % kPer16 == 0) {
+      // a lane's VPT values are contiguous: 16-byte loads (rows and the lane's offset are multiples of VPT elements)
+#pragma unroll
+      for (int c = 0; c < VPT / kPer16; ++c) {
+        const int64_t at = (live ? row * experts : 0) + first + c * kPer16;
+        if constexpr (DT == FP8K_F32) {
+          const float4 a = *reinterpret_cast<const float4*>((const float*)input + at);
+          const float4 b = *reinterpret_cast<const float4*>((const float*)bias + first + c * 4);
+          xin[c * 4] = a.x; xin[c * 4 + 1] = a.y; xin[c * 4 + 2] = a.z; xin[c * 4 + 3] = a.w;
+          bin[c * 4] = b.x; bin[c * 4 + 1] = b.y; bin[c * 4 + 2] = b.z; bin[c * 4 + 3] = b.w;
+        } else {
+          load8<DT>(input, at, *reinterpret_cast<float(*)[8]>(&xin[c * 8]));
+          load8<DT>(bias, first + c * 8, *reinterpret_cast<float(*)[8]>(&bin[c * 8]));
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) {
+        xin[i] = live ? gate_load<DT>(input, row * experts + first + i) : 0.f;
+        bin[i] = gate_load<DT>(bias, first + i);
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      score[i] = round_to<DT>(1.0f / (1.0f + expf(-xin[i])));
+      choice[i] = round_to<DT>(score[i] + bin[i]);
+    }
+  }
+
+  // drop the weakest groups: a group's weight does not change while other groups are dropped
+  {
+    float m1 = -__builtin_inff(), m2 = -__builtin_inff();
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      const float v = choice[i];
+      if (v > m1) { m2 = m1; m1 = v; }
+      else if (v > m2) m2 = v;
+    }
+    const float gsum = VPT > 1 ? round_to<DT>(m1 + m2) : m1;
+    bool dropped = false;
+    for (int k = 0; k < tpr - topk_group; ++k) {
+      float sum = dropped ? kCleared : gsum;
+      int grp = lane_in_row;
+      for (int mask = tpr >> 1; mask > 0; mask >>= 1) {
+        const float osum = __shfl_xor(sum, mask, tpr);
+        const int ogrp = __shfl_xor(grp, mask, tpr);
+        if (sum > osum || (osum == sum && ogrp > grp)) { sum = osum; grp = ogrp; }
+      }
+      dropped = dropped || lane_in_row == grp;
+    }
+    if (dropped) {
+#pragma unroll
+      for (int i = 0; i < VPT; ++i) choice[i] = kCleared;
+    }
+  }
+
+  // pick k is kept by lane k % tpr of the row in slot k / tpr, so that the row's lanes write their entries
+  // side by side once the normaliser is known
+  constexpr int kSlots = 4;
+  float keep_w[kSlots];
+  int keep_i[kSlots];
+#pragma unroll
+  for (int j = 0; j < kSlots; ++j) { keep_w[j] = 0.f; keep_i[j] = 0; }
+  const int take = topk - num_shared;
+  float wsum = 0.f;
+  for (int k = 0; k < take; ++k) {
+    // local argmax as a tree (the lower index wins ties, as a left-to-right scan would have it)
+    float tv[VPT];
+    int ti[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) { tv[i] = choice[i]; ti[i] = first + i; }
+#pragma unroll
+    for (int stride = 1; stride < VPT; stride *= 2) {
+#pragma unroll
+      for (int i = 0; i + stride < VPT; i += 2 * stride) {
+        if (tv[i + stride] > tv[i]) { tv[i] = tv[i + stride]; ti[i] = ti[i + stride]; }
+      }
+    }
+    float best = tv[0];
+    int idx = ti[0];
+    if (choice[0] == kCleared) { best = -__builtin_inff(); idx = first; }
+    for (int mask = tpr >> 1; mask > 0; mask >>= 1) {
+      const float obest = __shfl_xor(best, mask, tpr);
+      const int oidx = __shfl_xor(idx, mask, tpr);
+      if (obest > best || (obest == best && oidx < idx)) { best = obest; idx = oidx; }
+    }
+    const int owner = idx / VPT, slot = idx - owner * VPT;
+    float w = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+      if (i == slot) {
+        w = score[i];
+        if (lane_in_row == owner) choice[i] = -__builtin_inff();
+      }
+    }
+    w = __shfl(w, owner, tpr);
+    wsum += w;
+    const bool mine = lane_in_row == k % tpr;
+    const int slot_k = k / tpr;
+#pragma unroll
+    for (int j = 0; j < kSlots; ++j) {
+      if (mine && j == slot_k) { keep_w[j] = w; keep_i[j] = idx; }
+    }
+  }
+  if (!live) return;
+#pragma unroll
+  for (int j = 0; j < kSlots; ++j) {
+    const int k = j * tpr + lane_in_row;
+    float w = keep_w[j];
+    int id = keep_i[j];
+    if (k >= take) {  // shared experts follow the routed ones
+      w = (float)((double)wsum / rsf);
+      id = experts + (k - take);
+    }
+    if (k < topk) {
+      w = w / wsum;
+      if (scale_output) w = (float)((double)w * rsf);
+      out_w[row * topk + k] = w;
+      out_i[row * topk + k] = id;
+    }
+  }
+}
+
+extern "C" int fp8k_moe_fused_gate(const void* input, const void* bias, float* topk_weights, int32_t* topk_ids,
+                                   int64_t num_rows, int64_t num_experts, int64_t num_expert_group, int64_t topk_group,
+                                   int64_t topk, int64_t num_fused_shared_experts, double routed_scaling_factor,
+                                   int apply_routed_scaling_factor_on_output, int dtype, void* stream) {
+  clear_error();
+  const char* op = "moe_fused_gate";
+  FP8K_REQUIRE(num_rows >= 0 && num_experts > 0 && num_expert_group > 0, "%s: bad shape", op);
+  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "%s: bad dtype %d", op, dtype);
+  FP8K_REQUIRE((num_experts & (num_experts - 1)) == 0, "%s: num_experts must be a power of 2, but got %lld", op,
+               (long long)num_experts);
+  FP8K_REQUIRE(num_experts % num_expert_group == 0, "%s: num_experts must be divisible by num_expert_group, but got %lld / %lld",
+               op, (long long)num_experts, (long long)num_expert_group);
+  const int64_t vpt = num_experts / num_expert_group;
+  FP8K_REQUIRE(vpt <= 32, "%s: Per group experts: num_experts / num_expert_group = (%lld) exceeds the maximum supported (32)",
+               op, (long long)vpt);
+  FP8K_REQUIRE(num_expert_group <= 64, "%s: at most 64 expert groups (got %lld)", op, (long long)num_expert_group);
+  FP8K_REQUIRE(topk_group >= 1 && topk_group <= num_expert_group, "%s: topk_group out of range", op);
+  FP8K_REQUIRE(num_fused_shared_experts >= 0 && topk > num_fused_shared_experts &&
+                   topk - num_fused_shared_experts <= topk_group * vpt,
+               "%s: topk (%lld) does not fit the experts of the selected groups", op, (long long)topk);
+  FP8K_REQUIRE(topk <= 4 * num_expert_group, "%s: topk (%lld) larger than 4 x num_expert_group is not built", op, (long long)topk);
+  FP8K_REQUIRE(num_fused_shared_experts == 0 || routed_scaling_factor != 0.0,
+               "%s: shared experts need a non-zero routed_scaling_factor", op);
+  if (num_rows == 0) return FP8K_OK;
+  FP8K_REQUIRE(input && bias && topk_weights && topk_ids, "%s: null pointer", op);
+  FP8K_REQUIRE(num_rows * num_experts < (1LL << 40), "%s: input too large", op);
+  FP8K_REQUIRE(aligned(input, 16) && aligned(bias, 16), "%s: input and bias must be 16-byte aligned", op);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t lanes = num_rows * num_expert_group;
+  const dim3 grid((unsigned)((lanes + 255) / 256)), block(256);
+#define FP8K_GATE2(DT, V)                                                                                              \
+  hipLaunchKernelGGL((moe_fused_gate_kernel<DT, V>), grid, block, 0, st, input, bias, topk_weights, topk_ids, num_rows, \
+                     (int)num_expert_group, (int)topk_group, (int)topk, (int)num_fused_shared_experts,                  \
+                     routed_scaling_factor, apply_routed_scaling_factor_on_output)
+#define FP8K_GATE(DT)                \
+  switch (vpt) {                     \
+    case 1: FP8K_GATE2(DT, 1); break;   \
+    case 2: FP8K_GATE2(DT, 2); break;   \
+    case 4: FP8K_GATE2(DT, 4); break;   \
+    case 8: FP8K_GATE2(DT, 8); break;   \
+    case 16: FP8K_GATE2(DT, 16); break; \
+    default: FP8K_GATE2(DT, 32); break; \
+  }
+  switch (dtype) {
+    case FP8K_BF16: FP8K_GATE(FP8K_BF16); break;
+    case FP8K_F16: FP8K_GATE(FP8K_F16); break;
+    default: FP8K_GATE(FP8K_F32); break;
+  }
+#undef FP8K_GATE
+#undef FP8K_GATE2
+  return check_launch(op);
+}

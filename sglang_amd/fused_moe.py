@@ -253,3 +253,37 @@ def biased_grouped_topk_impl(
         if apply_routed_scaling_factor_on_output:
             topk_weights = topk_weights * routed_scaling_factor
     return topk_weights.to(torch.float32), topk_ids.to(torch.int32)
+
+
+def biased_grouped_topk(
+    hidden_states: torch.Tensor,
+    gating_output: torch.Tensor,
+    correction_bias: torch.Tensor,
+    topk: int,
+    renormalize: bool,
+    num_expert_group: Optional[int] = None,
+    topk_group: Optional[int] = None,
+    num_fused_shared_experts: int = 0,
+    routed_scaling_factor: Optional[float] = None,
+    apply_routed_scaling_factor_on_output: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: biased_grouped_topk_gpu, python/sglang/srt/layers/moe/topk.py:762-850: the fused gate kernel
+    where its shape limits hold (power-of-two expert count, at most 32 experts per group, renormalised weights),
+    the torch restatement otherwise."""
+    experts = gating_output.shape[1]
+    fits = (
+        renormalize and num_expert_group and topk_group and experts & (experts - 1) == 0
+        and experts % num_expert_group == 0 and experts // num_expert_group <= 32 and num_expert_group <= 64
+    )
+    if fits:
+        return _ops.moe_fused_gate(
+            gating_output.contiguous(), correction_bias.to(gating_output.dtype).contiguous(), num_expert_group, topk_group,
+            topk, num_fused_shared_experts, routed_scaling_factor if routed_scaling_factor is not None else 0.0,
+            apply_routed_scaling_factor_on_output,
+        )
+    if num_fused_shared_experts:
+        raise RuntimeError("biased_grouped_topk: shared-expert fusion needs the fused gate kernel's shapes")
+    return biased_grouped_topk_impl(
+        hidden_states, gating_output, correction_bias, topk, renormalize, num_expert_group, topk_group,
+        routed_scaling_factor, apply_routed_scaling_factor_on_output,
+    )

@@ -456,3 +456,38 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
             stream_ptr(A.device),
         )
     )
+
+
+def moe_fused_gate(
+    input_tensor: torch.Tensor,
+    bias: torch.Tensor,
+    num_expert_group: int,
+    topk_group: int,
+    topk: int,
+    num_fused_shared_experts: int = 0,
+    routed_scaling_factor: float = 0,
+    apply_routed_scaling_factor_on_output: bool = False,
+):
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:105-137 (csrc/moe/moe_fused_gate.cu).  Hierarchical top-k:
+    groups are ranked by the sum of their two best biased sigmoid scores, the best `topk_group` groups stay, the
+    `topk` best experts among them are taken; returns (weights float32 [rows, topk], ids int32 [rows, topk]).
+    `topk` includes `num_fused_shared_experts` trailing shared-expert entries."""
+    require_cuda(input_tensor, bias)
+    if input_tensor.dtype != bias.dtype:
+        raise RuntimeError("input and bias should have the same dtype")
+    if input_tensor.dim() != 2 or bias.dim() != 1 or bias.shape[0] != input_tensor.shape[1]:
+        raise RuntimeError("moe_fused_gate: input [num_rows, num_experts], bias [num_experts]")
+    if not (input_tensor.is_contiguous() and bias.is_contiguous()):
+        raise RuntimeError("moe_fused_gate: input and bias must be contiguous")
+    rows, experts = input_tensor.shape
+    output = torch.empty((rows, topk), device=input_tensor.device, dtype=torch.float32)
+    indices = torch.empty((rows, topk), device=input_tensor.device, dtype=torch.int32)
+    check(
+        lib.fp8k_moe_fused_gate(
+            input_tensor.data_ptr(), bias.data_ptr(), output.data_ptr(), indices.data_ptr(), rows, experts,
+            int(num_expert_group), int(topk_group), int(topk), int(num_fused_shared_experts),
+            float(routed_scaling_factor), 1 if apply_routed_scaling_factor_on_output else 0,
+            dtype_code(input_tensor.dtype), stream_ptr(input_tensor.device),
+        )
+    )
+    return output, indices

@@ -318,3 +318,64 @@ def test_fused_experts_deepseek_dims_few_tokens(dev):
     # routing agrees with the numpy restatement (as sets; top-k order is unspecified)
     w_ref, ids_ref = O.biased_grouped_topk(logits.cpu().numpy(), bias.cpu().numpy(), 8, 4, topk)
     np.testing.assert_array_equal(np.sort(ids_np, 1), np.sort(ids_ref, 1))
+
+
+@pytest.mark.parametrize("rows", [1, 7, 64, 1000])
+@pytest.mark.parametrize("params", [(128, 4, 2, 4), (256, 8, 4, 8), (512, 16, 8, 16), (64, 8, 3, 6)])
+@pytest.mark.parametrize("shared,scale_out", [(0, False), (1, True), (2, False)])
+def test_moe_fused_gate_vs_oracle(dev, rows, params, shared, scale_out):
+    """Reference: sgl-kernel/tests/test_moe_fused_gate.py:8-101 (float32 inputs, the DeepSeek-V3 tuple among them).
+    Ids must equal the oracle's in order (same tie rules), weights to 1e-5 (expf may differ in the last bit)."""
+    from sglang_amd.sgl_kernel import moe_fused_gate
+
+    E, G, tg, topk = params
+    g = torch.Generator().manual_seed(rows * 7 + E)
+    x = torch.rand((rows, E), generator=g)
+    bias = torch.rand((E,), generator=g)
+    w, ids = moe_fused_gate(x.to(dev), bias.to(dev), G, tg, topk + shared, shared, 2.5, scale_out)
+    torch.cuda.synchronize()
+    w_ref, ids_ref = O.moe_fused_gate(x.numpy(), bias.numpy(), G, tg, topk + shared, shared, 2.5, scale_out)
+    assert w.dtype == torch.float32 and ids.dtype == torch.int32 and tuple(w.shape) == (rows, topk + shared)
+    got_i, got_w = ids.cpu().numpy(), w.cpu().numpy()
+    same = (got_i == ids_ref).all(axis=1)
+    # a last-bit difference in expf can swap two near-equal choices: such rows must still hold the same set
+    for r in np.nonzero(~same)[0]:
+        assert sorted(got_i[r].tolist()) == sorted(ids_ref[r].tolist())
+    assert same.mean() >= 0.99
+    np.testing.assert_allclose(np.sort(got_w, axis=1), np.sort(w_ref, axis=1), rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype,name", [(torch.bfloat16, "bf16")])
+def test_moe_fused_gate_bf16_and_ties(dev, dtype, name):
+    """16-bit inputs make ties common (the arithmetic is done in the input type): the tie rules must hold."""
+    from sglang_amd.sgl_kernel import moe_fused_gate
+
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn((300, 256), generator=g).to(dtype)
+    bias = (torch.randn((256,), generator=g) * 0.1).to(dtype)
+    w, ids = moe_fused_gate(x.to(dev), bias.to(dev), 8, 4, 8)
+    w_ref, ids_ref = O.moe_fused_gate(x.float().numpy(), bias.float().numpy(), 8, 4, 8, in_dtype=name)
+    got_i = ids.cpu().numpy()
+    same = (got_i == ids_ref).all(axis=1)
+    for r in np.nonzero(~same)[0]:
+        assert sorted(got_i[r].tolist()) == sorted(ids_ref[r].tolist())
+    assert same.mean() >= 0.97
+    np.testing.assert_allclose(np.sort(w.cpu().numpy(), axis=1), np.sort(w_ref, axis=1), rtol=2e-2, atol=1e-3)
+    # all-equal inputs: groups 7..4 are dropped, experts 0..7 win
+    z = torch.zeros((3, 256), device=dev, dtype=dtype)
+    w0, i0 = moe_fused_gate(z, torch.zeros((256,), device=dev, dtype=dtype), 8, 4, 8)
+    assert i0.cpu().tolist() == [list(range(8))] * 3
+    assert torch.allclose(w0, torch.full_like(w0, 0.125))
+
+
+def test_moe_fused_gate_errors(dev):
+    from sglang_amd.sgl_kernel import moe_fused_gate
+
+    x = torch.zeros((4, 96), device=dev)
+    with pytest.raises(RuntimeError, match="power of 2"):
+        moe_fused_gate(x, torch.zeros((96,), device=dev), 4, 2, 4)
+    x = torch.zeros((4, 256), device=dev)
+    with pytest.raises(RuntimeError, match="exceeds the maximum supported"):
+        moe_fused_gate(x, torch.zeros((256,), device=dev), 4, 2, 4)
+    with pytest.raises(RuntimeError, match="same dtype"):
+        moe_fused_gate(x, torch.zeros((256,), device=dev, dtype=torch.bfloat16), 8, 4, 8)

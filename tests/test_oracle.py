@@ -281,3 +281,46 @@ def test_grouped_topk_properties():
     sm = gm.unsqueeze(-1).expand(50, 8, 32).reshape(50, 256)
     ti = scb.masked_fill(~sm.bool(), float("-inf")).topk(8, dim=-1)[1]
     assert np.array_equal(np.sort(ids, axis=1), np.sort(ti.numpy(), axis=1))
+
+
+@pytest.mark.parametrize("params", [(128, 4, 2, 4), (256, 8, 4, 8), (512, 16, 8, 16)])
+@pytest.mark.parametrize("shared", [0, 1, 2])
+@pytest.mark.parametrize("scale_out", [False, True])
+def test_moe_fused_gate_oracle_matches_grouped_topk(params, shared, scale_out):
+    """The check of the reference's own test (sgl-kernel/tests/test_moe_fused_gate.py:25-101): on float32 inputs
+    the fused gate must pick the same expert sets as biased_grouped_topk (here: a torch restatement built from
+    library sigmoid / topk / scatter calls) and give the same weights to 1e-2."""
+    E, G, tg, topk = params
+    rows = 33
+    g = torch.Generator().manual_seed(E + shared)
+    x = torch.rand((rows, E), generator=g)
+    bias = torch.rand((E,), generator=g)
+    w, ids = O.moe_fused_gate(x.numpy(), bias.numpy(), G, tg, topk + shared, shared, 2.5, scale_out)
+    sc = torch.sigmoid(x)
+    scb = sc + bias
+    gs = scb.view(rows, G, E // G).topk(2, dim=-1)[0].sum(-1)
+    gi = gs.topk(tg, dim=-1)[1]
+    gm = torch.zeros_like(gs).scatter_(1, gi, 1)
+    sm = gm.unsqueeze(-1).expand(rows, G, E // G).reshape(rows, E)
+    ti = scb.masked_fill(~sm.bool(), float("-inf")).topk(topk, dim=-1)[1]
+    tw = sc.gather(1, ti)
+    routed_sum = tw.sum(-1, keepdim=True)  # topk.py:726-731: the shared entries stay out of the normaliser
+    if shared:
+        tw = torch.cat([tw] + [routed_sum / 2.5] * shared, dim=1)
+        assert np.array_equal(ids[:, topk:], np.tile(np.arange(E, E + shared, dtype=np.int32), (rows, 1)))
+    tw = tw / routed_sum
+    if scale_out:
+        tw = tw * 2.5
+    assert np.array_equal(np.sort(ids[:, :topk], axis=1), np.sort(ti.numpy(), axis=1))
+    np.testing.assert_allclose(np.sort(w, axis=1), np.sort(tw.numpy(), axis=1), rtol=1e-2, atol=1e-3)
+    # routed weights sum to 1, every shared expert carries 1 / routed_scaling_factor (times the factor if applied)
+    np.testing.assert_allclose(w.sum(-1), (1.0 + shared / 2.5) * (2.5 if scale_out else 1.0), rtol=1e-5)
+
+
+def test_moe_fused_gate_oracle_tie_rules():
+    """Equal choices: the lower expert wins a place; equal group weights: the higher group is dropped first."""
+    x = np.zeros((1, 16), np.float32)
+    bias = np.zeros((16,), np.float32)
+    w, ids = O.moe_fused_gate(x, bias, 4, 2, 3)
+    assert ids[0].tolist() == [0, 1, 2]          # groups 3 and 2 dropped, then experts 0, 1, 2
+    np.testing.assert_allclose(w[0], 1.0 / 3.0, rtol=1e-6)
