@@ -296,6 +296,20 @@ def write_table(torch, dev, path):
             lines.append("| %d | %d | %d | %.1f | %.1f | %.1f | %.0f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100,
                                                                           gemm_bytes(M, N, K) / us / 1e3))
         del ws
+    lines += ["", "## configs[2] shapes at M=4096 with UE8M0 scales (packed activation exponents, power-of-two weight scales:",
+              "## the matrix core applies the block scales itself)", "",
+              "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s |", "|---|---|---|---|---|---|"]
+    for (N, K) in DSV3_NK:
+        nbuf, M = 3, 4096
+        ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
+        ws = [(w, torch.exp2(torch.ceil(torch.log2(sc)))) for w, sc in ws]
+        qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True,
+                                               scale_tma_aligned=True, scale_ue8m0=True) for s in range(nbuf)]
+        us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
+                                                                ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
+        tf = 2.0 * M * N * K / us / 1e6
+        lines.append("| %d | %d | %d | %.1f | %.1f | %.1f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100))
+        del ws
     lines += ["", "## configs[3] per-token fp8_scaled_mm, Llama-3-8B shapes", "",
               "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s |", "|---|---|---|---|---|---|"]
     for (N, K) in LLAMA_NK:

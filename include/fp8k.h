@@ -114,6 +114,21 @@ int fp8k_block_gemm(const void* A, const void* B, const float* As, const float* 
                     int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
                     int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
                     int64_t workspace_bytes, void* stream);
+
+/*
+ * The same product with power-of-two scales that the matrix core applies itself (no float promote per K block):
+ * As_packed int32 words of four UE8M0 exponent bytes, as fp8k_group_quant writes them with FP8K_SCALE_UE8M0_PACKED
+ * (row m, K blocks 4j..4j+3 in the word at As_packed[m*as_stride_m + j*as_stride_w]); Bs float32, every value a power of
+ * two (UE8M0-format checkpoints, or weights requantised with power-of-two scales).
+ * Counterpart in the reference: the DeepGEMM path with DEEPGEMM_SCALE_UE8M0
+ *   (python/sglang/srt/layers/quantization/fp8_utils.py:229-268, deep_gemm_wrapper/entrypoint.py:70-88).
+ * Built for M > 128 and K % 128 == 0 (other shapes: expand the exponents to floats and call fp8k_block_gemm).
+ * A Bs value that is not a power of two is used as if its mantissa were zero.
+ */
+int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t* As_packed, const float* Bs, void* C, int64_t M,
+                          int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_w,
+                          int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
+                          int64_t workspace_bytes, void* stream);
 int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*

@@ -189,6 +189,55 @@ extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, co
                                 : launch<kModeBlock, FP8K_F16, FP8K_F32>(a, pl, st);
 }
 
+extern "C" int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t* As_packed, const float* Bs, void* C,
+                                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m,
+                                     int64_t as_stride_w, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc,
+                                     int out_dtype, void* workspace, int64_t workspace_bytes_given, void* stream) {
+  clear_error();
+  const char* op = "block_gemm_ue8m0";
+  int rc = common_checks(op, A, B, C, M, N, K, lda, ldb, ldc, out_dtype);
+  if (rc) return rc;
+  if (M == 0 || N == 0) return FP8K_OK;
+  FP8K_REQUIRE(K > 0, "%s: K must be positive", op);
+  FP8K_REQUIRE(As_packed && Bs, "%s: null scale pointer", op);
+  FP8K_REQUIRE(as_stride_m >= 0 && as_stride_w >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0, "%s: negative scale stride", op);
+  const Plan pl = make_plan(M, N, K);
+  // the matrix core applies the scales only in the 256x256 tile kernel; smaller problems take the float-scale
+  // entry point with the exponents expanded to floats
+  FP8K_REQUIRE(pl.kind == 1, "%s: built for M > 128 with K a multiple of 128 (got M=%lld, K=%lld); expand the scales "
+               "and call fp8k_block_gemm", op, (long long)M, (long long)K);
+  const int64_t need = pl.ws_bytes;
+  if (need > 0 && (!workspace || workspace_bytes_given < need))
+    return fail(FP8K_ERR_WORKSPACE, "%s: workspace of %lld bytes required, %lld given", op, (long long)need,
+                (long long)(workspace ? workspace_bytes_given : 0));
+  GemmArgs a{};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.sx = reinterpret_cast<const float*>(As_packed); a.sw = Bs;
+  a.bias = nullptr; a.C = C; a.partial = (float*)workspace;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.sx_m = as_stride_m; a.sx_k = as_stride_w; a.sw_n = bs_stride_n; a.sw_k = bs_stride_k;
+  a.tiles_m = (a.M + kTileM - 1) / kTileM;
+  a.tiles_n = (a.N + kTileN - 1) / kTileN;
+  a.splits = pl.splits;
+  a.kb_per_split = pl.kb_per_split;
+  a.tail_first = pl.tail_first;
+  hipStream_t st = (hipStream_t)stream;
+  const int ntiles = a.tiles_m * a.tiles_n;
+  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
+  if (out_dtype == FP8K_BF16)
+    hipLaunchKernelGGL((gemm_tile256_kernel<kModeScaled, FP8K_BF16, FP8K_F32>), dim3(nwg), dim3(512), 0, st, a);
+  else
+    hipLaunchKernelGGL((gemm_tile256_kernel<kModeScaled, FP8K_F16, FP8K_F32>), dim3(nwg), dim3(512), 0, st, a);
+  rc = check_launch(op);
+  if (rc || pl.tail_first == ntiles) return rc;
+  if (out_dtype == FP8K_BF16)
+    hipLaunchKernelGGL((tile_reduce_kernel<kModeScaled, FP8K_BF16, FP8K_F32>), dim3((unsigned)((ntiles - pl.tail_first) * 64)),
+                       dim3(256), 0, st, a);
+  else
+    hipLaunchKernelGGL((tile_reduce_kernel<kModeScaled, FP8K_F16, FP8K_F32>), dim3((unsigned)((ntiles - pl.tail_first) * 64)),
+                       dim3(256), 0, st, a);
+  return check_launch("tile_reduce");
+}
+
 extern "C" int fp8k_scaled_mm(const void* A, const void* B, const float* sa, const float* sb, const void* bias, void* C,
                               int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int out_dtype,
                               int bias_dtype, void* workspace, int64_t workspace_bytes_given, void* stream) {

@@ -39,7 +39,9 @@ struct GemmArgs {
   int64_t sw_expert_stride;     // floats between experts in sw
 };
 
-enum { kModeBlock = 0, kModeRow = 1 };
+// kModeScaled: block mode with power-of-two scales applied by the matrix core itself (activation scales as packed
+// UE8M0 bytes, weight scales as float powers of two): no float promote, one accumulator over the whole K range
+enum { kModeBlock = 0, kModeRow = 1, kModeScaled = 2 };
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70); }  // vmcnt(0)
@@ -47,6 +49,11 @@ __device__ __forceinline__ void wait_vm0() { __builtin_amdgcn_s_waitcnt(0x0F70);
 __device__ __forceinline__ v16f mfma_32x32x64(v8i a, v8i b, v16f c) {
   // cbsz = blgp = 0: both operands e4m3; scale operands 0 select the unscaled instruction form
   return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
+}
+// the same with block scales: byte 0 of scale_a / scale_b is the E8M0 exponent (value 2^(e-127)) of the 32 K
+// elements that this lane holds of its A row / B column
+__device__ __forceinline__ v16f mfma_32x32x64_scaled(v8i a, v8i b, v16f c, int scale_a, int scale_b) {
+  return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, scale_a, 0, scale_b);
 }
 
 template <int OUT_DT>
@@ -219,6 +226,11 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   const float* sx1 = p.sx + (int64_t)mrow1 * p.sx_m + (int64_t)kb_begin * p.sx_k;
   const int nb = min(n0 + wn * 128, p.N - 1) >> 7;
   const float* swp = p.sw + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
+  // scaled mode: sx points at int32 words of four UE8M0 bytes (K blocks 4j..4j+3 of a row), sx_k = word stride
+  const uint32_t* sq0p = reinterpret_cast<const uint32_t*>(p.sx) + (int64_t)mrow0 * p.sx_m;
+  const uint32_t* sq1p = reinterpret_cast<const uint32_t*>(p.sx) + (int64_t)mrow1 * p.sx_m;
+  int sq[2] = {127, 127}, sqw = 127;      // exponent bytes of the block the current MFMAs belong to
+  uint32_t q0n = 0, q1n = 0;              // words holding the next block's activation exponents
 
   v16f acc[4][2];
 #pragma unroll
@@ -260,6 +272,9 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       for (int r = 0; r < 16; ++r) z[r] = 0.f;
       tt = mfma_32x32x64(W[0], X[ms][0], z);
       tt = mfma_32x32x64(W[1], X[ms][1], tt);
+    } else if (MODE == kModeScaled) {
+      a = mfma_32x32x64_scaled(W[0], X[ms][0], a, sqw, sq[ms]);
+      a = mfma_32x32x64_scaled(W[1], X[ms][1], a, sqw, sq[ms]);
     } else {
       a = mfma_32x32x64(W[0], X[ms][0], a);
       a = mfma_32x32x64(W[1], X[ms][1], a);
@@ -280,6 +295,9 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
       for (int r = 8; r < 16; ++r) ap[r] = __builtin_fmaf(tp[r], s, ap[r]);
+    } else if (MODE == kModeScaled) {
+      a = mfma_32x32x64_scaled(W[0], X[ms][0], a, sqw, sq[ms]);
+      a = mfma_32x32x64_scaled(W[1], X[ms][1], a, sqw, sq[ms]);
     } else {
       a = mfma_32x32x64(W[0], X[ms][0], a);
       a = mfma_32x32x64(W[1], X[ms][1], a);
@@ -298,12 +316,23 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
   for (int i = 0; i < 8; ++i) L(i);
   if (MODE == kModeBlock) { sc[0] = sx0[0]; sc[1] = sx1[0]; const float sb = swp[0]; sc[0] *= sb; sc[1] *= sb; }
+  auto exponents = [&](uint32_t w0, uint32_t w1, float sb, int kb_abs) {  // -> sq, sqw for K block kb_abs
+    const int sh = (kb_abs & 3) * 8;
+    sq[0] = (int)(w0 >> sh);
+    sq[1] = (int)(w1 >> sh);
+    sqw = (int)(__float_as_uint(sb) >> 23);
+  };
+  if (MODE == kModeScaled) exponents(sq0p[(int64_t)(kb_begin >> 2) * p.sx_k], sq1p[(int64_t)(kb_begin >> 2) * p.sx_k], swp[0], kb_begin);
   wait_vm0();
   __syncthreads();
   cur_stage = 1; cur_kstep = 1;
 #pragma unroll
   for (int i = 0; i < 8; ++i) L(i);
   if (MODE == kModeBlock) { const int kn = min(1, nkb - 1); s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k]; }
+  if (MODE == kModeScaled) {
+    const int kn = min(1, nkb - 1);
+    q0n = sq0p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; q1n = sq1p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
+  }
   RX(smem, 0); RX(smem, 1); RW(WA, smem, 0); RW(WB, smem, 1);
   SB();
   G(WA, 0, acc[0][0], tq[0]); SB();
@@ -329,11 +358,16 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]); SB();
     RX(stn, 1); RW(WB, stn, 1); L(2); L(3); SB();
     if (MODE == kModeBlock) { scn[0] = s0n * sbn; scn[1] = s1n * sbn; }
+    if (MODE == kModeScaled) exponents(q0n, q1n, sbn, kb_begin + it + 1);  // the groups from here on are block it+1's
     GF(WA, 0, acc[0][0], tq[0], acc[3][1], tq[1], sc[1]); SB();
     if (MODE == kModeBlock) {
       sc[0] = scn[0]; sc[1] = scn[1];
       const int kn = min(it + 2, nkb - 1);
       s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
+    }
+    if (MODE == kModeScaled) {
+      const int kn = min(it + 2, nkb - 1);
+      q0n = sq0p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; q1n = sq1p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
     }
     L(4); L(5); SB();
     GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();

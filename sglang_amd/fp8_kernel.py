@@ -153,6 +153,11 @@ def w8a8_block_fp8_matmul(
 
     A e4m3fn [..., K]; B e4m3fn [N, K] contiguous; As float32 [..., ceil(K/bk)]; Bs float32
     [ceil(N/bn), ceil(K/bk)]; block_size must be [128, 128] on this path.
+
+    As may also be the packed UE8M0 tensor that the group quant returns with scale_ue8m0=True (int32
+    [M, ceil(K/128/4)]); Bs must then hold powers of two (a UE8M0-format checkpoint, or weights requantised that
+    way, fp8_utils.py:441-515 in the reference) and the matrix core applies both scales itself - the counterpart
+    of the reference's DeepGEMM path with DEEPGEMM_SCALE_UE8M0 (fp8_utils.py:229-268).
     """
     assert len(block_size) == 2
     block_n, block_k = block_size
@@ -160,7 +165,8 @@ def w8a8_block_fp8_matmul(
         raise RuntimeError("w8a8_block_fp8_matmul: only block_size [128, 128] is built on this path")
     assert A.shape[-1] == B.shape[-1]
     assert A.shape[:-1] == As.shape[:-1] and A.is_contiguous()
-    assert (A.shape[-1] + block_k - 1) // block_k == As.shape[-1]
+    packed = As.dtype == torch.int32
+    assert packed or (A.shape[-1] + block_k - 1) // block_k == As.shape[-1]
     assert B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
     N, K = B.shape
     assert (N + block_n - 1) // block_n == Bs.shape[0]
@@ -168,8 +174,12 @@ def w8a8_block_fp8_matmul(
     M = A.numel() // A.shape[-1]
     C_shape = A.shape[:-1] + (N,)
     A2 = A.reshape(M, K)
+    if packed:
+        if As.dim() != 2:
+            raise RuntimeError("w8a8_block_fp8_matmul: packed UE8M0 scales need a 2-D activation")
+        return _ops._block_gemm_nk_ue8m0(A2, B, As, Bs, output_dtype).reshape(C_shape)
     As2 = As.reshape(M, As.shape[-1])
     if As2.dtype != torch.float32 or Bs.dtype != torch.float32:
-        raise RuntimeError("w8a8_block_fp8_matmul: packed UE8M0 GEMM scales are not built on this path")
+        raise RuntimeError("w8a8_block_fp8_matmul: scales must be float32 (or packed int32 UE8M0 activation scales)")
     out = _ops._block_gemm_nk(A2, B, As2, Bs, output_dtype)
     return out.reshape(C_shape)

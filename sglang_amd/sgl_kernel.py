@@ -332,6 +332,46 @@ def _block_gemm_nk(A, B, As, Bs, out_dtype):
     return out
 
 
+def unpack_ue8m0_scales(packed: torch.Tensor, num_groups: int) -> torch.Tensor:
+    """int32 words of four UE8M0 exponent bytes [M, ceil(G/4)] -> float32 powers of two [M, G]."""
+    shifts = torch.arange(0, 32, 8, device=packed.device, dtype=torch.int32)
+    exps = (packed.unsqueeze(-1) >> shifts) & 0xFF
+    return (exps.reshape(packed.shape[0], -1)[:, :num_groups] << 23).contiguous().view(torch.float32)
+
+
+def _block_gemm_nk_ue8m0(A, B, As_packed, Bs, out_dtype):
+    """Block GEMM with packed UE8M0 activation scales (as the group quant writes them with scale_ue8m0=True) and
+    power-of-two float32 weight scales: for M > 128 the matrix core applies the scales itself
+    (include/fp8k.h: fp8k_block_gemm_ue8m0); smaller batches expand the exponents and take the float-scale kernels."""
+    require_cuda(A, B, As_packed, Bs)
+    if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
+        raise RuntimeError("A and B must be Float8_e4m3fn")
+    if As_packed.dtype != torch.int32 or Bs.dtype != torch.float32:
+        raise RuntimeError("packed activation scales must be int32, weight scales float32")
+    out_code = _out_code(out_dtype)
+    M, K = A.shape
+    N = B.shape[0]
+    G = (K + 127) // 128
+    if As_packed.shape[0] != M or As_packed.shape[1] != (G + 3) // 4:
+        raise RuntimeError("packed activation scales must be [M, ceil(K/128/4)]")
+    if M <= 128 or K % 128 != 0 or N % 4 != 0:
+        return _block_gemm_nk(A, B, unpack_ue8m0_scales(As_packed, G), Bs, out_dtype)
+    if (N * 2) % 16 != 0:
+        raise RuntimeError("out must be multiple of 16 bytes for memory alignment")
+    out = torch.empty((M, N), dtype=out_dtype, device=A.device)
+    ws_bytes = lib.fp8k_block_gemm_workspace_bytes(M, N, K)
+    ws = _workspace(A.device, ws_bytes)
+    check(
+        lib.fp8k_block_gemm_ue8m0(
+            A.data_ptr(), B.data_ptr(), As_packed.data_ptr(), Bs.data_ptr(), out.data_ptr(), M, N, K, A.stride(0),
+            B.stride(0) if N > 1 else K, As_packed.stride(0), As_packed.stride(1), Bs.stride(0), Bs.stride(1),
+            out.stride(0), out_code, ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0,
+            stream_ptr(A.device),
+        )
+    )
+    return out
+
+
 # --------------------------------------------------------------------------------------------
 # fused-MoE helpers
 # --------------------------------------------------------------------------------------------

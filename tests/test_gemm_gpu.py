@@ -240,3 +240,28 @@ def test_gemm_errors(dev):
                       torch.ones(255, device=dev))
     out = fp8_blockwise_scaled_mm(a[:0], b.t(), sa[:0], sb, torch.bfloat16)
     assert out.shape == (0, 256)
+
+
+@pytest.mark.parametrize("M,N,K", [(129, 256, 256), (300, 512, 1024), (1024, 4608, 1536), (2048, 1536, 7168), (64, 512, 512)])
+def test_block_gemm_ue8m0_hardware_scales(dev, M, N, K):
+    """UE8M0 path (reference: the DeepGEMM branch with DEEPGEMM_SCALE_UE8M0, fp8_utils.py:229-268): activations
+    quantised with power-of-two scales (packed bytes), weight scales rounded up to powers of two; the matrix core
+    applies both.  Checked against the oracle's block matmul on the very same (unpacked) scales, <= 1e-2, and
+    against this library's float-scale kernel on the unpacked scales."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.sgl_kernel import unpack_ue8m0_scales
+
+    x = O.make_activation(M, K, seed=M)
+    w = O.make_weight(N, K, seed=N)
+    wq, ws = O.block_quant_weight(w)
+    ws2 = O.ceil_to_ue8m0(ws)                     # power-of-two weight scales (the bytes stay as they are:
+    xt = torch.from_numpy(x).to(dev).to(torch.bfloat16)  # only the GEMM's use of the scales is under test)
+    xq, xs_packed = sglang_per_token_group_quant_fp8(xt, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    B, Bs = fp8_tensor(wq, dev), torch.from_numpy(ws2).to(dev)
+    c = w8a8_block_fp8_matmul(xq, B, xs_packed, Bs, [128, 128], torch.bfloat16)
+    xs = unpack_ue8m0_scales(xs_packed, K // 128)
+    c_float = w8a8_block_fp8_matmul(xq, B, xs, Bs, [128, 128], torch.bfloat16)
+    torch.cuda.synchronize()
+    ref = O.w8a8_block_fp8_matmul(xq.view(torch.uint8).cpu().numpy(), wq, xs.cpu().numpy(), ws2, acc=np.float64)
+    assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
+    assert _rel_err(c.float().cpu().numpy(), c_float.float().cpu().numpy()) <= REL_TOL
