@@ -4,7 +4,7 @@ reach.  There is a single backend, so the dispatcher always returns the same fun
 """
 from __future__ import annotations
 
-from typing import Callable, List, Optional
+from typing import Callable, List, Optional, Tuple
 
 import torch
 
@@ -90,3 +90,88 @@ def apply_fp8_linear(
     output = _ops.fp8_scaled_mm(qinput, weight, x_scale.reshape(-1), weight_scale.reshape(-1).to(torch.float32),
                                 out_dtype=input.dtype, bias=bias_arg)
     return output.view(*output_shape)
+
+
+# --------------------------------------------------------------------------------------------
+# weight-side transforms (run once, after loading; plain tensor ops on whatever device holds the weights)
+# --------------------------------------------------------------------------------------------
+
+_FP8_MAX = 448.0
+
+
+def input_to_float8(x: torch.Tensor, dtype: torch.dtype = fp8_dtype) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_utils.py:356-372 - one scale for the whole tensor: q = sat(x * 448/amax), returns
+    (q, amax/448 as a float32 scalar tensor); amax is floored at 1e-12."""
+    lo, hi = x.aminmax()
+    amax = torch.maximum(lo.abs(), hi.abs()).float().clamp(min=1e-12)
+    to_q = _FP8_MAX / amax
+    q = (x.float() * to_q).clamp(min=-_FP8_MAX, max=_FP8_MAX).to(dtype).contiguous()
+    return q, to_q.float().reciprocal()
+
+
+def block_quant_dequant(x_q_block: torch.Tensor, x_s: torch.Tensor, block_size: List[int], dtype: torch.dtype) -> torch.Tensor:
+    """Reference: fp8_utils.py:418-438 - [..., n, k] block-quantised values times their [..., ceil(n/bn), ceil(k/bk)]
+    scales, in float32, cast to `dtype`."""
+    bn, bk = block_size
+    n, k = x_q_block.shape[-2:]
+    rows = torch.arange(n, device=x_s.device) // bn
+    cols = torch.arange(k, device=x_s.device) // bk
+    full = x_s.index_select(-2, rows).index_select(-1, cols)
+    return (x_q_block.to(torch.float32) * full).to(dtype)
+
+
+def _tensor_quant(x_f32: torch.Tensor, like: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    # the GPU path quantises with the library's per-tensor op, as the reference does with scaled_fp8_quant
+    if x_f32.is_cuda and x_f32.dim() == 2:
+        return scaled_fp8_quant(x_f32.contiguous())
+    return input_to_float8(x_f32, dtype=like.dtype)
+
+
+def block_quant_to_tensor_quant(x_q_block: torch.Tensor, x_s: torch.Tensor, block_size: List[int]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_utils.py:375-415 - [n, k] block-quantised weight -> the same weight with one scale."""
+    n, k = x_q_block.shape
+    assert x_s.shape[0] == (n + block_size[0] - 1) // block_size[0]
+    assert x_s.shape[1] == (k + block_size[1] - 1) // block_size[1]
+    return _tensor_quant(block_quant_dequant(x_q_block, x_s, block_size, torch.float32), x_q_block)
+
+
+def channel_quant_to_tensor_quant(x_q_channel: torch.Tensor, x_s: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_utils.py:589-599 - per-channel scales [n, 1] -> one scale."""
+    return _tensor_quant(x_q_channel.to(torch.float32) * x_s, x_q_channel)
+
+
+def per_block_cast_to_fp8(x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_utils.py:568-582 - 128x128 block quantisation with power-of-two scales:
+    scale = 2^ceil(log2(max(amax, 1e-4) / 448)), q = e4m3fn(x / scale).  x [m, n] -> (q [m, n], scale [ceil(m/128), ceil(n/128)])."""
+    assert x.dim() == 2
+    m, n = x.shape
+    mt, nt = (m + 127) // 128, (n + 127) // 128
+    padded = torch.zeros((mt * 128, nt * 128), dtype=x.dtype, device=x.device)
+    padded[:m, :n] = x
+    tiles = padded.view(mt, 128, nt, 128)
+    amax = tiles.abs().float().amax(dim=(1, 3), keepdim=True).clamp(1e-4)
+    scale = ceil_to_ue8m0(amax / _FP8_MAX)
+    q = (tiles * (1.0 / scale)).to(torch.float8_e4m3fn).view(mt * 128, nt * 128)[:m, :n].contiguous()
+    return q, scale.view(mt, nt)
+
+
+def quant_weight_ue8m0(weight_dequant: torch.Tensor, weight_block_size: List[int]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_utils.py:479-502 - per_block_cast_to_fp8 over the last two dimensions of a bf16 weight."""
+    assert list(weight_block_size) == [128, 128]
+    assert weight_dequant.dtype == torch.bfloat16, f"{weight_dequant.dtype=} {weight_dequant.shape=}"
+    *batch, n, k = weight_dequant.shape
+    if not batch:
+        return per_block_cast_to_fp8(weight_dequant)
+    parts = [per_block_cast_to_fp8(w) for w in weight_dequant.reshape(-1, n, k)]
+    q = torch.stack([p[0] for p in parts]).view(*batch, n, k)
+    sc = torch.stack([p[1] for p in parts]).view(*batch, (n + 127) // 128, (k + 127) // 128)
+    return q, sc
+
+
+def requant_weight_ue8m0(weight: torch.Tensor, weight_scale_inv: torch.Tensor, weight_block_size: List[int]) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_utils.py:453-476 - dequantise a block-FP8 weight to bf16 and quantise it again with
+    power-of-two block scales.  The reference then repacks the scales into DeepGEMM's int32 layout; here they stay
+    float32 [.., ceil(n/128), ceil(k/128)] powers of two, which is what the UE8M0 GEMM of this library takes."""
+    assert list(weight_block_size) == [128, 128]
+    deq = block_quant_dequant(weight, weight_scale_inv, weight_block_size, torch.bfloat16)
+    return quant_weight_ue8m0(deq, weight_block_size)

@@ -1,0 +1,68 @@
+"""Host-side weight transforms of fp8_utils (plain tensor code, runs on the CPU): checked against the numpy oracle
+and against what the mathematics fixes (power-of-two scales, exact round trips)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fp8_oracle as O
+
+
+def _fp8(a_u8):
+    return torch.from_numpy(np.ascontiguousarray(a_u8)).view(torch.float8_e4m3fn)
+
+
+def test_block_quant_dequant_and_tensor_requant():
+    from sglang_amd.fp8_utils import block_quant_dequant, block_quant_to_tensor_quant, channel_quant_to_tensor_quant
+
+    w = O.make_weight(300, 520, seed=3)                        # not multiples of 128: ragged edge tiles
+    wq, ws = O.block_quant_weight(w)
+    deq = block_quant_dequant(_fp8(wq), torch.from_numpy(ws), [128, 128], torch.float32).numpy()
+    ref = O.e4m3fn_to_f32(wq) * np.repeat(np.repeat(ws, 128, 0), 128, 1)[:300, :520]
+    np.testing.assert_array_equal(deq, ref.astype(np.float32))
+    q, s = block_quant_to_tensor_quant(_fp8(wq), torch.from_numpy(ws), [128, 128])
+    assert q.dtype == torch.float8_e4m3fn and s.numel() == 1
+    amax = np.abs(ref).max()
+    np.testing.assert_allclose(float(s), amax / 448.0, rtol=1e-6)
+    np.testing.assert_allclose(q.float().numpy() * float(s), ref, atol=float(s) * 16 + 1e-12)  # half an e4m3 ulp at 448
+    xs = torch.rand((300, 1)) * 0.01 + 1e-3
+    q2, s2 = channel_quant_to_tensor_quant(_fp8(wq), xs)
+    ref2 = O.e4m3fn_to_f32(wq) * xs.numpy()
+    np.testing.assert_allclose(float(s2), np.abs(ref2).max() / 448.0, rtol=1e-6)
+
+
+def test_per_block_cast_and_ue8m0_requant():
+    from sglang_amd.fp8_utils import per_block_cast_to_fp8, requant_weight_ue8m0
+
+    w = torch.from_numpy(O.make_weight(256, 384, seed=5)).to(torch.bfloat16)
+    q, sc = per_block_cast_to_fp8(w)
+    assert q.shape == w.shape and sc.shape == (2, 3)
+    m, e = np.frexp(sc.numpy())
+    assert np.all(m == 0.5)                                      # powers of two
+    blocks = w.float().view(2, 128, 3, 128).abs().amax(dim=(1, 3)).clamp(1e-4)
+    assert torch.all(sc >= blocks / 448.0) and torch.all(sc < blocks / 448.0 * 2)   # the smallest power of two that fits
+    ref_q = O.f32_to_e4m3fn((w.float() / sc.repeat_interleave(128, 0).repeat_interleave(128, 1)).numpy())
+    np.testing.assert_array_equal(q.view(torch.uint8).numpy(), ref_q)
+    # requant of a float-scale checkpoint: scales become powers of two, values stay within one e4m3 step of the
+    # bf16 dequantisation
+    wq, ws = O.block_quant_weight(O.make_weight(256, 256, seed=7))
+    q2, s2 = requant_weight_ue8m0(_fp8(wq), torch.from_numpy(ws), [128, 128])
+    assert np.all(np.frexp(s2.numpy())[0] == 0.5)
+    deq = O.e4m3fn_to_f32(wq) * np.repeat(np.repeat(ws, 128, 0), 128, 1)
+    back = q2.float().numpy() * np.repeat(np.repeat(s2.numpy(), 128, 0), 128, 1)
+    step = np.repeat(np.repeat(s2.numpy(), 128, 0), 128, 1) * 32  # largest e4m3 spacing (between 416 and 448) in scaled units
+    assert np.all(np.abs(back - deq) <= step * 0.5 + np.abs(deq) * 2 ** -8)
+    # batched weights [E, n, k]
+    q3, s3 = requant_weight_ue8m0(_fp8(np.stack([wq, wq])), torch.from_numpy(np.stack([ws, ws])), [128, 128])
+    assert q3.shape == (2, 256, 256) and s3.shape == (2, 2, 2) and torch.equal(q3[0], q2) and torch.equal(s3[1], s2)
+
+
+def test_input_to_float8():
+    from sglang_amd.fp8_utils import input_to_float8
+
+    x = torch.randn(64, 96) * 3
+    q, s = input_to_float8(x)
+    assert q.dtype == torch.float8_e4m3fn
+    np.testing.assert_allclose(float(s), float(x.abs().max()) / 448.0, rtol=1e-6)
+    assert float(q.float().abs().max()) == 448.0
+    q0, s0 = input_to_float8(torch.zeros(4, 4))
+    assert float(s0) == pytest.approx(1e-12 / 448.0) and torch.all(q0.float() == 0)

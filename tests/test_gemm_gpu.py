@@ -265,3 +265,25 @@ def test_block_gemm_ue8m0_hardware_scales(dev, M, N, K):
     ref = O.w8a8_block_fp8_matmul(xq.view(torch.uint8).cpu().numpy(), wq, xs.cpu().numpy(), ws2, acc=np.float64)
     assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
     assert _rel_err(c.float().cpu().numpy(), c_float.float().cpu().numpy()) <= REL_TOL
+
+
+def test_ue8m0_requantised_checkpoint_end_to_end(dev):
+    """A float-scale block-FP8 weight passed through requant_weight_ue8m0 (reference: fp8_utils.py:453-476) and then
+    the UE8M0 linear: equal to the oracle on the requantised weight to 1e-2, and close to the float-scale linear of
+    the original weight (both are 8-bit renderings of the same bf16 numbers)."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.fp8_utils import requant_weight_ue8m0, w8a8_block_fp8_linear
+    from sglang_amd.sgl_kernel import unpack_ue8m0_scales
+
+    M, N, K = 384, 768, 1024
+    x = torch.from_numpy(O.make_activation(M, K, seed=1)).to(dev).to(torch.bfloat16)
+    wq, ws = O.block_quant_weight(O.make_weight(N, K, seed=2))
+    W, Ws = fp8_tensor(wq, dev), torch.from_numpy(ws).to(dev)
+    W2, Ws2 = requant_weight_ue8m0(W, Ws, [128, 128])
+    xq, xs_packed = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    c = w8a8_block_fp8_matmul(xq, W2, xs_packed, Ws2, [128, 128], torch.bfloat16)
+    ref = O.w8a8_block_fp8_matmul(xq.view(torch.uint8).cpu().numpy(), W2.view(torch.uint8).cpu().numpy(),
+                                  unpack_ue8m0_scales(xs_packed, K // 128).cpu().numpy(), Ws2.cpu().numpy(), acc=np.float64)
+    assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
+    c_float = w8a8_block_fp8_linear(x, W, [128, 128], Ws)
+    assert _rel_err(c.float().cpu().numpy(), c_float.float().cpu().numpy()) <= 0.08
