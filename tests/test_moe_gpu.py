@@ -154,7 +154,8 @@ def _expert_weights(rng, E, N, K):
 @pytest.mark.parametrize("T,E,topk,N,K,block", [(5, 8, 2, 512, 256, 16), (64, 8, 2, 384, 512, 32), (300, 16, 4, 1024, 1024, 64),
                                                (700, 4, 2, 256, 384, 128), (3, 16, 8, 1024, 7168, 32),
                                                (700, 4, 2, 512, 384, 256), (300, 16, 4, 1024, 1024, 256)])
-def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block):
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16])
+def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block, out_dtype):
     """GEMM1 form (row = slot // top_k, no routed weight) and GEMM2 form (row = slot, times routed weight)."""
     from sglang_amd.fused_moe import moe_align_block_size
     from sglang_amd.sgl_kernel import moe_block_gemm
@@ -169,7 +170,7 @@ def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block):
     for top_k, rows in ((topk, T), (1, T * topk)):
         xq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((rows, K)).astype(np.float32) * 100, -448, 448))
         xs = (rng.uniform(0.5, 2.0, (rows, K // 128)) * 1e-2).astype(np.float32)
-        C = torch.full((T * topk, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        C = torch.full((T * topk, N), float("nan"), dtype=out_dtype, device=dev)
         mul = top_k == 1
         moe_block_gemm(fp8_tensor(xq, dev), Bq, C, torch.from_numpy(xs).to(dev), Bs, torch.from_numpy(tw).to(dev),
                        sorted_ids, expert_ids, npad, mul, top_k, block, ids.size)
