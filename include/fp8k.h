@@ -132,6 +132,14 @@ int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t* As_packed
 int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * Tuning and test aid (no counterpart in the reference): pins the kernel family that the dense GEMM entry points
+ * pick for later calls of this process.  kind -1: automatic (the default).  kind 4: the 128x128 tile kernel with K
+ * cut into `splits` runs (0 or 1: none).  kind 0..3: automatic choice among the other families only (generic, 256x256
+ * tiles, streaming, direct), `splits` ignored.  fp8k_*_workspace_bytes follows the pinned choice.  Not thread safe.
+ */
+void fp8k_tune_force_gemm_plan(int kind, int splits);
+
+/*
  * Per-token x per-channel FP8 GEMM:  C = (A . B^T) * sa[m] * sb[n] (+ bias[n]), fp32 accumulate.
  * Replaces torch.ops.sgl_kernel.fp8_scaled_mm
  *   (sgl-kernel/python/sgl_kernel/gemm.py:35-43, sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532).

@@ -3,23 +3,38 @@
 #include <algorithm>
 
 #include "gemm_direct.h"
+#include "gemm_tile128.h"
 
 namespace fp8k {
 
 struct Plan {
-  int kind;    // 0 = generic, 1 = tile256, 2 = weight-streaming through LDS (33..128 rows), 3 = direct (<= 32 rows)
+  int kind;    // 0 = generic, 1 = tile256, 2 = weight-streaming through LDS (33..128 rows), 3 = direct (<= 32 rows),
+               // 4 = tile128
   int splits;  // >1: split-K through the float workspace
   int kb_per_split;
-  int tm;      // rows per block of the streaming kernel
+  int tm;      // rows per block of the streaming kernels
   int tail_first;   // tile256: first tile that is cut along K (== number of tiles when none is)
   int64_t ws_bytes; // float workspace the plan needs
 };
 
 constexpr int kNumCU = 256;  // MI355X
 
-static Plan make_plan(int64_t M, int64_t N, int64_t K) {
+// tuning aid: force the kernel family (and the K split of the uniform-split families) of later calls
+static int g_force_kind = -1, g_force_splits = 0;
+
+static Plan plan_tile128(int64_t M, int64_t N, int kb, int splits) {
+  Plan pl{4, 1, 0, 0, 0, 0};
+  if (splits > kb) splits = kb;
+  if (splits < 1) splits = 1;
+  pl.kb_per_split = (kb + splits - 1) / splits;
+  pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
+  pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  return pl;
+}
+
+// the plan without the 128x128 tile kernel: direct / streaming / 256x256 tiles by the number of rows
+static Plan plan_base(int64_t M, int64_t N, int64_t K) {
   Plan pl{0, 1, 0, 0, 0, 0};
-  if (K % kTileK != 0 || N % 4 != 0) return pl;
   const int kb = (int)(K / kTileK);
   if (M <= 32 && M * K < (1LL << 31)) {
     // decode-sized: weights go HBM -> registers -> matrix core.  K is cut so that about 512 workgroups (two per
@@ -68,9 +83,93 @@ static Plan make_plan(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
+
+// Rough device-time models in microseconds, fitted to sweeps over M = 64..2048 on the DeepSeek-V3 and Llama
+// projection shapes; they only have to rank the two candidates where the gap is large.
+//  * 128x128 tiles: a workgroup spends 0.55 us per K block alone on the chip, up to 0.85 us when all CUs stream at
+//    once; first loads + tile write-out 2.5 us per round of tiles, launch 1 us; a K cut adds the reduction launch
+//    (4 us) and the float partials (written and read back, about 8 TB/s since they stay in the memory-side cache).
+//  * streaming kernel: 8-11 us fixed, the weights once at 5.5 TB/s, the same partials.
+//  * 256x256 tiles: 2 us per K block and tile, 8 us fixed, 6 us + partials for a cut last round.
+static double est_tile128(int64_t M, int64_t N, int kb, int* best_splits) {
+  const int64_t tiles = ((M + kT128 - 1) / kT128) * ((N + kT128 - 1) / kT128);
+  double best = 1e30;
+  for (int s = 1; s <= 8; ++s) {
+    if (s > 1 && (s > kb / 4 || tiles * s > kNumCU)) break;
+    const int64_t wgs = tiles * s;
+    const double rounds = (double)((wgs + kNumCU - 1) / kNumCU);
+    const int kbps = (kb + s - 1) / s;
+    const double tb = 0.55 + 0.30 * std::min(1.0, (double)wgs / kNumCU);
+    const double t = 1.0 + rounds * (kbps * tb + 2.5) + (s > 1 ? 4.0 + (double)s * M * N * 8.0 / 8e6 : 0.0);
+    if (t < best) { best = t; *best_splits = s; }
+  }
+  return best;
+}
+
+static double est_base(const Plan& pl, int64_t M, int64_t N, int64_t K) {
+  const int kb = (int)(K / kTileK);
+  if (pl.kind == 2)
+    return (M <= 64 ? 8.0 : 11.0) + (double)N * K / 5.5e6 + (pl.splits > 1 ? (double)pl.splits * M * N * 8.0 / 8e6 : 0.0);
+  const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
+  if (pl.splits == 1) return 8.0 + (double)((tiles + kNumCU - 1) / kNumCU) * kb * 2.0;
+  const int64_t rest = tiles % kNumCU;
+  return 8.0 + (double)(tiles / kNumCU) * kb * 2.0 + pl.kb_per_split * 2.0 + 6.0 +
+         (double)rest * pl.splits * (kTileM * kTileN * 4) * 2.0 / 8e6;
+}
+
+static Plan make_plan(int64_t M, int64_t N, int64_t K) {
+  Plan pl{0, 1, 0, 0, 0, 0};
+  if (K % kTileK != 0 || N % 4 != 0) return pl;
+  const int kb = (int)(K / kTileK);
+  if (g_force_kind == 4 && N % 8 == 0) return plan_tile128(M, N, kb, g_force_splits);
+  pl = plan_base(M, N, K);
+  if (g_force_kind >= 0 || M <= 32 || N % 8 != 0 || (pl.kind != 1 && pl.kind != 2)) return pl;
+  // a few hundred rows, or fewer 256x256 tiles than CUs: the 128x128 tile kernel when the model says it is
+  // clearly ahead (more clearly for the smallest batches, where the fixed costs it ignores weigh most)
+  int s128 = 1;
+  const double t128 = est_tile128(M, N, kb, &s128);
+  if (t128 < (M <= 64 ? 0.8 : 0.9) * est_base(pl, M, N, K)) return plan_tile128(M, N, kb, s128);
+  return pl;
+}
+
 static int64_t workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0) return 0;
   return make_plan(M, N, K).ws_bytes;
+}
+
+// the two tile kernels (plan kinds 1 and 4); `a` carries the operands, the plan the tiling
+template <int MODE, int OUT_DT, int BIAS_DT>
+static int launch_tiles(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
+  GemmArgs a = a0;
+  a.tiles_m = (a.M + kTileM - 1) / kTileM;
+  a.tiles_n = (a.N + kTileN - 1) / kTileN;
+  a.splits = pl.splits;
+  a.kb_per_split = pl.kb_per_split;
+  if (pl.kind == 4) {
+    a.tiles_m = (a.M + kT128 - 1) / kT128;
+    a.tiles_n = (a.N + kT128 - 1) / kT128;
+    const unsigned nwg = (unsigned)(((int64_t)a.tiles_m * a.tiles_n * pl.splits + 7) / 8 * 8);
+    if (pl.splits == 1) {
+      hipLaunchKernelGGL((gemm_tile128_kernel<MODE, OUT_DT, BIAS_DT, false>), dim3(nwg), dim3(512), 0, st, a);
+      return check_launch("gemm_tile128");
+    }
+    hipLaunchKernelGGL((gemm_tile128_kernel<MODE, OUT_DT, BIAS_DT, true>), dim3(nwg), dim3(512), 0, st, a);
+    int rc = check_launch("gemm_tile128");
+    if (rc) return rc;
+    const int64_t quads = (int64_t)a.M * (a.N / 4);
+    hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256),
+                       0, st, a);
+    return check_launch("splitk_reduce");
+  }
+  const int ntiles = a.tiles_m * a.tiles_n;
+  a.tail_first = pl.tail_first;
+  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
+  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
+  int rc = check_launch("gemm_tile256");
+  if (rc || pl.tail_first == ntiles) return rc;
+  hipLaunchKernelGGL((tile_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((ntiles - pl.tail_first) * 64)), dim3(256),
+                     0, st, a);
+  return check_launch("tile_reduce");
 }
 
 template <int MODE, int OUT_DT, int BIAS_DT>
@@ -128,15 +227,7 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
                        0, st, a);
     return check_launch("splitk_reduce");
   }
-  const int ntiles = a.tiles_m * a.tiles_n;
-  a.tail_first = pl.tail_first;
-  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
-  hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
-  int rc = check_launch("gemm_tile256");
-  if (rc || pl.tail_first == ntiles) return rc;
-  hipLaunchKernelGGL((tile_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((ntiles - pl.tail_first) * 64)), dim3(256),
-                     0, st, a);
-  return check_launch("tile_reduce");
+  return launch_tiles<MODE, OUT_DT, BIAS_DT>(a, pl, st);
 }
 
 static int common_checks(const char* op, const void* A, const void* B, void* C, int64_t M, int64_t N, int64_t K,
@@ -158,6 +249,8 @@ static int common_checks(const char* op, const void* A, const void* B, void* C, 
 }  // namespace fp8k
 
 using namespace fp8k;
+
+extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) { g_force_kind = kind; g_force_splits = splits; }
 
 extern "C" int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return workspace_bytes(M, N, K); }
 extern "C" int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return workspace_bytes(M, N, K); }
@@ -202,9 +295,9 @@ extern "C" int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t
   FP8K_REQUIRE(As_packed && Bs, "%s: null scale pointer", op);
   FP8K_REQUIRE(as_stride_m >= 0 && as_stride_w >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0, "%s: negative scale stride", op);
   const Plan pl = make_plan(M, N, K);
-  // the matrix core applies the scales only in the 256x256 tile kernel; smaller problems take the float-scale
+  // the matrix core applies the scales only in the tile kernels; smaller problems take the float-scale
   // entry point with the exponents expanded to floats
-  FP8K_REQUIRE(pl.kind == 1, "%s: built for M > 128 with K a multiple of 128 (got M=%lld, K=%lld); expand the scales "
+  FP8K_REQUIRE(pl.kind == 1 || pl.kind == 4, "%s: built for M > 128 with K a multiple of 128 (got M=%lld, K=%lld); expand the scales "
                "and call fp8k_block_gemm", op, (long long)M, (long long)K);
   const int64_t need = pl.ws_bytes;
   if (need > 0 && (!workspace || workspace_bytes_given < need))
@@ -215,27 +308,9 @@ extern "C" int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t
   a.bias = nullptr; a.C = C; a.partial = (float*)workspace;
   a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
   a.sx_m = as_stride_m; a.sx_k = as_stride_w; a.sw_n = bs_stride_n; a.sw_k = bs_stride_k;
-  a.tiles_m = (a.M + kTileM - 1) / kTileM;
-  a.tiles_n = (a.N + kTileN - 1) / kTileN;
-  a.splits = pl.splits;
-  a.kb_per_split = pl.kb_per_split;
-  a.tail_first = pl.tail_first;
   hipStream_t st = (hipStream_t)stream;
-  const int ntiles = a.tiles_m * a.tiles_n;
-  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
-  if (out_dtype == FP8K_BF16)
-    hipLaunchKernelGGL((gemm_tile256_kernel<kModeScaled, FP8K_BF16, FP8K_F32>), dim3(nwg), dim3(512), 0, st, a);
-  else
-    hipLaunchKernelGGL((gemm_tile256_kernel<kModeScaled, FP8K_F16, FP8K_F32>), dim3(nwg), dim3(512), 0, st, a);
-  rc = check_launch(op);
-  if (rc || pl.tail_first == ntiles) return rc;
-  if (out_dtype == FP8K_BF16)
-    hipLaunchKernelGGL((tile_reduce_kernel<kModeScaled, FP8K_BF16, FP8K_F32>), dim3((unsigned)((ntiles - pl.tail_first) * 64)),
-                       dim3(256), 0, st, a);
-  else
-    hipLaunchKernelGGL((tile_reduce_kernel<kModeScaled, FP8K_F16, FP8K_F32>), dim3((unsigned)((ntiles - pl.tail_first) * 64)),
-                       dim3(256), 0, st, a);
-  return check_launch("tile_reduce");
+  return out_dtype == FP8K_BF16 ? launch_tiles<kModeScaled, FP8K_BF16, FP8K_F32>(a, pl, st)
+                                : launch_tiles<kModeScaled, FP8K_F16, FP8K_F32>(a, pl, st);
 }
 
 extern "C" int fp8k_scaled_mm(const void* A, const void* B, const float* sa, const float* sb, const void* bias, void* C,
