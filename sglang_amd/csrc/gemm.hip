@@ -84,23 +84,31 @@ static Plan plan_base(int64_t M, int64_t N, int64_t K) {
 }
 
 
-// Rough device-time models in microseconds, fitted to sweeps over M = 64..2048 on the DeepSeek-V3 and Llama
+// Rough device-time models in microseconds, fitted to sweeps over M = 48..2048 on the DeepSeek-V3 and Llama
 // projection shapes; they only have to rank the two candidates where the gap is large.
-//  * 128x128 tiles: a workgroup spends 0.55 us per K block alone on the chip, up to 0.85 us when all CUs stream at
-//    once; first loads + tile write-out 2.5 us per round of tiles, launch 1 us; a K cut adds the reduction launch
-//    (4 us) and the float partials (written and read back, about 8 TB/s since they stay in the memory-side cache).
-//  * streaming kernel: 8-11 us fixed, the weights once at 5.5 TB/s, the same partials.
-//  * 256x256 tiles: 2 us per K block and tile, 8 us fixed, 6 us + partials for a cut last round.
+//  * 128x128 tiles: a workgroup spends 0.42 us per K block when its operands come out of the L2, up to 0.72 us
+//    when every CU streams lines that are new to the chip (the share of such lines falls with the number of
+//    tiles that share a weight or activation tile); first loads + tile write-out 2.5 us per round of tiles,
+//    launch 1 us; more than two rounds are left to the 256x256 kernel, two rounds measure about 15 % over the
+//    model; a K cut adds the reduction launch (4 us) and the float partials (written and read back at about
+//    5 TB/s).
+//  * streaming kernel: 8-11 us fixed, the weights once at 5.5 TB/s, its partials at about 8 TB/s.
+//  * 256x256 tiles: 1.6 us per K block and tile, 8 us fixed, 6 us + partials (8 TB/s) for a cut last round.
 static double est_tile128(int64_t M, int64_t N, int kb, int* best_splits) {
-  const int64_t tiles = ((M + kT128 - 1) / kT128) * ((N + kT128 - 1) / kT128);
+  const int64_t tm = (M + kT128 - 1) / kT128, tn = (N + kT128 - 1) / kT128;
+  const int64_t tiles = tm * tn;
+  const double cold = std::min(1.0, 1.0 / (double)tm + 1.0 / (double)tn);
   double best = 1e30;
   for (int s = 1; s <= 8; ++s) {
-    if (s > 1 && (s > kb / 4 || tiles * s > kNumCU)) break;
+    if (s > 1 && (s > kb / 4 || tiles * s > 216)) break;  // a K cut over more than ~85 % of the CUs measured slower
     const int64_t wgs = tiles * s;
-    const double rounds = (double)((wgs + kNumCU - 1) / kNumCU);
+    const int64_t rounds = (wgs + kNumCU - 1) / kNumCU;
+    if (rounds > 2) break;
     const int kbps = (kb + s - 1) / s;
-    const double tb = 0.55 + 0.30 * std::min(1.0, (double)wgs / kNumCU);
-    const double t = 1.0 + rounds * (kbps * tb + 2.5) + (s > 1 ? 4.0 + (double)s * M * N * 8.0 / 8e6 : 0.0);
+    const double tb = 0.42 + 0.30 * cold * std::min(1.0, (double)wgs / kNumCU);
+    double t = 1.0 + (double)rounds * (kbps * tb + 2.5);
+    if (rounds == 2) t *= 1.15;
+    if (s > 1) t += 4.0 + (double)s * M * N * 8.0 / 5e6;
     if (t < best) { best = t; *best_splits = s; }
   }
   return best;
@@ -111,9 +119,9 @@ static double est_base(const Plan& pl, int64_t M, int64_t N, int64_t K) {
   if (pl.kind == 2)
     return (M <= 64 ? 8.0 : 11.0) + (double)N * K / 5.5e6 + (pl.splits > 1 ? (double)pl.splits * M * N * 8.0 / 8e6 : 0.0);
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
-  if (pl.splits == 1) return 8.0 + (double)((tiles + kNumCU - 1) / kNumCU) * kb * 2.0;
+  if (pl.splits == 1) return 8.0 + (double)((tiles + kNumCU - 1) / kNumCU) * kb * 1.6;
   const int64_t rest = tiles % kNumCU;
-  return 8.0 + (double)(tiles / kNumCU) * kb * 2.0 + pl.kb_per_split * 2.0 + 6.0 +
+  return 8.0 + (double)(tiles / kNumCU) * kb * 1.6 + pl.kb_per_split * 1.6 + 6.0 +
          (double)rest * pl.splits * (kTileM * kTileN * 4) * 2.0 / 8e6;
 }
 
@@ -124,11 +132,10 @@ static Plan make_plan(int64_t M, int64_t N, int64_t K) {
   if (g_force_kind == 4 && N % 8 == 0) return plan_tile128(M, N, kb, g_force_splits);
   pl = plan_base(M, N, K);
   if (g_force_kind >= 0 || M <= 32 || N % 8 != 0 || (pl.kind != 1 && pl.kind != 2)) return pl;
-  // a few hundred rows, or fewer 256x256 tiles than CUs: the 128x128 tile kernel when the model says it is
-  // clearly ahead (more clearly for the smallest batches, where the fixed costs it ignores weigh most)
+  // a few hundred rows, or fewer 256x256 tiles than CUs: the 128x128 tile kernel when the model puts it ahead
   int s128 = 1;
   const double t128 = est_tile128(M, N, kb, &s128);
-  if (t128 < (M <= 64 ? 0.8 : 0.9) * est_base(pl, M, N, K)) return plan_tile128(M, N, kb, s128);
+  if (t128 < 0.92 * est_base(pl, M, N, K)) return plan_tile128(M, N, kb, s128);
   return pl;
 }
 

@@ -12,10 +12,11 @@
 // 0 and 1 fetch the 128 activation-row scales of the block, the others the weight scale), so that one partial
 // vmcnt wait covers everything a block needs.
 //
-// One barrier per K block.  After the barrier of block `it` a wave (a) refills the stage of block it-1 with
-// block it+3, (b) fetches its operands of block `it` from LDS into one of two register sets and (c) issues the
-// MFMAs of block it-1 from the other set, so the matrix core never waits for LDS.  The loop body is
-// branch-free: loads past the last K block are out of range or unread.
+// One barrier per K block.  After the barrier of block `it` a wave issues the four MFMAs of block it-1 from one
+// of two register sets, and between them (a) refills the stage of block it-1 with block it+3 and (b) fetches its
+// operands of block `it` from LDS into the other set: all eight waves pass the barrier together, and with the
+// LDS reads up front the LDS pipe and the matrix core would take turns instead of overlapping.  The loop body
+// is branch-free: loads past the last K block are out of range or unread.
 //
 // SPLIT: the K range is cut into p.splits runs, every (tile, run) pair is one workgroup, float partials go to
 // the workspace [split][M][N] for splitk_reduce_kernel.
@@ -131,89 +132,119 @@ __global__ __launch_bounds__(512, 1) void gemm_tile128_kernel(const GemmArgs p) 
     for (int r = 0; r < 16; ++r) acc[ns][r] = 0.f;
 
   // operands and scale of one K block, in registers
-  struct Operands { v8i W0[2], W1[2], X[2]; float sc; int sq, sqw; };
+  struct Operands { v8i W0[2], W1[2], X[2]; uint32_t sx, sw; };  // sx, sw: raw scale words as they lie in LDS
   Operands oa, ob;
   v16f tb_pend;       // block mode: second tile's product of the block before, not yet added to acc[1]
   float sc_pend = 0.f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) tb_pend[r] = 0.f;
 
-  // barrier of block `it`, then refill of the stage that block it-1 has left
-  auto top = [&](int it) {
-    const int kf = it + NST - 1;
-    const int fill = kf & (NST - 1);
-    SB();  // the MFMAs issued before stay in front of this wait: they are what hides the loads' latency
-    lds_barrier<(NST - 2) * kLoadsPerBlock>();
-    L(fill, kf, 0); L(fill, kf, 1); L(fill, kf, 2); L(fill, kf, 3);
-    LS(fill, kf);
-  };
-  auto fetch = [&](Operands& o, int it) {
-    const uint8_t* st = smem + (it & (NST - 1)) * kT128Stage;
-    o.W0[0] = frag(st, rdW, 0); o.X[0] = frag(st, rdX, 0);
-    o.W0[1] = frag(st, rdW, 1); o.X[1] = frag(st, rdX, 1);
-    o.W1[0] = frag(st, rdW + 32 * kTileK, 0); o.W1[1] = frag(st, rdW + 32 * kTileK, 1);
-    o.sc = 0.f; o.sq = 127; o.sqw = 127;
-    if (MODE == kModeBlock)
-      o.sc = *reinterpret_cast<const float*>(st + rdS) * *reinterpret_cast<const float*>(st + kT128SOff + 512);
-    if (MODE == kModeScaled) {
-      const int sh = ((kb_begin + it) & 3) * 8;
-      o.sq = (int)(*reinterpret_cast<const uint32_t*>(st + rdS) >> sh);
-      o.sqw = (int)(*reinterpret_cast<const uint32_t*>(st + kT128SOff + 512) >> 23);
-    }
-    SB();
-  };
-  auto compute = [&](const Operands& o) {
+  // the four MFMAs of K block `it` from registers; `between(i)` is issued after MFMA i (the LDS reads and global
+  // loads of the trip go there, so that they run in the shadow of the matrix core instead of before it)
+  auto compute = [&](const Operands& o, int it, auto&& between) {
     if (MODE == kModeBlock) {
+      const float sc = __uint_as_float(o.sx) * __uint_as_float(o.sw);
       v16f z, ta, tb;
 #pragma unroll
       for (int r = 0; r < 16; ++r) z[r] = 0.f;
       ta = mfma_32x32x64(o.W0[0], o.X[0], z);
+      between(0);
 #pragma unroll
       for (int r = 0; r < 8; ++r) acc[1][r] = __builtin_fmaf(tb_pend[r], sc_pend, acc[1][r]);
-      ta = mfma_32x32x64(o.W0[1], o.X[1], ta);
+      SB();
+      tb = mfma_32x32x64(o.W1[0], o.X[0], z);
+      between(1);
 #pragma unroll
       for (int r = 8; r < 16; ++r) acc[1][r] = __builtin_fmaf(tb_pend[r], sc_pend, acc[1][r]);
       SB();
-      tb = mfma_32x32x64(o.W1[0], o.X[0], z);
-#pragma unroll
-      for (int r = 0; r < 8; ++r) acc[0][r] = __builtin_fmaf(ta[r], o.sc, acc[0][r]);
+      ta = mfma_32x32x64(o.W0[1], o.X[1], ta);
+      between(2);
+      SB();
       tb = mfma_32x32x64(o.W1[1], o.X[1], tb);
+      between(3);
 #pragma unroll
-      for (int r = 8; r < 16; ++r) acc[0][r] = __builtin_fmaf(ta[r], o.sc, acc[0][r]);
+      for (int r = 0; r < 16; ++r) acc[0][r] = __builtin_fmaf(ta[r], sc, acc[0][r]);
       tb_pend = tb;
-      sc_pend = o.sc;
-    } else if (MODE == kModeScaled) {
-      acc[0] = mfma_32x32x64_scaled(o.W0[0], o.X[0], acc[0], o.sqw, o.sq);
-      acc[1] = mfma_32x32x64_scaled(o.W1[0], o.X[0], acc[1], o.sqw, o.sq);
-      acc[0] = mfma_32x32x64_scaled(o.W0[1], o.X[1], acc[0], o.sqw, o.sq);
-      acc[1] = mfma_32x32x64_scaled(o.W1[1], o.X[1], acc[1], o.sqw, o.sq);
+      sc_pend = sc;
     } else {
-      acc[0] = mfma_32x32x64(o.W0[0], o.X[0], acc[0]);
-      acc[1] = mfma_32x32x64(o.W1[0], o.X[0], acc[1]);
-      acc[0] = mfma_32x32x64(o.W0[1], o.X[1], acc[0]);
-      acc[1] = mfma_32x32x64(o.W1[1], o.X[1], acc[1]);
+      int sq = 127, sqw = 127;
+      if (MODE == kModeScaled) { sq = (int)(o.sx >> (((kb_begin + it) & 3) * 8)); sqw = (int)(o.sw >> 23); }
+      auto MM = [&](const v8i& a, const v8i& b, v16f c) -> v16f {
+        if (MODE == kModeScaled) return mfma_32x32x64_scaled(a, b, c, sqw, sq);
+        return mfma_32x32x64(a, b, c);
+      };
+      acc[0] = MM(o.W0[0], o.X[0], acc[0]);
+      between(0); SB();
+      acc[1] = MM(o.W1[0], o.X[0], acc[1]);
+      between(1); SB();
+      acc[0] = MM(o.W0[1], o.X[1], acc[0]);
+      between(2); SB();
+      acc[1] = MM(o.W1[1], o.X[1], acc[1]);
+      between(3);
     }
   };
+  // trip `it`: barrier of block `it`; refill of the stage that block it-1 has left with block it+3; operands of
+  // block `it` from LDS into `rd`; MFMAs of block it-1 from `use`
+  auto trip = [&](int it, Operands& rd, const Operands& use) {
+    const int kf = it + NST - 1;
+    const int fill = kf & (NST - 1);
+    const uint8_t* st = smem + (it & (NST - 1)) * kT128Stage;
+    SB();  // the MFMAs issued before stay in front of this wait: they are what hides the loads' latency
+    lds_barrier<(NST - 2) * kLoadsPerBlock>();
+    compute(use, it - 1, [&](int i) {
+      // all LDS reads in the first three gaps, so that they have returned when the wave reaches the next barrier
+      if (i == 0) {
+        rd.W0[0] = frag(st, rdW, 0); rd.X[0] = frag(st, rdX, 0);
+        rd.sx = 0; rd.sw = 0;
+        if (MODE != kModeRow) {  // combined a trip later: nothing here waits for these reads
+          rd.sx = *reinterpret_cast<const uint32_t*>(st + rdS);
+          rd.sw = *reinterpret_cast<const uint32_t*>(st + kT128SOff + 512);
+        }
+        L(fill, kf, 0);
+      } else if (i == 1) {
+        rd.W1[0] = frag(st, rdW + 32 * kTileK, 0); rd.W0[1] = frag(st, rdW, 1);
+        L(fill, kf, 1); L(fill, kf, 2);
+      } else if (i == 2) {
+        rd.X[1] = frag(st, rdX, 1); rd.W1[1] = frag(st, rdW + 32 * kTileK, 1);
+        L(fill, kf, 3);
+      } else {
+        LS(fill, kf);
+      }
+    });
+  };
 
-  // ---- prologue: blocks 0 .. 2 into stages 0 .. 2
+  // ---- prologue: blocks 0 .. 2 into stages 0 .. 2, block 0's operands into `oa`
 #pragma unroll
   for (int s = 0; s < NST - 1; ++s) {
     L(s, s, 0); L(s, s, 1); L(s, s, 2); L(s, s, 3);
     LS(s, s);
   }
+  {
+    SB();
+    lds_barrier<(NST - 2) * kLoadsPerBlock>();
+    L(NST - 1, NST - 1, 0); L(NST - 1, NST - 1, 1); L(NST - 1, NST - 1, 2); L(NST - 1, NST - 1, 3);
+    LS(NST - 1, NST - 1);
+    oa.W0[0] = frag(smem, rdW, 0); oa.X[0] = frag(smem, rdX, 0);
+    oa.W0[1] = frag(smem, rdW, 1); oa.X[1] = frag(smem, rdX, 1);
+    oa.W1[0] = frag(smem, rdW + 32 * kTileK, 0); oa.W1[1] = frag(smem, rdW + 32 * kTileK, 1);
+    oa.sx = 0; oa.sw = 0;
+    if (MODE != kModeRow) {
+      oa.sx = *reinterpret_cast<const uint32_t*>(smem + rdS);
+      oa.sw = *reinterpret_cast<const uint32_t*>(smem + kT128SOff + 512);
+    }
+  }
   // ---- block b is fetched in trip b and multiplied in trip b+1; even blocks live in `oa`, odd ones in `ob`
-  top(0);
-  fetch(oa, 0);
+  auto nothing = [](int) {};
   int it = 1;
   for (; it + 1 < nkb; it += 2) {
-    top(it); fetch(ob, it); compute(oa);
-    top(it + 1); fetch(oa, it + 1); compute(ob);
+    trip(it, ob, oa);
+    trip(it + 1, oa, ob);
   }
   if (it < nkb) {
-    top(it); fetch(ob, it); compute(oa);
-    compute(ob);
+    trip(it, ob, oa);
+    compute(ob, it, nothing);
   } else {
-    compute(oa);
+    compute(oa, it - 1, nothing);
   }
   if (MODE == kModeBlock) {
 #pragma unroll
