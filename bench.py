@@ -266,6 +266,24 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384)):
     return lines
 
 
+def gemm_lines(torch, dev, shapes):
+    """Block-FP8 GEMM alone at the given (M, N, K): device time, TFLOP/s and algorithmic GB/s."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    lines = ["| M | N | K | us | TFLOP/s | % of 5 PFLOP/s | GB/s (algorithmic) |", "|---|---|---|---|---|---|---|"]
+    for (M, N, K) in shapes:
+        nbuf = 3
+        ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
+        qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True)
+              for s in range(nbuf)]
+        us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
+                                                                ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
+        tf = 2.0 * M * N * K / us / 1e6
+        lines.append("| %d | %d | %d | %.1f | %.1f | %.1f | %.0f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100,
+                                                                      gemm_bytes(M, N, K) / us / 1e3))
+    return lines
+
+
 def write_table(torch, dev, path):
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
     from sglang_amd.sgl_kernel import fp8_scaled_mm
@@ -341,6 +359,8 @@ def main() -> int:
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--moe", type=str, default=None,
                     help="only time the fused MoE layer at these token counts (comma separated) and print its table")
+    ap.add_argument("--gemm", type=str, default=None,
+                    help="only time the block-FP8 GEMM at these shapes (MxNxK, comma separated) and print its table")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no cross-GPU step); --gpus %d is not "
@@ -357,6 +377,10 @@ def main() -> int:
 
     if args.moe:
         print("\n".join(moe_table(torch, dev, tuple(int(t) for t in args.moe.split(",")))))
+        return 0
+    if args.gemm:
+        shapes = [tuple(int(v) for v in t.split("x")) for t in args.gemm.split(",")]
+        print("\n".join(gemm_lines(torch, dev, shapes)))
         return 0
     ms_per_step, gemm_us = run_headline(torch, dev, args.steps, args.warmup)
     M, N, K = HEADLINE["M"], HEADLINE["N"], HEADLINE["K"]
