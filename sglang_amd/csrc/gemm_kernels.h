@@ -476,6 +476,48 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 }
 
 
+// Work item of a grouped (MoE) launch.  The number of blocks in use is device data; each XCD (workgroup id mod 8)
+// takes a contiguous run of those blocks, cut into windows of four.  Inside a window the blocks of one expert form
+// a group whose workgroups walk the blocks first and the n tiles second, so the workgroups that stream the same
+// weight tile are dispatched together and meet in L2 instead of fetching it once each.  The window's expert ids
+// are fetched with four independent loads: a workgroup starts with two dependent memory round trips (block count,
+// then the window) before it knows its tile, not one per neighbour it compares with.
+struct MoeItem {
+  int mb;       // block of token slots, -1: nothing to do
+  int tile_n;
+  int expert;
+};
+__device__ __forceinline__ MoeItem moe_work_item(const GemmArgs& p, int bid) {
+  constexpr int kWin = 4;
+  MoeItem it{-1, 0, -1};
+  const int used = min(p.num_post_pad[0] / p.block_m, p.m_blocks);
+  const int per_xcd = (used + 7) >> 3;
+  const int j = bid >> 3;
+  const int pos = j / p.tiles_n;                      // block position inside the XCD's run, before regrouping
+  if (pos >= per_xcd) return it;
+  const int first_blk = (bid & 7) * per_xcd, end_blk = min(first_blk + per_xcd, used);
+  if (first_blk + pos >= end_blk) return it;
+  const int w0 = pos & ~(kWin - 1);                   // first position of the window
+  int e[kWin];
+#pragma unroll
+  for (int i = 0; i < kWin; ++i) e[i] = first_blk + w0 + i < end_blk ? p.expert_ids[first_blk + w0 + i] : -2 - i;
+  const int pi = pos - w0;
+  int a = 0, b = kWin, ex = e[0];                     // group [a, b) of the window that holds position pi
+#pragma unroll
+  for (int i = 1; i < kWin; ++i) {
+    if (e[i] != e[i - 1]) {
+      if (i <= pi) { a = i; ex = e[i]; }
+      else if (b == kWin) b = i;
+    }
+  }
+  const int g = b - a;
+  const int r = j - (w0 + a) * p.tiles_n;             // slot inside the group: 0 .. g*tiles_n-1
+  it.tile_n = r / g;
+  it.mb = first_blk + w0 + a + (r - it.tile_n * g);
+  it.expert = ex;
+  return it;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Weight-streaming kernel for 33..128 activation rows: 256(n) x TM(m) x 128(k) tile, TM in {64, 128}.
 // Used for small dense batches (with split-K through a float workspace so that every CU streams a share
@@ -507,34 +549,15 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
 
   // ---- work item.  Workgroup ids are dealt round-robin to the 8 XCDs (one L2 each).
   // Dense: each XCD takes a contiguous run of items, consecutive ids walk the m blocks of one n tile.
-  // Grouped: the number of blocks in use is device data; each XCD takes a contiguous run of those
-  // blocks and walks all n tiles of a block before the next one, so the tiles that run together on
-  // an XCD share the block's activation rows, and the blocks of one expert share its weights.
+  // Grouped: see moe_work_item().
   int bid = blockIdx.x;
   int split = 0;
   int mb, tile_n;
+  int expert = 0;
   if (MOE) {
-    const int used = min(p.num_post_pad[0] / p.block_m, p.m_blocks);
-    const int per_xcd = (used + 7) >> 3;
-    const int j = bid >> 3;
-    const int mbl = j / p.tiles_n;
-    if (mbl >= per_xcd) return;
-    const int first_blk = (bid & 7) * per_xcd, end_blk = min(first_blk + per_xcd, used);
-    mb = first_blk + mbl;
-    if (mb >= end_blk) return;
-    // Blocks of one expert that sit next to each other in the run form groups of up to kShare; inside a
-    // group consecutive workgroup ids walk the blocks first and the n tiles second, so the workgroups that
-    // stream the same weight tile are dispatched together and meet in L2 instead of fetching it once each.
-    constexpr int kShare = 4;
-    const int e = p.expert_ids[mb];
-    int idx = 0;                       // position of this block inside its run of equal expert ids
-    while (mb - idx > first_blk && p.expert_ids[mb - idx - 1] == e) ++idx;
-    const int gfirst = mb - (idx & (kShare - 1));
-    int g = (idx & (kShare - 1)) + 1;  // group size: forward to the end of the run, at most kShare
-    while (g < kShare && gfirst + g < end_blk && p.expert_ids[gfirst + g] == e) ++g;
-    const int r = j - (gfirst - first_blk) * p.tiles_n;  // slot inside the group: 0 .. g*tiles_n-1
-    tile_n = r / g;
-    mb = gfirst + (r - tile_n * g);
+    const MoeItem item = moe_work_item(p, bid);
+    if (item.mb < 0) return;
+    mb = item.mb; tile_n = item.tile_n; expert = item.expert;
   } else {
     const int nitems = p.tiles_n * p.m_blocks;
     const int per_xcd = (nitems + 7) >> 3;
@@ -547,7 +570,6 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   const int n0 = tile_n * kTileN;
   const int block_m = MOE ? p.block_m : TM;
   const int slot0 = mb * block_m;
-  const int expert = MOE ? p.expert_ids[mb] : 0;
   const int nrows = MOE ? p.num_valid : p.M;  // exclusive bound of a valid slot
 
   const int kb_begin = SPLIT ? split * p.kb_per_split : 0;

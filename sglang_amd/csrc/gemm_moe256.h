@@ -29,29 +29,10 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int wn = w & 3, wm = w >> 2;
 
-  // ---- work item: each XCD takes a contiguous run of the blocks in use and walks all n tiles of a block
-  const int bid = blockIdx.x;
-  const int used = min(p.num_post_pad[0] / TM, p.m_blocks);
-  const int per_xcd = (used + 7) >> 3;
-  const int j = bid >> 3;
-  const int mbl = j / p.tiles_n;
-  if (mbl >= per_xcd) return;
-  const int first_blk = (bid & 7) * per_xcd, end_blk = min(first_blk + per_xcd, used);
-  int mb = first_blk + mbl;
-  if (mb >= end_blk) return;
-  // Blocks of one expert that sit next to each other in the run form groups of up to kShare; inside a group
-  // consecutive workgroup ids walk the blocks first and the n tiles second, so the workgroups that stream
-  // the same weight tile are dispatched together and share it in L2.
-  constexpr int kShare = 4;
-  const int expert = p.expert_ids[mb];
-  int idx = 0;  // position of this block inside its run of equal expert ids
-  while (mb - idx > first_blk && p.expert_ids[mb - idx - 1] == expert) ++idx;
-  const int gfirst = mb - (idx & (kShare - 1));
-  int g = (idx & (kShare - 1)) + 1;  // group size: forward to the end of the run, at most kShare
-  while (g < kShare && gfirst + g < end_blk && p.expert_ids[gfirst + g] == expert) ++g;
-  const int r = j - (gfirst - first_blk) * p.tiles_n;  // slot inside the group: 0 .. g*tiles_n-1
-  const int tile_n = r / g;
-  mb = gfirst + (r - tile_n * g);
+  // ---- work item (moe_work_item(): contiguous run of blocks per XCD, same-expert blocks of a window grouped)
+  const MoeItem item = moe_work_item(p, (int)blockIdx.x);
+  if (item.mb < 0) return;
+  const int mb = item.mb, tile_n = item.tile_n, expert = item.expert;
   const int n0 = tile_n * kTileN;
   const int slot0 = mb * TM;
   const int nrows = p.num_valid;
