@@ -31,6 +31,7 @@ inline bool aligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_
 
 // ---------------------------------------------------------------- device: types
 typedef int v2i __attribute__((ext_vector_type(2)));
+typedef float v2f __attribute__((ext_vector_type(2)));
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v8i __attribute__((ext_vector_type(8)));
 typedef float v4f __attribute__((ext_vector_type(4)));

@@ -18,7 +18,9 @@
 
 namespace fp8k {
 
-template <int OUT_DT>
+// PAIRS: the activation scales are row-major (stride 1 between K blocks, even stride between rows, base aligned to
+// 8 bytes; the host checks), and a lane fetches two K blocks per load.
+template <int OUT_DT, bool PAIRS>
 __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p) {
   constexpr int TM = 256, WST = 3, XST = 2, MS = 4, NS = 2, LW = 4;  // LW: wave loads per tile per stage
   constexpr int WBYTES = kTileN * kTileK, XBYTES = TM * kTileK;
@@ -121,27 +123,45 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
 
-  float sxa[MS], sxb[MS], sba = 0.f, sbb = 0.f;  // scales of the even / odd K blocks in flight
-  auto load_scales = [&](float (&sx)[MS], float& sb, int kb) {
+  v2f sxp[MS];                 // activation scales of the even ([0]) and odd ([1]) K block in flight
+  float sba = 0.f, sbb = 0.f;  // weight scales of the same two blocks
+  // Activation scales.  With row-major scales (one row's K blocks next to each other: sx_k == 1, even row stride)
+  // a lane fetches two K blocks per load, every other trip: the rows of a block are gathered, so every lane's
+  // load is a cache line of its own whatever the layout, and what counts is the number of load instructions
+  // (one per K block and 32 slots would take more of the CU's load path than the operand tiles themselves) and
+  // that a row's line is met again on the following trips.  Other layouts fall back to one load per K block.
+  constexpr bool pairs = PAIRS;
+  const rsrc_t rS = make_rsrc(p.sx, (uint32_t)(((xrows - 1) * p.sx_m + nkb) * 4));  // used by the paired loads only
+  auto load_sb = [&](float& sb, int kb) { sb = swp[(int64_t)min(kb, nkb - 1) * p.sw_k]; };
+  auto load_sx = [&](int parity, int kb) {
     const int kn = min(kb, nkb - 1);
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) sx[ms] = p.sx[sxo[ms] + (uint32_t)(kn * (int)p.sx_k)];
-    sb = swp[(int64_t)kn * p.sw_k];
+    for (int ms = 0; ms < MS; ++ms) sxp[ms][parity] = p.sx[sxo[ms] + (uint32_t)(kn * (int)p.sx_k)];
   };
-  load_scales(sxa, sba, 0);
-  load_scales(sxb, sbb, 1);
+  auto load_sx_pair = [&](int kb) {  // kb even: blocks kb and kb+1 (past the tensor: zero)
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms)
+      sxp[ms] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rS, (int)((sxo[ms] + (uint32_t)kb) * 4u), 0, 0));
+  };
+  if (pairs) load_sx_pair(0);
+  else { load_sx(0, 0); load_sx(1, 1); }
+  load_sb(sba, 0);
+  load_sb(sbb, 1);
   __builtin_amdgcn_sched_barrier(0);
   issue_x(0);
   issue_w(0);
   issue_w(1);
 
-  // one K block; (sx, sb) hold its scales on entry and are reloaded with those of block it+2
-  auto trip = [&](int it, float (&sx)[MS], float& sb) {
+  // one K block; its scales sit in sxp[.][parity] and sb on entry; the odd trips reload both blocks' activation
+  // scales in the paired form
+  auto trip = [&](int it, int parity, float& sb) {
     lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
     float sc[MS];
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) sc[ms] = sx[ms] * sb;
-    load_scales(sx, sb, it + 2);
+    for (int ms = 0; ms < MS; ++ms) sc[ms] = sxp[ms][parity] * sb;
+    if (!pairs) load_sx(parity, it + 2);
+    else if (parity) load_sx_pair(it + 1);
+    load_sb(sb, it + 2);
     __builtin_amdgcn_sched_barrier(0);  // scales, then activations, then weights
     issue_x(it + 1);                    // into the stage of block it-1, which every wave has left
     issue_w(it + 2);
@@ -172,10 +192,10 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   };
   int it = 0;
   for (; it + 1 < nkb; it += 2) {
-    trip(it, sxa, sba);
-    trip(it + 1, sxb, sbb);
+    trip(it, 0, sba);
+    trip(it + 1, 1, sbb);
   }
-  if (it < nkb) trip(it, sxa, sba);
+  if (it < nkb) trip(it, 0, sba);
   wait_vm0();     // the loads past the last K block still target the stages
   lds_barrier();  // every wave has left the stages: they become the output staging area
 

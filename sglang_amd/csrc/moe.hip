@@ -299,11 +299,18 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
   }
 #undef FP8K_MOE_DIRECT
   FP8K_REQUIRE(xrows * as_stride_m + (K / kTileK) * as_stride_k < 0xffffffffLL, "%s: activation scale tensor too large", op);
-  if (block_m == 256) {  // 129..256 and more slots per expert: both 128-row halves on one weight stage
-    if (out_dtype == FP8K_BF16)
-      hipLaunchKernelGGL((moe_stream256_kernel<FP8K_BF16>), dim3((unsigned)nwg), dim3(512), 0, st, a);
-    else
-      hipLaunchKernelGGL((moe_stream256_kernel<FP8K_F16>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+  if (block_m == 256) {
+    // row-major activation scales (what fused_experts_impl produces for 256-slot blocks) take the form that fetches
+    // two K blocks per load
+    const bool pairs = as_stride_k == 1 && (as_stride_m & 1) == 0 && aligned(As, 8);  // 129..256 and more slots per expert: both 128-row halves on one weight stage
+#define FP8K_MOE256(O) \
+  do { \
+    if (pairs) hipLaunchKernelGGL((moe_stream256_kernel<O, true>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
+    else hipLaunchKernelGGL((moe_stream256_kernel<O, false>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
+  } while (0)
+    if (out_dtype == FP8K_BF16) FP8K_MOE256(FP8K_BF16);
+    else FP8K_MOE256(FP8K_F16);
+#undef FP8K_MOE256
     return check_launch(op);
   }
 #define FP8K_MOE(TM, NST, NW, O) \

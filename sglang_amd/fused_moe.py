@@ -105,8 +105,9 @@ def invoke_fused_moe_kernel(
     assert B_scale is not None
     if A.dtype != torch.float8_e4m3fn:
         assert A_scale is None
-        # column-major scales: one coalesced load per K block for the lanes of a wave (any layout is accepted)
-        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1], column_major_scales=True)
+        # 256-slot blocks: row-major scales (the kernel gathers rows and fetches a row's scales two K blocks at a
+        # time); smaller blocks measured better with column-major ones
+        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] != 256)
     assert (A.shape[-1] + 127) // 128 == A_scale.shape[-1]
     assert (B.shape[-2] + 127) // 128 == B_scale.shape[-2]
     assert (B.shape[-1] + 127) // 128 == B_scale.shape[-1]
@@ -203,7 +204,8 @@ def fused_experts_impl(
         )
         # silu_and_mul fused into the requantisation (same bytes as silu_and_mul + group quant, one pass less
         # over the [tokens*topk, N] intermediate)
-        a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=True, fuse_silu_and_mul=True)
+        a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] != 256,
+                                                      fuse_silu_and_mul=True)
         invoke_fused_moe_kernel(
             a2_q, w2, None, ic3, a2_s, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
             num_tokens_post_padded, True, 1, config, use_fp8_w8a8=True, block_shape=block_shape,
