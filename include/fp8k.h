@@ -108,7 +108,8 @@ int fp8k_tensor_quant(const void* x, void* q, float* s, int64_t numel, int in_dt
  * As float, element (m,kb) at As[m*as_stride_m + kb*as_stride_k]; Bs float, element (nb,kb) at
  * Bs[nb*bs_stride_n + kb*bs_stride_k].  C [M,N] of out_dtype (F16/BF16), ldc elements between rows.
  * K % 16 == 0, lda % 16 == 0, ldb % 16 == 0, ldc*2 % 16 == 0.
- * workspace: device scratch of at least fp8k_block_gemm_workspace_bytes(M,N,K) bytes (may be 0 -> NULL ok).
+ * workspace: device scratch of at least fp8k_block_gemm_workspace_bytes(M,N,K) bytes (may be 0 -> NULL ok): float
+ *   partials of K-cut launches and, for more than 32 rows, room for a column-major copy of row-major scales_a.
  */
 int fp8k_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M, int64_t N,
                     int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,

@@ -72,7 +72,9 @@ def test_invalid_arguments_are_rejected_on_the_host():
     assert need > 0
     rc = lib.fp8k_block_gemm(p, p, p, p, p, 16, 7168, 16384, 16384, 16384, 128, 1, 128, 1, 7168, _lib.BF16, None, 0, None)
     assert rc == 4 and b"workspace" in lib.fp8k_last_error()
-    assert lib.fp8k_block_gemm_workspace_bytes(4096, 7168, 16384) == 0
+    # no K cut at this shape: only the area for a column-major copy of the activation scales
+    assert lib.fp8k_block_gemm_workspace_bytes(4096, 7168, 16384) == 4096 * 128 * 4
+    assert lib.fp8k_scaled_mm_workspace_bytes(4096, 7168, 16384) == 0
     rc = lib.fp8k_token_quant(p, p, p, 4, 100, _lib.BF16, None)
     assert rc == 1 and b"divisible by 8" in lib.fp8k_last_error()
     rc = lib.fp8k_scaled_mm(p, p, p, p, p, p, 4, 256, 256, 256, 256, 256, _lib.BF16, 7, None, 0, None)

@@ -101,8 +101,11 @@ def test_tile128_strided_output_rows(dev, tile128):
     for ldc in (N + 4, N + 8):
         C = torch.full((M, ldc), 7.0, dtype=torch.bfloat16, device=dev)
         tile128(1)
+        need = lib.fp8k_block_gemm_workspace_bytes(M, N, K)
+        ws = torch.empty(max(need, 1), dtype=torch.uint8, device=dev)
         check(lib.fp8k_block_gemm(A.data_ptr(), B.data_ptr(), As.data_ptr(), Bs.data_ptr(), C.data_ptr(), M, N, K, K, K,
-                                  As.stride(0), As.stride(1), Bs.stride(0), Bs.stride(1), ldc, 2, None, 0, stream_ptr(dev)))
+                                  As.stride(0), As.stride(1), Bs.stride(0), Bs.stride(1), ldc, 2, ws.data_ptr(), need,
+                                  stream_ptr(dev)))
         torch.cuda.synchronize()
         out = C.float().cpu().numpy()
         assert _rel_err(out[:, :N], ref) <= REL_TOL
