@@ -180,6 +180,8 @@ int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64, int64_t n
  * rows); As float (as_stride_m, as_stride_k); Bs float [E, ceil(N/128), K/128] (bs_stride_e, bs_stride_n,
  * bs_stride_k); C [num_valid_tokens, N] of out_dtype (ldc).  block_m in {16,32,64,128,256} is the block size
  * moe_align_block_size was called with; sorted_capacity = length of sorted_token_ids.  K % 128 == 0, N % 8 == 0.
+ * as_sorted != 0 (block_m >= 64): As holds one row per position of sorted_token_ids instead of one per token
+ * (see fp8k_moe_sort_scales).
  */
 int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
                         const int32_t* sorted_token_ids, const int32_t* expert_ids,
@@ -187,7 +189,18 @@ int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const flo
                         int64_t block_m, int64_t num_valid_tokens, int64_t top_k, int64_t num_experts, int64_t N,
                         int64_t K, int64_t lda, int64_t as_stride_m, int64_t as_stride_k, int64_t b_stride_e,
                         int64_t ldb, int64_t bs_stride_e, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc,
-                        int out_dtype, void* stream);
+                        int out_dtype, int as_sorted, void* stream);
+
+/*
+ * Activation scales in the order of sorted_token_ids (no counterpart in the reference, whose Triton kernel gathers
+ * them per K block): out[kb * sorted_capacity + i] = As[sorted_token_ids[i] / top_k, kb] for i below
+ * num_tokens_post_padded[0], 0 for padding entries.  Passing `out` to fp8k_moe_block_gemm with as_stride_m = 1,
+ * as_stride_k = sorted_capacity and as_sorted = 1 lets the lanes of a wave fetch their scales from one cache line
+ * instead of one line per token row.
+ */
+int fp8k_moe_sort_scales(const float* As, float* out, const int32_t* sorted_token_ids,
+                         const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t k_blocks, int64_t top_k,
+                         int64_t num_valid_tokens, int64_t as_stride_m, int64_t as_stride_k, void* stream);
 
 /*
  * out[r, c] = silu(x[r, c]) * x[r, d + c] for c < d, computed as the reference does for 16-bit types:

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libfp8k.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 F32, F16, BF16 = 0, 1, 2
 SCALE_F32, SCALE_UE8M0_PACKED = 0, 1
@@ -63,7 +63,8 @@ SIGNATURES = {
         _c_int,
         [_c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr],
     ),
-    "fp8k_moe_block_gemm": (_c_int, [_c_ptr] * 9 + [_c_i64] * 16 + [_c_int, _c_ptr]),
+    "fp8k_moe_block_gemm": (_c_int, [_c_ptr] * 9 + [_c_i64] * 16 + [_c_int, _c_int, _c_ptr]),
+    "fp8k_moe_sort_scales": (_c_int, [_c_ptr] * 4 + [_c_i64] * 6 + [_c_ptr]),
     "fp8k_silu_and_mul": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr]),
     "fp8k_moe_sum_reduce": (_c_int, [_c_ptr, _c_ptr] + [_c_i64] * 6 + [_c_f32, _c_int, _c_ptr]),
     "fp8k_moe_fused_gate": (

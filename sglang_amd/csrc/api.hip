@@ -18,4 +18,4 @@ void clear_error() { g_err[0] = 0; }
 }  // namespace fp8k
 
 extern "C" const char* fp8k_last_error(void) { return fp8k::g_err; }
-extern "C" int fp8k_abi_version(void) { return 1; }
+extern "C" int fp8k_abi_version(void) { return 2; }

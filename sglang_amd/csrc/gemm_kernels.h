@@ -35,6 +35,7 @@ struct GemmArgs {
   int num_valid;                // number of real slots (topk_ids.numel())
   int m_blocks;                 // dense: blocks of TM rows; grouped: capacity of sorted_ids in blocks
   int block_m;                  // grouped: slots per block in sorted_ids (<= TM)
+  int sx_sorted;                // grouped: sx holds one row per position of sorted_ids (row = position), not per token
   int64_t w_expert_stride;      // bytes between experts in W
   int64_t sw_expert_stride;     // floats between experts in sw
 };
@@ -662,7 +663,8 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   const float* sxp[MS];
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
-    const int64_t xr = out_ok[ms] ? (MOE ? out_slot[ms] / p.top_k : out_slot[ms]) : 0;
+    int64_t xr = out_ok[ms] ? (MOE ? out_slot[ms] / p.top_k : out_slot[ms]) : 0;
+    if (MOE && p.sx_sorted) xr = slot0 + mrow0 + ms * 32 + lr;
     sxp[ms] = p.sx + xr * p.sx_m + (int64_t)kb_begin * p.sx_k;
   }
   const int nb = min(n0 + wn * 32, p.N - 1) >> 7;

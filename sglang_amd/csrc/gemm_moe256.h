@@ -109,7 +109,8 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
     const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
-    sxo[ms] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u;
+    sxo[ms] = p.sx_sorted ? (uint32_t)((int64_t)(slot0 + wm * 128 + ms * 32 + lr) * p.sx_m)
+                          : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
   }
   const int nb = min(n0 + wn * 64, p.N - 1) >> 7;  // the wave's 64 weight rows lie inside one 128-row block
   const float* swp = p.sw + (int64_t)expert * p.sw_expert_stride + (int64_t)nb * p.sw_n;

@@ -238,13 +238,47 @@ extern "C" int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64
   return check_launch("moe_align_block_size");
 }
 
+// Activation scales in the order of sorted_token_ids: out[kb * capacity + i] = As[sorted_token_ids[i] / top_k, kb]
+// (0 for padding), for i < num_tokens_post_padded.  One lane per position walks its row's K blocks, so every
+// store instruction writes 256 contiguous bytes.
+__global__ __launch_bounds__(256) void moe_sort_scales_kernel(const float* __restrict__ As, float* __restrict__ out,
+                                                              const int32_t* __restrict__ sorted_ids,
+                                                              const int32_t* __restrict__ npad, int capacity, int kb,
+                                                              int top_k, int num_valid, int64_t sm, int64_t sk) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= min(npad[0], capacity)) return;
+  const int s = sorted_ids[i];
+  const bool ok = s < num_valid;
+  const float* row = As + (int64_t)(ok ? s / top_k : 0) * sm;
+  for (int k = 0; k < kb; ++k) out[(int64_t)k * capacity + i] = ok ? row[(int64_t)k * sk] : 0.f;
+}
+
+extern "C" int fp8k_moe_sort_scales(const float* As, float* out, const int32_t* sorted_token_ids,
+                                    const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t k_blocks,
+                                    int64_t top_k, int64_t num_valid_tokens, int64_t as_stride_m, int64_t as_stride_k,
+                                    void* stream) {
+  clear_error();
+  const char* op = "moe_sort_scales";
+  FP8K_REQUIRE(sorted_capacity >= 0 && sorted_capacity < 0x7fffffffLL && k_blocks >= 0 && k_blocks < 0x7fffffffLL,
+               "%s: bad shape", op);
+  FP8K_REQUIRE(top_k > 0 && num_valid_tokens >= 0 && num_valid_tokens < 0x7fffffffLL, "%s: bad shape", op);
+  FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0, "%s: negative scale stride", op);
+  if (sorted_capacity == 0 || k_blocks == 0) return FP8K_OK;
+  FP8K_REQUIRE(As && out && sorted_token_ids && num_tokens_post_padded, "%s: null pointer", op);
+  hipLaunchKernelGGL(moe_sort_scales_kernel, dim3((unsigned)((sorted_capacity + 255) / 256)), dim3(256), 0,
+                     (hipStream_t)stream, As, out, sorted_token_ids, num_tokens_post_padded, (int)sorted_capacity,
+                     (int)k_blocks, (int)top_k, (int)num_valid_tokens, as_stride_m, as_stride_k);
+  return check_launch(op);
+}
+
 extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
                                    const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                    const int32_t* num_tokens_post_padded, const float* topk_weights,
                                    int64_t sorted_capacity, int64_t block_m, int64_t num_valid_tokens, int64_t top_k,
                                    int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_m,
                                    int64_t as_stride_k, int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e,
-                                   int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* stream) {
+                                   int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, int as_sorted,
+                                   void* stream) {
   clear_error();
   const char* op = "moe_block_gemm";
   FP8K_REQUIRE(N > 0 && K > 0 && num_experts > 0 && top_k > 0, "%s: bad shape", op);
@@ -279,6 +313,8 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
   a.m_blocks = (int)(sorted_capacity / block_m);
   a.block_m = (int)block_m;
   a.w_expert_stride = b_stride_e; a.sw_expert_stride = bs_stride_e;
+  a.sx_sorted = as_sorted ? 1 : 0;
+  FP8K_REQUIRE(!as_sorted || block_m >= 64, "%s: scales in sorted order are taken with block_m >= 64", op);
   const bool direct = block_m <= 32;  // few rows per expert: weights go straight to registers, 128-row tiles
   if (direct) a.tiles_n = (int)((N + kDirTileN - 1) / kDirTileN);
   const int64_t per_xcd = (a.m_blocks + 7) / 8;
@@ -298,11 +334,12 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
     return check_launch(op);
   }
 #undef FP8K_MOE_DIRECT
-  FP8K_REQUIRE(xrows * as_stride_m + (K / kTileK) * as_stride_k < 0xffffffffLL, "%s: activation scale tensor too large", op);
+  FP8K_REQUIRE((as_sorted ? sorted_capacity : xrows) * as_stride_m + (K / kTileK) * as_stride_k < 0x3fffffffLL,
+               "%s: activation scale tensor too large", op);
   if (block_m == 256) {
     // row-major activation scales (what fused_experts_impl produces for 256-slot blocks) take the form that fetches
     // two K blocks per load
-    const bool pairs = as_stride_k == 1 && (as_stride_m & 1) == 0 && aligned(As, 8);  // 129..256 and more slots per expert: both 128-row halves on one weight stage
+    const bool pairs = !as_sorted && as_stride_k == 1 && (as_stride_m & 1) == 0 && aligned(As, 8);  // 129..256 and more slots per expert: both 128-row halves on one weight stage
 #define FP8K_MOE256(O) \
   do { \
     if (pairs) hipLaunchKernelGGL((moe_stream256_kernel<O, true>), dim3((unsigned)nwg), dim3(512), 0, st, a); \

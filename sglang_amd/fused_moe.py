@@ -63,6 +63,10 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}
 
 
+# block sizes from which the activation scales are first gathered into the order of sorted_token_ids
+SORT_SCALES_MIN_BLOCK = 64
+
+
 def invoke_fused_moe_kernel(
     A: torch.Tensor,
     B: torch.Tensor,
@@ -105,15 +109,20 @@ def invoke_fused_moe_kernel(
     assert B_scale is not None
     if A.dtype != torch.float8_e4m3fn:
         assert A_scale is None
-        # 256-slot blocks: row-major scales (the kernel gathers rows and fetches a row's scales two K blocks at a
-        # time); smaller blocks measured better with column-major ones
-        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] != 256)
+        # blocks of 64 slots and more: row-major scales, which moe_sort_scales reads a row at a time
+        A, A_scale = sglang_per_token_group_quant_fp8(A, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] < 64)
     assert (A.shape[-1] + 127) // 128 == A_scale.shape[-1]
     assert (B.shape[-2] + 127) // 128 == B_scale.shape[-2]
     assert (B.shape[-1] + 127) // 128 == B_scale.shape[-1]
+    block_m = int(config["BLOCK_SIZE_M"])
+    sort_scales = block_m >= SORT_SCALES_MIN_BLOCK
+    if sort_scales:
+        # the rows of a block are gathered: with the scales in the order of sorted_token_ids the lanes of a wave read
+        # theirs from one cache line instead of one line per token row
+        A_scale = _ops.moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k, topk_ids.numel())
     _ops.moe_block_gemm(
         A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-        mul_routed_weight, top_k, int(config["BLOCK_SIZE_M"]), topk_ids.numel(),
+        mul_routed_weight, top_k, block_m, topk_ids.numel(), scales_sorted=sort_scales,
     )
 
 
@@ -204,7 +213,7 @@ def fused_experts_impl(
         )
         # silu_and_mul fused into the requantisation (same bytes as silu_and_mul + group quant, one pass less
         # over the [tokens*topk, N] intermediate)
-        a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] != 256,
+        a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] < 64,
                                                       fuse_silu_and_mul=True)
         invoke_fused_moe_kernel(
             a2_q, w2, None, ic3, a2_s, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,

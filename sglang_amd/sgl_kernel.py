@@ -454,10 +454,30 @@ def moe_sum_reduce(input_tensor: torch.Tensor, output_tensor: torch.Tensor, rout
                                   dtype_code(input_tensor.dtype), stream_ptr(input_tensor.device)))
 
 
+def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: int, num_valid_tokens: int) -> torch.Tensor:
+    """Activation scales gathered into the order of sorted_token_ids (see include/fp8k.h: fp8k_moe_sort_scales):
+    returns a [len(sorted_token_ids), K/128] view with strides (1, len): row i holds the scales of slot
+    sorted_token_ids[i].  Pass it to moe_block_gemm with scales_sorted=True."""
+    require_cuda(A_scale, sorted_token_ids, num_tokens_post_padded)
+    if A_scale.dtype != torch.float32 or A_scale.dim() != 2:
+        raise RuntimeError("moe_sort_scales: A_scale must be Float32 [rows, K/128]")
+    cap, kb = sorted_token_ids.numel(), A_scale.shape[1]
+    out = torch.empty((kb, cap), dtype=torch.float32, device=A_scale.device)
+    check(
+        lib.fp8k_moe_sort_scales(
+            A_scale.data_ptr(), out.data_ptr(), sorted_token_ids.data_ptr(), num_tokens_post_padded.data_ptr(), cap, kb,
+            top_k, num_valid_tokens, A_scale.stride(0), A_scale.stride(1), stream_ptr(A_scale.device),
+        )
+    )
+    return out.t()
+
+
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                   mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int) -> None:
+                   mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int,
+                   scales_sorted: bool = False) -> None:
     """Grouped block-FP8 GEMM behind invoke_fused_moe_kernel (see include/fp8k.h: fp8k_moe_block_gemm).
-    A e4m3fn [rows, K]; B e4m3fn [E, N, K]; A_scale float32 [rows, K/128]; B_scale float32 [E, N/128, K/128];
+    A e4m3fn [rows, K]; B e4m3fn [E, N, K]; A_scale float32 [rows, K/128] (scales_sorted: one row per entry of
+    sorted_token_ids, from moe_sort_scales); B_scale float32 [E, N/128, K/128];
     C [num_valid_tokens, N] (any leading shape, flattened) bf16/fp16, written in place."""
     require_cuda(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded)
     if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
@@ -469,7 +489,7 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
     E, N, K = B.shape
     if A.shape[1] != K or (K > 1 and (A.stride(1) != 1 or B.stride(2) != 1)):
         raise RuntimeError("moe_block_gemm: K must be the contiguous dimension of A and B")
-    if A_scale.shape[0] != A.shape[0] or A_scale.shape[1] != (K + 127) // 128:
+    if A_scale.shape[0] != (sorted_token_ids.numel() if scales_sorted else A.shape[0]) or A_scale.shape[1] != (K + 127) // 128:
         raise RuntimeError("moe_block_gemm: A_scale shape does not match A")
     if B_scale.shape[0] != E or B_scale.shape[1] != (N + 127) // 128 or B_scale.shape[2] != (K + 127) // 128:
         raise RuntimeError("moe_block_gemm: B_scale shape does not match B")
@@ -493,7 +513,7 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
             topk_weights.data_ptr() if mul_routed_weight else None, sorted_token_ids.numel(), block_m,
             num_valid_tokens, top_k, E, N, K, A.stride(0), A_scale.stride(0), A_scale.stride(1), B.stride(0),
             B.stride(1), B_scale.stride(0), B_scale.stride(1), B_scale.stride(2), C2.stride(0), _out_code(C.dtype),
-            stream_ptr(A.device),
+            1 if scales_sorted else 0, stream_ptr(A.device),
         )
     )
 

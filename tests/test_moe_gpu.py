@@ -158,7 +158,7 @@ def _expert_weights(rng, E, N, K):
 def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block, out_dtype):
     """GEMM1 form (row = slot // top_k, no routed weight) and GEMM2 form (row = slot, times routed weight)."""
     from sglang_amd.fused_moe import moe_align_block_size
-    from sglang_amd.sgl_kernel import moe_block_gemm
+    from sglang_amd.sgl_kernel import moe_block_gemm, moe_sort_scales
 
     rng = np.random.default_rng(T * 7 + N)
     ids = _random_ids(rng, T, E, topk, 0.1 if T > 5 else 0.0)
@@ -188,6 +188,20 @@ def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block, out_dtype):
             ref[slots] = part * (tw.reshape(-1)[slots][:, None] if mul else 1.0)
         assert (got[flat == -1] == 0).all()
         assert _rel_err(got, ref) <= REL_TOL
+        if block >= 64:
+            # scales gathered into sorted-slot order first: same arithmetic, so the same bits
+            for xs_dev in (torch.from_numpy(xs).to(dev), torch.from_numpy(np.ascontiguousarray(xs.T)).to(dev).t()):
+                srt = moe_sort_scales(xs_dev, sorted_ids, npad, top_k, ids.size)
+                n_used = int(npad.item())
+                sid = sorted_ids.cpu().numpy()[:n_used]
+                live = sid < ids.size
+                assert srt.shape == (sorted_ids.numel(), K // 128)
+                np.testing.assert_array_equal(srt.cpu().numpy()[:n_used][live], xs[sid[live] // top_k])
+                C2 = torch.full((T * topk, N), float("nan"), dtype=out_dtype, device=dev)
+                moe_block_gemm(fp8_tensor(xq, dev), Bq, C2, srt, Bs, torch.from_numpy(tw).to(dev),
+                               sorted_ids, expert_ids, npad, mul, top_k, block, ids.size, scales_sorted=True)
+                torch.cuda.synchronize()
+                assert torch.equal(C2, C)
 
 
 def test_grouped_gemm_exact_on_integers(dev):
