@@ -238,6 +238,7 @@ extern "C" int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64
   return check_launch("moe_align_block_size");
 }
 
+namespace fp8k {
 // Activation scales in the order of sorted_token_ids: out[kb * capacity + i] = As[sorted_token_ids[i] / top_k, kb]
 // (0 for padding), for i < num_tokens_post_padded.  One lane per position walks its row's K blocks, so every
 // store instruction writes 256 contiguous bytes.
@@ -252,6 +253,7 @@ __global__ __launch_bounds__(256) void moe_sort_scales_kernel(const float* __res
   const float* row = As + (int64_t)(ok ? s / top_k : 0) * sm;
   for (int k = 0; k < kb; ++k) out[(int64_t)k * capacity + i] = ok ? row[(int64_t)k * sk] : 0.f;
 }
+}  // namespace fp8k
 
 extern "C" int fp8k_moe_sort_scales(const float* As, float* out, const int32_t* sorted_token_ids,
                                     const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t k_blocks,
