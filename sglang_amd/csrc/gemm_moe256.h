@@ -9,10 +9,12 @@
 //   LDS = 3 weight stages (32 KB each) + 2 activation stages (32 KB each) = 160 KB, the whole CU.
 //   Activation tiles are re-read by every n tile of the block and come from L2; one stage ahead is enough.
 //   Waves: 4 along n (64 weight rows) x 2 along m (128 slots), 2 x 4 MFMA tiles of 32x32 each (24 KB of LDS
-//   operands per 16 MFMAs); a half without real slots skips its MFMAs.
+//   operands per 16 MFMAs); 32-slot groups without real slots skip their MFMAs.
 // Load order inside a K block is scales, activations, weights, so that at the next barrier only the four
 // youngest weight loads of each wave may still be in flight (memory operations retire in order).
 #pragma once
+
+#include <type_traits>
 
 #include "gemm_kernels.h"
 
@@ -53,9 +55,6 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     }
     return;
   }
-  // real slots come first in a block: the upper half is in use iff its first slot is
-  const bool active = wm == 0 || __builtin_amdgcn_readfirstlane(p.sorted_ids[slot0 + 128]) < nrows;
-
   // ---- global -> LDS: a wave load covers 8 rows (lane: row lane/8, 16-byte chunk lane%8, stored at chunk
   // position c ^ ((row>>1)&7)); whole offsets travel in the bounds-checked per-lane operand
   const uint8_t* Wb = p.W + (int64_t)expert * p.w_expert_stride;
@@ -106,9 +105,11 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 
   // ---- scales: activation scale rows follow the activation rows
   uint32_t sxo[MS];  // element offsets into the activation scales (the host checks they fit 32 bits)
+  int nact = 0;      // 32-slot groups of the wave's half that hold real slots (a prefix: real slots come first)
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
     const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
+    nact += __builtin_amdgcn_readfirstlane(s) < nrows ? 1 : 0;
     sxo[ms] = p.sx_sorted ? (uint32_t)((int64_t)(slot0 + wm * 128 + ms * 32 + lr) * p.sx_m)
                           : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
   }
@@ -155,7 +156,8 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 
   // one K block; its scales sit in sxp[.][parity] and sb on entry; the odd trips reload both blocks' activation
   // scales in the paired form
-  auto trip = [&](int it, int parity, float& sb) {
+  auto trip = [&](auto na, int it, int parity, float& sb) {
+    constexpr int NA = decltype(na)::value;  // 32-slot groups of the wave's half with real slots
     lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
     float sc[MS];
 #pragma unroll
@@ -166,7 +168,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     __builtin_amdgcn_sched_barrier(0);  // scales, then activations, then weights
     issue_x(it + 1);                    // into the stage of block it-1, which every wave has left
     issue_w(it + 2);
-    if (!active) return;
+    if (NA == 0) return;
     const uint8_t* sw_ = smem + (it % WST) * WBYTES;
     const uint8_t* sx_ = smem + XBASE + (it & 1) * XBYTES;
     v8i wf[NS][2];
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       wf[ns][1] = frag(sw_, rdW + ns * 32 * kTileK, 1);
     }
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) {
+    for (int ms = 0; ms < NA; ++ms) {  // groups past the expert's last slot are padding
       const v8i x0 = frag(sx_, rdX + ms * 32 * kTileK, 0);
       const v8i x1 = frag(sx_, rdX + ms * 32 * kTileK, 1);
 #pragma unroll
@@ -191,12 +193,24 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       }
     }
   };
-  int it = 0;
-  for (; it + 1 < nkb; it += 2) {
-    trip(it, 0, sba);
-    trip(it + 1, 1, sbb);
+  auto run = [&](auto na) {
+    int it = 0;
+    for (; it + 1 < nkb; it += 2) {
+      trip(na, it, 0, sba);
+      trip(na, it + 1, 1, sbb);
+    }
+    if (it < nkb) trip(na, it, 0, sba);
+  };
+  // one copy of the loop per group count keeps every copy straight-line.  (The four-group copy needs all 256
+  // registers; the compiler parks a few epilogue values in scratch around it, outside the loops, where those
+  // accesses are older than every load the partial waits count.)
+  switch (nact) {  // wave-uniform
+    case 4: run(std::integral_constant<int, 4>{}); break;
+    case 3: run(std::integral_constant<int, 3>{}); break;
+    case 2: run(std::integral_constant<int, 2>{}); break;
+    case 1: run(std::integral_constant<int, 1>{}); break;
+    default: run(std::integral_constant<int, 0>{}); break;
   }
-  if (it < nkb) trip(it, 0, sba);
   wait_vm0();     // the loads past the last K block still target the stages
   lds_barrier();  // every wave has left the stages: they become the output staging area
 

@@ -204,6 +204,33 @@ def test_grouped_gemm_vs_oracle(dev, T, E, topk, N, K, block, out_dtype):
                 assert torch.equal(C2, C)
 
 
+def test_grouped_gemm_256_slot_blocks_every_group_count(dev):
+    """Experts whose last 256-slot block holds 1..8 groups of 32 slots (the kernel skips the padding groups)."""
+    from sglang_amd.fused_moe import moe_align_block_size
+    from sglang_amd.sgl_kernel import moe_block_gemm
+
+    rng = np.random.default_rng(11)
+    counts = [1, 32, 33, 65, 97, 128, 129, 161, 193, 225, 256, 257, 0, 300]
+    E, N, K, block = len(counts), 512, 384, 256
+    ids = rng.permutation(np.repeat(np.arange(E, dtype=np.int32), counts))[:, None]
+    T = ids.shape[0]
+    wq, ws = _expert_weights(rng, E, N, K)
+    xq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((T, K)).astype(np.float32) * 100, -448, 448))
+    xs = (rng.uniform(0.5, 2.0, (T, K // 128)) * 1e-2).astype(np.float32)
+    sorted_ids, expert_ids, npad = moe_align_block_size(torch.from_numpy(ids).to(dev), block, E)
+    C = torch.full((T, N), float("nan"), dtype=torch.bfloat16, device=dev)
+    moe_block_gemm(fp8_tensor(xq, dev), fp8_tensor(wq, dev), C, torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev),
+                   torch.ones((T, 1), device=dev), sorted_ids, expert_ids, npad, False, 1, block, T)
+    torch.cuda.synchronize()
+    got = C.float().cpu().numpy()
+    assert np.isfinite(got).all(), "some output row was not written"
+    for e in range(E):
+        rows = np.nonzero(ids[:, 0] == e)[0]
+        if rows.size:
+            ref = O.w8a8_block_fp8_matmul(xq[rows], wq[e], xs[rows], ws[e], out_dtype="f32", acc=np.float64)
+            assert _rel_err(got[rows], ref) <= REL_TOL, "expert %d with %d slots" % (e, rows.size)
+
+
 def test_grouped_gemm_exact_on_integers(dev):
     from sglang_amd.fused_moe import moe_align_block_size
     from sglang_amd.sgl_kernel import moe_block_gemm
