@@ -69,8 +69,6 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     const int g = w * LW + q;  // 8-row group, 0..31, of both tiles
     const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
     voW[q] = (uint32_t)((g * 8 + rl) * p.ldw + c * 16);
-    const int s = p.sorted_ids[slot0 + g * 8 + rl];
-    voX[q] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
   }
   auto issue_w = [&](int kstep) {
     uint8_t* base = smem + (kstep % WST) * WBYTES + w * (LW * 1024);
@@ -78,6 +76,15 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
     for (int q = 0; q < LW; ++q) buf_load16_to_lds(rW, voW[q] + ko, 0, base + q * 1024);
   };
+  issue_w(0);  // the weights do not wait for the slot table
+  issue_w(1);
+#pragma unroll
+  for (int q = 0; q < LW; ++q) {
+    const int g = w * LW + q;
+    const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
+    const int s = p.sorted_ids[slot0 + g * 8 + rl];
+    voX[q] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
+  }
   auto issue_x = [&](int kstep) {
     uint8_t* base = smem + XBASE + (kstep & 1) * XBYTES + w * (LW * 1024);
     const uint32_t ko = (uint32_t)kstep * kTileK;
@@ -151,8 +158,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   load_sb(sbb, 1);
   __builtin_amdgcn_sched_barrier(0);
   issue_x(0);
-  issue_w(0);
-  issue_w(1);
+  wait_vm0();  // the first trip's partial wait assumes the in-loop order of loads
 
   // one K block; its scales sit in sxp[.][parity] and sb on entry; the odd trips reload both blocks' activation
   // scales in the paired form
@@ -211,19 +217,29 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     case 1: run(std::integral_constant<int, 1>{}); break;
     default: run(std::integral_constant<int, 0>{}); break;
   }
+  // output rows and routed weights, fetched while the stages drain
+  const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  const int rr = lane >> 5, pc = lane & 31;
+  int oslots[MS], srow[16];
+  float rsw[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[slot0 + w * 32 + i * 2 + rr] : 0;
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) rsw[ms] = (p.topk_w && oslots[ms] < nrows) ? p.topk_w[oslots[ms]] : 1.f;
   wait_vm0();     // the loads past the last K block still target the stages
   lds_barrier();  // every wave has left the stages: they become the output staging area
 
   // ---- epilogue through LDS: [256 slots][256 n] 16-bit, 512 B per row, 16-byte chunks XOR-swizzled by the
   // row so that the accumulator-shaped 8-byte writes spread over all banks; every store instruction then
   // writes two whole 512-byte row segments
-  const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
     const int row = wm * 128 + ms * 32 + lr;
-    const int oslot = p.sorted_ids[slot0 + row];
+    const int oslot = oslots[ms];
     const bool ok = oslot < nrows;
-    const float rs = (p.topk_w && ok) ? p.topk_w[oslot] : 1.f;
+    const float rs = rsw[ms];
 #pragma unroll
     for (int nr = 0; nr < NS * 4; ++nr) {
       const int ns = nr >> 2, rg = nr & 3;
@@ -249,11 +265,10 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   }
   if (!wide) return;
   lds_barrier();
-  const int rr = lane >> 5, pc = lane & 31;
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
     const int row = w * 32 + i * 2 + rr;
-    const int s = p.sorted_ids[slot0 + row];
+    const int s = srow[i];
     const int n = n0 + (pc << 3);  // consecutive lanes store consecutive 16-byte chunks
     const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + ((pc ^ (row & 31)) << 4));
     if (s < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)s * p.ldc + n) = o;
