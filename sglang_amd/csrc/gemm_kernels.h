@@ -619,27 +619,45 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   }
   uint32_t voX[XL];
   bool xload[XL];
+  auto issue_w = [&](int kstep) {
+    uint8_t* base = smem + (kstep % NSTAGE) * STAGE;
+    const uint32_t ko = (uint32_t)kstep * kTileK;
+#pragma unroll
+    for (int j = 0; j < WL; ++j) buf_load16_to_lds(rW, voW[j] + ko, 0, base + (w * WL + j) * 1024);
+  };
+  auto issue_x = [&](int kstep) {
+    uint8_t* base = smem + (kstep % NSTAGE) * STAGE;
+    const uint32_t ko = (uint32_t)kstep * kTileK;
+#pragma unroll
+    for (int j = 0; j < XL; ++j)
+      buf_load16_to_lds(rX, voX[j] + ko, 0, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
+  };
+  auto issue = [&](int kstep) { issue_w(kstep); issue_x(kstep); };
+  // Grouped: the slot table is fetched first and the weights of the first stages behind it (loads retire in order:
+  // the table arrives without waiting for the weights, and the weights do not wait for the table).
+  int sid[XL];
 #pragma unroll
   for (int j = 0; j < XL; ++j) {
     const int grp = w * XL + j;             // 8-row group of the X tile
     xload[j] = grp < XG;                    // wave-uniform
     const int row = grp * 8 + rl;
+    sid[j] = nrows;
+    if (xload[j] && row < block_m) sid[j] = MOE ? p.sorted_ids[slot0 + row] : slot0 + row;
+  }
+  if (MOE) {
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s) issue_w(s);
+    __builtin_amdgcn_sched_barrier(0);
+  }
+#pragma unroll
+  for (int j = 0; j < XL; ++j) {
+    const int grp = w * XL + j;
     const int c = cp ^ (((grp & 1) << 2) + (rl >> 1));
-    int s = nrows;
-    if (xload[j] && row < block_m) s = MOE ? p.sorted_ids[slot0 + row] : slot0 + row;
-    const bool ok = s < nrows;
-    const int64_t xr = MOE ? s / p.top_k : s;
+    const bool ok = sid[j] < nrows;
+    const int64_t xr = MOE ? sid[j] / p.top_k : sid[j];
     voX[j] = ok ? (uint32_t)(xr * p.ldx + c * 16) : 0xF0000000u;
   }
-  auto issue = [&](int kstep) {
-    uint8_t* base = smem + (kstep % NSTAGE) * STAGE;
-    const uint32_t ko = (uint32_t)kstep * kTileK;
-#pragma unroll
-    for (int j = 0; j < WL; ++j) buf_load16_to_lds(rW, voW[j] + ko, 0, base + (w * WL + j) * 1024);
-#pragma unroll
-    for (int j = 0; j < XL; ++j)
-      buf_load16_to_lds(rX, voX[j] + ko, 0, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
-  };
 
   // ---- LDS -> MFMA operands
   const int swz = (lr >> 1) & 7;
@@ -677,7 +695,10 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
     for (int r = 0; r < 16; ++r) acc[ms][r] = 0.f;
 
 #pragma unroll
-  for (int s = 0; s < NSTAGE - 1; ++s) issue(s);
+  for (int s = 0; s < NSTAGE - 1; ++s) {
+    if (MOE) issue_x(s);  // the weights of these stages are on their way already
+    else issue(s);
+  }
   // Scales travel two K blocks ahead, and the loads of block it+2 are issued BEFORE the stage loads of the same
   // trip: memory operations retire in order, so a scale that is younger than a stage load could only be waited
   // for by draining that stage load too, which would serialise the whole pipeline on HBM latency.
@@ -693,6 +714,7 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
     load_scales(sxa, sba, 0);
     load_scales(sxb, sbb, 1);
   }
+  if (MOE) wait_vm0();  // the grouped prologue issues its loads in another order than the trips' partial waits assume
 
   // one K block; (sx, sb) hold its scales on entry and are reloaded with those of block it+2
   auto trip = [&](int it, float (&sx)[MS], float& sb) {
@@ -735,21 +757,32 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
     trip(it + 1, sxb, sbb);
   }
   if (it < nkb) trip(it, sxa, sba);
+  // routed weights and the output rows of the store loop, fetched while the stages drain
+  const bool wide = !SPLIT && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  float rsw[MS];
+  int srow[TM / NW / 2];
+  if (MOE) {
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) rsw[ms] = (p.topk_w && out_ok[ms]) ? p.topk_w[out_slot[ms]] : 1.f;
+#pragma unroll
+    for (int i = 0; i < TM / NW / 2; ++i) {
+      const int row = w * (TM / NW) + i * 2 + (lane >> 5);
+      srow[i] = (wide && row < block_m) ? p.sorted_ids[slot0 + row] : nrows;
+    }
+  }
   wait_vm0();  // drain the padding loads before the LDS allocation is released
 
   // ---- epilogue.  Finished 16-bit tiles leave through LDS ([TM rows][256 n], 512 B per row, 16-byte chunks
   // XOR-swizzled by the row) so that every store instruction writes two whole 512-byte row segments instead
   // of 8 bytes in each of 32 rows.
-  if (!SPLIT && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0) {
+  if (wide) {
     lds_barrier();  // every wave has left the stages
 #pragma unroll
     for (int ms = 0; ms < MS; ++ms) {
       const int row = mrow0 + ms * 32 + lr;
       float rs = 1.f;
-      if (out_ok[ms]) {
-        if (MODE == kModeRow) rs = p.sx[out_slot[ms]];
-        if (MOE && p.topk_w) rs = p.topk_w[out_slot[ms]];
-      }
+      if (MODE == kModeRow && out_ok[ms]) rs = p.sx[out_slot[ms]];
+      if (MOE) rs = rsw[ms];
 #pragma unroll
       for (int rg = 0; rg < 4; ++rg) {
         const int n = n0 + wn * 32 + rg * 8 + h * 4;
@@ -784,8 +817,7 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
 #pragma unroll
     for (int i = 0; i < TM / NW / 2; ++i) {
       const int row = w * (TM / NW) + i * 2 + rr;
-      int slot = slot0 + row;
-      if (MOE) slot = row < block_m ? p.sorted_ids[slot0 + row] : nrows;
+      const int slot = MOE ? srow[i] : slot0 + row;
       const int n = n0 + (pc << 3);
       const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + ((pc ^ (row & 31)) << 4));
       if (slot < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)slot * p.ldc + n) = o;
@@ -798,7 +830,7 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
     const int64_t orow = out_slot[ms];
     float rs = 1.f;
     if (MODE == kModeRow && !SPLIT) rs = p.sx[orow];
-    if (MOE && p.topk_w) rs = p.topk_w[orow];
+    if (MOE) rs = rsw[ms];
 #pragma unroll
     for (int rg = 0; rg < 4; ++rg) {
       const int n = n0 + wn * 32 + rg * 8 + h * 4;

@@ -76,13 +76,20 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
     for (int q = 0; q < LW; ++q) buf_load16_to_lds(rW, voW[q] + ko, 0, base + q * 1024);
   };
-  issue_w(0);  // the weights do not wait for the slot table
+  // slot table first, weights behind it: loads retire in order, so the table arrives without waiting for the
+  // weights, and the weights do not wait for the table
+  int sid[LW];
+#pragma unroll
+  for (int q = 0; q < LW; ++q) sid[q] = p.sorted_ids[slot0 + (w * LW + q) * 8 + rl];
+  __builtin_amdgcn_sched_barrier(0);
+  issue_w(0);
   issue_w(1);
+  __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
   for (int q = 0; q < LW; ++q) {
     const int g = w * LW + q;
     const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
-    const int s = p.sorted_ids[slot0 + g * 8 + rl];
+    const int s = sid[q];
     voX[q] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
   }
   auto issue_x = [&](int kstep) {
