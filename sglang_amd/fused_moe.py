@@ -54,7 +54,7 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
         bm = 16
     elif per_expert <= 16:
         bm = 32
-    elif per_expert <= 40:
+    elif per_expert <= 48:
         bm = 64
     elif per_expert <= 96:
         bm = 128
