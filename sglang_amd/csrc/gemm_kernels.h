@@ -81,7 +81,7 @@ __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
 // 256(n) x 256(m) x 128(k) workgroup tile, 8 wavefronts (2 along n x 4 along m), wave tile
 // 128(n) x 64(m) = 4 x 2 MFMA tiles of 32x32, K step 128 = two v_mfma_f32_32x32x64_f8f6f4.
 //
-// LDS: two stages of [W 256 rows x 128 B | X 256 rows x 128 B] = 2 x 64 KB, filled by
+// LDS: three weight stages and two activation stages of 256 rows x 128 B each = 160 KB, filled by
 // buffer_load_dwordx4 ... lds (no register staging; rows past the matrix edge are out of the
 // descriptor's range - the complete offset is in the range-checked per-lane operand - and arrive
 // as zeros without touching memory).  A 1 KB wave-load covers 8 rows; the 16-byte chunk c of
@@ -90,8 +90,12 @@ __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
 //
 // Pipeline.  One loop iteration is one barrier interval, and the barrier sits BEFORE the last
 // quarter of a K block: by then a wave has every operand of the block in registers, so after the
-// barrier (a) the stage it just left can be refilled with block it+2 at once and (b) the first
-// operands of block it+1 are fetched while the last four MFMAs of block it still run.  Operand
+// barrier (a) the activation stage it just left can be refilled with block it+2 and the weight
+// stage with block it+3 at once and (b) the first operands of block it+1 are fetched while the
+// last four MFMAs of block it still run.  A wave's loads retire in order and are issued as
+// activations, scales, weights: the wait in front of the barrier leaves its four weight loads in
+// flight, so the weights - whose lines come from HBM or the memory-side cache, where the
+// activations mostly hit the L2 - have two barrier intervals to arrive.  Operand
 // fetches are issued two MFMA groups ahead of their use; the eight 1 KB global loads of a wave are
 // spread over the first half of the interval, two per group, because the texture-address path
 // moves 64 B/clk per CU and a burst would stall the issuing wave.  The loop body is branch-free
@@ -103,8 +107,6 @@ __device__ __forceinline__ float load_scalar(const void* p, int64_t i) {
 // group g; row mode accumulates in place and scales in the epilogue.
 // ------------------------------------------------------------------------------------------------
 constexpr int kTileN = 256, kTileM = 256, kTileK = 128;
-constexpr int kStageBytes = (kTileN + kTileM) * kTileK;  // 64 KB
-constexpr int kXOff = kTileN * kTileK;                   // X tile offset inside a stage
 
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 // raw buffer descriptor: base pointer + byte range; loads past the range return zero
@@ -149,7 +151,10 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // dispatched when the whole tiles drain.
 template <int MODE, int OUT_DT, int BIAS_DT>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
-  __shared__ __attribute__((aligned(1024))) uint8_t smem[2 * kStageBytes];
+  // the whole LDS: three weight stages (the weights travel two K blocks ahead: their lines come from HBM or the
+  // memory-side cache) and two activation stages (one block ahead: mostly L2 hits)
+  constexpr int kWStage = kTileN * kTileK, kXStage = kTileM * kTileK, kXBase = 3 * kWStage;
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[3 * kWStage + 2 * kXStage];
 
   const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
@@ -209,7 +214,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 #pragma unroll
     for (int j = 0; j < 2; ++j) co[ks][j] = (uint32_t)(((ks * 4 + h * 2 + j) ^ swz) << 4);
   const uint32_t rdW = (uint32_t)((wn * 128 + lr) * kTileK);
-  const uint32_t rdX = (uint32_t)(kXOff + (wm * 64 + lr) * kTileK);
+  const uint32_t rdX = (uint32_t)((wm * 64 + lr) * kTileK);
   auto frag = [&](const uint8_t* st, uint32_t rowoff, int ks) -> v8i {
     const v4i lo = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][0]);
     const v4i hi = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][1]);
@@ -245,23 +250,23 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   v16f tq[2];
   float sc[2] = {0.f, 0.f}, scn[2] = {0.f, 0.f};
   float s0n = 0.f, s1n = 0.f, sbn = 0.f;
-  int cur_stage = 0, cur_kstep = 0;
 
 #define SB() __builtin_amdgcn_sched_barrier(0)
-  auto L = [&](int idx) {  // one 1 KB global->LDS load: idx 0..3 W slices, 4..7 X slices
-    uint8_t* base = smem + cur_stage * kStageBytes + w * 4096;
-    const uint32_t ko = (uint32_t)cur_kstep * kTileK;
-    const int j = idx & 3;
-    // the whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt from the
-    // range check, and rows past the matrix edge must read as zero, not touch memory)
-    if (idx < 4) buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + ko), 0, base + j * 1024);
-    else buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + ko), 0, base + kXOff + j * 1024);
+  // one 1 KB global->LDS load (slice j of the wave's 32 rows) of K block kstep into weight stage ws / activation
+  // stage xst.  The whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt
+  // from the range check, and rows past the matrix edge must read as zero, not touch memory).
+  auto LW = [&](int j, int kstep, int ws) {
+    buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + (uint32_t)kstep * kTileK), 0, smem + ws * kWStage + w * 4096 + j * 1024);
+  };
+  auto LX = [&](int j, int kstep, int xst) {
+    buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + (uint32_t)kstep * kTileK), 0,
+                      smem + kXBase + xst * kXStage + w * 4096 + j * 1024);
   };
   auto RW = [&](v8i(&dst)[2], const uint8_t* st, int ns) {
     dst[0] = frag(st, rdW + ns * 32 * kTileK, 0);
     dst[1] = frag(st, rdW + ns * 32 * kTileK, 1);
   };
-  auto RX = [&](const uint8_t* st, int ms) {
+  auto RX = [&](const uint8_t* st, int ms) {  // st: activation stage
     X[ms][0] = frag(st, rdX + ms * 32 * kTileK, 0);
     X[ms][1] = frag(st, rdX + ms * 32 * kTileK, 1);
   };
@@ -313,9 +318,10 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 
   if (nkb <= 0) return;
   // ---- prologue: block 0 into stage 0, block 1 into stage 1, groups (0,0)..(2,1) of block 0
-  cur_stage = 0; cur_kstep = 0;
 #pragma unroll
-  for (int i = 0; i < 8; ++i) L(i);
+  for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) LW(j, 0, 0);
   if (MODE == kModeBlock) { sc[0] = sx0[0]; sc[1] = sx1[0]; const float sb = swp[0]; sc[0] *= sb; sc[1] *= sb; }
   auto exponents = [&](uint32_t w0, uint32_t w1, float sb, int kb_abs) {  // -> sq, sqw for K block kb_abs
     const int sh = (kb_abs & 3) * 8;
@@ -326,15 +332,21 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   if (MODE == kModeScaled) exponents(sq0p[(int64_t)(kb_begin >> 2) * p.sx_k], sq1p[(int64_t)(kb_begin >> 2) * p.sx_k], swp[0], kb_begin);
   wait_vm0();
   __syncthreads();
-  cur_stage = 1; cur_kstep = 1;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) L(i);
+  // scales of block 1, then activations of block 1, weights of blocks 1 and 2: the order the loop keeps, so that at
+  // a barrier only a wave's four youngest loads - weights for the block after next - may still be in flight
   if (MODE == kModeBlock) { const int kn = min(1, nkb - 1); s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k]; }
   if (MODE == kModeScaled) {
     const int kn = min(1, nkb - 1);
     q0n = sq0p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; q1n = sq1p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
   }
-  RX(smem, 0); RX(smem, 1); RW(WA, smem, 0); RW(WB, smem, 1);
+  SB();
+#pragma unroll
+  for (int j = 0; j < 4; ++j) LX(j, 1, 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) LW(j, 1, 1);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) LW(j, 2, 2);
+  RX(smem + kXBase, 0); RX(smem + kXBase, 1); RW(WA, smem, 0); RW(WB, smem, 1);
   SB();
   G(WA, 0, acc[0][0], tq[0]); SB();
   GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();
@@ -346,21 +358,23 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   GF(WA, 1, acc[2][1], tq[1], acc[2][0], tq[0], sc[0]); SB();
   // pending: F(acc[2][1], tq[1], sc[1])
 
+  int w_ld = 0, w_rd = 1;  // weight stages: the one block it left (refilled with block it+3), the one of block it+1
   for (int it = 0; it < nkb - 1; ++it) {
-    const int stage = it & 1;
-    const uint8_t* stn = smem + (stage ^ 1) * kStageBytes;  // block it+1
-    wait_vm0_lgkm0();
-    __syncthreads();
+    const uint8_t* stW = smem + w_rd * kWStage;                     // block it+1
+    const uint8_t* stX = smem + kXBase + ((it + 1) & 1) * kXStage;
+    const int xl = it & 1;                                          // activation stage block it left
+    lds_barrier<4>();  // block it+1 has landed; the weights of block it+2 may still be on their way
     SB();
-    cur_stage = stage; cur_kstep = it + 2;
-    RW(WA, stn, 0); SB();
+    RW(WA, stW, 0); SB();
     GF(WB, 0, acc[3][0], tq[0], acc[2][1], tq[1], sc[1]); SB();
-    RX(stn, 0); L(0); L(1); SB();
+    RX(stX, 0); LX(0, it + 2, xl); LX(1, it + 2, xl); SB();
     GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]); SB();
-    RX(stn, 1); RW(WB, stn, 1); L(2); L(3); SB();
+    RX(stX, 1); RW(WB, stW, 1); LX(2, it + 2, xl); LX(3, it + 2, xl); SB();
     if (MODE == kModeBlock) { scn[0] = s0n * sbn; scn[1] = s1n * sbn; }
     if (MODE == kModeScaled) exponents(q0n, q1n, sbn, kb_begin + it + 1);  // the groups from here on are block it+1's
     GF(WA, 0, acc[0][0], tq[0], acc[3][1], tq[1], sc[1]); SB();
+    // the scales of block it+2 are requested after the activation loads and before the weight loads: the wait in
+    // front of their use then leaves exactly the weight loads in flight
     if (MODE == kModeBlock) {
       sc[0] = scn[0]; sc[1] = scn[1];
       const int kn = min(it + 2, nkb - 1);
@@ -370,14 +384,17 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       const int kn = min(it + 2, nkb - 1);
       q0n = sq0p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; q1n = sq1p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
     }
-    L(4); L(5); SB();
+    SB();
+    LW(0, it + 3, w_ld); LW(1, it + 3, w_ld); SB();
     GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();
-    RW(WA, stn, 2); L(6); L(7); SB();
+    RW(WA, stW, 2); LW(2, it + 3, w_ld); LW(3, it + 3, w_ld); SB();
     GF(WB, 0, acc[1][0], tq[0], acc[0][1], tq[1], sc[1]); SB();
     GF(WB, 1, acc[1][1], tq[1], acc[1][0], tq[0], sc[0]); SB();
-    RW(WB, stn, 3); SB();
+    RW(WB, stW, 3); SB();
     GF(WA, 0, acc[2][0], tq[0], acc[1][1], tq[1], sc[1]); SB();
     GF(WA, 1, acc[2][1], tq[1], acc[2][0], tq[0], sc[0]); SB();
+    w_ld = w_rd;
+    w_rd = w_rd == 2 ? 0 : w_rd + 1;
   }
   // ---- last block's tail
   GF(WB, 0, acc[3][0], tq[0], acc[2][1], tq[1], sc[1]);
@@ -389,6 +406,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   // Each wave re-lays its own 64 x 128 block out in a private 16 KB slot of the stage memory, 16-byte
   // chunks XOR-swizzled by the row so that both the 8-byte writes and the 16-byte reads spread over all banks.
   const bool wide = !is_split && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  wait_vm0();  // the loads past the last K block still target the stages: drain them before the stages are reused or released
   if (wide) {
     lds_barrier();  // every wave has taken its last operands out of the stages
     uint8_t* ep = smem + w * 16384;
