@@ -287,3 +287,23 @@ def test_ue8m0_requantised_checkpoint_end_to_end(dev):
     assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
     c_float = w8a8_block_fp8_linear(x, W, [128, 128], Ws)
     assert _rel_err(c.float().cpu().numpy(), c_float.float().cpu().numpy()) <= 0.08
+
+
+@pytest.mark.parametrize("case", ["a", "b", "c"])
+def test_linear_path_against_golden_vectors(dev, case):
+    """Quant and GEMM through the library against tests/golden/w8a8_vectors.npz, which torch library ops alone wrote
+    (tests/golden/make_vectors.py): quantised bytes and scales bit for bit, the product within the stated tolerance."""
+    import os
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+
+    G = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "w8a8_vectors.npz"))
+    x = torch.from_numpy(G[case + "_x_bf16_bits"].view(np.int16)).view(torch.bfloat16).to(dev)
+    for col in (False, True):
+        q, s = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=col)
+        torch.cuda.synchronize()
+        assert np.array_equal(q.view(torch.uint8).cpu().numpy(), G[case + "_q"])
+        assert np.array_equal(s.cpu().numpy(), G[case + "_s"])
+        y = w8a8_block_fp8_matmul(q, fp8_tensor(G[case + "_wq"], dev), s, torch.from_numpy(G[case + "_ws"]).to(dev),
+                                  [128, 128], torch.bfloat16)
+        torch.cuda.synchronize()
+        assert _rel_err(y.float().cpu().numpy(), G[case + "_y"]) <= REL_TOL

@@ -324,3 +324,26 @@ def test_moe_fused_gate_oracle_tie_rules():
     w, ids = O.moe_fused_gate(x, bias, 4, 2, 3)
     assert ids[0].tolist() == [0, 1, 2]          # groups 3 and 2 dropped, then experts 0, 1, 2
     np.testing.assert_allclose(w[0], 1.0 / 3.0, rtol=1e-6)
+
+
+def _bf16_bits_to_f32(bits):
+    return (bits.astype(np.uint32) << 16).view(np.float32)
+
+
+def _golden():
+    import os
+    return np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "w8a8_vectors.npz"))
+
+
+@pytest.mark.parametrize("case", ["a", "b", "c"])
+def test_oracle_against_golden_vectors(case):
+    """tests/golden/w8a8_vectors.npz was written by torch library ops alone (tests/golden/make_vectors.py)."""
+    G = _golden()
+    x = _bf16_bits_to_f32(G[case + "_x_bf16_bits"])
+    q, s = O.per_token_group_quant_fp8(x, 128)
+    assert np.array_equal(q, G[case + "_q"]) and np.array_equal(s, G[case + "_s"])
+    y = O.w8a8_block_fp8_matmul(G[case + "_q"], G[case + "_wq"], G[case + "_s"], G[case + "_ws"], out_dtype="f32", acc=np.float64)
+    np.testing.assert_allclose(y, G[case + "_y"], rtol=1e-6, atol=1e-30)
+    if case == "a":
+        wq, ws = O.block_quant_weight(_bf16_bits_to_f32(G["a_w_bf16_bits"]))
+        assert np.array_equal(wq, G["a_wq"]) and np.array_equal(ws, G["a_ws"])
