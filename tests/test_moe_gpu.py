@@ -2,7 +2,7 @@
 
 Integer stage (moe_align_block_size): exact, compared through the invariants the reference's own test
 uses (sgl-kernel/tests/test_moe_align.py:210-254) because the order inside an expert is unspecified.
-Floating-point stages: silu_and_mul within one bf16 ulp of the oracle (device expf vs numpy exp),
+Floating-point stages: silu within one bf16 ulp of the oracle's (hardware exp2 and reciprocal vs numpy exp),
 moe_sum_reduce exact (same float32 summation order), grouped GEMM and the whole layer within the
 path's 1e-2 max-relative-error bound.
 """
@@ -109,14 +109,16 @@ def test_silu_and_mul(dev, rows, d):
     torch.cuda.synchronize()
     got = out.float().cpu().numpy()
     ref = O.silu_and_mul(x)
-    # one bf16 ulp of the silu value (2^-8 relative) carried through the product
-    tol = np.abs(ref) * 2.0**-7 + 1e-30
+    # a silu value one bf16 ulp off (at most 2^-7 relative) carried through the product and its rounding
+    tol = np.abs(ref) * 2.0**-6 + 1e-30
     assert (np.abs(got - ref) <= tol).all()
-    assert (got != ref).mean() < 1e-3
+    # bf16 inputs take few distinct values: one whose silu lies within a float32 ulp of a bf16 tie (5.9375 ->
+    # 5.92187444, tie 5.921875) repeats a dozen times in the small case
+    assert (got != ref).mean() < 2e-3
     # the library routine on the same device agrees with the same bound
     xt = bf16_tensor(x, dev)
     lib_ref = (torch.nn.functional.silu(xt[:, :d].float()).to(torch.bfloat16) * xt[:, d:]).float().cpu().numpy()
-    assert (np.abs(got - lib_ref) <= np.abs(lib_ref) * 2.0**-7 + 1e-30).all()
+    assert (np.abs(got - lib_ref) <= np.abs(lib_ref) * 2.0**-6 + 1e-30).all()
 
 
 def test_silu_and_mul_other_dtypes_and_errors(dev):
@@ -128,6 +130,16 @@ def test_silu_and_mul_other_dtypes_and_errors(dev):
     xh = x.half()
     refh = torch.nn.functional.silu(xh[:, :32].float()).half() * xh[:, 32:]
     torch.testing.assert_close(silu_and_mul(xh), refh, rtol=2e-3, atol=1e-6)
+    # the ends of the range: exp(-v) over- and underflows, infinities and NaN behave as v / (1 + exp(-v)) does
+    edge = torch.tensor([0.0, -0.0, 1e-30, -1e-30, 20.0, -20.0, 80.0, -80.0, 88.0, -88.0, 90.0, -90.0, 104.0, -104.0, 1e4, -1e4,
+                         3e38, -3e38, float("inf"), float("-inf"), float("nan"), 1.0, -1.0, 0.5, -0.5, 7.0, -7.0, 15.0, -15.0,
+                         30.0, -30.0, 60.0, -60.0], device=dev)
+    xe = torch.cat([edge, torch.ones_like(edge)]).reshape(1, -1)
+    xe = torch.cat([xe[:, :edge.numel()], torch.zeros(1, (-edge.numel()) % 8, device=dev), xe[:, edge.numel():],
+                    torch.zeros(1, (-edge.numel()) % 8, device=dev)], dim=1)
+    got = silu_and_mul(xe)[0, :edge.numel()]
+    want = edge / (1.0 + torch.exp(-edge))
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-37, equal_nan=True)
     with pytest.raises(ValueError, match="multiple of 16 bytes"):
         silu_and_mul(torch.zeros(3, 12, device=dev, dtype=torch.bfloat16))
     assert silu_and_mul(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16)).shape == (0, 32)
