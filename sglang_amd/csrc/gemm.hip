@@ -32,42 +32,44 @@ static Plan plan_tile128(int64_t M, int64_t N, int kb, int splits) {
   return pl;
 }
 
-// the plan without the 128x128 tile kernel: direct / streaming / 256x256 tiles by the number of rows
-static Plan plan_base(int64_t M, int64_t N, int64_t K) {
-  Plan pl{0, 1, 0, 0, 0, 0};
+// decode-sized, up to 32 rows: weights go HBM -> registers -> matrix core.  K is cut so that about 512 workgroups
+// (two per CU, one round) stream at once, at least 8 K blocks each, while the float partials stay a small fraction
+// of the weight bytes
+static Plan plan_direct(int64_t M, int64_t N, int64_t K) {
+  Plan pl{3, 1, 0, 0, 0, 0};
   const int kb = (int)(K / kTileK);
-  if (M <= 32 && M * K < (1LL << 31)) {
-    // decode-sized: weights go HBM -> registers -> matrix core.  K is cut so that about 512 workgroups (two per
-    // CU, one round) stream at once, at least 8 K blocks each, while the float partials stay a small fraction of
-    // the weight bytes
-    pl.kind = 3;
-    pl.tm = M <= 16 ? 16 : 32;
-    const int64_t tiles_n = (N + kDirTileN - 1) / kDirTileN;
-    int64_t splits = std::max<int64_t>(1, 512 / tiles_n);
-    splits = std::min<int64_t>(splits, std::max<int64_t>(1, kb / kDirDepth));
-    splits = std::min<int64_t>(splits, std::max<int64_t>(1, K / (64 * M)));
-    const int kbps = (int)((kb + splits - 1) / splits);
-    pl.kb_per_split = kbps;
-    pl.splits = (kb + kbps - 1) / kbps;
-    pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
-    return pl;
-  }
-  if (M <= 128 && M * K < (1LL << 31)) {
-    // decode-sized: stream the weights once, every CU takes a K slice of one 256-row weight tile
-    pl.kind = 2;
-    pl.tm = M <= 64 ? 64 : 128;
-    const int64_t tiles_n = (N + kTileN - 1) / kTileN;
-    int splits = (int)(256 / tiles_n);
-    if (splits > kb / 4) splits = kb / 4;
-    if (splits < 1) splits = 1;
-    pl.kb_per_split = (kb + splits - 1) / splits;
-    pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
-    pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
-    return pl;
-  }
-  pl.kind = 1;
-  // One workgroup (one CU) per 256x256 tile.  The tiles of the last, partial round over the CUs are cut along K
-  // so that the round keeps every CU busy for 1/splits of a tile time (>= 4 K blocks per piece).
+  pl.tm = M <= 16 ? 16 : 32;
+  const int64_t tiles_n = (N + kDirTileN - 1) / kDirTileN;
+  int64_t splits = std::max<int64_t>(1, 512 / tiles_n);
+  splits = std::min<int64_t>(splits, std::max<int64_t>(1, kb / kDirDepth));
+  splits = std::min<int64_t>(splits, std::max<int64_t>(1, K / (64 * M)));
+  const int kbps = (int)((kb + splits - 1) / splits);
+  pl.kb_per_split = kbps;
+  pl.splits = (kb + kbps - 1) / kbps;
+  pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  return pl;
+}
+
+// up to 128 rows: stream the weights once, every CU takes a K slice of one 256-row weight tile
+static Plan plan_stream(int64_t M, int64_t N, int64_t K) {
+  Plan pl{2, 1, 0, 0, 0, 0};
+  const int kb = (int)(K / kTileK);
+  pl.tm = M <= 64 ? 64 : 128;
+  const int64_t tiles_n = (N + kTileN - 1) / kTileN;
+  int splits = (int)(256 / tiles_n);
+  if (splits > kb / 4) splits = kb / 4;
+  if (splits < 1) splits = 1;
+  pl.kb_per_split = (kb + splits - 1) / splits;
+  pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
+  pl.ws_bytes = pl.splits > 1 ? (int64_t)pl.splits * M * N * 4 : 0;
+  return pl;
+}
+
+// One workgroup (one CU) per 256x256 tile.  The tiles of the last, partial round over the CUs are cut along K
+// so that the round keeps every CU busy for 1/splits of a tile time (>= 4 K blocks per piece).
+static Plan plan_tile256(int64_t M, int64_t N, int64_t K) {
+  Plan pl{1, 1, 0, 0, 0, 0};
+  const int kb = (int)(K / kTileK);
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
   const int64_t rest = tiles % kNumCU;
   int splits = rest ? (int)(kNumCU / rest) : 1;
@@ -83,6 +85,20 @@ static Plan plan_base(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
+// the plan without the 128x128 tile kernel: direct / streaming / 256x256 tiles by the number of rows
+static Plan plan_base(int64_t M, int64_t N, int64_t K) {
+  const bool fits32 = M * K < (1LL << 31);
+  if (g_force_kind == 3 && M <= 32 && fits32) return plan_direct(M, N, K);
+  if (g_force_kind == 2 && M <= 128 && fits32) return plan_stream(M, N, K);
+  if (g_force_kind == 1) return plan_tile256(M, N, K);
+  // 17..32 rows of a large, deep weight matrix (measured on 18432 x 7168: 31 us against 34-37 us): the LDS-staged
+  // streaming kernel; the register-streaming kernel keeps every other shape of that size
+  const bool big = N * K >= 96000000LL && K >= 32 * kTileK;
+  if (M <= 32 && fits32 && !(M > 16 && big)) return plan_direct(M, N, K);
+  if (M <= 128 && fits32) return plan_stream(M, N, K);
+  return plan_tile256(M, N, K);
+}
+
 
 // Rough device-time models in microseconds, fitted to sweeps over M = 48..2048 on the DeepSeek-V3 and Llama
 // projection shapes; they only have to rank the two candidates where the gap is large.
@@ -92,7 +108,7 @@ static Plan plan_base(int64_t M, int64_t N, int64_t K) {
 //    launch 1 us; more than two rounds are left to the 256x256 kernel, two rounds measure about 15 % over the
 //    model; a K cut adds the reduction launch (4 us) and the float partials (written and read back at about
 //    5 TB/s).
-//  * streaming kernel: 8-11 us fixed, the weights once at 5.5 TB/s, its partials at about 8 TB/s.
+//  * streaming kernel: 10-11 us fixed, the weights once at 5.5 TB/s, its partials at about 8 TB/s.
 //  * 256x256 tiles: 1.6 us per K block and tile, 8 us fixed, 6 us + partials (8 TB/s) for a cut last round.
 static double est_tile128(int64_t M, int64_t N, int kb, int* best_splits) {
   const int64_t tm = (M + kT128 - 1) / kT128, tn = (N + kT128 - 1) / kT128;
@@ -100,7 +116,7 @@ static double est_tile128(int64_t M, int64_t N, int kb, int* best_splits) {
   const double cold = std::min(1.0, 1.0 / (double)tm + 1.0 / (double)tn);
   double best = 1e30;
   for (int s = 1; s <= 8; ++s) {
-    if (s > 1 && (s > kb / 4 || tiles * s > 216)) break;  // a K cut over more than ~85 % of the CUs measured slower
+    if (s > 1 && (s > kb / 4 || tiles * s > 256)) break;  // a K cut stays within one round of workgroups
     const int64_t wgs = tiles * s;
     const int64_t rounds = (wgs + kNumCU - 1) / kNumCU;
     if (rounds > 2) break;
@@ -117,7 +133,7 @@ static double est_tile128(int64_t M, int64_t N, int kb, int* best_splits) {
 static double est_base(const Plan& pl, int64_t M, int64_t N, int64_t K) {
   const int kb = (int)(K / kTileK);
   if (pl.kind == 2)
-    return (M <= 64 ? 8.0 : 11.0) + (double)N * K / 5.5e6 + (pl.splits > 1 ? (double)pl.splits * M * N * 8.0 / 8e6 : 0.0);
+    return (M <= 64 ? 10.0 : 11.0) + (double)N * K / 5.5e6 + (pl.splits > 1 ? (double)pl.splits * M * N * 8.0 / 8e6 : 0.0);
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
   if (pl.splits == 1) return 8.0 + (double)((tiles + kNumCU - 1) / kNumCU) * kb * 1.6;
   const int64_t rest = tiles % kNumCU;
