@@ -52,7 +52,7 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     per_expert = (M * topk + E - 1) // max(E, 1)
     if per_expert <= 4:
         bm = 16
-    elif per_expert <= 16:
+    elif per_expert <= 22:
         bm = 32
     elif per_expert <= 48:
         bm = 64
