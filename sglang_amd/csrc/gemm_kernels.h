@@ -7,6 +7,8 @@
 // as[m,kb]*bs[nb,kb] per lane, and the bf16 output is written as 8-byte runs along n.
 #pragma once
 
+#include <type_traits>
+
 #include "fp8k_common.h"
 
 namespace fp8k {
@@ -735,7 +737,8 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   if (MOE) wait_vm0();  // the grouped prologue issues its loads in another order than the trips' partial waits assume
 
   // one K block; (sx, sb) hold its scales on entry and are reloaded with those of block it+2
-  auto trip = [&](int it, float (&sx)[MS], float& sb) {
+  auto trip = [&](auto na, int it, float (&sx)[MS], float& sb) {
+    constexpr int NA = decltype(na)::value;  // 32-row groups of the wave that hold real rows (grouped form)
     // stage `it` has landed once at most NSTAGE-2 younger trips (stage + scale loads each) are still in flight
     constexpr int kInFlight = (NSTAGE - 2) * (LPW + SL);
     lds_barrier<kInFlight>();
@@ -747,12 +750,13 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
       __builtin_amdgcn_sched_barrier(0);  // keep the scale loads ahead of the stage loads
     }
     issue(it + NSTAGE - 1);  // refills the stage every wave finished before this barrier
+    if (NA == 0) return;
     const uint8_t* st = smem + (it % NSTAGE) * STAGE;
     v8i wf[2];
     wf[0] = frag(st, rdW, 0);
     wf[1] = frag(st, rdW, 1);
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) {
+    for (int ms = 0; ms < NA; ++ms) {
       const v8i x0 = frag(st, rdX + ms * 32 * kTileK, 0);
       const v8i x1 = frag(st, rdX + ms * 32 * kTileK, 1);
       if (MODE == kModeBlock) {
@@ -769,12 +773,27 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
       }
     }
   };
-  int it = 0;
-  for (; it + 1 < nkb; it += 2) {
-    trip(it, sxa, sba);
-    trip(it + 1, sxb, sbb);
+  auto run = [&](auto na) {
+    int it = 0;
+    for (; it + 1 < nkb; it += 2) {
+      trip(na, it, sxa, sba);
+      trip(na, it + 1, sxb, sbb);
+    }
+    if (it < nkb) trip(na, it, sxa, sba);
+  };
+  // Grouped form: the 32-row groups past an expert's last slot are padding (real slots come first in a block) and
+  // skip their MFMAs; one straight-line copy of the loop per group count.
+  int nact = MS;
+  if (MOE) {
+    nact = 0;
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) nact += __builtin_amdgcn_readfirstlane(out_slot[ms]) < nrows ? 1 : 0;
   }
-  if (it < nkb) trip(it, sxa, sba);
+  if (!MOE || nact == MS) run(std::integral_constant<int, MS>{});
+  else if (MS > 2 && nact == 3) run(std::integral_constant<int, (MS > 2 ? 3 : MS)>{});
+  else if (MS > 2 && nact == 2) run(std::integral_constant<int, 2>{});
+  else if (nact == 1) run(std::integral_constant<int, 1>{});
+  else run(std::integral_constant<int, 0>{});
   // routed weights and the output rows of the store loop, fetched while the stages drain
   const bool wide = !SPLIT && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
   float rsw[MS];
