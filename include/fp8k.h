@@ -138,6 +138,7 @@ int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * cut into `splits` runs (0 or 1: none).  kind 0: the choice by the number of rows alone, without the 128x128
  * kernel.  kind 1: 256x256 tiles; kind 2: the streaming kernel (up to 128 rows); kind 3: the direct kernel (up to 32
  * rows); where a pinned family cannot take the shape, the choice by rows stands.  `splits` is ignored for kinds 0..3.
+ * kind -2: automatic, but the last round of 256x256 tiles is kept whole instead of being computed in 128-row halves.
  * fp8k_*_workspace_bytes follows the pinned choice.  Not thread safe.
  */
 void fp8k_tune_force_gemm_plan(int kind, int splits);

@@ -13,7 +13,8 @@ struct Plan {
   int splits;  // >1: split-K through the float workspace
   int kb_per_split;
   int tm;      // rows per block of the streaming kernels
-  int tail_first;   // tile256: first tile that is cut along K (== number of tiles when none is)
+  int tail_first;   // tile256: first tile that is cut along K or into halves (== number of tiles when none is)
+  int halves;       // tile256: the tiles from tail_first on are computed as two 128-row halves
   int64_t ws_bytes; // float workspace the plan needs
 };
 
@@ -21,6 +22,7 @@ constexpr int kNumCU = 256;  // MI355X
 
 // tuning aid: force the kernel family (and the K split of the uniform-split families) of later calls
 static int g_force_kind = -1, g_force_splits = 0;
+static int g_tail_halves = 1;  // tuning aid: 0 keeps the last round of 256x256 tiles whole
 
 static Plan plan_tile128(int64_t M, int64_t N, int kb, int splits) {
   Plan pl{4, 1, 0, 0, 0, 0};
@@ -82,6 +84,12 @@ static Plan plan_tile256(int64_t M, int64_t N, int64_t K) {
   pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
   pl.tail_first = (int)(pl.splits > 1 ? tiles - rest : tiles);
   pl.ws_bytes = pl.splits > 1 ? rest * pl.splits * (int64_t)(kTileM * kTileN) * 4 : 0;
+  // A last round that fills at most half the CUs and is not worth a K cut: its tiles run as two 128-row halves, one
+  // workgroup each (half the matrix-core time per K block, nothing to reduce).
+  if (pl.splits == 1 && tiles > kNumCU && rest > 0 && rest <= kNumCU / 2 && M > kTileM / 2 && g_tail_halves) {
+    pl.halves = 1;
+    pl.tail_first = (int)(tiles - rest);
+  }
   return pl;
 }
 
@@ -206,10 +214,11 @@ static int launch_tiles(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   }
   const int ntiles = a.tiles_m * a.tiles_n;
   a.tail_first = pl.tail_first;
-  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * pl.splits);
+  a.tail_halves = pl.halves;
+  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * (pl.halves ? 2 : pl.splits));
   hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
   int rc = check_launch("gemm_tile256");
-  if (rc || pl.tail_first == ntiles) return rc;
+  if (rc || pl.tail_first == ntiles || pl.halves) return rc;
   hipLaunchKernelGGL((tile_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((ntiles - pl.tail_first) * 64)), dim3(256),
                      0, st, a);
   return check_launch("tile_reduce");
@@ -293,7 +302,11 @@ static int common_checks(const char* op, const void* A, const void* B, void* C, 
 
 using namespace fp8k;
 
-extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) { g_force_kind = kind; g_force_splits = splits; }
+extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) {
+  g_tail_halves = kind != -2;  // -2: automatic choice with the last round of 256x256 tiles kept whole
+  g_force_kind = kind == -2 ? -1 : kind;
+  g_force_splits = splits;
+}
 
 extern "C" int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return block_gemm_workspace_bytes(M, N, K); }
 extern "C" int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return workspace_bytes(M, N, K); }

@@ -27,7 +27,8 @@ struct GemmArgs {
   int tiles_m, tiles_n;
   int splits;         // K is cut into `splits` runs of kb_per_split K-blocks
   int kb_per_split;
-  int tail_first;     // tile256 only: tiles [tail_first, tiles) are the ones cut along K
+  int tail_first;     // tile256 only: tiles [tail_first, tiles) are the ones cut along K or into halves
+  int tail_halves;    // tile256 only: those tiles are computed as two 128-row halves, one workgroup each (no K cut)
   // grouped (MoE) form of the streaming kernel; all null / zero for a dense GEMM
   const int32_t* sorted_ids;    // [m_blocks * TM] token slots, padded with values >= num_valid
   const int32_t* expert_ids;    // [m_blocks] expert of each block of TM slots, -1 = not on this rank
@@ -150,7 +151,10 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
 // Tiles [tail_first, tiles) - the last, partial round over the chip's CUs - are cut into `splits` K ranges, one
 // workgroup each, so that the round takes 1/splits of a tile time; they leave float partials in the workspace
 // ([tile - tail_first][split][256 m][256 n]) for tile_reduce_kernel.  Their workgroup ids come last, so they are
-// dispatched when the whole tiles drain.
+// dispatched when the whole tiles drain.  With tail_halves the tiles of the last round are instead computed as two
+// 128-row halves, one workgroup each: the four waves of the lower half of the tile do the MFMAs (one per SIMD, so
+// a K block takes half the matrix-core time), the other four only take part in the loads, and nothing has to be
+// reduced afterwards.
 template <int MODE, int OUT_DT, int BIAS_DT>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
   // the whole LDS: three weight stages (the weights travel two K blocks ahead: their lines come from HBM or the
@@ -163,26 +167,33 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   const int wn = w & 1, wm = w >> 1;
 
   const int bid = blockIdx.x;
-  int t = 0, split = 0;
-  bool is_split = false;
+  int t = 0, split = 0, half = 0;
+  bool is_split = false, is_half = false;
   int tile_m, tile_n;
   {
     const int ntiles = p.tiles_m * p.tiles_n;
     const int per_xcd = (p.tail_first + 7) >> 3;
-    is_split = bid >= per_xcd * 8;
-    if (!is_split) {
+    if (bid < per_xcd * 8) {
       t = (bid & 7) * per_xcd + (bid >> 3);
       if (t >= p.tail_first) return;
     } else {
       const int b2 = bid - per_xcd * 8;
-      t = p.tail_first + b2 / p.splits;
-      split = b2 % p.splits;
+      if (p.tail_halves) {
+        is_half = true;
+        t = p.tail_first + (b2 >> 1);
+        half = b2 & 1;
+      } else {
+        is_split = true;
+        t = p.tail_first + b2 / p.splits;
+        split = b2 % p.splits;
+      }
       if (t >= ntiles) return;
     }
     tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
   }
-  const int m0 = tile_m * kTileM, n0 = tile_n * kTileN;
-  const int nrows = p.M;   // exclusive bound of a valid output row
+  const int m0 = tile_m * kTileM + half * (kTileM / 2), n0 = tile_n * kTileN;
+  if (m0 >= p.M) return;                                              // upper half of a tile past the last row
+  const int nrows = is_half ? min(p.M, m0 + kTileM / 2) : p.M;        // exclusive bound of a valid output row
 
   const int kb_begin = is_split ? split * p.kb_per_split : 0;
   const int kb_end = is_split ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
@@ -193,7 +204,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the
   // matrix edge are out of range and read as zero
   const uint8_t* Wb = p.W;
-  const int rowsW = min(kTileN, p.N - n0), rowsX = min(kTileM, p.M - m0);
+  const int rowsW = min(kTileN, p.N - n0), rowsX = min(is_half ? kTileM / 2 : kTileM, p.M - m0);
   const int kbytes = p.K - kb_begin * kTileK;
   const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
   const rsrc_t rX = make_rsrc(p.X + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
@@ -319,6 +330,36 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   };
 
   if (nkb <= 0) return;
+  if (is_half && wm >= 2) {
+    // half tile: the waves of the upper 128 rows issue their share of the loads (their activation rows are out of
+    // range and arrive as zeros) and keep the barriers, with the same order and counts of loads as the others
+#pragma unroll
+    for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+    wait_vm0();
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) LX(j, 1, 1);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) LW(j, 1, 1);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) LW(j, 2, 2);
+    int w_ld = 0, w_rd = 1;
+    for (int it = 0; it < nkb - 1; ++it) {
+      lds_barrier<4>();
+      SB();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LX(j, it + 2, it & 1);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LW(j, it + 3, w_ld);
+      w_ld = w_rd;
+      w_rd = w_rd == 2 ? 0 : w_rd + 1;
+    }
+    wait_vm0();
+    if ((p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0) lds_barrier();  // the others' epilogue barrier
+    return;
+  }
   // ---- prologue: block 0 into stage 0, block 1 into stage 1, groups (0,0)..(2,1) of block 0
 #pragma unroll
   for (int j = 0; j < 4; ++j) LX(j, 0, 0);

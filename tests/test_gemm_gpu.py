@@ -152,6 +152,23 @@ def test_block_gemm_exact_on_integers(dev, M, N, K):
     np.testing.assert_array_equal(c16, O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="f16", acc=np.float64))
 
 
+@pytest.mark.parametrize("M", [3700, 3840, 4000])
+def test_block_gemm_last_round_in_half_tiles_exact(dev, M):
+    """More 256x256 tiles than CUs with a last round that fills less than half of them: those tiles run as two
+    128-row halves.  M = 3700 leaves a tile whose upper half lies past the last row, 4000 one whose upper half holds
+    32 rows, 3840 (a multiple of 256) none that is ragged.  Integer data: exact."""
+    N, K = 18432, 256
+    rng = np.random.default_rng(M)
+    xq = O.f32_to_e4m3fn(rng.integers(-4, 5, (M, K)).astype(np.float32))
+    wq = O.f32_to_e4m3fn(rng.integers(-4, 5, (N, K)).astype(np.float32))
+    xs = (2.0 ** rng.integers(-3, 3, (M, K // 128))).astype(np.float32)
+    ws = (2.0 ** rng.integers(-3, 3, (N // 128, K // 128))).astype(np.float32)
+    tiles = ((M + 255) // 256) * (N // 256)
+    assert tiles > 256 and 0 < tiles % 256 <= 128
+    c = _run_block(xq, xs, wq, ws, dev)
+    np.testing.assert_array_equal(c, O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="bf16", acc=np.float64))
+
+
 def test_block_gemm_scale_layouts_agree(dev):
     xq, xs, wq, ws = _quantised_problem(200, 512, 1024, 9)
     a = _run_block(xq, xs, wq, ws, dev, col_major_as=False)
