@@ -193,6 +193,23 @@ def test_block_gemm_unaligned_shapes(dev, N, K):
     assert _rel_err(c, ref) <= REL_TOL
 
 
+def test_block_gemm_random_shapes_every_plan(dev):
+    """Sixty seeded random shapes (M 1..1500, N a multiple of 8 up to 6144, K a multiple of 128 up to 2304) with
+    random scale layouts: whatever kernel family and K cut the plan picks, exact on integer data."""
+    rng = np.random.default_rng(20250101)
+    for case in range(60):
+        M = int(rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(300, 1500)]))
+        N = int(rng.integers(1, 769)) * 8
+        K = int(rng.integers(1, 19)) * 128
+        xq = O.f32_to_e4m3fn(rng.integers(-4, 5, (M, K)).astype(np.float32))
+        wq = O.f32_to_e4m3fn(rng.integers(-4, 5, (N, K)).astype(np.float32))
+        xs = (2.0 ** rng.integers(-3, 3, (M, K // 128))).astype(np.float32)
+        ws = (2.0 ** rng.integers(-3, 3, ((N + 127) // 128, K // 128))).astype(np.float32)
+        ref = O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype="bf16", acc=np.float64)
+        c = _run_block(xq, xs, wq, ws, dev, col_major_as=bool(case & 1))
+        assert np.array_equal(c, ref), "case %d: M=%d N=%d K=%d" % (case, M, N, K)
+
+
 def _run_scaled_mm(aq, bq, sa, sb, dev, out_dtype=torch.bfloat16, bias=None):
     from sglang_amd.sgl_kernel import fp8_scaled_mm
 

@@ -243,6 +243,49 @@ def test_grouped_gemm_256_slot_blocks_every_group_count(dev):
             assert _rel_err(got[rows], ref) <= REL_TOL, "expert %d with %d slots" % (e, rows.size)
 
 
+def test_grouped_gemm_random_routings_exact(dev):
+    """Forty seeded random routings (1..600 tokens, 2..40 experts, top-1..6, every block size, skewed and absent
+    experts, ids of -1) on integer data with power-of-two scales: exact, with per-token and with sorted scales."""
+    from sglang_amd.fused_moe import moe_align_block_size
+    from sglang_amd.sgl_kernel import moe_block_gemm, moe_sort_scales
+
+    rng = np.random.default_rng(20250102)
+    for case in range(40):
+        T = int(rng.choice([rng.integers(1, 8), rng.integers(8, 100), rng.integers(100, 600)]))
+        E = int(rng.integers(2, 41))
+        topk = int(rng.integers(1, min(6, E) + 1))
+        block = int(rng.choice([16, 32, 64, 128, 256]))
+        N, K = int(rng.integers(1, 9)) * 128, int(rng.integers(1, 7)) * 128
+        p = rng.dirichlet(np.full(E, 0.5))  # skewed: some experts get nothing
+        ids = np.stack([rng.choice(E, size=topk, replace=False, p=p / p.sum()) if (p > 0).sum() >= topk
+                        else rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+        ids[rng.random(ids.shape) < 0.05] = -1
+        wq = O.f32_to_e4m3fn(rng.integers(-4, 5, (E, N, K)).astype(np.float32))
+        ws = (2.0 ** rng.integers(-3, 3, (E, N // 128, K // 128))).astype(np.float32)
+        xq = O.f32_to_e4m3fn(rng.integers(-4, 5, (T, K)).astype(np.float32))
+        xs = (2.0 ** rng.integers(-3, 3, (T, K // 128))).astype(np.float32)
+        sorted_ids, expert_ids, npad = moe_align_block_size(torch.from_numpy(ids).to(dev), block, E)
+        A, B = fp8_tensor(xq, dev), fp8_tensor(wq, dev)
+        As, Bs = torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev)
+        tw = torch.ones((T, topk), device=dev)
+        outs = []
+        for sort in ([False, True] if block >= 64 else [False]):
+            C = torch.full((T * topk, N), float("nan"), dtype=torch.bfloat16, device=dev)
+            sc = moe_sort_scales(As, sorted_ids, npad, topk, ids.size) if sort else As
+            moe_block_gemm(A, B, C, sc, Bs, tw, sorted_ids, expert_ids, npad, False, topk, block, ids.size, scales_sorted=sort)
+            torch.cuda.synchronize()
+            outs.append(C.float().cpu().numpy())
+        flat = ids.reshape(-1)
+        for got in outs:
+            for e in range(E):
+                slots = np.nonzero(flat == e)[0]
+                if slots.size:
+                    ref = O.w8a8_block_fp8_matmul(xq[slots // topk], wq[e], xs[slots // topk], ws[e], out_dtype="bf16", acc=np.float64)
+                    assert np.array_equal(got[slots], ref), "case %d: T=%d E=%d topk=%d block=%d N=%d K=%d expert %d" % (
+                        case, T, E, topk, block, N, K, e)
+            assert (got[flat == -1] == 0).all(), "case %d: rows of dropped slots must be zero" % case
+
+
 def test_grouped_gemm_exact_on_integers(dev):
     from sglang_amd.fused_moe import moe_align_block_size
     from sglang_amd.sgl_kernel import moe_block_gemm
