@@ -45,6 +45,10 @@ static Plan plan_direct(int64_t M, int64_t N, int64_t K) {
   int64_t splits = std::max<int64_t>(1, 512 / tiles_n);
   splits = std::min<int64_t>(splits, std::max<int64_t>(1, kb / kDirDepth));
   splits = std::min<int64_t>(splits, std::max<int64_t>(1, K / (64 * M)));
+  // 128 and more n tiles keep half the CUs streaming on their own: no K cut and no reduction launch (18432 x 7168:
+  // 26.6 us against 28.6 us with three cuts; two cuts, 288 workgroups, leave the CUs unevenly loaded: 33 us)
+  if (tiles_n >= 128) splits = 1;
+  if (g_force_kind == 3 && g_force_splits > 0) splits = std::min<int64_t>(g_force_splits, kb);  // tuning aid
   const int kbps = (int)((kb + splits - 1) / splits);
   pl.kb_per_split = kbps;
   pl.splits = (kb + kbps - 1) / kbps;
@@ -99,10 +103,7 @@ static Plan plan_base(int64_t M, int64_t N, int64_t K) {
   if (g_force_kind == 3 && M <= 32 && fits32) return plan_direct(M, N, K);
   if (g_force_kind == 2 && M <= 128 && fits32) return plan_stream(M, N, K);
   if (g_force_kind == 1) return plan_tile256(M, N, K);
-  // 17..32 rows of a large, deep weight matrix (measured on 18432 x 7168: 31 us against 34-37 us): the LDS-staged
-  // streaming kernel; the register-streaming kernel keeps every other shape of that size
-  const bool big = N * K >= 96000000LL && K >= 32 * kTileK;
-  if (M <= 32 && fits32 && !(M > 16 && big)) return plan_direct(M, N, K);
+  if (M <= 32 && fits32) return plan_direct(M, N, K);
   if (M <= 128 && fits32) return plan_stream(M, N, K);
   return plan_tile256(M, N, K);
 }
