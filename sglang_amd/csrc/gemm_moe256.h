@@ -226,24 +226,26 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   }
   // output rows and routed weights, fetched while the stages drain
   const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
-  const int rr = lane >> 5, pc = lane & 31;
+  const int er = lane >> 3, ec = lane & 7;  // store loop: row inside a group of 8, 16-byte chunk of the wave's 128 bytes
   int oslots[MS], srow[16];
   float rsw[MS];
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
 #pragma unroll
-  for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[slot0 + w * 32 + i * 2 + rr] : 0;
+  for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[slot0 + wm * 128 + i * 8 + er] : 0;
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) rsw[ms] = (p.topk_w && oslots[ms] < nrows) ? p.topk_w[oslots[ms]] : 1.f;
   wait_vm0();     // the loads past the last K block still target the stages
   lds_barrier();  // every wave has left the stages: they become the output staging area
 
-  // ---- epilogue through LDS: [256 slots][256 n] 16-bit, 512 B per row, 16-byte chunks XOR-swizzled by the
-  // row so that the accumulator-shaped 8-byte writes spread over all banks; every store instruction then
-  // writes two whole 512-byte row segments
+  // ---- epilogue through LDS.  A wave re-lays its own 128 slots x 64 n block out in a private 16 KB slot (128 B per
+  // row, 16-byte chunk c of row r at position c ^ ((r >> 1) & 7), so that the accumulator-shaped 8-byte writes and
+  // the 16-byte reads spread over all banks): no second workgroup barrier, and every store instruction writes eight
+  // whole 128-byte lines.
+  uint8_t* const ep = smem + w * 16384;
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
-    const int row = wm * 128 + ms * 32 + lr;
+    const int row = ms * 32 + lr;  // inside the wave's 128 slots
     const int oslot = oslots[ms];
     const bool ok = oslot < nrows;
     const float rs = rsw[ms];
@@ -262,8 +264,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
           o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
           o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
         }
-        const int chunk = (wn * 8 + nr) ^ (row & 31);
-        *reinterpret_cast<uint2*>(smem + row * 512 + chunk * 16 + h * 8) = o;
+        *reinterpret_cast<uint2*>(ep + row * 128 + ((nr ^ ((row >> 1) & 7)) << 4) + h * 8) = o;
       } else {
         const int n = n0 + wn * 64 + nr * 8 + h * 4;
         if (ok && n < p.N) store4<OUT_DT>(p.C, (int64_t)oslot * p.ldc + n, v[0], v[1], v[2], v[3]);
@@ -271,13 +272,13 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     }
   }
   if (!wide) return;
-  lds_barrier();
+  __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
 #pragma unroll
   for (int i = 0; i < 16; ++i) {
-    const int row = w * 32 + i * 2 + rr;
+    const int row = i * 8 + er;
     const int s = srow[i];
-    const int n = n0 + (pc << 3);  // consecutive lanes store consecutive 16-byte chunks
-    const uint4 o = *reinterpret_cast<const uint4*>(smem + row * 512 + ((pc ^ (row & 31)) << 4));
+    const int n = n0 + wn * 64 + (ec << 3);
+    const uint4 o = *reinterpret_cast<const uint4*>(ep + row * 128 + ((ec ^ ((row >> 1) & 7)) << 4));
     if (s < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)s * p.ldc + n) = o;
   }
 }
