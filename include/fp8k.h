@@ -134,13 +134,14 @@ int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
  * Tuning and test aid (no counterpart in the reference): pins the kernel family that the dense GEMM entry points
- * pick for later calls of this process.  kind -1: automatic (the default).  kind 4: the 128x128 tile kernel with K
+ * pick for later calls made by the calling thread (the setting is thread-local; other threads keep the automatic
+ * choice).  kind -1: automatic (the default).  kind 4: the 128x128 tile kernel with K
  * cut into `splits` runs (0 or 1: none).  kind 0: the choice by the number of rows alone, without the 128x128
  * kernel.  kind 1: 256x256 tiles; kind 2: the streaming kernel (up to 128 rows); kind 3: the direct kernel (up to 32
  * rows, `splits` > 0 pins its K cut too); where a pinned family cannot take the shape, the choice by rows stands.
  * `splits` is ignored for kinds 0..2.
  * kind -2: automatic, but the last round of 256x256 tiles is kept whole instead of being computed in 128-row halves.
- * fp8k_*_workspace_bytes follows the pinned choice.  Not thread safe.
+ * fp8k_*_workspace_bytes, called from the same thread, follows the pinned choice.
  */
 void fp8k_tune_force_gemm_plan(int kind, int splits);
 

@@ -1,6 +1,7 @@
 // Host side of the FP8 GEMM entry points: argument checks mirrored from the reference ops, kernel
 // choice, launch.  No allocation, no synchronisation.
 #include <algorithm>
+#include <atomic>
 
 #include "gemm_direct.h"
 #include "gemm_tile128.h"
@@ -18,11 +19,30 @@ struct Plan {
   int64_t ws_bytes; // float workspace the plan needs
 };
 
-constexpr int kNumCU = 256;  // MI355X
+// Compute units of the current device, read once per device (a read-only cache; 256 on MI355X, which is also the
+// answer when no device is visible, so that the workspace queries work on a machine without a GPU).
+static int num_cu() {
+  constexpr int kMaxDev = 64;
+  static std::atomic<int> cache[kMaxDev];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  int n = cache[dev].load(std::memory_order_relaxed);
+  if (n > 0) return n;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
+    (void)hipGetLastError();
+    n = 256;
+  }
+  cache[dev].store(n, std::memory_order_relaxed);
+  return n;
+}
 
-// tuning aid: force the kernel family (and the K split of the uniform-split families) of later calls
-static int g_force_kind = -1, g_force_splits = 0;
-static int g_tail_halves = 1;  // tuning aid: 0 keeps the last round of 256x256 tiles whole
+// tuning aid: force the kernel family (and the K split of the uniform-split families) of later calls made by the
+// calling thread; other threads keep the automatic choice
+static thread_local int g_force_kind = -1, g_force_splits = 0;
+static thread_local int g_tail_halves = 1;  // tuning aid: 0 keeps the last round of 256x256 tiles whole
 
 static Plan plan_tile128(int64_t M, int64_t N, int kb, int splits) {
   Plan pl{4, 1, 0, 0, 0, 0};
@@ -77,20 +97,20 @@ static Plan plan_tile256(int64_t M, int64_t N, int64_t K) {
   Plan pl{1, 1, 0, 0, 0, 0};
   const int kb = (int)(K / kTileK);
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
-  const int64_t rest = tiles % kNumCU;
-  int splits = rest ? (int)(kNumCU / rest) : 1;
+  const int64_t rest = tiles % num_cu();
+  int splits = rest ? (int)(num_cu() / rest) : 1;
   if (splits > kb / 4) splits = kb / 4;
   if (splits < 1) splits = 1;
   // With at least one full round before it, the cut only pays when the tile time it saves (about 2 us per K block)
   // outweighs writing and re-reading the float partials (256 KB per piece): measured break-even.
-  if (tiles > kNumCU && kb * (splits - 1) * 8 <= rest * splits * splits) splits = 1;
+  if (tiles > num_cu() && kb * (splits - 1) * 8 <= rest * splits * splits) splits = 1;
   pl.kb_per_split = (kb + splits - 1) / splits;
   pl.splits = (kb + pl.kb_per_split - 1) / pl.kb_per_split;
   pl.tail_first = (int)(pl.splits > 1 ? tiles - rest : tiles);
   pl.ws_bytes = pl.splits > 1 ? rest * pl.splits * (int64_t)(kTileM * kTileN) * 4 : 0;
   // A last round that fills at most half the CUs and is not worth a K cut: its tiles run as two 128-row halves, one
   // workgroup each (half the matrix-core time per K block, nothing to reduce).
-  if (pl.splits == 1 && tiles > kNumCU && rest > 0 && rest <= kNumCU / 2 && M > kTileM / 2 && g_tail_halves) {
+  if (pl.splits == 1 && tiles > num_cu() && rest > 0 && rest <= num_cu() / 2 && M > kTileM / 2 && g_tail_halves) {
     pl.halves = 1;
     pl.tail_first = (int)(tiles - rest);
   }
@@ -127,10 +147,10 @@ static double est_tile128(int64_t M, int64_t N, int kb, int* best_splits) {
   for (int s = 1; s <= 8; ++s) {
     if (s > 1 && (s > kb / 4 || tiles * s > 256)) break;  // a K cut stays within one round of workgroups
     const int64_t wgs = tiles * s;
-    const int64_t rounds = (wgs + kNumCU - 1) / kNumCU;
+    const int64_t rounds = (wgs + num_cu() - 1) / num_cu();
     if (rounds > 2) break;
     const int kbps = (kb + s - 1) / s;
-    const double tb = 0.42 + 0.30 * cold * std::min(1.0, (double)wgs / kNumCU);
+    const double tb = 0.42 + 0.30 * cold * std::min(1.0, (double)wgs / num_cu());
     double t = 1.0 + (double)rounds * (kbps * tb + 2.5);
     if (rounds == 2) t *= 1.15;
     if (s > 1) t += 4.0 + (double)s * M * N * 8.0 / 5e6;
@@ -144,9 +164,9 @@ static double est_base(const Plan& pl, int64_t M, int64_t N, int64_t K) {
   if (pl.kind == 2)
     return (M <= 64 ? 10.0 : 11.0) + (double)N * K / 5.5e6 + (pl.splits > 1 ? (double)pl.splits * M * N * 8.0 / 8e6 : 0.0);
   const int64_t tiles = ((M + kTileM - 1) / kTileM) * ((N + kTileN - 1) / kTileN);
-  if (pl.splits == 1) return 8.0 + (double)((tiles + kNumCU - 1) / kNumCU) * kb * 1.6;
-  const int64_t rest = tiles % kNumCU;
-  return 8.0 + (double)(tiles / kNumCU) * kb * 1.6 + pl.kb_per_split * 1.6 + 6.0 +
+  if (pl.splits == 1) return 8.0 + (double)((tiles + num_cu() - 1) / num_cu()) * kb * 1.6;
+  const int64_t rest = tiles % num_cu();
+  return 8.0 + (double)(tiles / num_cu()) * kb * 1.6 + pl.kb_per_split * 1.6 + 6.0 +
          (double)rest * pl.splits * (kTileM * kTileN * 4) * 2.0 / 8e6;
 }
 

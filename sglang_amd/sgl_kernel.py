@@ -18,19 +18,37 @@ FP8_DTYPE = torch.float8_e4m3fn
 FP8_MAX = 448.0
 FP8_MIN = -448.0
 
-_workspaces: dict = {}
+_workspaces: dict = {}   # (device index, stream handle) -> the buffer handed out on that stream
+_retired: list = []      # every buffer ever handed out and since outgrown: kept alive for the life of the process
 
 
 def _workspace(device: torch.device, nbytes: int) -> Optional[torch.Tensor]:
-    """Per-(device, stream) split-K scratch, grown on demand and reused (never freed mid-graph)."""
+    """Scratch of the GEMM entry points (float partials of K-cut launches, the column-major scale copy), one buffer per
+    (device, stream) so that GEMMs on two streams never share one.
+
+    A buffer that has been handed out is never released: a HIP graph captured earlier still holds its address, and its
+    replays write partials there.  When a later call needs more, a larger buffer takes its place for new launches and
+    the old one is parked in `_retired`.  Growth is geometric (at least double, at least 32 MiB), so a process parks
+    a handful of buffers at most.  Allocation under stream capture goes through torch's allocator like the GEMM's
+    output tensor does, into the capturing graph's pool; `reserve_workspace` sizes the buffer ahead of a capture."""
     if nbytes <= 0:
         return None
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     buf = _workspaces.get(key)
     if buf is None or buf.numel() < nbytes:
-        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        size = max(nbytes, 32 << 20, 2 * buf.numel() if buf is not None else 0)
+        if buf is not None:
+            _retired.append(buf)
+        buf = torch.empty(size, dtype=torch.uint8, device=device)
         _workspaces[key] = buf
     return buf
+
+
+def reserve_workspace(device: torch.device, nbytes: int) -> None:
+    """Make the current stream's GEMM scratch on `device` at least `nbytes` large (see fp8k_*_workspace_bytes in
+    include/fp8k.h for what a shape needs); call it before capturing a graph to keep the allocation out of the
+    capture."""
+    _workspace(torch.device(device), int(nbytes))
 
 
 # --------------------------------------------------------------------------------------------

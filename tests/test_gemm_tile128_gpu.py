@@ -117,11 +117,13 @@ def test_automatic_plan_matches_pinned_kernels(dev):
     (same summation order), and stay within tolerance of the other families' result."""
     from sglang_amd._lib import lib
 
-    for (M, N, K) in ((128, 4608, 1536), (512, 1024, 1024), (256, 7168, 2304)):
-        xq, xs, wq, ws = _quantised_problem(M, N, K, seed=M)
+    try:
+        for (M, N, K) in ((128, 4608, 1536), (512, 1024, 1024), (256, 7168, 2304)):
+            xq, xs, wq, ws = _quantised_problem(M, N, K, seed=M)
+            lib.fp8k_tune_force_gemm_plan(-1, 0)
+            auto = _run_block(xq, xs, wq, ws, dev)
+            lib.fp8k_tune_force_gemm_plan(1, 0)
+            other = _run_block(xq, xs, wq, ws, dev)
+            assert _rel_err(auto, other) <= REL_TOL
+    finally:
         lib.fp8k_tune_force_gemm_plan(-1, 0)
-        auto = _run_block(xq, xs, wq, ws, dev)
-        lib.fp8k_tune_force_gemm_plan(1, 0)
-        other = _run_block(xq, xs, wq, ws, dev)
-        lib.fp8k_tune_force_gemm_plan(-1, 0)
-        assert _rel_err(auto, other) <= REL_TOL

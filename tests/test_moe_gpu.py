@@ -374,47 +374,105 @@ def test_fused_experts_with_absent_experts_and_no_combine(dev):
     np.testing.assert_array_equal(out.float().cpu().numpy(), O.moe_sum_reduce(per_slot.float().cpu().numpy(), 1.0))
 
 
-def test_fused_experts_deepseek_dims_few_tokens(dev):
-    """256 experts, hidden 7168, intermediate 2048, top-8 grouped-sigmoid routing; weights are generated
-    on the device (11 GB) and only the experts the tokens hit are copied back for the oracle."""
-    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl
+class _LazyExperts:
+    """Expert-indexed view of a device tensor that copies one expert to the host when the oracle asks for it."""
 
-    T, E, H, I, topk = 3, 256, 7168, 2048, 8
+    def __init__(self, t, as_u8):
+        self.t, self.as_u8, self.shape = t, as_u8, tuple(t.shape)
+
+    def __getitem__(self, e):
+        v = self.t[e]
+        return (v.view(torch.uint8) if self.as_u8 else v).cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def deepseek_experts(dev):
+    """256 experts, hidden 7168, intermediate 2048: 11 GB of random e4m3fn weights generated on the device (no NaN
+    codes) with float32 block scales; shared by the full-size tests below and released afterwards."""
+    E, H, I = 256, 7168, 2048
     g = torch.Generator(device=dev)
     g.manual_seed(0)
 
     def rand_fp8(shape):
         b = torch.randint(0, 256, shape, generator=g, device=dev, dtype=torch.uint8)
-        b = torch.where((b & 0x7F) == 0x7F, b & 0xFE, b)  # no NaN codes
-        return b.view(torch.float8_e4m3fn)
+        return torch.where((b & 0x7F) == 0x7F, b & 0xFE, b).view(torch.float8_e4m3fn)
 
     w1 = rand_fp8((E, 2 * I, H))
     w2 = rand_fp8((E, H, I))
     w1s = torch.rand((E, 2 * I // 128, H // 128), generator=g, device=dev) * 2e-4 + 1e-4
     w2s = torch.rand((E, H // 128, I // 128), generator=g, device=dev) * 2e-4 + 1e-4
-    x = O.make_activation(T, H, 0)
-    logits = torch.randn((T, E), generator=g, device=dev)
     bias = torch.randn((E,), generator=g, device=dev) * 0.1
+    yield dict(E=E, H=H, I=I, w1=w1, w2=w2, w1s=w1s, w2s=w2s, bias=bias, gen=g)
+    del w1, w2
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("T", [1, 3, 32, 256, 4096])
+def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
+    """The fused MoE layer at its full DeepSeek-V3 dimensions (256 experts, hidden 7168, intermediate 2048, top-8
+    grouped-sigmoid routing over 8 groups / 4 groups kept) for 1, 3, 32, 256 and 4096 tokens: these token counts
+    take the 16-, 32-, 64-slot and 256-slot grouped kernels in turn (asserted below).  A token's output depends on
+    nothing but its own row, its eight experts and its routed weights, so the oracle is evaluated on a sample of
+    tokens (all of them up to 3 tokens) with only the experts those tokens hit copied back; the whole output must
+    be finite, and permuting the tokens must permute the result (exactly where the kernel choice per expert is
+    unchanged, which holds for a permutation: every expert keeps its slot count)."""
+    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl, get_default_config
+
+    d = deepseek_experts
+    E, H, topk = d["E"], d["H"], 8
+    want_block = {1: 16, 3: 16, 32: 16, 256: 32, 4096: 256}[T]
+    assert get_default_config(T, E, topk)["BLOCK_SIZE_M"] == want_block
+    x = O.make_activation(T, H, T)
+    logits = torch.randn((T, E), generator=d["gen"], device=dev)
     xt = bf16_tensor(x, dev)
-    tw, ids = biased_grouped_topk_impl(xt, logits, bias, topk, True, 8, 4)
-    out = fused_experts_impl(xt, w1, w2, tw, ids, use_fp8_w8a8=True, w1_scale=w1s, w2_scale=w2s, block_shape=[128, 128],
-                             routed_scaling_factor=2.5)
+    tw, ids = biased_grouped_topk_impl(xt, logits, d["bias"], topk, True, 8, 4)
+    kw = dict(use_fp8_w8a8=True, w1_scale=d["w1s"], w2_scale=d["w2s"], block_shape=[128, 128], routed_scaling_factor=2.5)
+    out = fused_experts_impl(xt, d["w1"], d["w2"], tw, ids, **kw)
     torch.cuda.synchronize()
+    assert out.shape == (T, H) and out.dtype == torch.bfloat16
+    assert bool(torch.isfinite(out).all())
     ids_np, tw_np = ids.cpu().numpy(), tw.cpu().numpy()
 
-    class Lazy:
-        def __init__(self, t, as_u8):
-            self.t, self.as_u8, self.shape = t, as_u8, tuple(t.shape)
-
-        def __getitem__(self, e):
-            v = self.t[e]
-            return (v.view(torch.uint8) if self.as_u8 else v).cpu().numpy()
-
-    ref = O.fused_moe_block_fp8(x, Lazy(w1, True), Lazy(w1s, False), Lazy(w2, True), Lazy(w2s, False), tw_np, ids_np, 2.5)
-    assert _rel_err(out.float().cpu().numpy(), ref) <= REL_TOL
+    rng = np.random.default_rng(T)
+    sample = np.arange(T) if T <= 3 else np.unique(np.concatenate([[0, T - 1], rng.integers(0, T, 4)]))
+    ref = O.fused_moe_block_fp8(x[sample], _LazyExperts(d["w1"], True), _LazyExperts(d["w1s"], False),
+                                _LazyExperts(d["w2"], True), _LazyExperts(d["w2s"], False), tw_np[sample], ids_np[sample], 2.5)
+    got = out[torch.from_numpy(sample).to(dev)].float().cpu().numpy()
+    assert _rel_err(got, ref) <= REL_TOL, _rel_err(got, ref)
     # routing agrees with the numpy restatement (as sets; top-k order is unspecified)
-    w_ref, ids_ref = O.biased_grouped_topk(logits.cpu().numpy(), bias.cpu().numpy(), 8, 4, topk)
-    np.testing.assert_array_equal(np.sort(ids_np, 1), np.sort(ids_ref, 1))
+    _, ids_ref = O.biased_grouped_topk(logits.cpu().numpy()[sample], d["bias"].cpu().numpy(), 8, 4, topk)
+    np.testing.assert_array_equal(np.sort(ids_np[sample], 1), np.sort(ids_ref, 1))
+    if T > 3:
+        perm = torch.from_numpy(rng.permutation(T)).to(dev)
+        out_p = fused_experts_impl(xt[perm].contiguous(), d["w1"], d["w2"], tw[perm].contiguous(), ids[perm].contiguous(), **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(out_p, out[perm])
+
+
+@pytest.mark.parametrize("T,block", [(1024, 64), (2048, 128)])
+def test_fused_experts_deepseek_dims_other_block_sizes(dev, deepseek_experts, T, block):
+    """The 64- and 128-slot grouped streaming kernels at the full expert dimensions (the default choice takes them
+    between 1024 and 3072 tokens): a sample of tokens against the oracle."""
+    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl, get_default_config
+
+    d = deepseek_experts
+    E, H, topk = d["E"], d["H"], 8
+    assert get_default_config(T, E, topk)["BLOCK_SIZE_M"] == block
+    x = O.make_activation(T, H, T)
+    logits = torch.randn((T, E), generator=d["gen"], device=dev)
+    xt = bf16_tensor(x, dev)
+    tw, ids = biased_grouped_topk_impl(xt, logits, d["bias"], topk, True, 8, 4)
+    out = fused_experts_impl(xt, d["w1"], d["w2"], tw, ids, use_fp8_w8a8=True, w1_scale=d["w1s"], w2_scale=d["w2s"],
+                             block_shape=[128, 128], routed_scaling_factor=2.5)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(out).all())
+    rng = np.random.default_rng(T)
+    sample = np.unique(np.concatenate([[0, T - 1], rng.integers(0, T, 3)]))
+    ref = O.fused_moe_block_fp8(x[sample], _LazyExperts(d["w1"], True), _LazyExperts(d["w1s"], False),
+                                _LazyExperts(d["w2"], True), _LazyExperts(d["w2s"], False), tw.cpu().numpy()[sample],
+                                ids.cpu().numpy()[sample], 2.5)
+    got = out[torch.from_numpy(sample).to(dev)].float().cpu().numpy()
+    assert _rel_err(got, ref) <= REL_TOL, _rel_err(got, ref)
 
 
 @pytest.mark.parametrize("rows", [1, 7, 64, 1000])

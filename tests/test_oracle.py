@@ -347,3 +347,138 @@ def test_oracle_against_golden_vectors(case):
     if case == "a":
         wq, ws = O.block_quant_weight(_bf16_bits_to_f32(G["a_w_bf16_bits"]))
         assert np.array_equal(wq, G["a_wq"]) and np.array_equal(ws, G["a_ws"])
+
+
+# ---------------------------------------------------------------- composites: linear with bias, fused MoE, bf16 gate
+def _t_group_quant(x_bf16):
+    """Per-token-group quant as a chain of torch library ops on a bf16 tensor (the arithmetic of
+    python/sglang/test/test_block_fp8.py:23-48, written against the library, not against the oracle)."""
+    g = x_bf16.reshape(-1, 128)
+    amax = g.abs().amax(dim=-1, keepdim=True).clamp(min=1e-10).to(torch.float32)
+    s = amax / 448.0
+    q = torch.clamp(g / s, -448.0, 448.0).to(torch.float8_e4m3fn)
+    return q.reshape(x_bf16.shape), s.reshape(x_bf16.shape[0], -1)
+
+
+def _t_block_matmul_f64(q, s, wq, ws):
+    """Dequantise with broadcast scales and multiply in float64 (sgl-kernel/tests/test_fp8_blockwise_gemm.py:19-59)."""
+    a = q.to(torch.float64) * s.to(torch.float64).repeat_interleave(128, dim=1)
+    b = wq.to(torch.float64) * ws.to(torch.float64).repeat_interleave(128, dim=0).repeat_interleave(128, dim=1)
+    return a @ b.t()
+
+
+def test_block_fp8_linear_bias_branch_and_nd_input():
+    """python/sglang/srt/layers/quantization/fp8_utils.py:306-326: the bias is added to the bf16 GEMM result with a
+    bf16 tensor add (one more rounding), and leading dimensions are flattened and restored."""
+    x = O.make_activation(12, 512, 21).reshape(3, 4, 512)
+    wq, ws = O.block_quant_weight(O.make_weight(256, 512, 21))
+    bias = O.to_bf16(np.random.default_rng(21).standard_normal(256).astype(np.float32))
+    plain = O.block_fp8_linear(x, wq, ws)
+    got = O.block_fp8_linear(x, wq, ws, bias)
+    assert plain.shape == got.shape == (3, 4, 256)
+    ref = (torch.from_numpy(plain).bfloat16() + torch.from_numpy(bias).bfloat16()).float().numpy()
+    assert np.array_equal(got, ref)
+    assert not np.array_equal(got, plain + bias)  # the second rounding is visible on this data
+    # the flattened problem gives the same rows
+    assert np.array_equal(O.block_fp8_linear(x.reshape(12, 512), wq, ws, bias), got.reshape(12, 256))
+    # and the un-biased result is the torch-ops pipeline's, up to float32-vs-float64 summation at bf16 ties
+    q, s = _t_group_quant(torch.from_numpy(x.reshape(12, 512)).bfloat16())
+    y = _t_block_matmul_f64(q, s, torch.from_numpy(wq).view(torch.float8_e4m3fn), torch.from_numpy(ws))
+    y = y.to(torch.float32).bfloat16().float().numpy()
+    assert (y == plain.reshape(12, 256)).mean() > 0.995
+    assert np.abs(y - plain.reshape(12, 256)).max() <= 2.0**-7 * np.abs(y).max()
+
+
+@pytest.mark.parametrize("T,E,H,I,topk,rsf", [(20, 4, 256, 128, 2, 2.5), (33, 8, 384, 256, 3, 1.0)])
+def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf):
+    """fused_moe_block_fp8 against the same layer spelled with torch library ops, expert by expert as
+    torch_w8a8_block_fp8_moe does (python/sglang/test/test_block_fp8.py:418-447), with the roundings of the fused
+    path (fused_moe.py:498-639): GEMM1 -> bf16, silu -> bf16 -> times up -> bf16, requant, GEMM2 times the routed
+    weight in float32 -> bf16, float32 sum over the top-k in ascending k times routed_scaling_factor -> bf16.
+    The GEMMs run in float64 here and in float32 tile sums in the oracle, so a result that sits within a float32 ulp
+    of a bf16 tie may round the other way; everything else must agree bit for bit."""
+    rng = np.random.default_rng(T + E)
+    x = O.make_activation(T, H, T)
+    w13q = np.empty((E, 2 * I, H), np.uint8); w13s = np.empty((E, 2 * I // 128, H // 128), np.float32)
+    w2q = np.empty((E, H, I), np.uint8); w2s = np.empty((E, H // 128, I // 128), np.float32)
+    for e in range(E):
+        w13q[e], w13s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((2 * I, H)).astype(np.float32) * 0.05))
+        w2q[e], w2s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((H, I)).astype(np.float32) * 0.05))
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    ids[rng.random(ids.shape) < 0.1] = -1          # experts on another rank contribute nothing
+    tw = rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32)
+    got = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf)
+
+    xt = torch.from_numpy(x).bfloat16()
+    xq, xs = _t_group_quant(xt)
+    per_slot = torch.zeros((T, topk, H), dtype=torch.bfloat16)
+    t_ids, t_w = torch.from_numpy(ids), torch.from_numpy(tw)
+    for e in range(E):
+        tok, slot = torch.nonzero(t_ids == e, as_tuple=True)
+        if tok.numel() == 0:
+            continue
+        W1, S1 = torch.from_numpy(w13q[e]).view(torch.float8_e4m3fn), torch.from_numpy(w13s[e])
+        W2, S2 = torch.from_numpy(w2q[e]).view(torch.float8_e4m3fn), torch.from_numpy(w2s[e])
+        h1 = _t_block_matmul_f64(xq[tok].float(), xs[tok], W1, S1).to(torch.float32).bfloat16()
+        act = torch.nn.functional.silu(h1[:, :I].float()).bfloat16() * h1[:, I:]
+        aq, a_s = _t_group_quant(act)
+        h2 = _t_block_matmul_f64(aq.float(), a_s, W2, S2).to(torch.float32)
+        per_slot[tok, slot] = (h2 * t_w[tok, slot].unsqueeze(1)).bfloat16()
+    acc = torch.zeros((T, H), dtype=torch.float32)
+    for k in range(topk):
+        acc = acc + per_slot[:, k].float()
+    ref = (acc * rsf).bfloat16().float().numpy()
+
+    assert got.shape == ref.shape == (T, H)
+    assert (got == ref).mean() > 0.99, (got == ref).mean()
+    assert np.abs(got - ref).max() <= 2.0**-6 * np.abs(ref).max()
+    # rows whose every expert is absent are exactly zero
+    dead = (ids == -1).all(axis=1)
+    assert (got[dead] == 0).all()
+    # what a plausible mistake would change: no routed weight, weight applied after the sum, no scaling factor
+    assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, np.ones_like(tw), ids, rsf), rtol=1e-2)
+    if rsf != 1.0:
+        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0), rtol=1e-2)
+
+
+def _t_fused_gate_bf16(x, bias, G, topk_group, topk):
+    """The gate of sgl-kernel/csrc/moe/moe_fused_gate.cu:52-257 with bf16 tensors and torch library ops: every
+    intermediate (sigmoid, score + bias, the sum of a group's two best) is a bf16 tensor; the weakest group is
+    dropped repeatedly (ties: the higher group), the best expert taken repeatedly (ties: the lower expert;
+    torch.argmax returns the first maximum)."""
+    rows, E = x.shape
+    score = torch.sigmoid(x)                                # bf16 in, bf16 out
+    choice = (score + bias).reshape(rows, G, E // G).clone()
+    for _ in range(G - topk_group):
+        top2 = choice.float().topk(2, dim=-1)[0].bfloat16()
+        sums = (top2[..., 0] + top2[..., 1]).float()
+        sums = torch.where(torch.isinf(sums), torch.full_like(sums, float("inf")), sums)
+        worst = (G - 1) - torch.argmin(sums.flip(-1), dim=-1)   # last minimum = highest group among equals
+        choice[torch.arange(rows), worst] = float("inf")
+    flat = choice.float().reshape(rows, E)
+    flat = torch.where(flat == float("inf"), torch.full_like(flat, float("-inf")), flat)
+    ids = torch.empty((rows, topk), dtype=torch.int64)
+    for k in range(topk):
+        ids[:, k] = torch.argmax(flat, dim=-1)
+        flat[torch.arange(rows), ids[:, k]] = float("-inf")
+    w = score.float().gather(1, ids)
+    return (w / w.sum(-1, keepdim=True)).numpy(), ids.numpy().astype(np.int32)
+
+
+@pytest.mark.parametrize("E,G,tg,topk", [(256, 8, 4, 8), (128, 4, 2, 4)])
+def test_moe_fused_gate_bf16_branch_against_torch_bf16_ops(E, G, tg, topk):
+    """in_dtype="bf16": the oracle's rounding points against bf16 tensor arithmetic.  bf16 scores tie often, so
+    the tie rules are exercised on every row."""
+    g = torch.Generator().manual_seed(E)
+    x = torch.randn((200, E), generator=g).bfloat16()
+    bias = (torch.randn((E,), generator=g) * 0.1).bfloat16()
+    w, ids = O.moe_fused_gate(x.float().numpy(), bias.float().numpy(), G, tg, topk, in_dtype="bf16")
+    w_ref, ids_ref = _t_fused_gate_bf16(x, bias, G, tg, topk)
+    # torch's bf16 sigmoid and numpy's float32 exp can differ in the last float32 bit, which moves a bf16 score only
+    # at a tie: allow a handful of rows to differ, as sets they must still agree on all but those
+    same = (ids == ids_ref).all(axis=1)
+    assert same.mean() >= 0.98, same.mean()
+    np.testing.assert_allclose(w[same], w_ref[same], rtol=1e-6, atol=1e-7)
+    # the bf16 rounding matters: the float32 gate picks other experts on some rows of the same data
+    _, ids32 = O.moe_fused_gate(x.float().numpy(), bias.float().numpy(), G, tg, topk, in_dtype="f32")
+    assert (ids32 != ids).any()

@@ -59,9 +59,27 @@ def test_group_quant_sweep_4096(dev, seed, layout):
     _check(x, dev, 128, layout)
 
 
-def test_group_quant_16384_row_major(dev):
-    x = O.make_activation(16384, 7168, seed=0)
-    _check(x, dev, 128, (False, False, False))
+def test_group_quant_16384_every_layout(dev):
+    """The largest size of the bandwidth sweep (bf16 [16384, 7168]) in all four scale layouts.  At this size the
+    expected bytes and scales come from the C restatement of the oracle (OpenMP), which tests/test_oracle.py holds
+    bit for bit against the numpy one."""
+    from oracle import c_oracle
+
+    M, K, G = 16384, 7168, 56
+    x = O.make_activation(M, K, seed=0)
+    lib = c_oracle.load()
+    eps = float(O.clamp_eps(1e-10, "bf16"))
+    for layout in _layouts():
+        cm, al, ue = layout
+        q_ref, s_ref = c_oracle.group_quant_bf16(lib, O.bf16_bits(x), 128, eps, ue)
+        q, s = _run_group_quant(x, dev, 128, layout)
+        assert torch.equal(q.view(torch.uint8).cpu(), torch.from_numpy(q_ref)), layout
+        if ue:
+            assert s.dtype == torch.int32 and s.shape == (M, G // 4) and s.stride() == (1, M)
+            np.testing.assert_array_equal(s.cpu().numpy(), O.pack_ue8m0_scales(s_ref))
+        else:
+            assert s.shape == (M, G) and (s.stride() == (1, M) if cm else s.is_contiguous())
+            np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
 
 
 @pytest.mark.parametrize("group", [16, 32, 64, 128, 256, 512])
