@@ -133,6 +133,21 @@ int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t* As_packed
 int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * fp8k_block_gemm for callers that cannot allocate device memory or pass a workspace: code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same arguments and the
+ * same result, bit for bit, as fp8k_block_gemm, without the workspace pair: the scratch (float partials of K-cut
+ * launches, the column-major copy of row-major activation scales) is a fixed 80 MiB array in device memory that is
+ * part of this library - one copy on every GPU that loads it, held until the process ends.  The call allocates and
+ * frees nothing.  The first call on a device looks up the array's device address (hipGetSymbolAddress) and keeps it;
+ * make that call outside a graph capture.  A shape whose fp8k_block_gemm_workspace_bytes exceeds 80 MiB is refused
+ * with FP8K_ERR_WORKSPACE.  All calls on one GPU share the one array: calls that overlap in time on the same GPU
+ * (two streams, two threads) race; nothing in the array has to be cleared between calls.
+ */
+int fp8k_block_gemm_noalloc(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M,
+                            int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
+                            int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* stream);
+
+/*
  * Tuning and test aid (no counterpart in the reference): pins the kernel family that the dense GEMM entry points
  * pick for later calls made by the calling thread (the setting is thread-local; other threads keep the automatic
  * choice).  kind -1: automatic (the default).  kind 4: the 128x128 tile kernel with K

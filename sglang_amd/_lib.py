@@ -53,6 +53,7 @@ SIGNATURES = {
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 10 + [_c_int, _c_ptr, _c_i64, _c_ptr],
     ),
     "fp8k_block_gemm_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64]),
+    "fp8k_block_gemm_noalloc": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 10 + [_c_int, _c_ptr]),
     "fp8k_scaled_mm": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 6 + [_c_int, _c_int, _c_ptr, _c_i64, _c_ptr],

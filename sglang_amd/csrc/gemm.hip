@@ -2,6 +2,7 @@
 // choice, launch.  No allocation, no synchronisation.
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 
 #include "gemm_direct.h"
 #include "gemm_tile128.h"
@@ -332,11 +333,10 @@ extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) {
 extern "C" int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return block_gemm_workspace_bytes(M, N, K); }
 extern "C" int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K) { return workspace_bytes(M, N, K); }
 
-extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M,
-                               int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
-                               int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
-                               int64_t workspace_bytes_given, void* stream) {
-  clear_error();
+static int block_gemm_impl(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M, int64_t N,
+                           int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
+                           int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
+                           int64_t workspace_bytes_given, void* stream) {
   int rc = common_checks("fp8_blockwise_scaled_mm", A, B, C, M, N, K, lda, ldb, ldc, out_dtype);
   if (rc) return rc;
   if (M == 0 || N == 0) return FP8K_OK;
@@ -366,6 +366,62 @@ extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, co
   }
   return out_dtype == FP8K_BF16 ? launch<kModeBlock, FP8K_BF16, FP8K_F32>(a, pl, st)
                                 : launch<kModeBlock, FP8K_F16, FP8K_F32>(a, pl, st);
+}
+
+extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M,
+                               int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
+                               int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* workspace,
+                               int64_t workspace_bytes_given, void* stream) {
+  clear_error();
+  return block_gemm_impl(A, B, As, Bs, C, M, N, K, lda, ldb, as_stride_m, as_stride_k, bs_stride_n, bs_stride_k, ldc,
+                         out_dtype, workspace, workspace_bytes_given, stream);
+}
+
+// ---- the same GEMM for callers that cannot allocate: its scratch is a fixed array in device memory, one copy per GPU
+// that loads this library, held until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress; kernels and every other use take the device address that call returns, kept per device.
+constexpr int64_t kStaticScratchBytes = 80ll << 20;  // 64 MiB of float partials (one 256x256 tile per CU) + 16 MiB of copied scales
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static int static_scratch(void** out) {
+  constexpr int kMaxDev = 64;
+  static std::mutex mu;
+  static void* ptrs[kMaxDev];  // device address of `scratch` on each device, resolved on the first call there
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FP8K_ERR_LAUNCH, "fp8k_block_gemm_noalloc: hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= kMaxDev) return fail(FP8K_ERR_UNSUPPORTED, "fp8k_block_gemm_noalloc: device index %d not supported", dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptrs[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p)
+      return fail(FP8K_ERR_LAUNCH, "fp8k_block_gemm_noalloc: hipGetSymbolAddress: %s", hipGetErrorString(e));
+    ptrs[dev] = p;
+  }
+  *out = ptrs[dev];
+  return FP8K_OK;
+}
+
+extern "C" int fp8k_block_gemm_noalloc(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M,
+                                       int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m,
+                                       int64_t as_stride_k, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc,
+                                       int out_dtype, void* stream) {
+  clear_error();
+  const int64_t need = block_gemm_workspace_bytes(M, N, K);
+  if (need > kStaticScratchBytes)
+    return fail(FP8K_ERR_WORKSPACE, "fp8k_block_gemm_noalloc: M=%lld N=%lld K=%lld needs %lld bytes of scratch, the built-in "
+                "buffer holds %lld; use fp8k_block_gemm with a caller-owned workspace", (long long)M, (long long)N,
+                (long long)K, (long long)need, (long long)kStaticScratchBytes);
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = static_scratch(&ws);
+    if (rc) return rc;
+  }
+  // nothing in the buffer has to start at zero: every float partial and every copied scale that a launch reads was
+  // written by the same call
+  return block_gemm_impl(A, B, As, Bs, C, M, N, K, lda, ldb, as_stride_m, as_stride_k, bs_stride_n, bs_stride_k, ldc,
+                         out_dtype, ws, need > 0 ? kStaticScratchBytes : 0, stream);
 }
 
 extern "C" int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t* As_packed, const float* Bs, void* C,
