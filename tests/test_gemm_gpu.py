@@ -225,8 +225,6 @@ def _run_scaled_mm(aq, bq, sa, sb, dev, out_dtype=torch.bfloat16, bias=None):
 @pytest.mark.parametrize("N,K", [(6144, 4096), (4096, 14336)])
 @pytest.mark.parametrize("with_bias", [False, True])
 def test_scaled_mm_llama_shapes(dev, M, N, K, with_bias):
-    if M == 2048 and K == 14336 and with_bias:
-        pytest.skip("covered without bias; keeps the CPU oracle time down")
     rng = np.random.default_rng(M + N)
     x = O.make_activation(M, K, M)
     aq, sa = O.per_token_quant_fp8(x)
