@@ -237,7 +237,19 @@ static int launch_tiles(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
   const int ntiles = a.tiles_m * a.tiles_n;
   a.tail_first = pl.tail_first;
   a.tail_halves = pl.halves;
-  const unsigned nwg = (unsigned)((pl.tail_first + 7) / 8 * 8 + (ntiles - pl.tail_first) * (pl.halves ? 2 : pl.splits));
+  const int ncu8 = std::max(8, num_cu() / 8 * 8);
+  const int tail_units = (ntiles - pl.tail_first) * (pl.halves ? 2 : pl.splits);
+  unsigned nwg;
+  if (pl.tail_first > ncu8) {
+    // more whole tiles than CUs: one walking workgroup per CU, which also takes a unit of the tail at the end
+    a.walkers = ncu8;
+    a.tail_shared = 1;
+    nwg = (unsigned)std::max(ncu8, tail_units);
+  } else {
+    a.walkers = (pl.tail_first + 7) / 8 * 8;
+    a.tail_shared = 0;
+    nwg = (unsigned)(a.walkers + tail_units);
+  }
   hipLaunchKernelGGL((gemm_tile256_kernel<MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
   int rc = check_launch("gemm_tile256");
   if (rc || pl.tail_first == ntiles || pl.halves) return rc;
@@ -344,6 +356,8 @@ static int block_gemm_impl(const void* A, const void* B, const float* As, const 
   FP8K_REQUIRE(As && Bs, "fp8_blockwise_scaled_mm: null scale pointer");
   FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0,
                "fp8_blockwise_scaled_mm: negative scale stride");
+  FP8K_REQUIRE((M - 1) * as_stride_m + ((K + kTileK - 1) / kTileK - 1) * as_stride_k < (1LL << 31),
+               "fp8_blockwise_scaled_mm: scales_a spans more than 2^31 elements");
   const Plan pl = make_plan(M, N, K);
   const int64_t kb = (K + kTileK - 1) / kTileK;
   const int64_t need = wants_scale_copy(pl, M) ? align256(pl.ws_bytes) + M * kb * 4 : pl.ws_bytes;
@@ -436,6 +450,7 @@ extern "C" int fp8k_block_gemm_ue8m0(const void* A, const void* B, const int32_t
   FP8K_REQUIRE(K > 0, "%s: K must be positive", op);
   FP8K_REQUIRE(As_packed && Bs, "%s: null scale pointer", op);
   FP8K_REQUIRE(as_stride_m >= 0 && as_stride_w >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0, "%s: negative scale stride", op);
+  FP8K_REQUIRE((M - 1) * as_stride_m + ((K + kTileK - 1) / kTileK / 4) * as_stride_w < (1LL << 31), "%s: scales span more than 2^31 elements", op);
   const Plan pl = make_plan(M, N, K);
   // the matrix core applies the scales only in the tile kernels; smaller problems take the float-scale
   // entry point with the exponents expanded to floats

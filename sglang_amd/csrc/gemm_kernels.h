@@ -29,6 +29,8 @@ struct GemmArgs {
   int kb_per_split;
   int tail_first;     // tile256 only: tiles [tail_first, tiles) are the ones cut along K or into halves
   int tail_halves;    // tile256 only: those tiles are computed as two 128-row halves, one workgroup each (no K cut)
+  int walkers;        // tile256 only: workgroups [0, walkers) walk the whole tiles (a multiple of 8)
+  int tail_shared;    // tile256 only: unit u of the tail belongs to workgroup u (after its walk), else to workgroup walkers + u
   // grouped (MoE) form of the streaming kernel; all null / zero for a dense GEMM
   const int32_t* sorted_ids;    // [m_blocks * TM] token slots, padded with values >= num_valid
   const int32_t* expert_ids;    // [m_blocks] expert of each block of TM slots, -1 = not on this rank
@@ -147,14 +149,19 @@ __device__ __forceinline__ void tile_coords(int t, int tiles_m, int tiles_n, int
   tile_n = tin / gsz;
 }
 
-// Tiles [0, tail_first) are computed whole, one per workgroup, each XCD walking a contiguous run of them.
-// Tiles [tail_first, tiles) - the last, partial round over the chip's CUs - are cut into `splits` K ranges, one
-// workgroup each, so that the round takes 1/splits of a tile time; they leave float partials in the workspace
-// ([tile - tail_first][split][256 m][256 n]) for tile_reduce_kernel.  Their workgroup ids come last, so they are
-// dispatched when the whole tiles drain.  With tail_halves the tiles of the last round are instead computed as two
-// 128-row halves, one workgroup each: the four waves of the lower half of the tile do the MFMAs (one per SIMD, so
-// a K block takes half the matrix-core time), the other four only take part in the loads, and nothing has to be
-// reduced afterwards.
+// scheduling barrier: the compiler moves nothing across it (used by the hand-ordered K loops here and in gemm_tile128.h)
+#define SB() __builtin_amdgcn_sched_barrier(0)
+
+// Work of a launch.  Tiles [0, tail_first) are computed whole.  The first `walkers` workgroups (a multiple of 8,
+// at most one per CU) walk them: workgroup (xcd, c) takes tiles xcd*per_xcd + c, + walkers/8, ... of its XCD's
+// contiguous run, and requests the first K block of its next tile before it writes the finished one out, so the
+// new tile's first lines travel while the old tile leaves through LDS and neither a workgroup launch nor a cold
+// first load sits between two tiles.  Tiles [tail_first, tiles) - the last, partial round over the chip's CUs - are
+// either cut into `splits` K ranges that leave float partials in the workspace ([tile - tail_first][split][256 m]
+// [256 n]) for tile_reduce_kernel, or (tail_halves) computed as two 128-row halves: the four waves of the lower
+// half of the tile do the MFMAs (one per SIMD, so a K block takes half the matrix-core time), the other four only
+// take part in the loads, and nothing has to be reduced afterwards.  Unit u of that tail goes to workgroup u after
+// its walk (tail_shared: more whole tiles than CUs) or to workgroup walkers + u.
 template <int MODE, int OUT_DT, int BIAS_DT>
 __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) {
   // the whole LDS: three weight stages (the weights travel two K blocks ahead: their lines come from HBM or the
@@ -167,373 +174,437 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   const int wn = w & 1, wm = w >> 1;
 
   const int bid = blockIdx.x;
-  int t = 0, split = 0, half = 0;
-  bool is_split = false, is_half = false;
-  int tile_m, tile_n;
-  {
-    const int ntiles = p.tiles_m * p.tiles_n;
+  // ---- this workgroup's items: the whole tiles of its walk, then at most one unit of the tail
+  int walk_next = 0, walk_step = 1, walk_first = 0, walk_end = 0;
+  if (bid < p.walkers) {
     const int per_xcd = (p.tail_first + 7) >> 3;
-    if (bid < per_xcd * 8) {
-      t = (bid & 7) * per_xcd + (bid >> 3);
-      if (t >= p.tail_first) return;
-    } else {
-      const int b2 = bid - per_xcd * 8;
-      if (p.tail_halves) {
-        is_half = true;
-        t = p.tail_first + (b2 >> 1);
-        half = b2 & 1;
-      } else {
-        is_split = true;
-        t = p.tail_first + b2 / p.splits;
-        split = b2 % p.splits;
-      }
-      if (t >= ntiles) return;
+    walk_next = bid >> 3;
+    walk_step = p.walkers >> 3;
+    walk_first = (bid & 7) * per_xcd;
+    walk_end = min(walk_first + per_xcd, p.tail_first);
+  }
+  int tail_unit = p.tail_shared ? bid : bid - p.walkers;
+  {
+    const int units = (p.tiles_m * p.tiles_n - p.tail_first) * (p.tail_halves ? 2 : p.splits);
+    if (tail_unit >= units) tail_unit = -1;
+  }
+  struct Item { int t, split, half; bool is_split, is_half; };
+  auto next_item = [&](Item& it) -> bool {
+    if (walk_first + walk_next < walk_end) {
+      it = Item{walk_first + walk_next, 0, 0, false, false};
+      walk_next += walk_step;
+      return true;
     }
+    if (tail_unit >= 0) {
+      if (p.tail_halves) it = Item{p.tail_first + (tail_unit >> 1), 0, tail_unit & 1, false, true};
+      else it = Item{p.tail_first + tail_unit / p.splits, tail_unit % p.splits, 0, true, false};
+      tail_unit = -1;
+      return true;
+    }
+    return false;
+  };
+  Item item;
+  if (!next_item(item)) return;
+
+  bool first_item = true;  // no item before this one has requested its first K block
+  for (;;) {
+    const int t = item.t, split = item.split, half = item.half;
+    const bool is_split = item.is_split, is_half = item.is_half;
+    // The lane-dependent constants are derived anew for every tile from a lane id the compiler cannot see through:
+    // hoisted out of the tile loop they would all stay live across it and push the K loop's operands into scratch.
+    int ln = lane;
+    asm volatile("" : "+v"(ln));
+    // ---- lane constants of the global -> LDS loads and of the LDS -> MFMA operand fetches
+    const int rl = ln >> 3, cp = ln & 7;
+    uint32_t voW[2], voX[2];
+#pragma unroll
+    for (int par = 0; par < 2; ++par) {
+      const int c = cp ^ ((par << 2) + (rl >> 1));
+      voW[par] = (uint32_t)(rl * p.ldw + c * 16);
+      voX[par] = (uint32_t)(rl * p.ldx + c * 16);
+    }
+    const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = (uint32_t)(w * 32 * p.ldx);
+    const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = (uint32_t)(8 * p.ldx);
+    const int lr = ln & 31, h = ln >> 5;
+    const int swz = (lr >> 1) & 7;
+    // lane part of an operand fetch address: row lr of a 32-row group, 16-byte chunk (ks, j) at its swizzled place.
+    // Stage, wave position and group are uniform and reach the address through scalar registers, so weights and
+    // activations share these four registers.
+    uint32_t fa[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) fa[ks][j] = (uint32_t)(lr * kTileK + (((ks * 4 + h * 2 + j) ^ swz) << 4));
+    auto frag = [&](const uint8_t* grp, int ks) -> v8i {  // grp: first row of the 32-row group inside its stage (uniform)
+      const v4i lo = *reinterpret_cast<const v4i*>(grp + fa[ks][0]);
+      const v4i hi = *reinterpret_cast<const v4i*>(grp + fa[ks][1]);
+      v8i r;
+      r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+      r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+      return r;
+    };
+
+    // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the matrix edge are out
+    // of range and read as zero
+    rsrc_t rW = make_rsrc(p.W, 0), rX = make_rsrc(p.X, 0);
+    auto tile_rsrcs = [&](int tile, int hf, bool halved, int kb0) {
+      int tm, tn;
+      tile_coords(tile, p.tiles_m, p.tiles_n, tm, tn);
+      const int mm = tm * kTileM + hf * (kTileM / 2), nn = tn * kTileN;
+      const int rowsW = min(kTileN, p.N - nn), rowsX = min(halved ? kTileM / 2 : kTileM, p.M - mm);
+      const int kbytes = p.K - kb0 * kTileK;
+      rW = make_rsrc(p.W + (int64_t)nn * p.ldw + (int64_t)kb0 * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
+      rX = make_rsrc(p.X + (int64_t)mm * p.ldx + (int64_t)kb0 * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
+    };
+    // one 1 KB global->LDS load (slice j of the wave's 32 rows) of K block kstep into weight stage ws / activation
+    // stage xst.  The whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt
+    // from the range check, and rows past the matrix edge must read as zero, not touch memory).
+    auto LW = [&](int j, int kstep, int ws) {
+      buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + (uint32_t)kstep * kTileK), 0, smem + ws * kWStage + w * 4096 + j * 1024);
+    };
+    auto LX = [&](int j, int kstep, int xst) {
+      buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + (uint32_t)kstep * kTileK), 0,
+                        smem + kXBase + xst * kXStage + w * 4096 + j * 1024);
+    };
+
+    int tile_m, tile_n;
     tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
-  }
-  const int m0 = tile_m * kTileM + half * (kTileM / 2), n0 = tile_n * kTileN;
-  if (m0 >= p.M) return;                                              // upper half of a tile past the last row
-  const int nrows = is_half ? min(p.M, m0 + kTileM / 2) : p.M;        // exclusive bound of a valid output row
+    const int m0 = tile_m * kTileM + half * (kTileM / 2), n0 = tile_n * kTileN;
+    if (m0 >= p.M) return;                                              // upper half of a tile past the last row
+    const int nrows = is_half ? min(p.M, m0 + kTileM / 2) : p.M;        // exclusive bound of a valid output row
 
-  const int kb_begin = is_split ? split * p.kb_per_split : 0;
-  const int kb_end = is_split ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
-  const int nkb = kb_end - kb_begin;
+    const int kb_begin = is_split ? split * p.kb_per_split : 0;
+    const int kb_end = is_split ? min(p.K / kTileK, kb_begin + p.kb_per_split) : p.K / kTileK;
+    const int nkb = kb_end - kb_begin;
 
-  auto slot_at = [&](int i) -> int { return m0 + i; };
+    auto slot_at = [&](int i) -> int { return m0 + i; };
+    tile_rsrcs(t, half, is_half, kb_begin);
 
-  // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the
-  // matrix edge are out of range and read as zero
-  const uint8_t* Wb = p.W;
-  const int rowsW = min(kTileN, p.N - n0), rowsX = min(is_half ? kTileM / 2 : kTileM, p.M - m0);
-  const int kbytes = p.K - kb_begin * kTileK;
-  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
-  const rsrc_t rX = make_rsrc(p.X + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
-  const int rl = lane >> 3, cp = lane & 7;
-  uint32_t voW[2], voX[2];
-#pragma unroll
-  for (int par = 0; par < 2; ++par) {
-    const int c = cp ^ ((par << 2) + (rl >> 1));
-    voW[par] = (uint32_t)(rl * p.ldw + c * 16);
-    voX[par] = (uint32_t)(rl * p.ldx + c * 16);
-  }
-  const uint32_t soW = (uint32_t)(w * 32 * p.ldw), soX = (uint32_t)(w * 32 * p.ldx);
-  const uint32_t stepW = (uint32_t)(8 * p.ldw), stepX = (uint32_t)(8 * p.ldx);
-  // ---- LDS -> MFMA operands
-  const int lr = lane & 31, h = lane >> 5;
-  const int swz = (lr >> 1) & 7;
-  uint32_t co[2][2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) co[ks][j] = (uint32_t)(((ks * 4 + h * 2 + j) ^ swz) << 4);
-  const uint32_t rdW = (uint32_t)((wn * 128 + lr) * kTileK);
-  const uint32_t rdX = (uint32_t)((wm * 64 + lr) * kTileK);
-  auto frag = [&](const uint8_t* st, uint32_t rowoff, int ks) -> v8i {
-    const v4i lo = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][0]);
-    const v4i hi = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][1]);
-    v8i r;
-    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-    return r;
-  };
+    // ---- scales (block mode)
+    // activation rows whose scales this lane applies (any valid row for padding lanes)
+    const int mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
+    const int mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
+    // element offsets of this lane's two scale rows (32 bits: the host checks M * K/128 against 2^31)
+    const uint32_t sxo0 = (uint32_t)((int64_t)mrow0 * p.sx_m + (int64_t)kb_begin * p.sx_k);
+    const uint32_t sxo1 = (uint32_t)((int64_t)mrow1 * p.sx_m + (int64_t)kb_begin * p.sx_k);
+    const uint32_t sxk = (uint32_t)p.sx_k;
+    const int nb = min(n0 + wn * 128, p.N - 1) >> 7;
+    const float* swp = p.sw + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
+    // scaled mode: sx points at int32 words of four UE8M0 bytes (K blocks 4j..4j+3 of a row), sx_k = word stride
+    const uint32_t* sqp = reinterpret_cast<const uint32_t*>(p.sx);
+    const uint32_t sqo0 = (uint32_t)((int64_t)mrow0 * p.sx_m), sqo1 = (uint32_t)((int64_t)mrow1 * p.sx_m);
+    int sq[2] = {127, 127}, sqw = 127;      // exponent bytes of the block the current MFMAs belong to
+    uint32_t q0n = 0, q1n = 0;              // words holding the next block's activation exponents
 
-  // ---- scales (block mode)
-  // activation rows whose scales this lane applies (any valid row for padding lanes)
-  const int mrow0 = min(m0 + wm * 64 + lr, p.M - 1);
-  const int mrow1 = min(m0 + wm * 64 + 32 + lr, p.M - 1);
-  const float* sx0 = p.sx + (int64_t)mrow0 * p.sx_m + (int64_t)kb_begin * p.sx_k;
-  const float* sx1 = p.sx + (int64_t)mrow1 * p.sx_m + (int64_t)kb_begin * p.sx_k;
-  const int nb = min(n0 + wn * 128, p.N - 1) >> 7;
-  const float* swp = p.sw + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
-  // scaled mode: sx points at int32 words of four UE8M0 bytes (K blocks 4j..4j+3 of a row), sx_k = word stride
-  const uint32_t* sq0p = reinterpret_cast<const uint32_t*>(p.sx) + (int64_t)mrow0 * p.sx_m;
-  const uint32_t* sq1p = reinterpret_cast<const uint32_t*>(p.sx) + (int64_t)mrow1 * p.sx_m;
-  int sq[2] = {127, 127}, sqw = 127;      // exponent bytes of the block the current MFMAs belong to
-  uint32_t q0n = 0, q1n = 0;              // words holding the next block's activation exponents
+    v16f acc[4][2];
+#pragma unroll
+    for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
 
-  v16f acc[4][2];
-#pragma unroll
-  for (int ns = 0; ns < 4; ++ns)
-#pragma unroll
-    for (int ms = 0; ms < 2; ++ms)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
+    // Operand registers: X[ms][ks] the four activation fragments of a K block, W[ks] the two fragments of ONE weight
+    // group.  A K block is walked as four steps, one per weight group ns, each step the MFMAs (ms, ks) = (0,0) (1,0)
+    // (0,1) (1,1): W[0] is free after the second and W[1] after the fourth, and each is refilled in place with the
+    // next group's fragment two MFMAs before its first use.  (A second set of weight registers would push the block
+    // mode past 256 registers, and scratch reloads inside the K loop cannot coexist with its partial vmcnt waits.)
+    v8i X[2][2], W[2];
+    v16f tq[2];
+    float sc[2] = {0.f, 0.f}, scn[2] = {0.f, 0.f};
+    float s0n = 0.f, s1n = 0.f, sbn = 0.f;
 
-  v8i X[2][2], WA[2], WB[2];   // [.][ks]
-  v16f tq[2];
-  float sc[2] = {0.f, 0.f}, scn[2] = {0.f, 0.f};
-  float s0n = 0.f, s1n = 0.f, sbn = 0.f;
-
-#define SB() __builtin_amdgcn_sched_barrier(0)
-  // one 1 KB global->LDS load (slice j of the wave's 32 rows) of K block kstep into weight stage ws / activation
-  // stage xst.  The whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt
-  // from the range check, and rows past the matrix edge must read as zero, not touch memory).
-  auto LW = [&](int j, int kstep, int ws) {
-    buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + (uint32_t)kstep * kTileK), 0, smem + ws * kWStage + w * 4096 + j * 1024);
-  };
-  auto LX = [&](int j, int kstep, int xst) {
-    buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + (uint32_t)kstep * kTileK), 0,
-                      smem + kXBase + xst * kXStage + w * 4096 + j * 1024);
-  };
-  auto RW = [&](v8i(&dst)[2], const uint8_t* st, int ns) {
-    dst[0] = frag(st, rdW + ns * 32 * kTileK, 0);
-    dst[1] = frag(st, rdW + ns * 32 * kTileK, 1);
-  };
-  auto RX = [&](const uint8_t* st, int ms) {  // st: activation stage
-    X[ms][0] = frag(st, rdX + ms * 32 * kTileK, 0);
-    X[ms][1] = frag(st, rdX + ms * 32 * kTileK, 1);
-  };
-  // one group = the two K-halves of one 32x32 tile
-  auto G = [&](const v8i(&W)[2], int ms, v16f& a, v16f& tt) {
-    if (MODE == kModeBlock) {
-      v16f z;
+    auto RW = [&](int ks, const uint8_t* st, int ns) { W[ks] = frag(st + (wn * 128 + ns * 32) * kTileK, ks); };
+    auto RX = [&](int ms, int ks, const uint8_t* st) { X[ms][ks] = frag(st + (wm * 64 + ms * 32) * kTileK, ks); };
+    // one MFMA of step ns.  Block mode: the products of a step gather in tq[ms] (K half 0 starts from zero, K half 1
+    // adds), to be folded into acc[ns][ms] with the block's scale during the next step; the other modes accumulate
+    // in place.
+    auto M = [&](int ms, int ks, int ns) {
+      if (MODE == kModeBlock) {
+        if (ks == 0) {
+          v16f z;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) z[r] = 0.f;
-      tt = mfma_32x32x64(W[0], X[ms][0], z);
-      tt = mfma_32x32x64(W[1], X[ms][1], tt);
-    } else if (MODE == kModeScaled) {
-      a = mfma_32x32x64_scaled(W[0], X[ms][0], a, sqw, sq[ms]);
-      a = mfma_32x32x64_scaled(W[1], X[ms][1], a, sqw, sq[ms]);
-    } else {
-      a = mfma_32x32x64(W[0], X[ms][0], a);
-      a = mfma_32x32x64(W[1], X[ms][1], a);
+          for (int r = 0; r < 16; ++r) z[r] = 0.f;
+          tq[ms] = mfma_32x32x64(W[0], X[ms][0], z);
+        } else {
+          tq[ms] = mfma_32x32x64(W[1], X[ms][1], tq[ms]);
+        }
+      } else if (MODE == kModeScaled) {
+        acc[ns][ms] = mfma_32x32x64_scaled(W[ks], X[ms][ks], acc[ns][ms], sqw, sq[ms]);
+      } else {
+        acc[ns][ms] = mfma_32x32x64(W[ks], X[ms][ks], acc[ns][ms]);
+      }
+    };
+    // the 16 scale-FMAs that fold a finished product into its accumulator (block mode only)
+    auto F = [&](v16f& a, const v16f& tt, float sv) {
+      if (MODE == kModeBlock) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) a[r] = __builtin_fmaf(tt[r], sv, a[r]);
+      }
+    };
+
+    if (nkb <= 0) return;
+    if (is_half && wm >= 2) {
+      // half tile (always a workgroup's last item): the waves of the upper 128 rows issue their share of the loads
+      // (their activation rows are out of range and arrive as zeros) and keep the barriers, with the same order and
+      // counts of loads as the others
+      if (first_item) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+      }
+      wait_vm0();
+      __syncthreads();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LX(j, 1, 1);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LW(j, 1, 1);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LW(j, 2, 2);
+      int w_ld = 0, w_rd = 1;
+      for (int it = 0; it < nkb - 1; ++it) {
+        lds_barrier<4>();
+        SB();
+#pragma unroll
+        for (int j = 0; j < 4; ++j) LX(j, it + 2, it & 1);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) LW(j, it + 3, w_ld);
+        w_ld = w_rd;
+        w_rd = w_rd == 2 ? 0 : w_rd + 1;
+      }
+      wait_vm0();
+      lds_barrier();  // the others' barrier in front of the write-out
+      return;
     }
-  };
-  // group g's two MFMAs with the previous group's 16 scale-FMAs split around them
-  auto GF = [&](const v8i(&W)[2], int ms, v16f& a, v16f& tt, v16f& ap, const v16f& tp, float s) {
-    if (MODE == kModeBlock) {
-      v16f z;
+    // ---- prologue: block 0 into stage 0, block 1 into stage 1, steps 0..2 of block 0.  Block 0 of every item but a
+    // workgroup's first was requested before the previous item's write-out.
+    if (first_item) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) z[r] = 0.f;
-      tt = mfma_32x32x64(W[0], X[ms][0], z);
-      __builtin_amdgcn_sched_barrier(0);
+      for (int j = 0; j < 4; ++j) LX(j, 0, 0);
 #pragma unroll
-      for (int r = 0; r < 8; ++r) ap[r] = __builtin_fmaf(tp[r], s, ap[r]);
-      __builtin_amdgcn_sched_barrier(0);
-      tt = mfma_32x32x64(W[1], X[ms][1], tt);
-      __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int r = 8; r < 16; ++r) ap[r] = __builtin_fmaf(tp[r], s, ap[r]);
-    } else if (MODE == kModeScaled) {
-      a = mfma_32x32x64_scaled(W[0], X[ms][0], a, sqw, sq[ms]);
-      a = mfma_32x32x64_scaled(W[1], X[ms][1], a, sqw, sq[ms]);
-    } else {
-      a = mfma_32x32x64(W[0], X[ms][0], a);
-      a = mfma_32x32x64(W[1], X[ms][1], a);
+      for (int j = 0; j < 4; ++j) LW(j, 0, 0);
     }
-  };
-  auto F = [&](v16f& a, const v16f& tt, float s) {
-    if (MODE == kModeBlock) {
-#pragma unroll
-      for (int r = 0; r < 16; ++r) a[r] = __builtin_fmaf(tt[r], s, a[r]);
-    }
-  };
-
-  if (nkb <= 0) return;
-  if (is_half && wm >= 2) {
-    // half tile: the waves of the upper 128 rows issue their share of the loads (their activation rows are out of
-    // range and arrive as zeros) and keep the barriers, with the same order and counts of loads as the others
-#pragma unroll
-    for (int j = 0; j < 4; ++j) LX(j, 0, 0);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+    if (MODE == kModeBlock) { sc[0] = p.sx[sxo0]; sc[1] = p.sx[sxo1]; const float sb = swp[0]; sc[0] *= sb; sc[1] *= sb; }
+    auto exponents = [&](uint32_t w0, uint32_t w1, float sb, int kb_abs) {  // -> sq, sqw for K block kb_abs
+      const int sh = (kb_abs & 3) * 8;
+      sq[0] = (int)(w0 >> sh);
+      sq[1] = (int)(w1 >> sh);
+      sqw = (int)(__float_as_uint(sb) >> 23);
+    };
+    if (MODE == kModeScaled) exponents(sqp[sqo0 + (uint32_t)(kb_begin >> 2) * sxk], sqp[sqo1 + (uint32_t)(kb_begin >> 2) * sxk], swp[0], kb_begin);
     wait_vm0();
     __syncthreads();
+    // scales of block 1, then activations of block 1, weights of blocks 1 and 2: the order the loop keeps, so that at
+    // a barrier only a wave's four youngest loads - weights for the block after next - may still be in flight
+    if (MODE == kModeBlock) { const int kn = min(1, nkb - 1); s0n = p.sx[sxo0 + (uint32_t)kn * sxk]; s1n = p.sx[sxo1 + (uint32_t)kn * sxk]; sbn = swp[(int64_t)kn * p.sw_k]; }
+    if (MODE == kModeScaled) {
+      const int kn = min(1, nkb - 1);
+      q0n = sqp[sqo0 + (uint32_t)((kb_begin + kn) >> 2) * sxk]; q1n = sqp[sqo1 + (uint32_t)((kb_begin + kn) >> 2) * sxk]; sbn = swp[(int64_t)kn * p.sw_k];
+    }
+    SB();
 #pragma unroll
     for (int j = 0; j < 4; ++j) LX(j, 1, 1);
 #pragma unroll
     for (int j = 0; j < 4; ++j) LW(j, 1, 1);
 #pragma unroll
     for (int j = 0; j < 4; ++j) LW(j, 2, 2);
-    int w_ld = 0, w_rd = 1;
+    RX(0, 0, smem + kXBase); RX(1, 0, smem + kXBase); RW(0, smem, 0);
+    RX(0, 1, smem + kXBase); RX(1, 1, smem + kXBase); RW(1, smem, 0);
+    SB();
+    // steps 0..2 of block 0
+    M(0, 0, 0); SB();
+    M(1, 0, 0); SB();
+    RW(0, smem, 1); SB();
+    M(0, 1, 0); SB();
+    M(1, 1, 0); SB();
+    RW(1, smem, 1); SB();
+    F(acc[0][0], tq[0], sc[0]); SB();
+    M(0, 0, 1); SB();
+    F(acc[0][1], tq[1], sc[1]); SB();
+    M(1, 0, 1); SB();
+    RW(0, smem, 2); SB();
+    M(0, 1, 1); SB();
+    M(1, 1, 1); SB();
+    RW(1, smem, 2); SB();
+    F(acc[1][0], tq[0], sc[0]); SB();
+    M(0, 0, 2); SB();
+    F(acc[1][1], tq[1], sc[1]); SB();
+    M(1, 0, 2); SB();
+    RW(0, smem, 3); SB();
+    M(0, 1, 2); SB();
+    M(1, 1, 2); SB();
+    RW(1, smem, 3); SB();
+    // pending: F(acc[2][0], tq[0], sc[0]), F(acc[2][1], tq[1], sc[1])
+
+    int w_ld = 0, w_rd = 1;  // weight stages: the one block it left (refilled with block it+3), the one of block it+1
     for (int it = 0; it < nkb - 1; ++it) {
-      lds_barrier<4>();
+      const uint8_t* stW = smem + w_rd * kWStage;                     // block it+1
+      const uint8_t* stX = smem + kXBase + ((it + 1) & 1) * kXStage;
+      const int xl = it & 1;                                          // activation stage block it left
+      lds_barrier<4>();  // block it+1 has landed; the weights of block it+2 may still be on their way
       SB();
-#pragma unroll
-      for (int j = 0; j < 4; ++j) LX(j, it + 2, it & 1);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) LW(j, it + 3, w_ld);
+      // ---- step 3 of block it; every operand register is refilled from block it+1 after its last use
+      F(acc[2][0], tq[0], sc[0]); SB();
+      M(0, 0, 3); SB();
+      RX(0, 0, stX); LX(0, it + 2, xl); LX(1, it + 2, xl); SB();
+      F(acc[2][1], tq[1], sc[1]); SB();
+      M(1, 0, 3); SB();
+      RX(1, 0, stX); RW(0, stW, 0); LX(2, it + 2, xl); LX(3, it + 2, xl); SB();
+      M(0, 1, 3); SB();
+      RX(0, 1, stX); SB();
+      M(1, 1, 3); SB();
+      RX(1, 1, stX); RW(1, stW, 0); SB();
+      if (MODE == kModeBlock) { scn[0] = s0n * sbn; scn[1] = s1n * sbn; }
+      // ---- step 0 of block it+1; the pending products still belong to block it
+      F(acc[3][0], tq[0], sc[0]); SB();
+      if (MODE == kModeScaled) exponents(q0n, q1n, sbn, kb_begin + it + 1);  // the MFMAs from here on are block it+1's
+      M(0, 0, 0); SB();
+      F(acc[3][1], tq[1], sc[1]); SB();
+      M(1, 0, 0); SB();
+      // the scales of block it+2 are requested after the activation loads and before the weight loads: the wait in
+      // front of their use then leaves exactly the weight loads in flight
+      if (MODE == kModeBlock) {
+        sc[0] = scn[0]; sc[1] = scn[1];
+        const int kn = min(it + 2, nkb - 1);
+        s0n = p.sx[sxo0 + (uint32_t)kn * sxk]; s1n = p.sx[sxo1 + (uint32_t)kn * sxk]; sbn = swp[(int64_t)kn * p.sw_k];
+      }
+      if (MODE == kModeScaled) {
+        const int kn = min(it + 2, nkb - 1);
+        q0n = sqp[sqo0 + (uint32_t)((kb_begin + kn) >> 2) * sxk]; q1n = sqp[sqo1 + (uint32_t)((kb_begin + kn) >> 2) * sxk]; sbn = swp[(int64_t)kn * p.sw_k];
+      }
+      SB();
+      RW(0, stW, 1); LW(0, it + 3, w_ld); LW(1, it + 3, w_ld); SB();
+      M(0, 1, 0); SB();
+      M(1, 1, 0); SB();
+      RW(1, stW, 1); LW(2, it + 3, w_ld); LW(3, it + 3, w_ld); SB();
+      // ---- steps 1 and 2 of block it+1
+      F(acc[0][0], tq[0], sc[0]); SB();
+      M(0, 0, 1); SB();
+      F(acc[0][1], tq[1], sc[1]); SB();
+      M(1, 0, 1); SB();
+      RW(0, stW, 2); SB();
+      M(0, 1, 1); SB();
+      M(1, 1, 1); SB();
+      RW(1, stW, 2); SB();
+      F(acc[1][0], tq[0], sc[0]); SB();
+      M(0, 0, 2); SB();
+      F(acc[1][1], tq[1], sc[1]); SB();
+      M(1, 0, 2); SB();
+      RW(0, stW, 3); SB();
+      M(0, 1, 2); SB();
+      M(1, 1, 2); SB();
+      RW(1, stW, 3); SB();
       w_ld = w_rd;
       w_rd = w_rd == 2 ? 0 : w_rd + 1;
     }
-    wait_vm0();
-    if ((p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0) lds_barrier();  // the others' epilogue barrier
-    return;
-  }
-  // ---- prologue: block 0 into stage 0, block 1 into stage 1, groups (0,0)..(2,1) of block 0
-#pragma unroll
-  for (int j = 0; j < 4; ++j) LX(j, 0, 0);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) LW(j, 0, 0);
-  if (MODE == kModeBlock) { sc[0] = sx0[0]; sc[1] = sx1[0]; const float sb = swp[0]; sc[0] *= sb; sc[1] *= sb; }
-  auto exponents = [&](uint32_t w0, uint32_t w1, float sb, int kb_abs) {  // -> sq, sqw for K block kb_abs
-    const int sh = (kb_abs & 3) * 8;
-    sq[0] = (int)(w0 >> sh);
-    sq[1] = (int)(w1 >> sh);
-    sqw = (int)(__float_as_uint(sb) >> 23);
-  };
-  if (MODE == kModeScaled) exponents(sq0p[(int64_t)(kb_begin >> 2) * p.sx_k], sq1p[(int64_t)(kb_begin >> 2) * p.sx_k], swp[0], kb_begin);
-  wait_vm0();
-  __syncthreads();
-  // scales of block 1, then activations of block 1, weights of blocks 1 and 2: the order the loop keeps, so that at
-  // a barrier only a wave's four youngest loads - weights for the block after next - may still be in flight
-  if (MODE == kModeBlock) { const int kn = min(1, nkb - 1); s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k]; }
-  if (MODE == kModeScaled) {
-    const int kn = min(1, nkb - 1);
-    q0n = sq0p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; q1n = sq1p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
-  }
-  SB();
-#pragma unroll
-  for (int j = 0; j < 4; ++j) LX(j, 1, 1);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) LW(j, 1, 1);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) LW(j, 2, 2);
-  RX(smem + kXBase, 0); RX(smem + kXBase, 1); RW(WA, smem, 0); RW(WB, smem, 1);
-  SB();
-  G(WA, 0, acc[0][0], tq[0]); SB();
-  GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();
-  RW(WA, smem, 2); SB();
-  GF(WB, 0, acc[1][0], tq[0], acc[0][1], tq[1], sc[1]); SB();
-  GF(WB, 1, acc[1][1], tq[1], acc[1][0], tq[0], sc[0]); SB();
-  RW(WB, smem, 3); SB();
-  GF(WA, 0, acc[2][0], tq[0], acc[1][1], tq[1], sc[1]); SB();
-  GF(WA, 1, acc[2][1], tq[1], acc[2][0], tq[0], sc[0]); SB();
-  // pending: F(acc[2][1], tq[1], sc[1])
+    // ---- step 3 of the last block
+    F(acc[2][0], tq[0], sc[0]); SB();
+    M(0, 0, 3); SB();
+    F(acc[2][1], tq[1], sc[1]); SB();
+    M(1, 0, 3); SB();
+    M(0, 1, 3); SB();
+    M(1, 1, 3); SB();
+    F(acc[3][0], tq[0], sc[0]);
+    F(acc[3][1], tq[1], sc[1]);
 
-  int w_ld = 0, w_rd = 1;  // weight stages: the one block it left (refilled with block it+3), the one of block it+1
-  for (int it = 0; it < nkb - 1; ++it) {
-    const uint8_t* stW = smem + w_rd * kWStage;                     // block it+1
-    const uint8_t* stX = smem + kXBase + ((it + 1) & 1) * kXStage;
-    const int xl = it & 1;                                          // activation stage block it left
-    lds_barrier<4>();  // block it+1 has landed; the weights of block it+2 may still be on their way
-    SB();
-    RW(WA, stW, 0); SB();
-    GF(WB, 0, acc[3][0], tq[0], acc[2][1], tq[1], sc[1]); SB();
-    RX(stX, 0); LX(0, it + 2, xl); LX(1, it + 2, xl); SB();
-    GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]); SB();
-    RX(stX, 1); RW(WB, stW, 1); LX(2, it + 2, xl); LX(3, it + 2, xl); SB();
-    if (MODE == kModeBlock) { scn[0] = s0n * sbn; scn[1] = s1n * sbn; }
-    if (MODE == kModeScaled) exponents(q0n, q1n, sbn, kb_begin + it + 1);  // the groups from here on are block it+1's
-    GF(WA, 0, acc[0][0], tq[0], acc[3][1], tq[1], sc[1]); SB();
-    // the scales of block it+2 are requested after the activation loads and before the weight loads: the wait in
-    // front of their use then leaves exactly the weight loads in flight
-    if (MODE == kModeBlock) {
-      sc[0] = scn[0]; sc[1] = scn[1];
-      const int kn = min(it + 2, nkb - 1);
-      s0n = sx0[(int64_t)kn * p.sx_k]; s1n = sx1[(int64_t)kn * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
+    // Finished tiles leave through LDS so that every store instruction writes whole 256-byte row segments
+    // (the accumulator layout alone gives 8 bytes per row per lane: 32 partial lines per instruction).
+    // Each wave re-lays its own 64 x 128 block out, 32 rows at a time, in a private 8 KB slot of weight stages 1 and
+    // 2, 16-byte chunks XOR-swizzled by the row so that both the 8-byte writes and the 16-byte reads spread over all
+    // banks; weight stage 0 and activation stage 0 meanwhile receive the first K block of the next item.
+    const bool wide = !is_split && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+    wait_vm0();     // the loads past the last K block still target the stages: drain them before the stages are reused
+    lds_barrier();  // every wave has taken its last operands out of the stages, and every stale load has landed
+    Item next;
+    const bool has_next = next_item(next);
+    if (has_next) {
+      tile_rsrcs(next.t, next.half, next.is_half, next.is_split ? next.split * p.kb_per_split : 0);
+      SB();
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+      SB();
     }
-    if (MODE == kModeScaled) {
-      const int kn = min(it + 2, nkb - 1);
-      q0n = sq0p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; q1n = sq1p[(int64_t)((kb_begin + kn) >> 2) * p.sx_k]; sbn = swp[(int64_t)kn * p.sw_k];
-    }
-    SB();
-    LW(0, it + 3, w_ld); LW(1, it + 3, w_ld); SB();
-    GF(WA, 1, acc[0][1], tq[1], acc[0][0], tq[0], sc[0]); SB();
-    RW(WA, stW, 2); LW(2, it + 3, w_ld); LW(3, it + 3, w_ld); SB();
-    GF(WB, 0, acc[1][0], tq[0], acc[0][1], tq[1], sc[1]); SB();
-    GF(WB, 1, acc[1][1], tq[1], acc[1][0], tq[0], sc[0]); SB();
-    RW(WB, stW, 3); SB();
-    GF(WA, 0, acc[2][0], tq[0], acc[1][1], tq[1], sc[1]); SB();
-    GF(WA, 1, acc[2][1], tq[1], acc[2][0], tq[0], sc[0]); SB();
-    w_ld = w_rd;
-    w_rd = w_rd == 2 ? 0 : w_rd + 1;
-  }
-  // ---- last block's tail
-  GF(WB, 0, acc[3][0], tq[0], acc[2][1], tq[1], sc[1]);
-  GF(WB, 1, acc[3][1], tq[1], acc[3][0], tq[0], sc[0]);
-  F(acc[3][1], tq[1], sc[1]);
 
-  // Finished tiles leave through LDS so that every store instruction writes whole 256-byte row segments
-  // (the accumulator layout alone gives 8 bytes per row per lane: 32 partial lines per instruction).
-  // Each wave re-lays its own 64 x 128 block out in a private 16 KB slot of the stage memory, 16-byte
-  // chunks XOR-swizzled by the row so that both the 8-byte writes and the 16-byte reads spread over all banks.
-  const bool wide = !is_split && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
-  wait_vm0();  // the loads past the last K block still target the stages: drain them before the stages are reused or released
-  if (wide) {
-    lds_barrier();  // every wave has taken its last operands out of the stages
-    uint8_t* ep = smem + w * 16384;
+    // value (ns, rg) of row slot ms of this lane, scaled / biased (row mode) and packed to two 16-bit pairs
+    auto out_pair = [&](int ns, int ms, int rg, float sa) -> uint2 {
+      const int n = n0 + wn * 128 + ns * 32 + rg * 8 + h * 4;
+      float v[4];
 #pragma unroll
-    for (int ms = 0; ms < 2; ++ms) {
-      const int r = ms * 32 + lr;
-      const int m = slot_at(wm * 64 + r);
-      float sa = 1.f;
-      if (MODE == kModeRow && m < nrows) sa = p.sx[m];
+      for (int q = 0; q < 4; ++q) v[q] = acc[ns][ms][rg * 4 + q];
+      if (MODE == kModeRow) {
+        float4 sb = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (n < p.N) sb = *reinterpret_cast<const float4*>(p.sw + n);
+        v[0] = v[0] * sb.x * sa; v[1] = v[1] * sb.y * sa; v[2] = v[2] * sb.z * sa; v[3] = v[3] * sb.w * sa;
+        if (p.bias && n < p.N) {
 #pragma unroll
-      for (int ns = 0; ns < 4; ++ns) {
+          for (int q = 0; q < 4; ++q) v[q] += load_scalar<BIAS_DT>(p.bias, n + q);
+        }
+      }
+      uint2 o;
+      if (OUT_DT == FP8K_BF16) {
+        o.x = pack_bf16x2(v[0], v[1]);
+        o.y = pack_bf16x2(v[2], v[3]);
+      } else {
+        o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+        o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+      }
+      return o;
+    };
+
+    if (wide) {
+      uint8_t* ep = smem + kWStage + w * 8192;  // 32 rows x 256 B per pass
 #pragma unroll
-        for (int rg = 0; rg < 4; ++rg) {
-          const int n = n0 + wn * 128 + ns * 32 + rg * 8 + h * 4;
-          float v[4];
+      for (int ms = 0; ms < 2; ++ms) {
+        const int mrow = slot_at(wm * 64 + ms * 32 + lr);
+        float sa = 1.f;
+        if (MODE == kModeRow && mrow < nrows) sa = p.sx[mrow];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) v[q] = acc[ns][ms][rg * 4 + q];
-          if (MODE == kModeRow) {
-            float4 sb = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (n < p.N) sb = *reinterpret_cast<const float4*>(p.sw + n);
-            v[0] = v[0] * sb.x * sa; v[1] = v[1] * sb.y * sa; v[2] = v[2] * sb.z * sa; v[3] = v[3] * sb.w * sa;
-            if (p.bias && n < p.N) {
+        for (int ns = 0; ns < 4; ++ns)
 #pragma unroll
-              for (int q = 0; q < 4; ++q) v[q] += load_scalar<BIAS_DT>(p.bias, n + q);
+          for (int rg = 0; rg < 4; ++rg)
+            *reinterpret_cast<uint2*>(ep + lr * 256 + (((ns * 4 + rg) ^ (lr & 15)) << 4) + h * 8) = out_pair(ns, ms, rg, sa);
+        __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
+        const int rr = ln >> 4, pc = ln & 15;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int r = i * 4 + rr;
+          const uint4 o = *reinterpret_cast<const uint4*>(ep + r * 256 + ((pc ^ (r & 15)) << 4));
+          const int m = slot_at(wm * 64 + ms * 32 + r);
+          const int n = n0 + wn * 128 + (pc << 3);  // consecutive lanes store consecutive 16-byte chunks
+          if (m < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)m * p.ldc + n) = o;
+        }
+        __builtin_amdgcn_wave_barrier();
+      }
+    } else {
+#pragma unroll
+      for (int ms = 0; ms < 2; ++ms) {
+        const int ml = wm * 64 + ms * 32 + lr;  // row inside the tile
+        const int m = slot_at(ml);               // output row
+        if (m >= nrows) continue;
+        const float sa = (MODE == kModeRow && !is_split) ? p.sx[m] : 1.f;
+#pragma unroll
+        for (int ns = 0; ns < 4; ++ns) {
+#pragma unroll
+          for (int rg = 0; rg < 4; ++rg) {
+            const int n = n0 + wn * 128 + ns * 32 + rg * 8 + h * 4;
+            if (n >= p.N) continue;
+            if (is_split) {
+              float* tile_part = p.partial + ((int64_t)(t - p.tail_first) * p.splits + split) * (kTileM * kTileN);
+              *reinterpret_cast<float4*>(tile_part + ml * kTileN + (n - n0)) =
+                  make_float4(acc[ns][ms][rg * 4], acc[ns][ms][rg * 4 + 1], acc[ns][ms][rg * 4 + 2], acc[ns][ms][rg * 4 + 3]);
+            } else {
+              *reinterpret_cast<uint2*>((u16*)p.C + (int64_t)m * p.ldc + n) = out_pair(ns, ms, rg, sa);
             }
           }
-          uint2 o;
-          if (OUT_DT == FP8K_BF16) {
-            o.x = pack_bf16x2(v[0], v[1]);
-            o.y = pack_bf16x2(v[2], v[3]);
-          } else {
-            o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-            o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
-          }
-          const int chunk = (ns * 4 + rg) ^ (r & 15);
-          *reinterpret_cast<uint2*>(ep + r * 256 + chunk * 16 + h * 8) = o;
         }
       }
     }
-    __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
-    const int rr = lane >> 4, pc = lane & 15;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      const int r = i * 4 + rr;
-      const uint4 o = *reinterpret_cast<const uint4*>(ep + r * 256 + ((pc ^ (r & 15)) << 4));
-      const int m = slot_at(wm * 64 + r);
-      const int n = n0 + wn * 128 + (pc << 3);  // consecutive lanes store consecutive 16-byte chunks
-      if (m < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)m * p.ldc + n) = o;
-    }
-    return;
-  }
-
-#pragma unroll
-  for (int ms = 0; ms < 2; ++ms) {
-    const int ml = wm * 64 + ms * 32 + lr;  // row inside the tile
-    const int m = slot_at(ml);               // output row
-    if (m >= nrows) continue;
-    float sa = 1.f;
-    if (MODE == kModeRow && !is_split) sa = p.sx[m];
-#pragma unroll
-    for (int ns = 0; ns < 4; ++ns) {
-#pragma unroll
-      for (int rg = 0; rg < 4; ++rg) {
-        const int n = n0 + wn * 128 + ns * 32 + rg * 8 + h * 4;
-        if (n >= p.N) continue;
-        float v[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) v[r] = acc[ns][ms][rg * 4 + r];
-        if (is_split) {
-          float* tile_part = p.partial + ((int64_t)(t - p.tail_first) * p.splits + split) * (kTileM * kTileN);
-          *reinterpret_cast<float4*>(tile_part + ml * kTileN + (n - n0)) = make_float4(v[0], v[1], v[2], v[3]);
-        } else {
-          if (MODE == kModeRow) {
-            const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
-            v[0] = v[0] * sb.x * sa; v[1] = v[1] * sb.y * sa; v[2] = v[2] * sb.z * sa; v[3] = v[3] * sb.w * sa;
-            if (p.bias) {
-#pragma unroll
-              for (int r = 0; r < 4; ++r) v[r] += load_scalar<BIAS_DT>(p.bias, n + r);
-            }
-          }
-          store4<OUT_DT>(p.C, (int64_t)m * p.ldc + n, v[0], v[1], v[2], v[3]);
-        }
-      }
-    }
+    if (!has_next) return;
+    item = next;
+    first_item = false;
   }
 }
 
