@@ -21,8 +21,10 @@
 namespace fp8k {
 
 // PAIRS: the activation scales are row-major (stride 1 between K blocks, even stride between rows, base aligned to
-// 8 bytes; the host checks), and a lane fetches two K blocks per load.
-template <int OUT_DT, bool PAIRS>
+// 8 bytes; the host checks), and a lane fetches two K blocks per load.  SORTED: one scale row per position of
+// sorted_token_ids (what the layer passes): the rows of a wave's four 32-slot groups are a uniform step apart, so one
+// offset register serves them.
+template <int OUT_DT, bool PAIRS, bool SORTED>
 __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p) {
   constexpr int TM = 256, WST = 3, XST = 2, MS = 4, NS = 2, LW = 4;  // LW: wave loads per tile per stage
   constexpr int WBYTES = kTileN * kTileK, XBYTES = TM * kTileK;
@@ -63,18 +65,21 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   const int64_t xrows = (int64_t)((p.num_valid + p.top_k - 1) / p.top_k);
   const rsrc_t rX = make_rsrc(p.X, (uint32_t)((xrows - 1) * p.ldx + p.K));
   const int rl = lane >> 3, cp = lane & 7;
-  uint32_t voW[LW], voX[LW];
+  // the wave's 8-row groups g = 4w + q: groups q and q + 2 differ by 16 rows and share the chunk swizzle, so two
+  // lane offsets serve the four weight loads (the 16-row step is uniform and joins the K offset)
+  uint32_t voW[2], voX[LW];
 #pragma unroll
-  for (int q = 0; q < LW; ++q) {
+  for (int q = 0; q < 2; ++q) {
     const int g = w * LW + q;  // 8-row group, 0..31, of both tiles
     const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
     voW[q] = (uint32_t)((g * 8 + rl) * p.ldw + c * 16);
   }
+  const uint32_t w16 = (uint32_t)(16 * p.ldw);
   auto issue_w = [&](int kstep) {
     uint8_t* base = smem + (kstep % WST) * WBYTES + w * (LW * 1024);
     const uint32_t ko = (uint32_t)kstep * kTileK;
 #pragma unroll
-    for (int q = 0; q < LW; ++q) buf_load16_to_lds(rW, voW[q] + ko, 0, base + q * 1024);
+    for (int q = 0; q < LW; ++q) buf_load16_to_lds(rW, voW[q & 1] + (ko + (q >> 1) * w16), 0, base + q * 1024);
   };
   // slot table first, weights behind it: loads retire in order, so the table arrives without waiting for the
   // weights, and the weights do not wait for the table
@@ -101,16 +106,16 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 
   // ---- LDS -> MFMA operands
   const int swz = (lr >> 1) & 7;
-  uint32_t co[2][2];
+  // lane part of an operand fetch address (row lr of a 32-row group, swizzled 16-byte chunk); stage, wave position
+  // and group are uniform, so weights and activations share these four registers
+  uint32_t fa[2][2];
 #pragma unroll
   for (int ks = 0; ks < 2; ++ks)
 #pragma unroll
-    for (int q = 0; q < 2; ++q) co[ks][q] = (uint32_t)(((ks * 4 + h * 2 + q) ^ swz) << 4);
-  const uint32_t rdW = (uint32_t)((wn * 64 + lr) * kTileK);
-  const uint32_t rdX = (uint32_t)((wm * 128 + lr) * kTileK);
-  auto frag = [&](const uint8_t* st, uint32_t rowoff, int ks) -> v8i {
-    const v4i lo = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][0]);
-    const v4i hi = *reinterpret_cast<const v4i*>(st + rowoff + co[ks][1]);
+    for (int q = 0; q < 2; ++q) fa[ks][q] = (uint32_t)(lr * kTileK + (((ks * 4 + h * 2 + q) ^ swz) << 4));
+  auto frag = [&](const uint8_t* grp, int ks) -> v8i {  // grp: first row of the 32-row group inside its stage (uniform)
+    const v4i lo = *reinterpret_cast<const v4i*>(grp + fa[ks][0]);
+    const v4i hi = *reinterpret_cast<const v4i*>(grp + fa[ks][1]);
     v8i r;
     r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
     r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
@@ -124,9 +129,10 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   for (int ms = 0; ms < MS; ++ms) {
     const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
     nact += __builtin_amdgcn_readfirstlane(s) < nrows ? 1 : 0;
-    sxo[ms] = p.sx_sorted ? (uint32_t)((int64_t)(slot0 + wm * 128 + ms * 32 + lr) * p.sx_m)
-                          : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
+    sxo[ms] = SORTED ? (uint32_t)((int64_t)(slot0 + wm * 128 + lr) * p.sx_m)  // + ms * 32 rows, added as a uniform
+                     : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
   }
+  const uint32_t sx32 = SORTED ? (uint32_t)(32 * p.sx_m) : 0u;  // step between the scale rows of two 32-slot groups
   const int nb = min(n0 + wn * 64, p.N - 1) >> 7;  // the wave's 64 weight rows lie inside one 128-row block
   const float* swp = p.sw + (int64_t)expert * p.sw_expert_stride + (int64_t)nb * p.sw_n;
   const int nkb = p.K / kTileK;
@@ -139,30 +145,34 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
 
-  v2f sxp[MS];                 // activation scales of the even ([0]) and odd ([1]) K block in flight
-  float sba = 0.f, sbb = 0.f;  // weight scales of the same two blocks
-  // Activation scales.  With row-major scales (one row's K blocks next to each other: sx_k == 1, even row stride)
-  // a lane fetches two K blocks per load, every other trip: the rows of a block are gathered, so every lane's
-  // load is a cache line of its own whatever the layout, and what counts is the number of load instructions
-  // (one per K block and 32 slots would take more of the CU's load path than the operand tiles themselves) and
-  // that a row's line is met again on the following trips.  Other layouts fall back to one load per K block.
+  // Scales.  PAIRS: sxp[ms] holds the activation scales of an even K block and the odd one after it, fetched with
+  // one 8-byte load every other trip; with row-major scales the rows of a block are gathered, so every lane's load is
+  // a cache line of its own whatever the layout, and what counts is the number of load instructions and that a
+  // row's line is met again on the following trips.  Otherwise sxn[ms] / sbn hold the scales of the NEXT K block,
+  // requested one trip ahead in front of that trip's stage loads: at the next barrier everything older than the
+  // four youngest weight loads has landed, the scales among it.
   constexpr bool pairs = PAIRS;
+  v2f sxp[MS];
+  float sxn[MS], sbn = 0.f;
+  float sba = 0.f, sbb = 0.f;  // PAIRS: weight scales of the even / odd block in flight
   const rsrc_t rS = make_rsrc(p.sx, (uint32_t)(((xrows - 1) * p.sx_m + nkb) * 4));  // used by the paired loads only
   auto load_sb = [&](float& sb, int kb) { sb = swp[(int64_t)min(kb, nkb - 1) * p.sw_k]; };
-  auto load_sx = [&](int parity, int kb) {
-    const int kn = min(kb, nkb - 1);
+  // through a buffer descriptor: a 32-bit lane offset and a uniform offset, no 64-bit address per lane and group
+  const rsrc_t rSall = make_rsrc(p.sx, 0xFFFFFFFFu);
+  auto load_sx = [&](int kb) {
+    const uint32_t ko = (uint32_t)(min(kb, nkb - 1) * (int)p.sx_k);
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) sxp[ms][parity] = p.sx[sxo[ms] + (uint32_t)(kn * (int)p.sx_k)];
+    for (int ms = 0; ms < MS; ++ms)
+      sxn[ms] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rSall, (int)(sxo[SORTED ? 0 : ms] * 4u),
+                                                                              (int)((ko + (uint32_t)ms * sx32) * 4u), 0));
   };
   auto load_sx_pair = [&](int kb) {  // kb even: blocks kb and kb+1 (past the tensor: zero)
 #pragma unroll
     for (int ms = 0; ms < MS; ++ms)
       sxp[ms] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rS, (int)((sxo[ms] + (uint32_t)kb) * 4u), 0, 0));
   };
-  if (pairs) load_sx_pair(0);
-  else { load_sx(0, 0); load_sx(1, 1); }
-  load_sb(sba, 0);
-  load_sb(sbb, 1);
+  if (pairs) { load_sx_pair(0); load_sb(sba, 0); load_sb(sbb, 1); }
+  else { load_sx(0); load_sb(sbn, 0); }
   __builtin_amdgcn_sched_barrier(0);
   issue_x(0);
   wait_vm0();  // the first trip's partial wait assumes the in-loop order of loads
@@ -173,11 +183,17 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     constexpr int NA = decltype(na)::value;  // 32-slot groups of the wave's half with real slots
     lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
     float sc[MS];
+    if (pairs) {
 #pragma unroll
-    for (int ms = 0; ms < MS; ++ms) sc[ms] = sxp[ms][parity] * sb;
-    if (!pairs) load_sx(parity, it + 2);
-    else if (parity) load_sx_pair(it + 1);
-    load_sb(sb, it + 2);
+      for (int ms = 0; ms < MS; ++ms) sc[ms] = sxp[ms][parity] * sb;
+      if (parity) load_sx_pair(it + 1);
+      load_sb(sb, it + 2);
+    } else {
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
+      load_sx(it + 1);
+      load_sb(sbn, it + 1);
+    }
     __builtin_amdgcn_sched_barrier(0);  // scales, then activations, then weights
     issue_x(it + 1);                    // into the stage of block it-1, which every wave has left
     issue_w(it + 2);
@@ -187,13 +203,13 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     v8i wf[NS][2];
 #pragma unroll
     for (int ns = 0; ns < NS; ++ns) {
-      wf[ns][0] = frag(sw_, rdW + ns * 32 * kTileK, 0);
-      wf[ns][1] = frag(sw_, rdW + ns * 32 * kTileK, 1);
+      wf[ns][0] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 0);
+      wf[ns][1] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 1);
     }
 #pragma unroll
     for (int ms = 0; ms < NA; ++ms) {  // groups past the expert's last slot are padding
-      const v8i x0 = frag(sx_, rdX + ms * 32 * kTileK, 0);
-      const v8i x1 = frag(sx_, rdX + ms * 32 * kTileK, 1);
+      const v8i x0 = frag(sx_ + (wm * 128 + ms * 32) * kTileK, 0);
+      const v8i x1 = frag(sx_ + (wm * 128 + ms * 32) * kTileK, 1);
 #pragma unroll
       for (int ns = 0; ns < NS; ++ns) {
         v16f z;
@@ -224,13 +240,17 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     case 1: run(std::integral_constant<int, 1>{}); break;
     default: run(std::integral_constant<int, 0>{}); break;
   }
-  // output rows and routed weights, fetched while the stages drain
+  // output rows and routed weights, fetched while the stages drain.  The lane id is taken anew (from the execution
+  // mask, no register kept for it): lane-derived values that stayed live across the K loops would be parked in scratch
+  // and reloaded inside them, and scratch reloads count against the partial vmcnt waits.
   const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
-  const int er = lane >> 3, ec = lane & 7;  // store loop: row inside a group of 8, 16-byte chunk of the wave's 128 bytes
+  const int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+  const int lr_e = lane_e & 31, h_e = lane_e >> 5;
+  const int er = lane_e >> 3, ec = lane_e & 7;  // store loop: row inside a group of 8, 16-byte chunk of the wave's 128 bytes
   int oslots[MS], srow[16];
   float rsw[MS];
 #pragma unroll
-  for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
+  for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr_e];
 #pragma unroll
   for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[slot0 + wm * 128 + i * 8 + er] : 0;
 #pragma unroll
@@ -245,7 +265,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   uint8_t* const ep = smem + w * 16384;
 #pragma unroll
   for (int ms = 0; ms < MS; ++ms) {
-    const int row = ms * 32 + lr;  // inside the wave's 128 slots
+    const int row = ms * 32 + lr_e;  // inside the wave's 128 slots
     const int oslot = oslots[ms];
     const bool ok = oslot < nrows;
     const float rs = rsw[ms];
@@ -264,9 +284,9 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
           o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
           o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
         }
-        *reinterpret_cast<uint2*>(ep + row * 128 + ((nr ^ ((row >> 1) & 7)) << 4) + h * 8) = o;
+        *reinterpret_cast<uint2*>(ep + row * 128 + ((nr ^ ((row >> 1) & 7)) << 4) + h_e * 8) = o;
       } else {
-        const int n = n0 + wn * 64 + nr * 8 + h * 4;
+        const int n = n0 + wn * 64 + nr * 8 + h_e * 4;
         if (ok && n < p.N) store4<OUT_DT>(p.C, (int64_t)oslot * p.ldc + n, v[0], v[1], v[2], v[3]);
       }
     }

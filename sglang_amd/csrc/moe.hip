@@ -344,8 +344,9 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
     const bool pairs = !as_sorted && as_stride_k == 1 && (as_stride_m & 1) == 0 && aligned(As, 8);  // 129..256 and more slots per expert: both 128-row halves on one weight stage
 #define FP8K_MOE256(O) \
   do { \
-    if (pairs) hipLaunchKernelGGL((moe_stream256_kernel<O, true>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
-    else hipLaunchKernelGGL((moe_stream256_kernel<O, false>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
+    if (pairs) hipLaunchKernelGGL((moe_stream256_kernel<O, true, false>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
+    else if (as_sorted) hipLaunchKernelGGL((moe_stream256_kernel<O, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
+    else hipLaunchKernelGGL((moe_stream256_kernel<O, false, false>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
   } while (0)
     if (out_dtype == FP8K_BF16) FP8K_MOE256(FP8K_BF16);
     else FP8K_MOE256(FP8K_F16);
