@@ -293,7 +293,7 @@ def gemm_lines(torch, dev, shapes):
 
 def write_table(torch, dev, path):
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
-    from sglang_amd.sgl_kernel import fp8_scaled_mm
+    from sglang_amd.sgl_kernel import fp8_scaled_mm, mark_ue8m0
 
     lines = ["# Per-shape report (one MI355X, synthetic data, rotating buffers; device time by HIP events around a",
              "# HIP graph that replays the launches back to back, so host launch cost is excluded)", ""]
@@ -327,7 +327,7 @@ def write_table(torch, dev, path):
     for (N, K) in DSV3_NK:
         nbuf, M = 3, 4096
         ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
-        ws = [(w, torch.exp2(torch.ceil(torch.log2(sc)))) for w, sc in ws]
+        ws = [(w, mark_ue8m0(torch.exp2(torch.ceil(torch.log2(sc))))) for w, sc in ws]
         qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True,
                                                scale_tma_aligned=True, scale_ue8m0=True) for s in range(nbuf)]
         us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],

@@ -11,15 +11,18 @@ All three are the 128x128 block-scaled product `out = sum_kb (a_kb . b_kb^T) * a
 accumulation.  The grouped forms run on the grouped MoE GEMM: the group of every row becomes its "expert id"
 (rows to skip get an id the aligner ignores, so they are neither computed nor written), moe_align_block_size
 sorts the rows into per-group blocks, and each row is its own token slot (top_k = 1, no routed weight).
-float32 scales only; packed UE8M0 scale tensors (the Blackwell layout) are not accepted.
+Scales are float32, or packed UE8M0 words (int32: [.., m, ceil(k/128/4)] for the activations, one row per weight row
+[.., n, ceil(k/128/4)] for the weights, the layout the reference prepares for DeepGEMM on Blackwell, fp8_kernel.py:
+1018-1043); the grouped kernels take float scales, so packed words are expanded to powers of two first.
 """
 from typing import Tuple
 
 import torch
 
-from . import sgl_kernel as _ops
+from . import custom_ops as _ops
 from .fp8_kernel import w8a8_block_fp8_matmul
 from .fused_moe import get_default_config, moe_align_block_size
+from .sgl_kernel import unpack_ue8m0_scales, unpack_ue8m0_weight_scales
 
 _IGNORED = -2  # moe_align_block_size drops ids below -1
 
@@ -28,8 +31,18 @@ def _check_pair(name: str, x: Tuple[torch.Tensor, torch.Tensor]) -> None:
     q, s = x
     if q.dtype != torch.float8_e4m3fn:
         raise RuntimeError("%s: data must be float8_e4m3fn" % name)
-    if s.dtype != torch.float32:
-        raise RuntimeError("%s: scales must be float32 (packed UE8M0 scales are not built on this path)" % name)
+    if s.dtype not in (torch.float32, torch.int32):
+        raise RuntimeError("%s: scales must be float32 or packed int32 UE8M0 words" % name)
+
+
+def _float_scales(a, a_s, b, b_s):
+    """Packed UE8M0 words -> float32 powers of two (activations per row, weights per 128-row block)."""
+    k = a.shape[-1]
+    if a_s.dtype == torch.int32:
+        a_s = unpack_ue8m0_scales(a_s, (k + 127) // 128)
+    if b_s.dtype == torch.int32:
+        b_s = unpack_ue8m0_weight_scales(b_s, k)
+    return a_s, b_s
 
 
 def gemm_nt_f8f8bf16(lhs: Tuple[torch.Tensor, torch.Tensor], rhs: Tuple[torch.Tensor, torch.Tensor], out: torch.Tensor):
@@ -62,6 +75,7 @@ def grouped_gemm_nt_f8f8bf16_contig(
     _check_pair("rhs", rhs)
     a, a_s = lhs
     b, b_s = rhs
+    a_s, b_s = _float_scales(a, a_s, b, b_s)
     if a.dim() != 2 or b.dim() != 3 or m_indices.numel() != a.shape[0]:
         raise RuntimeError("grouped_gemm_nt_f8f8bf16_contig: lhs [m,k], rhs [G,n,k], m_indices [m]")
     idx = m_indices.to(torch.int32)
@@ -79,6 +93,7 @@ def grouped_gemm_nt_f8f8bf16_masked(
     _check_pair("rhs", rhs)
     a, a_s = lhs
     b, b_s = rhs
+    a_s, b_s = _float_scales(a, a_s, b, b_s)
     if a.dim() != 3 or b.dim() != 3 or a.shape[0] != b.shape[0] or masked_m.numel() != a.shape[0]:
         raise RuntimeError("grouped_gemm_nt_f8f8bf16_masked: lhs [G,m_max,k], rhs [G,n,k], masked_m [G]")
     G, m_max, k = a.shape

@@ -6,7 +6,7 @@ of the masked expert runner (moe_runner/deep_gemm.py): grouped GEMM, silu_and_mu
 """
 import torch
 
-from . import sgl_kernel as _ops
+from . import custom_ops as _ops
 from .fp8_kernel import fp8_max, fp8_min
 
 

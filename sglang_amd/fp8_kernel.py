@@ -9,7 +9,8 @@ from typing import List, Optional, Tuple
 
 import torch
 
-from . import sgl_kernel as _ops
+from . import custom_ops as _ops
+from . import sgl_kernel as _k
 
 fp8_dtype = torch.float8_e4m3fn
 fp8_max = 448.0
@@ -154,10 +155,13 @@ def w8a8_block_fp8_matmul(
     A e4m3fn [..., K]; B e4m3fn [N, K] contiguous; As float32 [..., ceil(K/bk)]; Bs float32
     [ceil(N/bn), ceil(K/bk)]; block_size must be [128, 128] on this path.
 
-    As may also be the packed UE8M0 tensor that the group quant returns with scale_ue8m0=True (int32
-    [M, ceil(K/128/4)]); Bs must then hold powers of two (a UE8M0-format checkpoint, or weights requantised that
-    way, fp8_utils.py:441-515 in the reference) and the matrix core applies both scales itself - the counterpart
-    of the reference's DeepGEMM path with DEEPGEMM_SCALE_UE8M0 (fp8_utils.py:229-268).
+    UE8M0 scales (reference: the int32 forms admitted at fp8_kernel.py:1018-1043 and consumed by the DeepGEMM path,
+    fp8_utils.py:229-268): As may be the packed tensor that the group quant returns with scale_ue8m0=True (int32
+    [M, ceil(K/128/4)]), Bs the packed weight scales (int32 [N, ceil(K/128/4)], the rows of a block alike).  When
+    both operands' scales are known to be powers of two - Bs packed, or float32 and declared with
+    sgl_kernel.mark_ue8m0 (requant_weight_ue8m0 / quant_weight_ue8m0 return it so) - the matrix core applies the
+    exponents itself.  Packed activation scales next to ordinary float32 weight scales are expanded to floats and
+    take the float-scale kernels: a float scale is never read as a bare exponent.
     """
     assert len(block_size) == 2
     block_n, block_k = block_size
@@ -169,17 +173,29 @@ def w8a8_block_fp8_matmul(
     assert packed or (A.shape[-1] + block_k - 1) // block_k == As.shape[-1]
     assert B.ndim == 2 and B.is_contiguous() and Bs.ndim == 2
     N, K = B.shape
-    assert (N + block_n - 1) // block_n == Bs.shape[0]
-    assert (K + block_k - 1) // block_k == Bs.shape[1]
+    kb = (K + block_k - 1) // block_k
+    bs_pow2 = False
+    if Bs.dtype == torch.int32:
+        assert Bs.shape[0] == N and Bs.shape[1] == (kb + 3) // 4
+        Bs = _k.unpack_ue8m0_weight_scales(Bs, K)
+        bs_pow2 = True
+    else:
+        assert (N + block_n - 1) // block_n == Bs.shape[0]
+        assert kb == Bs.shape[1]
+        bs_pow2 = _k.is_ue8m0(Bs)
     M = A.numel() // A.shape[-1]
     C_shape = A.shape[:-1] + (N,)
     A2 = A.reshape(M, K)
     if packed:
         if As.dim() != 2:
             raise RuntimeError("w8a8_block_fp8_matmul: packed UE8M0 scales need a 2-D activation")
-        return _ops._block_gemm_nk_ue8m0(A2, B, As, Bs, output_dtype).reshape(C_shape)
+        if Bs.dtype != torch.float32:
+            raise RuntimeError("w8a8_block_fp8_matmul: weight scales must be float32 or packed int32 UE8M0")
+        if bs_pow2:
+            return _ops.block_gemm_nk_ue8m0(A2, B, As, Bs, output_dtype).reshape(C_shape)
+        return _ops.block_gemm_nk(A2, B, _k.unpack_ue8m0_scales(As, kb), Bs, output_dtype).reshape(C_shape)
     As2 = As.reshape(M, As.shape[-1])
     if As2.dtype != torch.float32 or Bs.dtype != torch.float32:
-        raise RuntimeError("w8a8_block_fp8_matmul: scales must be float32 (or packed int32 UE8M0 activation scales)")
-    out = _ops._block_gemm_nk(A2, B, As2, Bs, output_dtype)
+        raise RuntimeError("w8a8_block_fp8_matmul: scales must be float32 (or packed int32 UE8M0 scales)")
+    out = _ops.block_gemm_nk(A2, B, As2, Bs, output_dtype)
     return out.reshape(C_shape)

@@ -8,7 +8,8 @@ from typing import Callable, List, Optional, Tuple
 
 import torch
 
-from . import sgl_kernel as _ops
+from . import custom_ops as _ops
+from .sgl_kernel import mark_ue8m0, unpack_ue8m0_weight_scales  # noqa: F401  (re-exported for weight loading)
 from .fp8_kernel import (
     fp8_dtype,
     scaled_fp8_quant,
@@ -161,17 +162,19 @@ def quant_weight_ue8m0(weight_dequant: torch.Tensor, weight_block_size: List[int
     assert weight_dequant.dtype == torch.bfloat16, f"{weight_dequant.dtype=} {weight_dequant.shape=}"
     *batch, n, k = weight_dequant.shape
     if not batch:
-        return per_block_cast_to_fp8(weight_dequant)
+        q, sc = per_block_cast_to_fp8(weight_dequant)
+        return q, mark_ue8m0(sc.contiguous(), check=False)  # powers of two by construction
     parts = [per_block_cast_to_fp8(w) for w in weight_dequant.reshape(-1, n, k)]
     q = torch.stack([p[0] for p in parts]).view(*batch, n, k)
     sc = torch.stack([p[1] for p in parts]).view(*batch, (n + 127) // 128, (k + 127) // 128)
-    return q, sc
+    return q, mark_ue8m0(sc.contiguous(), check=False)  # powers of two by construction
 
 
 def requant_weight_ue8m0(weight: torch.Tensor, weight_scale_inv: torch.Tensor, weight_block_size: List[int]) -> Tuple[torch.Tensor, torch.Tensor]:
     """Reference: fp8_utils.py:453-476 - dequantise a block-FP8 weight to bf16 and quantise it again with
     power-of-two block scales.  The reference then repacks the scales into DeepGEMM's int32 layout; here they stay
-    float32 [.., ceil(n/128), ceil(k/128)] powers of two, which is what the UE8M0 GEMM of this library takes."""
+    float32 [.., ceil(n/128), ceil(k/128)] powers of two, declared as such (sgl_kernel.mark_ue8m0), which is what the
+    UE8M0 GEMM of this library takes."""
     assert list(weight_block_size) == [128, 128]
     deq = block_quant_dequant(weight, weight_scale_inv, weight_block_size, torch.bfloat16)
     return quant_weight_ue8m0(deq, weight_block_size)

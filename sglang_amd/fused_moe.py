@@ -15,7 +15,7 @@ from typing import Any, Dict, List, Optional, Tuple
 
 import torch
 
-from . import sgl_kernel as _ops
+from . import custom_ops as _ops
 from .fp8_kernel import sglang_per_token_group_quant_fp8
 
 CHUNK_SIZE = 64 * 1024  # tokens per pass, as in the reference (fused_moe.py:423)
@@ -241,29 +241,28 @@ def biased_grouped_topk_impl(
     routed_scaling_factor: Optional[float] = None,
     apply_routed_scaling_factor_on_output: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Routing harness in plain torch (reference: python/sglang/srt/layers/moe/topk.py:665-738): sigmoid
-    scores, group score = sum of the two best biased scores, keep topk_group groups, top-k experts
-    among them, weights = un-biased scores, renormalised.  Not a kernel of this path."""
-    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
-    scores = gating_output.sigmoid()
-    num_token = scores.shape[0]
-    scores_for_choice = scores.view(num_token, -1) + correction_bias.unsqueeze(0)
-    group_scores = scores_for_choice.view(num_token, num_expert_group, -1).topk(2, dim=-1)[0].sum(dim=-1)
-    group_idx = torch.topk(group_scores, k=topk_group, dim=-1, sorted=False)[1]
-    group_mask = torch.zeros_like(group_scores)
-    group_mask.scatter_(1, group_idx, 1)
-    score_mask = (
-        group_mask.unsqueeze(-1).expand(num_token, num_expert_group, scores.shape[-1] // num_expert_group)
-        .reshape(num_token, -1)
-    )
-    tmp_scores = scores_for_choice.masked_fill(~score_mask.bool(), float("-inf"))
-    _, topk_ids = torch.topk(tmp_scores, k=topk, dim=-1, sorted=False)
-    topk_weights = scores.gather(1, topk_ids)
+    """Grouped top-k routing with a selection bias in plain tensor ops, for the shapes the fused gate kernel does not
+    take (same interface and selection rule as python/sglang/srt/layers/moe/topk.py:665-738): an expert's choice value
+    is sigmoid(logit) + bias; a group is worth the sum of its two best choice values; only experts of the
+    `topk_group` best groups compete for the `topk` places; the routing weights are the un-biased sigmoid values of
+    the winners, normalised to sum 1 when `renormalize`."""
+    tokens, experts = gating_output.shape
+    assert hidden_states.shape[0] == tokens, "Number of tokens mismatch"
+    per_group = experts // num_expert_group
+    prob = torch.sigmoid(gating_output)
+    choice = (prob + correction_bias).view(tokens, num_expert_group, per_group)
+    group_worth = torch.topk(choice, 2, dim=2).values.sum(dim=2)                      # [tokens, groups]
+    kept_groups = torch.topk(group_worth, topk_group, dim=1, sorted=False).indices     # [tokens, topk_group]
+    group_open = torch.zeros((tokens, num_expert_group), dtype=torch.bool, device=choice.device)
+    group_open.scatter_(1, kept_groups, True)
+    candidates = torch.where(group_open.unsqueeze(2), choice, choice.new_full((), float("-inf"))).view(tokens, experts)
+    winners = torch.topk(candidates, topk, dim=1, sorted=False).indices
+    weights = torch.gather(prob, 1, winners)
     if renormalize:
-        topk_weights = topk_weights / topk_weights.sum(dim=-1, keepdim=True)
+        weights = weights / weights.sum(dim=1, keepdim=True)
         if apply_routed_scaling_factor_on_output:
-            topk_weights = topk_weights * routed_scaling_factor
-    return topk_weights.to(torch.float32), topk_ids.to(torch.int32)
+            weights = weights * routed_scaling_factor
+    return weights.float(), winners.int()
 
 
 def biased_grouped_topk(

@@ -351,16 +351,46 @@ def _block_gemm_nk(A, B, As, Bs, out_dtype):
 
 
 def unpack_ue8m0_scales(packed: torch.Tensor, num_groups: int) -> torch.Tensor:
-    """int32 words of four UE8M0 exponent bytes [M, ceil(G/4)] -> float32 powers of two [M, G]."""
+    """int32 words of four UE8M0 exponent bytes [..., M, ceil(G/4)] -> float32 powers of two [..., M, G]
+    (byte g % 4 of word g // 4 is the exponent of group g; decode is byte << 23, fp8_utils.py:549-550 of the reference)."""
     shifts = torch.arange(0, 32, 8, device=packed.device, dtype=torch.int32)
     exps = (packed.unsqueeze(-1) >> shifts) & 0xFF
-    return (exps.reshape(packed.shape[0], -1)[:, :num_groups] << 23).contiguous().view(torch.float32)
+    return (exps.reshape(*packed.shape[:-1], -1)[..., :num_groups] << 23).contiguous().view(torch.float32)
+
+
+def unpack_ue8m0_weight_scales(packed: torch.Tensor, K: int) -> torch.Tensor:
+    """Packed UE8M0 weight scales in the layout the reference hands to DeepGEMM - int32 [..., N, ceil(K/128/4)], one
+    row per weight row, the 128 rows of a block carrying the same words (fp8_kernel.py:1036-1043, inverse transform
+    fp8_utils.py:529-564) - to float32 powers of two [..., ceil(N/128), K/128], one row per 128-row block."""
+    kb = (K + 127) // 128
+    return unpack_ue8m0_scales(packed[..., ::128, :], kb)
+
+
+def is_ue8m0(scales: torch.Tensor) -> bool:
+    """True for a float32 scale tensor that has been declared to hold powers of two only (mark_ue8m0)."""
+    return bool(getattr(scales, "_fp8k_ue8m0", False))
+
+
+def mark_ue8m0(scales: torch.Tensor, check: bool = True) -> torch.Tensor:
+    """Declare a float32 weight-scale tensor to hold positive powers of two only, which lets the block GEMM hand the
+    exponents to the matrix core instead of multiplying.  With `check` (the default; one device synchronisation, meant
+    for weight-loading time) every mantissa is verified to be zero first.  Returns the same tensor."""
+    if scales.dtype != torch.float32:
+        raise RuntimeError("mark_ue8m0: float32 scales expected")
+    if check:
+        bits = scales.contiguous().view(torch.int32)
+        if bool(((bits & 0x7FFFFF) != 0).any()) or bool((bits <= 0).any()):
+            raise RuntimeError("mark_ue8m0: the scales are not all positive powers of two")
+    scales._fp8k_ue8m0 = True
+    return scales
 
 
 def _block_gemm_nk_ue8m0(A, B, As_packed, Bs, out_dtype):
-    """Block GEMM with packed UE8M0 activation scales (as the group quant writes them with scale_ue8m0=True) and
-    power-of-two float32 weight scales: for M > 128 the matrix core applies the scales itself
-    (include/fp8k.h: fp8k_block_gemm_ue8m0); smaller batches expand the exponents and take the float-scale kernels."""
+    """Block GEMM with packed UE8M0 activation scales (as the group quant writes them with scale_ue8m0=True) and float32
+    weight scales that are powers of two: the matrix core applies both scales itself (include/fp8k.h:
+    fp8k_block_gemm_ue8m0).  A weight scale with a non-zero mantissa would lose it here, so callers route to this
+    function only for scales known to be powers of two (see fp8_kernel.w8a8_block_fp8_matmul); up to 128 rows, where the
+    kernels have no such mode, the exponents are expanded and the float-scale kernels run - the same numbers."""
     require_cuda(A, B, As_packed, Bs)
     if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
         raise RuntimeError("A and B must be Float8_e4m3fn")

@@ -87,7 +87,37 @@ def test_grouped_masked(dev, G, m_max, masked, N, K):
 def test_wrapper_errors(dev):
     from sglang_amd.deep_gemm_wrapper import gemm_nt_f8f8bf16
 
-    a = torch.zeros((4, 128), device=dev, dtype=torch.float8_e4m3fn)
-    s_packed = torch.zeros((4, 1), device=dev, dtype=torch.int32)
-    with pytest.raises(RuntimeError, match="float32"):
-        gemm_nt_f8f8bf16((a, s_packed), (a, torch.ones((1, 1), device=dev)), torch.empty((4, 4), device=dev, dtype=torch.bfloat16))
+    a = torch.zeros((8, 128), device=dev, dtype=torch.float8_e4m3fn)
+    out = torch.empty((8, 8), device=dev, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="float32 or packed int32"):
+        gemm_nt_f8f8bf16((a, torch.zeros((8, 1), device=dev, dtype=torch.float16)), (a, torch.ones((1, 1), device=dev)), out)
+    with pytest.raises(RuntimeError, match="float8_e4m3fn"):
+        gemm_nt_f8f8bf16((a.view(torch.uint8), torch.ones((8, 1), device=dev)), (a, torch.ones((1, 1), device=dev)), out)
+    # packed activation scales are taken (exponent 127 = scale 1)
+    s_packed = torch.full((8, 1), 127, device=dev, dtype=torch.int32)
+    gemm_nt_f8f8bf16((a, s_packed), (a, torch.ones((1, 1), device=dev)), out)
+    assert bool((out == 0).all())
+
+
+def test_grouped_masked_with_packed_ue8m0_scales(dev):
+    """Both scale tensors as packed UE8M0 words (activations per row, weights per weight row): the result is the
+    oracle's on the powers of two they encode."""
+    from sglang_amd.deep_gemm_wrapper import grouped_gemm_nt_f8f8bf16_masked
+
+    rng = np.random.default_rng(9)
+    G, m_max, N, K = 4, 96, 256, 640
+    masked = np.array([96, 0, 40, 7], dtype=np.int32)
+    aq, bq = _codes(rng, (G, m_max, K)), _codes(rng, (G, N, K))
+    a_s = (2.0 ** rng.integers(-9, -4, (G, m_max, K // 128))).astype(np.float32)
+    b_s = (2.0 ** rng.integers(-9, -4, (G, N // 128, K // 128))).astype(np.float32)
+    a_p = torch.from_numpy(np.stack([O.pack_ue8m0_scales(x) for x in a_s])).to(dev)
+    b_p = torch.from_numpy(np.stack([O.pack_ue8m0_scales(np.repeat(x, 128, axis=0)) for x in b_s])).to(dev)
+    out = torch.full((G, m_max, N), 7.0, device=dev, dtype=torch.bfloat16)
+    grouped_gemm_nt_f8f8bf16_masked((fp8_tensor(aq, dev), a_p), (fp8_tensor(bq, dev), b_p), out, torch.from_numpy(masked).to(dev), 40)
+    got = out.float().cpu().numpy()
+    for g in range(G):
+        m = int(masked[g])
+        if m:
+            ref = O.w8a8_block_fp8_matmul(aq[g, :m], bq[g], a_s[g, :m], b_s[g], acc=np.float64)
+            assert _rel(got[g, :m], ref) <= REL_TOL
+        assert (got[g, m:] == 7.0).all()

@@ -66,3 +66,30 @@ def test_input_to_float8():
     assert float(q.float().abs().max()) == 448.0
     q0, s0 = input_to_float8(torch.zeros(4, 4))
     assert float(s0) == pytest.approx(1e-12 / 448.0) and torch.all(q0.float() == 0)
+
+
+def test_ue8m0_unpack_and_marking():
+    """Packed UE8M0 words -> float32 powers of two, for activations ([M, ceil(G/4)]) and for weights in the per-row
+    layout the reference hands to DeepGEMM ([N, ceil(G/4)], the 128 rows of a block alike); mark_ue8m0 accepts powers
+    of two only."""
+    from sglang_amd.sgl_kernel import is_ue8m0, mark_ue8m0, unpack_ue8m0_scales, unpack_ue8m0_weight_scales
+
+    rng = np.random.default_rng(5)
+    s = (2.0 ** rng.integers(-30, 10, (7, 6))).astype(np.float32)
+    packed = torch.from_numpy(O.pack_ue8m0_scales(s))
+    np.testing.assert_array_equal(unpack_ue8m0_scales(packed, 6).numpy(), s)
+    s3 = (2.0 ** rng.integers(-20, 5, (3, 5, 9))).astype(np.float32)   # a leading group dimension, ragged word count
+    p3 = torch.from_numpy(np.stack([O.pack_ue8m0_scales(x) for x in s3]))
+    np.testing.assert_array_equal(unpack_ue8m0_scales(p3, 9).numpy(), s3)
+    # weights: [N/128, K/128] block scales repeated over the 128 rows of a block, then packed per row
+    ws = (2.0 ** rng.integers(-14, -6, (3, 10))).astype(np.float32)
+    per_row = torch.from_numpy(O.pack_ue8m0_scales(np.repeat(ws, 128, axis=0)))
+    assert per_row.shape == (384, 3)
+    np.testing.assert_array_equal(unpack_ue8m0_weight_scales(per_row, 10 * 128).numpy(), ws)
+    t = torch.from_numpy(ws.copy())
+    assert not is_ue8m0(t)
+    assert mark_ue8m0(t) is t and is_ue8m0(t)
+    with pytest.raises(RuntimeError, match="powers of two"):
+        mark_ue8m0(torch.tensor([[1.0, 3.0]]))
+    with pytest.raises(RuntimeError, match="powers of two"):
+        mark_ue8m0(torch.tensor([[1.0, 0.0]]))

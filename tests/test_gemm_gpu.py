@@ -281,7 +281,7 @@ def test_block_gemm_ue8m0_hardware_scales(dev, M, N, K):
     applies both.  Checked against the oracle's block matmul on the very same (unpacked) scales, <= 1e-2, and
     against this library's float-scale kernel on the unpacked scales."""
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
-    from sglang_amd.sgl_kernel import unpack_ue8m0_scales
+    from sglang_amd.sgl_kernel import mark_ue8m0, unpack_ue8m0_scales
 
     x = O.make_activation(M, K, seed=M)
     w = O.make_weight(N, K, seed=N)
@@ -289,7 +289,7 @@ def test_block_gemm_ue8m0_hardware_scales(dev, M, N, K):
     ws2 = O.ceil_to_ue8m0(ws)                     # power-of-two weight scales (the bytes stay as they are:
     xt = torch.from_numpy(x).to(dev).to(torch.bfloat16)  # only the GEMM's use of the scales is under test)
     xq, xs_packed = sglang_per_token_group_quant_fp8(xt, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
-    B, Bs = fp8_tensor(wq, dev), torch.from_numpy(ws2).to(dev)
+    B, Bs = fp8_tensor(wq, dev), mark_ue8m0(torch.from_numpy(ws2).to(dev))
     c = w8a8_block_fp8_matmul(xq, B, xs_packed, Bs, [128, 128], torch.bfloat16)
     xs = unpack_ue8m0_scales(xs_packed, K // 128)
     c_float = w8a8_block_fp8_matmul(xq, B, xs, Bs, [128, 128], torch.bfloat16)
@@ -305,7 +305,7 @@ def test_ue8m0_requantised_checkpoint_end_to_end(dev):
     the original weight (both are 8-bit renderings of the same bf16 numbers)."""
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
     from sglang_amd.fp8_utils import requant_weight_ue8m0, w8a8_block_fp8_linear
-    from sglang_amd.sgl_kernel import unpack_ue8m0_scales
+    from sglang_amd.sgl_kernel import mark_ue8m0, unpack_ue8m0_scales
 
     M, N, K = 384, 768, 1024
     x = torch.from_numpy(O.make_activation(M, K, seed=1)).to(dev).to(torch.bfloat16)
@@ -319,6 +319,49 @@ def test_ue8m0_requantised_checkpoint_end_to_end(dev):
     assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
     c_float = w8a8_block_fp8_linear(x, W, [128, 128], Ws)
     assert _rel_err(c.float().cpu().numpy(), c_float.float().cpu().numpy()) <= 0.08
+
+
+@pytest.mark.parametrize("M", [40, 128, 129, 700])
+def test_packed_ue8m0_scales_next_to_ordinary_float_weight_scales(dev, M):
+    """Packed UE8M0 activation scales with float32 weight scales that are NOT powers of two: a float scale is never
+    read as a bare exponent, whatever the batch size (below and above the 128 rows from which the tile kernels could
+    apply exponents in hardware) - the result is the oracle's on the expanded scales (<= 1e-2) and, bit for bit, that
+    of the float-scale call on the expanded scales."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.sgl_kernel import unpack_ue8m0_scales
+
+    N, K = 768, 1024
+    x = torch.from_numpy(O.make_activation(M, K, seed=M)).to(dev).to(torch.bfloat16)
+    wq, ws = O.block_quant_weight(O.make_weight(N, K, seed=N))     # amax/448 scales: mantissas all over the place
+    xq, xs_packed = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    B, Bs = fp8_tensor(wq, dev), torch.from_numpy(ws).to(dev)
+    c = w8a8_block_fp8_matmul(xq, B, xs_packed, Bs, [128, 128], torch.bfloat16)
+    xs = unpack_ue8m0_scales(xs_packed, K // 128)
+    ref = O.w8a8_block_fp8_matmul(xq.view(torch.uint8).cpu().numpy(), wq, xs.cpu().numpy(), ws, acc=np.float64)
+    assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
+    assert torch.equal(c, w8a8_block_fp8_matmul(xq, B, xs, Bs, [128, 128], torch.bfloat16))
+
+
+@pytest.mark.parametrize("M", [64, 300])
+def test_packed_ue8m0_weight_scales(dev, M):
+    """Weight scales as packed UE8M0 words, one row per weight row (the layout the reference prepares for DeepGEMM,
+    fp8_kernel.py:1036-1043), with packed activation scales: equal to the float form of the same powers of two."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.sgl_kernel import mark_ue8m0, unpack_ue8m0_scales
+
+    N, K = 512, 1280
+    x = torch.from_numpy(O.make_activation(M, K, seed=M)).to(dev).to(torch.bfloat16)
+    wq, ws = O.block_quant_weight(O.make_weight(N, K, seed=N))
+    ws2 = O.ceil_to_ue8m0(ws)
+    packed_rows = torch.from_numpy(O.pack_ue8m0_scales(np.repeat(ws2, 128, axis=0))).to(dev)   # [N, ceil(10/4)]
+    xq, xs_packed = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
+    B = fp8_tensor(wq, dev)
+    c = w8a8_block_fp8_matmul(xq, B, xs_packed, packed_rows, [128, 128], torch.bfloat16)
+    c_float = w8a8_block_fp8_matmul(xq, B, xs_packed, mark_ue8m0(torch.from_numpy(ws2).to(dev)), [128, 128], torch.bfloat16)
+    assert torch.equal(c, c_float)
+    ref = O.w8a8_block_fp8_matmul(xq.view(torch.uint8).cpu().numpy(), wq,
+                                  unpack_ue8m0_scales(xs_packed, K // 128).cpu().numpy(), ws2, acc=np.float64)
+    assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
 
 
 @pytest.mark.parametrize("case", ["a", "b", "c"])

@@ -73,14 +73,14 @@ def test_tile128_scaled_mm(dev, tile128, M, N, K, with_bias, splits):
 def test_tile128_ue8m0(dev, tile128, M, N, K, splits):
     """Packed UE8M0 activation exponents and power-of-two weight scales applied by the matrix core."""
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
-    from sglang_amd.sgl_kernel import unpack_ue8m0_scales
+    from sglang_amd.sgl_kernel import mark_ue8m0, unpack_ue8m0_scales
 
     x = O.make_activation(M, K, seed=M)
     wq, ws = O.block_quant_weight(O.make_weight(N, K, seed=N))
     ws2 = O.ceil_to_ue8m0(ws)
     xt = torch.from_numpy(x).to(dev).to(torch.bfloat16)
     xq, xs_packed = sglang_per_token_group_quant_fp8(xt, 128, column_major_scales=True, scale_tma_aligned=True, scale_ue8m0=True)
-    B, Bs = fp8_tensor(wq, dev), torch.from_numpy(ws2).to(dev)
+    B, Bs = fp8_tensor(wq, dev), mark_ue8m0(torch.from_numpy(ws2).to(dev))
     tile128(splits)
     c = w8a8_block_fp8_matmul(xq, B, xs_packed, Bs, [128, 128], torch.bfloat16)
     torch.cuda.synchronize()
