@@ -92,6 +92,16 @@ def _time_graph(torch, fn, iters, replays=3, warm_launches=0):
     for i in range(max(2, warm_launches)):  # a cold chip clocks memory-bound kernels up to 15 % slower
         fn(i)
     torch.cuda.synchronize()
+    # after host-side work (the CPU legs of the report) the chip has idled: keep it under this load for about 60 ms so
+    # that its clocks have settled when the timed replays start
+    t_settle = time.perf_counter()
+    i = 0
+    while time.perf_counter() - t_settle < 0.06:
+        fn(i)
+        i += 1
+        if i % 16 == 0:
+            torch.cuda.synchronize()
+    torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
         for i in range(iters):
@@ -243,7 +253,53 @@ def _rand_fp8(torch, shape, gen, dev):
     return torch.where((b & 0x7F) == 0x7F, b & 0xFE, b).view(torch.float8_e4m3fn)  # no NaN codes
 
 
-def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384)):
+# ---------------------------------------------------------------------------------------------------------------
+# CPU column of the per-shape report: this build's own torch-CPU restatement of the reference's torch-native path
+# (per-token-group quant formula of python/sglang/test/test_block_fp8.py:23-48, block-tile matmul loop of :273-325:
+# k_tiles x n_tiles float32 matmuls with the scale applied per tile), timed on this machine's host cores.  It belongs
+# to the cpu_baseline leg; its result on the same tensors is also what the GPU output is compared with in the report.
+# ---------------------------------------------------------------------------------------------------------------
+CPU_ROW_CAP = 128  # rows of a shape that the interpreter-bound CPU loop is timed on (stated in the report)
+
+
+def _median_time(fn, runs=5):
+    fn()
+    ts = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[len(ts) // 2]
+
+
+def cpu_group_quant(torch, x):
+    g = x.reshape(-1, 128)
+    amax = g.abs().amax(dim=-1, keepdim=True).clamp(min=1e-10).to(torch.float32)
+    s = amax / 448.0
+    q = (g / s).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    return q.reshape(x.shape), s.reshape(x.shape[0], -1)
+
+
+def cpu_block_matmul(torch, q, s, wq, ws):
+    """C[:, j-block] += (A_i @ B_ji^T) * As[:, i] * Bs[j, i], tile by tile in float32, bf16 out."""
+    M, K = q.shape
+    N = wq.shape[0]
+    A = q.to(torch.float32)
+    B = wq.to(torch.float32)
+    C = torch.zeros((M, N), dtype=torch.float32)
+    for i in range(K // 128):
+        a = A[:, i * 128:(i + 1) * 128]
+        for j in range((N + 127) // 128):
+            C[:, j * 128:(j + 1) * 128] += (a @ B[j * 128:(j + 1) * 128, i * 128:(i + 1) * 128].t()) * s[:, i:i + 1] * ws[j, i]
+    return C.to(torch.bfloat16)
+
+
+def _rel_err(torch, got, ref):
+    return float((got.float() - ref.float()).abs().max() / ref.float().abs().max().clamp(min=1e-30))
+
+
+def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=False):
     """BASELINE configs[4]: 256 experts, hidden 7168, intermediate 2048, top-8 grouped-sigmoid routing."""
     from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl
 
@@ -257,9 +313,12 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384)):
     bias = torch.randn((E,), generator=g, device=dev) * 0.01  # near-balanced routing, as a trained router gives
     lines = ["", "## configs[4] block-FP8 fused MoE layer (E=256, H=7168, I=2048, top-8 of 8 groups / top-4 groups)", "",
              "whole layer: align + quant + grouped GEMM w13 + silu_and_mul + quant + grouped GEMM w2 + top-k sum; "
-             "bytes = fp8 weights of the experts hit (44.04 MB each)", "",
-             "| M | experts hit | us | TFLOP/s | weight GB/s | % of 8 TB/s |", "|---|---|---|---|---|---|"]
+             "bytes = fp8 weights of the experts hit (44.04 MB each); roofline = those bytes at 8 TB/s (HBM-bound at every M);",
+             "CPU: the same layer in torch-CPU ops, expert by expert, on the first token only (8 experts) - us per token", "",
+             "| M | experts hit | us | TFLOP/s | weight GB/s | fraction of HBM roofline | max rel err vs CPU (token 0) | CPU us / token |",
+             "|---|---|---|---|---|---|---|---|"]
     for M in token_counts:
+        print("[table] configs[4] M=%d" % M, file=sys.stderr, flush=True)
         x = _activation(torch, M, H, M, dev)
         logits = torch.randn((M, E), generator=g, device=dev)
         tw, ids = biased_grouped_topk_impl(x, logits, bias, topk, True, 8, 4)
@@ -268,8 +327,28 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384)):
         us = _time_graph(torch, lambda i: fused_experts_impl(x, w1, w2, tw, ids, **kw), 10 if M < 4096 else 5)
         flops = 2.0 * M * topk * 3 * I * H
         wbytes = hit * 3 * I * H
-        lines.append("| %d | %d | %.1f | %.1f | %.0f | %.1f |" % (M, hit, us, flops / us / 1e6, wbytes / us / 1e3,
-                                                                 wbytes / us / 1e3 / PEAK_HBM_GBS * 100))
+        err, cpu_us = "", ""
+        if cpu and M in (1, 32, 256, 4096):
+            out = fused_experts_impl(x, w1, w2, tw, ids, **kw)[0].cpu()
+            x0 = x[:1].cpu()
+
+            def layer_cpu():
+                xq, xs = cpu_group_quant(torch, x0)
+                acc = torch.zeros((1, H), dtype=torch.float32)
+                for k in range(topk):
+                    e = int(ids[0, k])
+                    h1 = cpu_block_matmul(torch, xq, xs, w1[e].cpu(), w1s[e].cpu())
+                    act = torch.nn.functional.silu(h1[:, :I].float()).to(torch.bfloat16) * h1[:, I:]
+                    aq, a_s = cpu_group_quant(torch, act)
+                    h2 = cpu_block_matmul(torch, aq, a_s, w2[e].cpu(), w2s[e].cpu()).float()
+                    acc = acc + (h2 * float(tw[0, k])).to(torch.bfloat16).float()
+                return (acc * 2.5).to(torch.bfloat16)
+
+            t = _median_time(layer_cpu, runs=1)
+            err = "%.1e" % _rel_err(torch, out, layer_cpu()[0])
+            cpu_us = "%.0f" % (t * 1e6)
+        lines.append("| %d | %d | %.1f | %.1f | %.0f | %.2f | %s | %s |" % (
+            M, hit, us, flops / us / 1e6, wbytes / us / 1e3, wbytes / us / 1e3 / PEAK_HBM_GBS, err, cpu_us))
     return lines
 
 
@@ -291,39 +370,108 @@ def gemm_lines(torch, dev, shapes):
     return lines
 
 
-def write_table(torch, dev, path):
+def _bound(flops, nbytes):
+    """(name, floor in us) of the binding roofline: dense-FP8 MFMA peak or HBM peak, whichever takes longer."""
+    t_mfma, t_hbm = flops / (PEAK_FP8_TFLOPS * 1e6), nbytes / (PEAK_HBM_GBS * 1e3)
+    return ("mfma", t_mfma) if t_mfma >= t_hbm else ("hbm", t_hbm)
+
+
+def write_table(torch, dev, path, cpu=True):
+    """Per-shape report of configs[0]..[4]: GPU time, throughput, fraction of the binding roofline, and next to it the
+    torch-native restatement on this machine's host cores (rows capped at CPU_ROW_CAP) with the GPU result's maximum
+    relative error against it on those rows."""
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
+    from sglang_amd.fp8_utils import w8a8_block_fp8_linear
     from sglang_amd.sgl_kernel import fp8_scaled_mm, mark_ue8m0
 
-    lines = ["# Per-shape report (one MI355X, synthetic data, rotating buffers; device time by HIP events around a",
-             "# HIP graph that replays the launches back to back, so host launch cost is excluded)", ""]
-    lines += ["## configs[1] per-token-group quant, K=7168, group 128", "",
-              "| M | layout | us | GB/s | % of 8 TB/s |", "|---|---|---|---|---|"]
+    lines = ["# Per-shape report (one MI355X, synthetic data, rotating buffers)", "",
+             "GPU: device time by HIP events around a HIP graph that replays the launches back to back (host launch cost excluded).",
+             "Roofline: the binding one of dense-FP8 MFMA peak (5 PFLOP/s) and HBM peak (8 TB/s) for the shape's algorithmic",
+             "FLOPs (2 M N K) and bytes (operands + output + scales); `frac` = that floor / measured time.",
+             "CPU: this build's torch-CPU restatement of the reference's torch-native path (group quant formula + k_tiles x",
+             "n_tiles block-tile float32 matmul loop), median of 5 runs after one warm-up, at most %d rows of the shape" % CPU_ROW_CAP,
+             "(the loop is interpreter-bound); host: torch.get_num_threads() = %d, os.cpu_count() = %d." % (
+                 torch.get_num_threads(), os.cpu_count()),
+             "`err` = max |gpu - cpu| / max |cpu| on the rows the CPU computed (quant: bytes and scales compared for equality).", ""]
+
+    # ---- configs[0]
+    lines += ["## configs[0] single W8A8 block-FP8 linear (x bf16 [32,4096], W [4096,4096], seed 0), quant + GEMM", "",
+              "| M | N | K | GPU us | TFLOP/s | bound | frac | err | CPU us | CPU GFLOP/s |", "|---|---|---|---|---|---|---|---|---|---|"]
+    M, N, K = 32, 4096, 4096
+    x = _activation(torch, M, K, 0, dev)
+    wq, wsc = _block_quant_weight(torch, N, K, 0, dev)
+    us = _time_graph(torch, lambda i: w8a8_block_fp8_linear(x, wq, [128, 128], wsc), 20)
+    bname, floor = _bound(2.0 * M * N * K, 2 * M * K + N * K + 2 * M * N)
+    err, cpu_us, cpu_gf = "", "", ""
+    if cpu:
+        xc, wqc, wsc_c = x.cpu(), wq.cpu(), wsc.cpu()
+        t = _median_time(lambda: cpu_block_matmul(torch, *cpu_group_quant(torch, xc), wqc, wsc_c))
+        ref = cpu_block_matmul(torch, *cpu_group_quant(torch, xc), wqc, wsc_c)
+        err = "%.1e" % _rel_err(torch, w8a8_block_fp8_linear(x, wq, [128, 128], wsc).cpu(), ref)
+        cpu_us, cpu_gf = "%.0f" % (t * 1e6), "%.1f" % (2.0 * M * N * K / t / 1e9)
+    lines.append("| %d | %d | %d | %.1f | %.1f | %s | %.3f | %s | %s | %s |" % (M, N, K, us, 2.0 * M * N * K / us / 1e6, bname, floor / us,
+                                                                              err, cpu_us, cpu_gf))
+
+    # ---- configs[1]
+    lines += ["", "## configs[1] per-token-group quant, K=7168, group 128 (bound: HBM)", "",
+              "| M | layout | GPU us | GB/s | frac of 8 TB/s | bytes+scales equal to CPU | CPU us | CPU GB/s |", "|---|---|---|---|---|---|---|---|"]
     for M in (1, 64, 512, 4096, 16384):
+        print("[table] configs[1] M=%d" % M, file=sys.stderr, flush=True)
         nbuf = 3 if M >= 4096 else 8
         xs = [_activation(torch, M, 7168, s, dev) for s in range(nbuf)]
+        cpu_us, cpu_gbs, ref = "", "", None
+        if cpu:
+            rows = min(M, 4096)
+            xc = xs[0][:rows].cpu()
+            t = _median_time(lambda: cpu_group_quant(torch, xc), runs=5 if rows <= 512 else 3)
+            ref = cpu_group_quant(torch, xc)
+            cpu_us, cpu_gbs = "%.0f" % (t * 1e6), "%.2f" % (quant_bytes(rows, 7168) / t / 1e9)
         for name, kw in QUANT_LAYOUTS:
             us = _time_graph(torch, _quant_launcher(torch, xs, kw), 30, warm_launches=100)
             gbs = quant_bytes(M, 7168, name == "ue8m0_packed") / us / 1e3
-            lines.append("| %d | %s | %.1f | %.0f | %.1f |" % (M, name, us, gbs, gbs / PEAK_HBM_GBS * 100))
+            same = ""
+            if ref is not None and name != "ue8m0_packed":
+                q, s = sglang_per_token_group_quant_fp8(xs[0], 128, **kw)
+                rows = ref[0].shape[0]
+                same = "yes" if (torch.equal(q[:rows].cpu().view(torch.uint8), ref[0].view(torch.uint8))
+                                 and torch.equal(s[:rows].cpu().contiguous(), ref[1])) else "NO"
+            lines.append("| %d | %s | %.1f | %.0f | %.3f | %s | %s | %s |" % (M, name, us, gbs, gbs / PEAK_HBM_GBS, same,
+                                                                         cpu_us if name == "row_major_f32" else "",
+                                                                         cpu_gbs if name == "row_major_f32" else ""))
         del xs
+
+    # ---- configs[2]
     lines += ["", "## configs[2] block-FP8 GEMM, DeepSeek-V3 shapes", "",
-              "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s | GB/s (algorithmic) |", "|---|---|---|---|---|---|---|"]
+              "| M | N | K | GPU us | TFLOP/s | GB/s (algorithmic) | bound | frac | err | CPU us (rows) | CPU GFLOP/s |",
+              "|---|---|---|---|---|---|---|---|---|---|---|"]
     for (N, K) in DSV3_NK:
+        print("[table] configs[2] N=%d K=%d" % (N, K), file=sys.stderr, flush=True)
         nbuf = 3
         ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
+        wq_c, ws_c = (ws[0][0].cpu(), ws[0][1].cpu()) if cpu else (None, None)
         for M in (1, 16, 128, 1024, 4096):
             qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True)
                   for s in range(nbuf)]
             us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
                                                                     ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
             tf = 2.0 * M * N * K / us / 1e6
-            lines.append("| %d | %d | %d | %.1f | %.1f | %.1f | %.0f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100,
-                                                                          gemm_bytes(M, N, K) / us / 1e3))
+            bname, floor = _bound(2.0 * M * N * K, gemm_bytes(M, N, K))
+            err, cpu_us, cpu_gf = "", "", ""
+            if cpu:
+                rows = min(M, CPU_ROW_CAP)
+                qc, sc_ = qs[0][0][:rows].cpu(), qs[0][1][:rows].cpu().contiguous()
+                t = _median_time(lambda: cpu_block_matmul(torch, qc, sc_, wq_c, ws_c), runs=3)
+                ref = cpu_block_matmul(torch, qc, sc_, wq_c, ws_c)
+                got = w8a8_block_fp8_matmul(qs[0][0], ws[0][0], qs[0][1], ws[0][1], [128, 128], torch.bfloat16)[:rows].cpu()
+                err = "%.1e" % _rel_err(torch, got, ref)
+                cpu_us, cpu_gf = "%.0f (%d)" % (t * 1e6, rows), "%.1f" % (2.0 * rows * N * K / t / 1e9)
+            lines.append("| %d | %d | %d | %.1f | %.1f | %.0f | %s | %.3f | %s | %s | %s |" % (
+                M, N, K, us, tf, gemm_bytes(M, N, K) / us / 1e3, bname, floor / us, err, cpu_us, cpu_gf))
         del ws
+
     lines += ["", "## configs[2] shapes at M=4096 with UE8M0 scales (packed activation exponents, power-of-two weight scales:",
               "## the matrix core applies the block scales itself)", "",
-              "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s |", "|---|---|---|---|---|---|"]
+              "| M | N | K | GPU us | TFLOP/s | frac of 5 PFLOP/s |", "|---|---|---|---|---|---|"]
     for (N, K) in DSV3_NK:
         nbuf, M = 3, 4096
         ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
@@ -333,22 +481,36 @@ def write_table(torch, dev, path):
         us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
                                                                 ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
         tf = 2.0 * M * N * K / us / 1e6
-        lines.append("| %d | %d | %d | %.1f | %.1f | %.1f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100))
+        lines.append("| %d | %d | %d | %.1f | %.1f | %.3f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS))
         del ws
-    lines += ["", "## configs[3] per-token fp8_scaled_mm, Llama-3-8B shapes", "",
-              "| M | N | K | us | TFLOP/s | % of 5 PFLOP/s |", "|---|---|---|---|---|---|"]
+
+    # ---- configs[3]
+    lines += ["", "## configs[3] per-token fp8_scaled_mm, Llama-3-8B shapes (CPU: (A.float() @ B.float().T) * sa * sb in torch)", "",
+              "| M | N | K | GPU us | TFLOP/s | bound | frac | err | CPU us (rows) | CPU GFLOP/s |", "|---|---|---|---|---|---|---|---|---|---|"]
     for (N, K) in LLAMA_NK:
+        print("[table] configs[3] N=%d K=%d" % (N, K), file=sys.stderr, flush=True)
         nbuf = 3
         bs = [(torch.randn((N, K), device=dev) * 50).clamp(-448, 448).to(torch.float8_e4m3fn) for _ in range(nbuf)]
         sb = torch.rand(N, device=dev) * 1e-3
+        b_c, sb_c = (bs[0].cpu().float(), sb.cpu()) if cpu else (None, None)
         for M in (1, 8, 64, 512, 2048, 8192):
             a = [(torch.randn((M, K), device=dev) * 50).clamp(-448, 448).to(torch.float8_e4m3fn) for _ in range(nbuf)]
             sa = torch.rand(M, device=dev)
             us = _time_graph(torch, lambda i: fp8_scaled_mm(a[i % nbuf], bs[i % nbuf].t(), sa, sb, torch.bfloat16), 20)
             tf = 2.0 * M * N * K / us / 1e6
-            lines.append("| %d | %d | %d | %.1f | %.1f | %.1f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100))
+            bname, floor = _bound(2.0 * M * N * K, M * K + N * K + 2 * M * N + 4 * (M + N))
+            err, cpu_us, cpu_gf = "", "", ""
+            if cpu:
+                rows = min(M, CPU_ROW_CAP)
+                a_c, sa_c = a[0][:rows].cpu(), sa[:rows].cpu()
+                fn = lambda: ((a_c.float() @ b_c.t()) * sa_c[:, None] * sb_c[None, :]).to(torch.bfloat16)
+                t = _median_time(fn, runs=3)
+                got = fp8_scaled_mm(a[0], bs[0].t(), sa, sb, torch.bfloat16)[:rows].cpu()
+                err = "%.1e" % _rel_err(torch, got, fn())
+                cpu_us, cpu_gf = "%.0f (%d)" % (t * 1e6, rows), "%.1f" % (2.0 * rows * N * K / t / 1e9)
+            lines.append("| %d | %d | %d | %.1f | %.1f | %s | %.3f | %s | %s | %s |" % (M, N, K, us, tf, bname, floor / us, err, cpu_us, cpu_gf))
         del bs
-    lines += moe_table(torch, dev)
+    lines += moe_table(torch, dev, cpu=cpu)
     os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
@@ -397,7 +559,7 @@ def main() -> int:
     quant = run_quant_roofline(torch, dev)
     q_us, q_gbs = quant["row_major_f32"]
     if args.table:
-        write_table(torch, dev, args.table)
+        write_table(torch, dev, args.table, cpu=not args.no_cpu)
     if args.copy_calibration:
         src = torch.ones(64 << 20, dtype=torch.int32, device=dev)
         dst = torch.empty_like(src)
