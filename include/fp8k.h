@@ -173,6 +173,29 @@ int fp8k_scaled_mm(const void* A, const void* B, const float* sa, const float* s
 int64_t fp8k_scaled_mm_workspace_bytes(int64_t M, int64_t N, int64_t K);
 
 /*
+ * Per-tensor FP8 quantisation of a strided [H, S, D] tensor into a contiguous [H, S, D] one (the activations of the
+ * MLA absorbed products): *s must be zero on entry and receives max(absmax, eps) / 448 (atomic max), then
+ * q = clamp(x * (1 / *s)).
+ * Replaces per_tensor_quant_mla_fp8 (python/sglang/srt/layers/quantization/fp8_kernel.py:1172-1266, two Triton kernels).
+ * Row (h, s) of x starts at x[h * x_stride_h + s * x_stride_s] (elements) and is contiguous; D % 8 == 0, rows 16-byte aligned.
+ */
+int fp8k_tensor_quant_mla(const void* x, void* q, float* s, int64_t H, int64_t S, int64_t D, int64_t x_stride_h,
+                          int64_t x_stride_s, float eps, int in_dtype, void* stream);
+
+/*
+ * Batched FP8 GEMM with one scale per operand: C[b] = (A[b] . B[b]^T) * sa[m] * sb[n], float32 accumulation.
+ * Replaces torch.ops.sgl_kernel.bmm_fp8 (sgl-kernel/python/sgl_kernel/gemm.py:45-82, sgl-kernel/csrc/gemm/bmm_fp8.cu),
+ * whose per-tensor scales the caller broadcasts to the vectors sa [M] and sb [N] (shared by all batch entries).
+ * A e4m3fn [batch, M, K]: entry b at A + b * a_stride_b bytes, lda bytes between rows.  B e4m3fn [batch, N, K] with K
+ * contiguous - the same memory as the reference's column-major [batch, K, N] - entry b at B + b * b_stride_b, ldb
+ * between rows.  C [batch, M, N] of out_dtype: entry b at C + b * c_stride_b elements, ldc elements between rows.
+ * K % 128 == 0, N % 8 == 0, batch <= 65535.  No workspace.
+ */
+int fp8k_bmm_fp8(const void* A, const void* B, const float* sa, const float* sb, void* C, int64_t batch, int64_t M,
+                 int64_t N, int64_t K, int64_t a_stride_b, int64_t lda, int64_t b_stride_b, int64_t ldb,
+                 int64_t c_stride_b, int64_t ldc, int out_dtype, void* stream);
+
+/*
  * Token alignment for the fused-MoE grouped GEMM (integer work).
  * Replaces torch.ops.sgl_kernel.moe_align_block_size
  *   (sgl-kernel/python/sgl_kernel/moe.py:6-25, sgl-kernel/csrc/moe/moe_align_kernel.cu:302-366); the caller

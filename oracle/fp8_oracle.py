@@ -219,6 +219,29 @@ def per_tensor_quant_fp8(x, static_scale=None):
     return f32_to_e4m3fn(y), np.array([s], dtype=np.float32)
 
 
+def per_tensor_quant_mla_fp8(x, eps=1e-12):
+    """Reference: _per_tensor_quant_mla_fp8_stage1/2, python/sglang/srt/layers/quantization/fp8_kernel.py:1172-1266:
+    every row contributes max(rowabsmax, eps) / 448 to an atomic maximum, then q = clamp(x * (1 / scale)) in float32.
+    x float32 [H, S, D] (values of the input type) -> (q uint8 [H, S, D], scale float32 [1])."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    rowmax = np.maximum(np.abs(x).max(axis=-1), np.float32(eps)).astype(np.float32)
+    s = np.float32((rowmax / np.float32(FP8_MAX)).astype(np.float32).max())
+    inv = np.float32(1.0) / s
+    y = np.clip((x * inv).astype(np.float32), np.float32(FP8_MIN), np.float32(FP8_MAX))
+    return f32_to_e4m3fn(y), np.array([s], dtype=np.float32)
+
+
+def bmm_fp8(Aq, Bq, a_scale, b_scale, out_dtype="bf16"):
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:66-82 with the check of sgl-kernel/tests/test_bmm_fp8.py:21-39
+    (torch.bmm of the de-quantised operands).  Aq uint8 [b, m, k]; Bq uint8 [b, n, k] (the op's column-major [b, k, n]
+    is this memory); one float32 scale per operand.  out[b] = (A[b] @ B[b]^T) * a_scale * b_scale."""
+    A = e4m3fn_to_f32(Aq).astype(np.float64)
+    B = e4m3fn_to_f32(Bq).astype(np.float64)
+    C = np.einsum("bmk,bnk->bmn", A, B).astype(np.float32)
+    C = C * np.float32(a_scale) * np.float32(b_scale)
+    return _cast_out(C, out_dtype)
+
+
 # --------------------------------------------------------------------------
 # offline weight quant (test/srt/cpu/utils.py:39-87 semantics: amax/448 per block)
 # --------------------------------------------------------------------------

@@ -44,6 +44,8 @@ SIGNATURES = {
     ),
     "fp8k_token_quant": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_int, _c_ptr]),
     "fp8k_tensor_quant": (_c_int, [_c_ptr, _c_ptr, _c_ptr, _c_i64, _c_int, _c_int, _c_ptr]),
+    "fp8k_tensor_quant_mla": (_c_int, [_c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 5 + [_c_f32, _c_int, _c_ptr]),
+    "fp8k_bmm_fp8": (_c_int, [_c_ptr] * 5 + [_c_i64] * 10 + [_c_int, _c_ptr]),
     "fp8k_block_gemm": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 10 + [_c_int, _c_ptr, _c_i64, _c_ptr],

@@ -505,3 +505,37 @@ extern "C" int fp8k_scaled_mm(const void* A, const void* B, const float* sa, con
   return FP8K_SMM(FP8K_F16, FP8K_F16);
 #undef FP8K_SMM
 }
+
+// ---- batched per-tensor-scaled FP8 GEMM (the MLA absorbed products): every batch entry is a row-mode GEMM on the
+// 128x128 tile kernel (grid y = entry), whose per-row / per-column scale vectors are shared by all entries.
+extern "C" int fp8k_bmm_fp8(const void* A, const void* B, const float* sa, const float* sb, void* C, int64_t batch, int64_t M,
+                            int64_t N, int64_t K, int64_t a_stride_b, int64_t lda, int64_t b_stride_b, int64_t ldb,
+                            int64_t c_stride_b, int64_t ldc, int out_dtype, void* stream) {
+  clear_error();
+  const char* op = "bmm_fp8";
+  int rc = common_checks(op, A, B, C, M, N, K, lda, ldb, ldc, out_dtype);
+  if (rc) return rc;
+  FP8K_REQUIRE(batch >= 0 && batch <= 65535, "%s: batch must be in [0, 65535] (got %lld)", op, (long long)batch);
+  if (batch == 0 || M == 0 || N == 0) return FP8K_OK;
+  FP8K_REQUIRE(K > 0 && K % kTileK == 0, "%s: K must be a positive multiple of 128 (got %lld)", op, (long long)K);
+  FP8K_REQUIRE(N % 8 == 0, "%s: N must be a multiple of 8 (got %lld)", op, (long long)N);
+  FP8K_REQUIRE(sa && sb, "%s: null scale pointer", op);
+  FP8K_REQUIRE(aligned(sb, 16), "%s: the column scale vector must be 16-byte aligned", op);
+  FP8K_REQUIRE(a_stride_b % 16 == 0 && b_stride_b % 16 == 0 && (c_stride_b * 2) % 16 == 0 && a_stride_b >= 0 && b_stride_b >= 0 &&
+               c_stride_b >= 0, "%s: batch strides must be non-negative multiples of 16 bytes", op);
+  GemmArgs a{};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.sx = sa; a.sw = sb; a.bias = nullptr; a.C = C; a.partial = nullptr;
+  a.M = (int)M; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = ldc;
+  a.batch_x = a_stride_b; a.batch_w = b_stride_b; a.batch_c = c_stride_b;
+  a.tiles_m = (int)((M + kT128 - 1) / kT128);
+  a.tiles_n = (int)((N + kT128 - 1) / kT128);
+  a.splits = 1;
+  a.kb_per_split = (int)(K / kTileK);
+  const unsigned nwg = (unsigned)(((int64_t)a.tiles_m * a.tiles_n + 7) / 8 * 8);
+  hipStream_t st = (hipStream_t)stream;
+  if (out_dtype == FP8K_BF16)
+    hipLaunchKernelGGL((gemm_tile128_kernel<kModeRow, FP8K_BF16, FP8K_F32, false>), dim3(nwg, (unsigned)batch), dim3(512), 0, st, a);
+  else
+    hipLaunchKernelGGL((gemm_tile128_kernel<kModeRow, FP8K_F16, FP8K_F32, false>), dim3(nwg, (unsigned)batch), dim3(512), 0, st, a);
+  return check_launch(op);
+}

@@ -43,6 +43,9 @@ struct GemmArgs {
   int sx_sorted;                // grouped: sx holds one row per position of sorted_ids (row = position), not per token
   int64_t w_expert_stride;      // bytes between experts in W
   int64_t sw_expert_stride;     // floats between experts in sw
+  // batched form of the 128x128 tile kernel (grid y = batch entry); zero for a single GEMM
+  int64_t batch_x, batch_w;     // bytes between batch entries of X and W
+  int64_t batch_c;              // elements between batch entries of C
 };
 
 // kModeScaled: block mode with power-of-two scales applied by the matrix core itself (activation scales as packed

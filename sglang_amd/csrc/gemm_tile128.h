@@ -65,8 +65,12 @@ __global__ __launch_bounds__(512, 1) void gemm_tile128_kernel(const GemmArgs p) 
   // ---- global -> LDS: wave w brings rows [16w, 16w+16) of both tiles, two 1 KB loads (8 rows) each
   const int rowsW = min(kT128, p.N - n0), rowsX = min(kT128, p.M - m0);
   const int kbytes = p.K - kb_begin * kTileK;
-  const rsrc_t rW = make_rsrc(p.W + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
-  const rsrc_t rX = make_rsrc(p.X + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
+  // batched launches (grid y): every batch entry has its own operands and output, the scales are shared
+  const uint8_t* const Wb = p.W + (int64_t)blockIdx.y * p.batch_w;
+  const uint8_t* const Xb = p.X + (int64_t)blockIdx.y * p.batch_x;
+  u16* const Cb = (u16*)p.C + (int64_t)blockIdx.y * p.batch_c;
+  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw + (int64_t)kb_begin * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
+  const rsrc_t rX = make_rsrc(Xb + (int64_t)m0 * p.ldx + (int64_t)kb_begin * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
   const int rl = lane >> 3, cp = lane & 7;
   uint32_t voW[2], voX[2];
 #pragma unroll
@@ -300,7 +304,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile128_kernel(const GemmArgs p) 
   const int m_own = m0 + wm * 32 + lr;
   float sa = 1.f;
   if (MODE == kModeRow && m_own < nrows) sa = p.sx[m_own];
-  const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+  const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(Cb) & 15) == 0;
   if (wide) {
     wait_vm0_lgkm0();                // own stray loads have landed ...
     __builtin_amdgcn_s_barrier();    // ... and so have everyone's; every wave has taken its last operands
@@ -323,7 +327,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile128_kernel(const GemmArgs p) 
       const uint4 o = *reinterpret_cast<const uint4*>(ep + r * 128 + ((pc ^ (r & 7)) << 4));
       const int m = m0 + wm * 32 + r;
       const int n = n0 + wn * 64 + (pc << 3);
-      if (m < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)m * p.ldc + n) = o;
+      if (m < nrows && n < p.N) *reinterpret_cast<uint4*>(Cb + (int64_t)m * p.ldc + n) = o;
     }
     return;
   }
@@ -337,7 +341,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile128_kernel(const GemmArgs p) 
       const int n = n0 + wn * 64 + ns * 32 + rg * 8 + h * 4;
       if (n >= p.N) continue;
       const uint2 o = finish4(ns, rg, n, sa);
-      *reinterpret_cast<uint2*>((u16*)p.C + (int64_t)m_own * p.ldc + n) = o;
+      *reinterpret_cast<uint2*>(Cb + (int64_t)m_own * p.ldc + n) = o;
     }
 }
 

@@ -460,6 +460,47 @@ __global__ __launch_bounds__(256) void tensor_quant_kernel(const void* __restric
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// per-tensor quant of a strided [H, S, D] tensor into a contiguous one (the MLA absorbed products): a workgroup takes
+// whole rows (h, s) in grid-stride, a lane 8 elements at a time
+// ------------------------------------------------------------------------------------------------
+template <int DT, bool QUANT>
+__global__ __launch_bounds__(256) void rows_tensor_quant_kernel(const void* __restrict__ x, uint8_t* __restrict__ q,
+                                                                float* __restrict__ s, int64_t rows, int S, int D,
+                                                                int64_t stride_h, int64_t stride_s, float eps) {
+  __shared__ float red[4];
+  const int chunks = D / 8;                 // per row; the host checks D % 8 == 0 and the alignment of every row
+  const int64_t total = rows * chunks;
+  const int64_t step = (int64_t)gridDim.x * 256;
+  const float inv = QUANT ? 1.0f / s[0] : 0.f;
+  float m = 0.f;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    const int64_t row = i / chunks;
+    const int c = (int)(i - row * chunks);
+    const int64_t hh = row / S, ss = row - hh * S;
+    Raw8<DT> t;
+    t.load(x, hh * stride_h + ss * stride_s + c * 8);
+    float a[8];
+    t.unpack(a);
+    if (QUANT) {
+      float y[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) y[j] = fmaxf(fminf(a[j] * inv, kFp8Max), -kFp8Max);
+      uint2 o;
+      o.x = cvt4_fp8(y[0], y[1], y[2], y[3]);
+      o.y = cvt4_fp8(y[4], y[5], y[6], y[7]);
+      *reinterpret_cast<uint2*>(q + row * D + c * 8) = o;
+    } else {
+      m = fmaxf(m, absmax8(a));
+    }
+  }
+  if (!QUANT) {
+    m = block_max_256(fmaxf(m, eps), red);
+    // non-negative floats order like their bit patterns
+    if (threadIdx.x == 0) atomicMax(reinterpret_cast<unsigned int*>(s), __float_as_uint(m / kFp8Max));
+  }
+}
+
 }  // namespace fp8k
 
 using namespace fp8k;
@@ -637,4 +678,37 @@ extern "C" int fp8k_tensor_quant(const void* x, void* q, float* s, int64_t numel
   }
 #undef FP8K_TQ
   return check_launch("tensor_quant");
+}
+
+extern "C" int fp8k_tensor_quant_mla(const void* x, void* q, float* s, int64_t H, int64_t S, int64_t D, int64_t x_stride_h,
+                                     int64_t x_stride_s, float eps, int in_dtype, void* stream) {
+  clear_error();
+  const char* op = "per_tensor_quant_mla_fp8";
+  FP8K_REQUIRE(H >= 0 && S >= 0 && D >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "%s: bad input dtype %d", op, in_dtype);
+  FP8K_REQUIRE(S <= 0x7fffffffLL && D <= 0x7fffffffLL, "%s: shape too large", op);
+  if (H * S * D == 0) return FP8K_OK;
+  const int64_t esz = in_dtype == FP8K_F32 ? 4 : 2;
+  FP8K_REQUIRE(x && q && s, "%s: null pointer", op);
+  FP8K_REQUIRE(D % 8 == 0, "%s: the last dimension (%lld) must be divisible by 8", op, (long long)D);
+  FP8K_REQUIRE(x_stride_h >= 0 && x_stride_s >= 0 && (x_stride_h * esz) % 16 == 0 && (x_stride_s * esz) % 16 == 0 && aligned(x, 16) &&
+               aligned(q, 8), "%s: rows of x must be 16-byte aligned, q 8-byte aligned", op);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t rows = H * S;
+  const int64_t want = (rows * (D / 8) + 255) / 256;
+  dim3 grid((unsigned)(want < 1 ? 1 : (want > 2048 ? 2048 : want))), block(256);
+#define FP8K_MLAQ(DT)                                                                                                    \
+  do {                                                                                                                   \
+    hipLaunchKernelGGL((rows_tensor_quant_kernel<DT, false>), grid, block, 0, st, x, (uint8_t*)q, s, rows, (int)S, (int)D, \
+                       x_stride_h, x_stride_s, eps);                                                                     \
+    hipLaunchKernelGGL((rows_tensor_quant_kernel<DT, true>), grid, block, 0, st, x, (uint8_t*)q, s, rows, (int)S, (int)D,  \
+                       x_stride_h, x_stride_s, eps);                                                                     \
+  } while (0)
+  switch (in_dtype) {
+    case FP8K_BF16: FP8K_MLAQ(FP8K_BF16); break;
+    case FP8K_F16: FP8K_MLAQ(FP8K_F16); break;
+    default: FP8K_MLAQ(FP8K_F32); break;
+  }
+#undef FP8K_MLAQ
+  return check_launch(op);
 }

@@ -64,6 +64,15 @@ _register("block_gemm_nk(Tensor A, Tensor B, Tensor As, Tensor Bs, ScalarType ou
 _register("block_gemm_nk_ue8m0(Tensor A, Tensor B, Tensor As_packed, Tensor Bs, ScalarType out_dtype) -> Tensor",
           _k._block_gemm_nk_ue8m0, _nk_fake)
 
+_register("tensor_quant_mla(Tensor x, Tensor(a!) x_q, Tensor(b!) x_s, float eps) -> ()", _k.tensor_quant_mla, _none)
+
+
+def _bmm_impl(A, B, A_scale, B_scale, dtype, out) -> None:
+    _k.bmm_fp8(A, B, A_scale, B_scale, dtype, out)
+
+
+_register("bmm_fp8(Tensor A, Tensor B, Tensor A_scale, Tensor B_scale, ScalarType dtype, Tensor(a!) out) -> ()", _bmm_impl, _none)
+
 # ---- fused-MoE stages
 _register(
     "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor(a!) sorted_token_ids, "
@@ -142,6 +151,17 @@ def block_gemm_nk(A, B, As, Bs, out_dtype) -> torch.Tensor:
 
 def block_gemm_nk_ue8m0(A, B, As_packed, Bs, out_dtype) -> torch.Tensor:
     return _ops.block_gemm_nk_ue8m0(A, B, As_packed, Bs, out_dtype)
+
+
+def tensor_quant_mla(x, x_q, x_s, eps: float) -> None:
+    _ops.tensor_quant_mla(x, x_q, x_s, float(eps))
+
+
+def bmm_fp8(A, B, A_scale, B_scale, dtype, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if out is None:
+        out = torch.empty((A.shape[0], A.shape[1], B.shape[2]), device=A.device, dtype=dtype)
+    _ops.bmm_fp8(A, B, A_scale, B_scale, dtype, out)
+    return out
 
 
 def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,

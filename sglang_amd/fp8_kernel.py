@@ -142,6 +142,47 @@ def scaled_fp8_quant(
     return output, scale
 
 
+def per_tensor_quant_mla_fp8(x: torch.Tensor, x_s_out: torch.Tensor, eps: float = 1e-12) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:1221-1266 - tensor-wise quantisation specialised for the MLA absorbed products: x is a
+    (possibly transposed) [num_head, num_seq, head_size] view, the result is contiguous.  x_s_out: one float32 that
+    must be zero on entry (the maximum is accumulated atomically) and receives max(absmax, eps) / 448."""
+    assert x.dim() == 3, "`x` is not a 3d-tensor"
+    assert x_s_out.shape == (1,) and x_s_out.dtype == torch.float32 and x_s_out.device == x.device
+    x_q = x.new_empty(x.size(), dtype=fp8_dtype)
+    if x.numel() > 0:
+        _ops.tensor_quant_mla(x, x_q, x_s_out, eps)
+    return x_q, x_s_out
+
+
+def per_token_group_quant_mla_deep_gemm_masked_fp8(
+    x: torch.Tensor, group_size: int = 128, eps: float = 1e-12, dtype: torch.dtype = fp8_dtype
+):
+    """Reference: fp8_kernel.py:1319-1362 - per-token-group quantisation of a [b, m, k] tensor into the masked layout
+    of the grouped GEMM: x_q [b, ceil256(m), k], scales [b, ceil256(m), k/g] stored as [b, k/g, ceil256(m)] (m
+    contiguous), masked_m [b] = m.  Returns (x_q, scales, masked_m, m, aligned_m); rows at or past m are not written.
+    x is first laid out as [b, aligned_m, k] (one copy, which also takes care of transposed inputs); the quantisation
+    is the masked form of the group quant kernel.  An all-zero group gets the scale of the eps clamp in the input
+    type (bf16(eps) / 448 for a bf16 input, where the reference's Triton kernel has eps / 448); its bytes are zero."""
+    assert x.dim() == 3, "`x` is not a 3d-tensor"
+    if dtype != fp8_dtype:
+        raise RuntimeError("per_token_group_quant_mla_deep_gemm_masked_fp8: only float8_e4m3fn is built on gfx950")
+    b, m, k = x.shape
+    aligned_m = (m + 255) // 256 * 256  # 256 is the largest row block of the grouped GEMM
+    num_tiles_k = k // group_size
+    assert num_tiles_k * group_size == k, f"k % {group_size} must be zero"
+    x_q = x.new_empty((b, aligned_m, k), dtype=dtype)
+    x_s = x.new_empty((b, num_tiles_k, aligned_m), dtype=torch.float32)
+    masked_m = torch.full((b,), m, dtype=torch.int32, device=x.device)
+    if b * m > 0:
+        if m == aligned_m and x.is_contiguous():
+            xp = x
+        else:
+            xp = x.new_empty((b, aligned_m, k))
+            xp[:, :m].copy_(x)
+        _ops.sgl_per_token_group_quant_8bit(xp, x_q, x_s.transpose(1, 2), group_size, eps, fp8_min, fp8_max, False, False, masked_m)
+    return x_q, x_s.transpose(1, 2), masked_m, m, aligned_m
+
+
 def w8a8_block_fp8_matmul(
     A: torch.Tensor,
     B: torch.Tensor,

@@ -318,6 +318,64 @@ def fp8_scaled_mm(mat_a, mat_b, scales_a, scales_b, out_dtype, bias=None):
     return out
 
 
+def tensor_quant_mla(x: torch.Tensor, x_q: torch.Tensor, x_s: torch.Tensor, eps: float) -> None:
+    """Per-tensor quant of a strided [H, S, D] tensor into the contiguous x_q; x_s (one float32, zero on entry) receives
+    max(absmax, eps) / 448.  Native side of fp8_kernel.per_tensor_quant_mla_fp8 (include/fp8k.h: fp8k_tensor_quant_mla)."""
+    require_cuda(x, x_q, x_s)
+    if x.dim() != 3 or x.stride(2) != 1:
+        raise RuntimeError("per_tensor_quant_mla_fp8: x must be 3-D with a contiguous last dimension")
+    if x_q.dtype != FP8_DTYPE or not x_q.is_contiguous() or x_q.shape != x.shape:
+        raise RuntimeError("per_tensor_quant_mla_fp8: x_q must be contiguous float8_e4m3fn of x's shape")
+    if x_s.dtype != torch.float32 or x_s.numel() != 1:
+        raise RuntimeError("per_tensor_quant_mla_fp8: x_s must be one float32")
+    H, S, D = x.shape
+    check(lib.fp8k_tensor_quant_mla(x.data_ptr(), x_q.data_ptr(), x_s.data_ptr(), H, S, D, x.stride(0), x.stride(1), float(eps),
+                                    dtype_code(x.dtype), stream_ptr(x.device)))
+
+
+def bmm_fp8(A: torch.Tensor, B: torch.Tensor, A_scale: torch.Tensor, B_scale: torch.Tensor, dtype: torch.dtype,
+            out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:66-82 (a cuBLASLt batched GEMM there).  A e4m3fn [b, m, k] with k
+    contiguous, B e4m3fn [b, k, n] column-major per entry (k contiguous: a [b, n, k] weight transposed), one float32
+    scale per operand; returns / fills out [b, m, n] = (A @ B) * A_scale * B_scale in `dtype`.  No host synchronisation:
+    the scalar scales are broadcast to vectors on the device."""
+    require_cuda(A, B, A_scale, B_scale, out)
+    if A.dim() != 3 or B.dim() != 3 or A.shape[0] != B.shape[0] or A.shape[2] != B.shape[1]:
+        raise RuntimeError("bmm_fp8: A [b, m, k] and B [b, k, n] expected")
+    if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
+        raise RuntimeError("bmm_fp8: A and B must be float8_e4m3fn (e5m2 is not built on this path)")
+    b, m, k = A.shape
+    n = B.shape[2]
+    if (k > 1 and A.stride(2) != 1) or (k > 1 and B.stride(1) != 1):
+        raise RuntimeError("bmm_fp8: A must be row-major and B column-major in their last two dimensions")
+    if A_scale.numel() != 1 or B_scale.numel() != 1:
+        raise RuntimeError("bmm_fp8: one scale per operand expected")
+    out_code = _out_code(dtype)
+    if out is None:
+        out = torch.empty((b, m, n), device=A.device, dtype=dtype)
+    elif out.shape != (b, m, n) or out.dtype != dtype or (n > 1 and out.stride(2) != 1):
+        raise RuntimeError("bmm_fp8: out must be [b, m, n] of the result dtype with a contiguous last dimension")
+    if b == 0 or m == 0 or n == 0:
+        return out
+    if k % 128 != 0 or n % 8 != 0:
+        # the kernel walks K in blocks of 128 and writes 8 columns at a time: zero padding changes no sum
+        kp, np_ = (k + 127) // 128 * 128, (n + 7) // 8 * 8
+        Ap = A.new_zeros((b, m, kp), dtype=torch.uint8)
+        Ap[:, :, :k] = A.view(torch.uint8)
+        Bp = B.new_zeros((b, np_, kp), dtype=torch.uint8)
+        Bp[:, :n, :k] = B.view(torch.uint8).transpose(1, 2)
+        res = bmm_fp8(Ap.view(FP8_DTYPE), Bp.view(FP8_DTYPE).transpose(1, 2), A_scale, B_scale, dtype)
+        out.copy_(res[:, :, :n])
+        return out
+    sa = A_scale.reshape(1).to(torch.float32).expand(m).contiguous()
+    sb = B_scale.reshape(1).to(torch.float32).expand(n).contiguous()
+    check(lib.fp8k_bmm_fp8(A.data_ptr(), B.data_ptr(), sa.data_ptr(), sb.data_ptr(), out.data_ptr(), b, m, n, k,
+                           A.stride(0) if b > 1 else m * k, A.stride(1) if m > 1 else k, B.stride(0) if b > 1 else n * k,
+                           B.stride(2) if n > 1 else k, out.stride(0) if b > 1 else m * n, out.stride(1) if m > 1 else n,
+                           out_code, stream_ptr(A.device)))
+    return out
+
+
 def _block_gemm_nk(A, B, As, Bs, out_dtype):
     """Block GEMM on the Triton-side layout: B [N,K] row-major, Bs [ceil(N/128), ceil(K/128)].
 

@@ -482,3 +482,48 @@ def test_moe_fused_gate_bf16_branch_against_torch_bf16_ops(E, G, tg, topk):
     # the bf16 rounding matters: the float32 gate picks other experts on some rows of the same data
     _, ids32 = O.moe_fused_gate(x.float().numpy(), bias.float().numpy(), G, tg, topk, in_dtype="f32")
     assert (ids32 != ids).any()
+
+
+def test_per_tensor_quant_mla_against_torch_ops_and_closed_form():
+    """per_tensor_quant_mla_fp8 (fp8_kernel.py:1172-1266) restated with torch ops on a transposed bf16 view: per-row
+    max(absmax, eps) / 448, the maximum of those, x * (1 / s) clamped and converted by torch's e4m3fn cast."""
+    g = torch.Generator().manual_seed(3)
+    x = (torch.randn(24, 6, 128, generator=g) * 3).to(torch.bfloat16).transpose(0, 1)  # [H=6, S=24, D=128], strided
+    rows = x.float().abs().amax(-1).clamp(min=1e-12) / 448.0
+    s = rows.max()
+    q = (x.float() * (1.0 / s)).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    oq, os_ = O.per_tensor_quant_mla_fp8(x.float().numpy())
+    assert os_.shape == (1,) and os_[0] == np.float32(s.item())
+    assert np.array_equal(oq, q.view(torch.uint8).numpy())
+    # closed forms: the element of largest magnitude lands on +-448; an all-zero tensor gets eps / 448 and zero bytes
+    y = np.zeros((2, 3, 16), np.float32)
+    y[1, 2, 5] = -7.0
+    y[0, 0, 0] = 3.5
+    q2, s2 = O.per_tensor_quant_mla_fp8(y)
+    assert s2[0] == np.float32(7.0) / np.float32(448.0)
+    assert O.e4m3fn_to_f32(q2)[1, 2, 5] == -448.0 and O.e4m3fn_to_f32(q2)[0, 0, 0] == 224.0
+    q3, s3 = O.per_tensor_quant_mla_fp8(np.zeros((1, 2, 8), np.float32))
+    assert s3[0] == np.float32(1e-12) / np.float32(448.0) and not q3.any()
+
+
+def test_bmm_fp8_against_torch_bmm_and_brute_force():
+    """bmm_fp8 the way sgl-kernel/tests/test_bmm_fp8.py checks it: torch.bmm of the de-quantised operands (float64 here),
+    times both scales; plus a triple loop on a tiny case, which a transposed operand or a dropped scale would fail."""
+    rng = np.random.default_rng(5)
+    b, m, n, k = 3, 5, 7, 16
+    aq = rng.integers(0, 0x70, (b, m, k), dtype=np.uint8) | (rng.integers(0, 2, (b, m, k), dtype=np.uint8) << 7)
+    bq = rng.integers(0, 0x70, (b, n, k), dtype=np.uint8) | (rng.integers(0, 2, (b, n, k), dtype=np.uint8) << 7)
+    sa, sb = np.float32(0.0123), np.float32(0.25)
+    got = O.bmm_fp8(aq, bq, sa, sb, "f32")
+    A = torch.from_numpy(aq).view(torch.float8_e4m3fn).double()
+    B = torch.from_numpy(bq).view(torch.float8_e4m3fn).double().transpose(1, 2)  # [b, k, n] column-major, as the op takes it
+    ref = (torch.bmm(A, B) * float(sa) * float(sb)).numpy()
+    assert np.allclose(got, ref, rtol=1e-6, atol=0)
+    brute = np.zeros((b, m, n))
+    a_f, b_f = O.e4m3fn_to_f32(aq).astype(np.float64), O.e4m3fn_to_f32(bq).astype(np.float64)
+    for i in range(b):
+        for r in range(m):
+            for c in range(n):
+                brute[i, r, c] = sum(a_f[i, r, t] * b_f[i, c, t] for t in range(k)) * float(sa) * float(sb)
+    assert np.allclose(got, brute, rtol=1e-6, atol=0)
+    assert np.array_equal(O.bmm_fp8(aq, bq, sa, sb, "bf16"), O.to_bf16(got))
