@@ -235,6 +235,51 @@ int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const flo
                         int out_dtype, int as_sorted, void* stream);
 
 /*
+ * Expert-major row layout for the grouped GEMM (integer work): the (token, k) slots of topk_ids int32 [numel] sorted by
+ * expert into contiguous, un-padded row ranges.
+ * Replaces torch.ops.sgl_kernel.prepare_moe_input (sgl-kernel/python/sgl_kernel/moe.py:217-240,
+ *   sgl-kernel/csrc/moe/prepare_moe_input.cu:12-167).
+ * expert_offsets [E + 1] (start row of every expert, then the total); blockscale_offsets [E + 1] or null (the same with
+ * every count rounded up to 128); problem_sizes1 [E, 3] = (rows, 2n, k); problem_sizes2 [E, 3] = (rows, k, n);
+ * input_permutation [numel]: token (slot / topk) whose copy sits in that row; output_permutation [numel]: row of the
+ * slot.  As in the reference the order of the rows inside one expert is not defined (atomic cursors).  Ids outside
+ * [0, num_experts) take no row.  num_experts <= 4096.  One workgroup, no scratch memory (the reference allocates a
+ * zeroed counter buffer per call).
+ */
+int fp8k_moe_prepare_input(const int32_t* topk_ids, int64_t numel, int64_t topk, int64_t num_experts, int64_t n, int64_t k,
+                           int32_t* expert_offsets, int32_t* blockscale_offsets, int32_t* problem_sizes1,
+                           int32_t* problem_sizes2, int32_t* input_permutation, int32_t* output_permutation, void* stream);
+
+/*
+ * output[d, :] = input[dst2src_map[d], :] for contiguous rows of row_bytes bytes (moved 16 bytes a lane when rows and
+ * pointers are multiples of 16 bytes, 4 or 1 otherwise).  Replaces torch.ops.sgl_kernel.shuffle_rows (sgl-kernel/python/sgl_kernel/gemm.py:302-309,
+ * prepare_moe_input.cu:169-250).  A map entry outside [0, src_rows) leaves its destination row untouched.
+ */
+int fp8k_shuffle_rows(const void* input, const int32_t* dst2src_map, void* output, int64_t src_rows, int64_t dst_rows,
+                      int64_t row_bytes, void* stream);
+
+/*
+ * output[t, :] = sum_j factors[t * topk + j] * input[permutation[t * topk + j], :], float32 sum in ascending j, one
+ * rounding to the element type; factors (same element type as the data) may be null (= 1).
+ * Replaces torch.ops.sgl_kernel.apply_shuffle_mul_sum (sgl-kernel/python/sgl_kernel/moe.py:243-251,
+ * prepare_moe_input.cu:252-392).  cols % 8 == 0; rows whose permutation entry is outside [0, input_rows) are skipped.
+ */
+int fp8k_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors, int64_t m,
+                               int64_t topk, int64_t cols, int64_t input_rows, int dtype, void* stream);
+
+/*
+ * Block table (sorted_token_ids / expert_ids / num_tokens_post_padded, as fp8k_moe_align_block_size writes them) for the
+ * expert-major layout: expert e owns rows [expert_starts[e], expert_starts[e] + problem_sizes[3 * e]).  With it
+ * fp8k_moe_block_gemm (top_k = 1, num_valid_tokens = rows) is the grouped GEMM of
+ * torch.ops.sgl_kernel.fp8_blockwise_scaled_grouped_mm (sgl-kernel/python/sgl_kernel/moe.py:175-214,
+ * sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu), which takes exactly these two tensors; the reference's pointer
+ * arrays, stride vectors and scale-layout buffers are CUTLASS plumbing with no counterpart here.
+ */
+int fp8k_moe_blocks_from_offsets(const int32_t* expert_starts, const int32_t* problem_sizes, int64_t num_experts, int64_t rows,
+                                 int64_t block_m, int32_t* sorted_token_ids, int64_t sorted_capacity, int32_t* expert_ids,
+                                 int64_t expert_capacity, int32_t* num_tokens_post_pad, void* stream);
+
+/*
  * Activation scales in the order of sorted_token_ids (no counterpart in the reference, whose Triton kernel gathers
  * them per K block): out[kb * sorted_capacity + i] = As[sorted_token_ids[i] / top_k, kb] for i below
  * num_tokens_post_padded[0], 0 for padding entries.  Passing `out` to fp8k_moe_block_gemm with as_stride_m = 1,

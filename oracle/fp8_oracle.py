@@ -496,6 +496,87 @@ def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scalin
 
 
 # --------------------------------------------------------------------------
+# expert-major ("CUTLASS") form of the fused experts
+# --------------------------------------------------------------------------
+
+
+def prepare_moe_input(topk_ids, num_experts, n, k):
+    """Reference: sgl-kernel/csrc/moe/prepare_moe_input.cu:12-141.  topk_ids int32 [m, topk] ->
+    (expert_offsets [E+1], blockscale_offsets [E+1], problem_sizes1 [E,3], problem_sizes2 [E,3], a_map, c_map).
+    The reference hands out the rows of an expert through an atomic counter, so their order inside the expert is not
+    defined; this restatement takes the slots in ascending order (one of the orders the reference can produce)."""
+    ids = np.asarray(topk_ids, dtype=np.int64)
+    topk = ids.shape[1]
+    flat = ids.reshape(-1)
+    counts = np.array([(flat == e).sum() for e in range(num_experts)], dtype=np.int32)
+    offsets = np.zeros(num_experts + 1, dtype=np.int32)
+    offsets[1:] = np.cumsum(counts)
+    bs_offsets = np.zeros(num_experts + 1, dtype=np.int32)
+    bs_offsets[1:] = np.cumsum((counts + 127) // 128 * 128)
+    ps1 = np.stack([counts, np.full_like(counts, 2 * n), np.full_like(counts, k)], axis=1).astype(np.int32)
+    ps2 = np.stack([counts, np.full_like(counts, k), np.full_like(counts, n)], axis=1).astype(np.int32)
+    a_map = np.zeros(flat.size, dtype=np.int32)
+    c_map = np.zeros(flat.size, dtype=np.int32)
+    cursor = offsets[:-1].copy()
+    for i, e in enumerate(flat):
+        if 0 <= e < num_experts:
+            a_map[cursor[e]] = i // topk
+            c_map[i] = cursor[e]
+            cursor[e] += 1
+    return offsets, bs_offsets, ps1, ps2, a_map, c_map
+
+
+def shuffle_rows(x, dst2src_map):
+    """Reference: prepare_moe_input.cu:169-193: out[d] = x[dst2src_map[d]]."""
+    return np.ascontiguousarray(np.asarray(x)[np.asarray(dst2src_map, dtype=np.int64)])
+
+
+def apply_shuffle_mul_sum(x, permutation, factors, out_dtype="bf16"):
+    """Reference: prepare_moe_input.cu:252-310: out[t] = T(sum_j f32(factors[t*topk+j]) * f32(x[perm[t*topk+j]])), float32
+    accumulation in ascending j (the product of two 16-bit values is exact in float32, so a fused multiply-add and a
+    multiply followed by an add give the same sum).  x float32 values of the element type [m*topk, k]; permutation
+    [m, topk]; factors float32 values of the element type [m, topk] or None."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    perm = np.asarray(permutation, dtype=np.int64)
+    m, topk = perm.shape
+    acc = np.zeros((m, x.shape[1]), dtype=np.float32)
+    for j in range(topk):
+        f = np.float32(1.0) if factors is None else np.asarray(factors, dtype=np.float32)[:, j][:, None]
+        acc = (acc + (f * x[perm[:, j]]).astype(np.float32)).astype(np.float32)
+    return _cast_out(acc, out_dtype)
+
+
+def fp8_blockwise_scaled_grouped_mm(Aq, Bq, As, Bs, expert_offsets, problem_sizes, out_dtype="bf16", acc=np.float32):
+    """Reference: sgl-kernel/csrc/moe/fp8_blockwise_moe_kernel.cu with the check of sgl-kernel/tests/
+    test_fp8_blockwise_moe.py:109-216: for every expert e, rows [expert_offsets[e], + problem_sizes[e, 0]) of A times
+    that expert's weight, 1x128 scales on A and 128x128 scales on B.  Aq uint8 [rows, K]; Bq uint8 [E, N, K];
+    As f32 [rows, K/128]; Bs f32 [E, N/128, K/128].  Rows that no expert owns stay zero."""
+    E, N, _ = Bq.shape
+    out = np.zeros((Aq.shape[0], N), dtype=np.float32)
+    for e in range(E):
+        r0, cnt = int(expert_offsets[e]), int(problem_sizes[e][0])
+        if cnt:
+            out[r0:r0 + cnt] = w8a8_block_fp8_matmul(Aq[r0:r0 + cnt], Bq[e], As[r0:r0 + cnt], Bs[e], (128, 128), out_dtype, acc=acc)
+    return out
+
+
+def cutlass_fused_experts_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, out_dtype="bf16"):
+    """Reference: cutlass_fused_experts_fp8, python/sglang/srt/layers/moe/cutlass_moe.py:119-247: prepare_moe_input ->
+    group quant of x -> rows replicated into expert order -> grouped GEMM 1 (out dtype) -> silu_and_mul -> group quant
+    -> grouped GEMM 2 (out dtype) -> apply_shuffle_mul_sum with topk_weights cast to the out dtype.
+    x bf16 values [m, k]; w13q uint8 [E, 2n, k]; w2q uint8 [E, k, n]; topk_w float32 [m, topk]."""
+    E = w13q.shape[0]
+    n = w2q.shape[2]
+    k = x.shape[1]
+    offsets, _, ps1, ps2, a_map, c_map = prepare_moe_input(topk_ids, E, n, k)
+    xq, xs = per_token_group_quant_fp8(x, 128)
+    c1 = fp8_blockwise_scaled_grouped_mm(shuffle_rows(xq, a_map), w13q, shuffle_rows(xs, a_map), w13s, offsets, ps1, out_dtype)
+    iq, is_ = per_token_group_quant_fp8(silu_and_mul(c1), 128)
+    c2 = fp8_blockwise_scaled_grouped_mm(iq, w2q, is_, w2s, offsets, ps2, out_dtype)
+    return apply_shuffle_mul_sum(c2, c_map.reshape(topk_ids.shape), _cast_out(np.asarray(topk_w, np.float32), out_dtype), out_dtype)
+
+
+# --------------------------------------------------------------------------
 # seeded synthetic inputs of the benchmark configurations
 # --------------------------------------------------------------------------
 

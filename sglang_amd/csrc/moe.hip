@@ -621,3 +621,259 @@ extern "C" int fp8k_moe_fused_gate(const void* input, const void* bias, float* t
 #undef FP8K_GATE2
   return check_launch(op);
 }
+
+namespace fp8k {
+
+// ------------------------------------------------------------------------------------------------
+// Expert-major MoE layout: the rows of every expert contiguous and un-padded, described by start offsets.
+//
+// moe_prepare_kernel: one workgroup.  Histogram of the expert of every (token, k) slot with LDS atomics, exclusive
+// scan by the first wavefront, then every slot takes the next free row of its expert (LDS cursor): the order of
+// the rows inside an expert is not defined, the rows themselves do not depend on it.
+//   expert_offsets [E + 1], optional blockscale_offsets [E + 1] (counts rounded up to 128),
+//   problem_sizes1 [E, 3] = (rows, 2n, k), problem_sizes2 [E, 3] = (rows, k, n),
+//   input_permutation[row] = token of the slot in that row, output_permutation[slot] = row.
+// Ids outside [0, E) take no row and leave their output_permutation entry untouched.
+// ------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kAlignThreads) void moe_prepare_kernel(const int32_t* __restrict__ ids, int numel, int topk,
+                                                                    int E, int n, int k, int32_t* __restrict__ offsets,
+                                                                    int32_t* __restrict__ bs_offsets,
+                                                                    int32_t* __restrict__ ps1, int32_t* __restrict__ ps2,
+                                                                    int32_t* __restrict__ in_perm,
+                                                                    int32_t* __restrict__ out_perm) {
+  __shared__ int32_t counts[kAlignMaxBuckets];
+  __shared__ int32_t cursor[kAlignMaxBuckets];
+  __shared__ int32_t rounded[kAlignMaxBuckets];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += kAlignThreads) counts[e] = 0;
+  __syncthreads();
+  for (int i = tid; i < numel; i += kAlignThreads) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (tid < 64) {
+    const int per = (E + 63) / 64;
+    const int e0 = tid * per, e1 = min(E, e0 + per);
+    int sum = 0, rsum = 0;
+    for (int e = e0; e < e1; ++e) { sum += counts[e]; rsum += (counts[e] + 127) / 128 * 128; }
+    int incl = sum, rincl = rsum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off), rv = __shfl_up(rincl, off);
+      if (tid >= off) { incl += v; rincl += rv; }
+    }
+    int run = incl - sum, rrun = rincl - rsum;
+    for (int e = e0; e < e1; ++e) {
+      cursor[e] = run; rounded[e] = rrun;
+      run += counts[e]; rrun += (counts[e] + 127) / 128 * 128;
+    }
+    if (tid == 63) { offsets[E] = incl; if (bs_offsets) bs_offsets[E] = rincl; }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += kAlignThreads) {
+    offsets[e] = cursor[e];
+    if (bs_offsets) bs_offsets[e] = rounded[e];
+    ps1[e * 3] = counts[e]; ps1[e * 3 + 1] = 2 * n; ps1[e * 3 + 2] = k;
+    ps2[e * 3] = counts[e]; ps2[e * 3 + 1] = k; ps2[e * 3 + 2] = n;
+  }
+  __syncthreads();
+  for (int i = tid; i < numel; i += kAlignThreads) {
+    const int e = ids[i];
+    if (e >= 0 && e < E) {
+      const int row = atomicAdd(&cursor[e], 1);
+      in_perm[row] = i / topk;
+      out_perm[i] = row;
+    }
+  }
+}
+
+// out[d, :] = in[map[d], :], rows moved in units of T (16 bytes a lane when the rows allow it); a map entry outside
+// [0, src_rows) leaves its destination row untouched.
+template <typename T>
+__global__ __launch_bounds__(256) void shuffle_rows_kernel(const T* __restrict__ in, const int32_t* __restrict__ map,
+                                                           T* __restrict__ out, int64_t src_rows, int64_t dst_rows,
+                                                           int chunks) {
+  const int64_t total = dst_rows * chunks;
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    const int64_t d = i / chunks;
+    const int c = (int)(i - d * chunks);
+    const int64_t s = map[d];
+    if (s >= 0 && s < src_rows) out[d * chunks + c] = in[s * chunks + c];
+  }
+}
+
+// out[t, :] = T( sum_j float(factor[t * topk + j]) * float(in[perm[t * topk + j], :]) ), ascending j, float32 sum
+template <int DT>
+__global__ __launch_bounds__(256) void shuffle_mul_sum_kernel(const void* __restrict__ in, void* __restrict__ out,
+                                                              const int32_t* __restrict__ perm, const void* __restrict__ factors,
+                                                              int64_t m, int topk, int cols, int64_t in_rows) {
+  const int chunks = cols / 8;
+  const int64_t total = m * chunks;
+  const int64_t step = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    const int64_t t = i / chunks;
+    const int c = (int)(i - t * chunks) * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < topk; ++j) {
+      const int64_t slot = t * topk + j;
+      const int64_t r = perm[slot];
+      if (r < 0 || r >= in_rows) continue;
+      float f = 1.0f;
+      if (factors) {
+        if (DT == FP8K_F32) f = ((const float*)factors)[slot];
+        else if (DT == FP8K_BF16) f = __uint_as_float((uint32_t)((const u16*)factors)[slot] << 16);
+        else f = f16_bits_to_f32(((const u16*)factors)[slot]);
+      }
+      float v[8];
+      load8<DT>(in, r * cols + c, v);
+#pragma unroll
+      for (int q = 0; q < 8; ++q) acc[q] = fmaf(f, v[q], acc[q]);
+    }
+    store8<DT>(out, t * cols + c, acc);
+  }
+}
+
+// Block table of the grouped GEMM for the expert-major layout: expert e owns rows [starts[e], starts[e] + sizes[3e]).
+// Every expert's rows are cut into blocks of `block` slots (the last one padded with the id `rows`), experts in
+// ascending order.  One workgroup: scan of the block counts by the first wavefront, then one pass over the slots.
+__global__ __launch_bounds__(kAlignThreads) void moe_offset_blocks_kernel(const int32_t* __restrict__ starts,
+                                                                          const int32_t* __restrict__ sizes, int E, int rows,
+                                                                          int block, int32_t* __restrict__ sorted,
+                                                                          int32_t* __restrict__ expert_ids,
+                                                                          int32_t* __restrict__ post_pad, int max_blocks) {
+  __shared__ int32_t first_block[kAlignMaxBuckets + 1];
+  const int tid = threadIdx.x;
+  if (tid < 64) {
+    const int per = (E + 63) / 64;
+    const int e0 = tid * per, e1 = min(E, e0 + per);
+    int sum = 0;
+    for (int e = e0; e < e1; ++e) sum += (max(sizes[e * 3], 0) + block - 1) / block;
+    int incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off);
+      if (tid >= off) incl += v;
+    }
+    int run = incl - sum;
+    for (int e = e0; e < e1; ++e) {
+      first_block[e] = run;
+      run += (max(sizes[e * 3], 0) + block - 1) / block;
+    }
+    if (tid == 63) first_block[E] = incl;
+  }
+  __syncthreads();
+  const int nblocks = min(first_block[E], max_blocks);
+  if (tid == 0) post_pad[0] = nblocks * block;
+  for (int b = tid; b < nblocks; b += kAlignThreads) {
+    int lo = 0, hi = E;  // first expert with first_block[e + 1] > b
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (first_block[mid + 1] <= b) lo = mid + 1;
+      else hi = mid;
+    }
+    expert_ids[b] = lo;
+  }
+  __syncthreads();
+  const int total = nblocks * block;
+  for (int i = tid; i < total; i += kAlignThreads) {
+    const int b = i / block;
+    int lo = 0, hi = E;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (first_block[mid + 1] <= b) lo = mid + 1;
+      else hi = mid;
+    }
+    const int within = i - first_block[lo] * block;
+    const int row = starts[lo] + within;
+    sorted[i] = (within < sizes[lo * 3] && row >= 0 && row < rows) ? row : rows;
+  }
+}
+
+}  // namespace fp8k
+
+extern "C" int fp8k_moe_prepare_input(const int32_t* topk_ids, int64_t numel, int64_t topk, int64_t num_experts, int64_t n,
+                                      int64_t k, int32_t* expert_offsets, int32_t* blockscale_offsets,
+                                      int32_t* problem_sizes1, int32_t* problem_sizes2, int32_t* input_permutation,
+                                      int32_t* output_permutation, void* stream) {
+  clear_error();
+  const char* op = "prepare_moe_input";
+  FP8K_REQUIRE(numel >= 0 && numel < 0x7fffffffLL && topk >= 1 && numel % topk == 0,
+               "%s: topk_ids must hold a whole number of rows of topk ids (numel %lld, topk %lld)", op, (long long)numel,
+               (long long)topk);
+  FP8K_REQUIRE(num_experts >= 1 && num_experts <= kAlignMaxBuckets, "%s: num_experts must be in [1, %d] (got %lld)", op,
+               kAlignMaxBuckets, (long long)num_experts);
+  FP8K_REQUIRE(n >= 0 && k >= 0 && 2 * n <= 0x7fffffffLL && k <= 0x7fffffffLL, "%s: bad n / k", op);
+  FP8K_REQUIRE(expert_offsets && problem_sizes1 && problem_sizes2, "%s: null output pointer", op);
+  FP8K_REQUIRE(numel == 0 || (topk_ids && input_permutation && output_permutation), "%s: null pointer", op);
+  hipLaunchKernelGGL(moe_prepare_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, topk_ids, (int)numel,
+                     (int)topk, (int)num_experts, (int)n, (int)k, expert_offsets, blockscale_offsets, problem_sizes1,
+                     problem_sizes2, input_permutation, output_permutation);
+  return check_launch(op);
+}
+
+extern "C" int fp8k_shuffle_rows(const void* input, const int32_t* dst2src_map, void* output, int64_t src_rows,
+                                 int64_t dst_rows, int64_t row_bytes, void* stream) {
+  clear_error();
+  const char* op = "shuffle_rows";
+  FP8K_REQUIRE(src_rows >= 0 && dst_rows >= 0 && row_bytes >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(row_bytes <= 0x7fffffffLL, "%s: rows longer than 2 GiB are not supported", op);
+  if (dst_rows == 0 || row_bytes == 0) return FP8K_OK;
+  FP8K_REQUIRE(input && dst2src_map && output, "%s: null pointer", op);
+  hipStream_t st = (hipStream_t)stream;
+#define FP8K_SHUF(T)                                                                                                       \
+  hipLaunchKernelGGL(shuffle_rows_kernel<T>, dim3(stream_grid(dst_rows * (row_bytes / (int64_t)sizeof(T)))), dim3(256), 0, \
+                     st, (const T*)input, dst2src_map, (T*)output, src_rows, dst_rows, (int)(row_bytes / (int64_t)sizeof(T)))
+  if (row_bytes % 16 == 0 && aligned(input, 16) && aligned(output, 16)) FP8K_SHUF(uint4);
+  else if (row_bytes % 4 == 0 && aligned(input, 4) && aligned(output, 4)) FP8K_SHUF(uint32_t);
+  else FP8K_SHUF(uint8_t);
+#undef FP8K_SHUF
+  return check_launch(op);
+}
+
+extern "C" int fp8k_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors,
+                                          int64_t m, int64_t topk, int64_t cols, int64_t input_rows, int dtype, void* stream) {
+  clear_error();
+  const char* op = "apply_shuffle_mul_sum";
+  FP8K_REQUIRE(m >= 0 && topk >= 0 && cols >= 0 && input_rows >= 0 && topk <= 0x7fffffffLL, "%s: negative shape", op);
+  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "%s: bad dtype %d", op, dtype);
+  FP8K_REQUIRE(cols % 8 == 0 && cols <= 0x7fffffffLL, "%s: the row length (%lld) must be a multiple of 8", op, (long long)cols);
+  if (m == 0 || cols == 0) return FP8K_OK;
+  FP8K_REQUIRE(output && (topk == 0 || (input && permutation)), "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(input, 16) && aligned(output, 16), "%s: pointers must be 16-byte aligned", op);
+  const dim3 grid(stream_grid(m * (cols / 8))), block(256);
+  hipStream_t st = (hipStream_t)stream;
+#define FP8K_SMS(DT) \
+  hipLaunchKernelGGL(shuffle_mul_sum_kernel<DT>, grid, block, 0, st, input, output, permutation, factors, m, (int)topk, (int)cols, input_rows)
+  switch (dtype) {
+    case FP8K_BF16: FP8K_SMS(FP8K_BF16); break;
+    case FP8K_F16: FP8K_SMS(FP8K_F16); break;
+    default: FP8K_SMS(FP8K_F32); break;
+  }
+#undef FP8K_SMS
+  return check_launch(op);
+}
+
+extern "C" int fp8k_moe_blocks_from_offsets(const int32_t* expert_starts, const int32_t* problem_sizes, int64_t num_experts,
+                                            int64_t rows, int64_t block_m, int32_t* sorted_token_ids, int64_t sorted_capacity,
+                                            int32_t* expert_ids, int64_t expert_capacity, int32_t* num_tokens_post_pad,
+                                            void* stream) {
+  clear_error();
+  const char* op = "moe_blocks_from_offsets";
+  FP8K_REQUIRE(num_experts >= 1 && num_experts <= kAlignMaxBuckets, "%s: num_experts must be in [1, %d] (got %lld)", op,
+               kAlignMaxBuckets, (long long)num_experts);
+  FP8K_REQUIRE(rows >= 0 && rows < 0x7fffffffLL && block_m >= 1 && block_m <= 1024, "%s: bad rows / block size", op);
+  FP8K_REQUIRE(expert_starts && problem_sizes && sorted_token_ids && expert_ids && num_tokens_post_pad, "%s: null pointer", op);
+  // the kernel never writes past the capacities (blocks beyond them are dropped); sizes that sum to `rows` need at most this
+  const int64_t used = rows < num_experts ? rows : num_experts;
+  const int64_t worst = rows + used * (block_m - 1);
+  FP8K_REQUIRE(sorted_capacity >= worst / block_m * block_m && expert_capacity >= worst / block_m,
+               "%s: block table too small (%lld slots, %lld blocks; %lld slots may be needed)", op, (long long)sorted_capacity,
+               (long long)expert_capacity, (long long)(worst / block_m * block_m));
+  const int64_t max_blocks = sorted_capacity / block_m < expert_capacity ? sorted_capacity / block_m : expert_capacity;
+  hipLaunchKernelGGL(moe_offset_blocks_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, expert_starts,
+                     problem_sizes, (int)num_experts, (int)rows, (int)block_m, sorted_token_ids, expert_ids,
+                     num_tokens_post_pad, (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks));
+  return check_launch(op);
+}

@@ -73,6 +73,25 @@ def _bmm_impl(A, B, A_scale, B_scale, dtype, out) -> None:
 
 _register("bmm_fp8(Tensor A, Tensor B, Tensor A_scale, Tensor B_scale, ScalarType dtype, Tensor(a!) out) -> ()", _bmm_impl, _none)
 
+# ---- expert-major MoE layout (the CUTLASS-shaped path)
+_register(
+    "prepare_moe_input(Tensor topk_ids, Tensor(a!) expert_offsets, Tensor(b!)? blockscale_offsets, Tensor(c!) problem_sizes1, "
+    "Tensor(d!) problem_sizes2, Tensor(e!) input_permutation, Tensor(f!) output_permutation, int num_experts, int n, int k) -> ()",
+    lambda topk_ids, expert_offsets, blockscale_offsets, problem_sizes1, problem_sizes2, input_permutation, output_permutation,
+    num_experts, n, k: _k.prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, input_permutation,
+                                            output_permutation, num_experts, n, k, blockscale_offsets),
+    _none,
+)
+_register("shuffle_rows(Tensor input, Tensor dst2src_map, Tensor(a!) output) -> ()", _k.shuffle_rows_out, _none)
+_register("apply_shuffle_mul_sum(Tensor input, Tensor(a!) output, Tensor permutation, Tensor? factors) -> ()",
+          _k.apply_shuffle_mul_sum, _none)
+_register(
+    "fp8_blockwise_scaled_grouped_mm(Tensor(a!) output, Tensor a_ptrs, Tensor b_ptrs, Tensor out_ptrs, Tensor a_scales_ptrs, "
+    "Tensor b_scales_ptrs, Tensor a, Tensor b, Tensor scales_a, Tensor scales_b, Tensor stride_a, Tensor stride_b, "
+    "Tensor stride_c, Tensor layout_sfa, Tensor layout_sfb, Tensor problem_sizes, Tensor expert_offsets, Tensor workspace) -> ()",
+    _k.fp8_blockwise_scaled_grouped_mm, _none,
+)
+
 # ---- fused-MoE stages
 _register(
     "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor(a!) sorted_token_ids, "
@@ -162,6 +181,30 @@ def bmm_fp8(A, B, A_scale, B_scale, dtype, out: Optional[torch.Tensor] = None) -
         out = torch.empty((A.shape[0], A.shape[1], B.shape[2]), device=A.device, dtype=dtype)
     _ops.bmm_fp8(A, B, A_scale, B_scale, dtype, out)
     return out
+
+
+def prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, input_permutation, output_permutation,
+                      num_experts, n, k, blockscale_offsets: Optional[torch.Tensor] = None) -> None:
+    _ops.prepare_moe_input(topk_ids, expert_offsets, blockscale_offsets, problem_sizes1, problem_sizes2, input_permutation,
+                           output_permutation, num_experts, n, k)
+
+
+def shuffle_rows(input_tensor, dst2src_map, output_tensor_shape) -> torch.Tensor:
+    output_tensor = torch.empty(output_tensor_shape, device=input_tensor.device, dtype=input_tensor.dtype)
+    _ops.shuffle_rows(input_tensor, dst2src_map, output_tensor)
+    return output_tensor
+
+
+def apply_shuffle_mul_sum(input, output, permutation, factors) -> None:
+    _ops.apply_shuffle_mul_sum(input, output, permutation, factors)
+
+
+def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b,
+                                    stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes, expert_offsets,
+                                    workspace) -> None:
+    _ops.fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a,
+                                         scales_b, stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes,
+                                         expert_offsets, workspace)
 
 
 def moe_align_block_size(topk_ids, num_experts, block_size, sorted_token_ids, experts_ids, num_tokens_post_pad,

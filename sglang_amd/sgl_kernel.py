@@ -624,6 +624,128 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
     )
 
 
+def prepare_moe_input(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, input_permutation, output_permutation,
+                      num_experts, n, k, blockscale_offsets: Optional[torch.Tensor] = None) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:217-240 (csrc/moe/prepare_moe_input.cu).  Sorts the (token, k)
+    slots of topk_ids int32 [m, topk] by expert into contiguous row ranges: expert_offsets int32 [E + 1],
+    problem_sizes1 / 2 int32 [E, 3] = (rows, 2n, k) / (rows, k, n), input_permutation [m * topk] (row -> token),
+    output_permutation [m * topk] (slot -> row).  The order of the rows inside an expert is not defined."""
+    require_cuda(topk_ids, expert_offsets, problem_sizes1, problem_sizes2, input_permutation, output_permutation,
+                 blockscale_offsets)
+    if topk_ids.dtype != torch.int32 or topk_ids.dim() != 2 or not topk_ids.is_contiguous():
+        raise RuntimeError("prepare_moe_input: topk_ids must be contiguous int32 [m, topk]")
+    numel = topk_ids.numel()
+    for name, t, need in (("expert_offsets", expert_offsets, num_experts + 1), ("problem_sizes1", problem_sizes1, 3 * num_experts),
+                          ("problem_sizes2", problem_sizes2, 3 * num_experts), ("input_permutation", input_permutation, numel),
+                          ("output_permutation", output_permutation, numel), ("blockscale_offsets", blockscale_offsets, num_experts + 1)):
+        if t is None:
+            continue
+        if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < need:
+            raise RuntimeError("prepare_moe_input: %s must be contiguous int32 with at least %d entries" % (name, need))
+    check(lib.fp8k_moe_prepare_input(topk_ids.data_ptr(), numel, max(topk_ids.shape[1], 1), num_experts, n, k,
+                                     expert_offsets.data_ptr(), None if blockscale_offsets is None else blockscale_offsets.data_ptr(),
+                                     problem_sizes1.data_ptr(), problem_sizes2.data_ptr(), input_permutation.data_ptr(),
+                                     output_permutation.data_ptr(), stream_ptr(topk_ids.device)))
+
+
+def shuffle_rows_out(input_tensor: torch.Tensor, dst2src_map: torch.Tensor, output_tensor: torch.Tensor) -> None:
+    """output[d] = input[dst2src_map[d]] for 2-D contiguous tensors of one dtype (the op behind shuffle_rows)."""
+    require_cuda(input_tensor, dst2src_map, output_tensor)
+    if input_tensor.dtype != output_tensor.dtype:
+        raise RuntimeError("shuffle_rows: input and output tensors must have the same data type")
+    if input_tensor.dim() != 2 or output_tensor.dim() != 2 or input_tensor.shape[1] != output_tensor.shape[1]:
+        raise RuntimeError("shuffle_rows: 2-D tensors with the same row length expected")
+    if not (input_tensor.is_contiguous() and output_tensor.is_contiguous()):
+        raise RuntimeError("shuffle_rows: input and output must be contiguous")
+    if dst2src_map.dtype != torch.int32 or not dst2src_map.is_contiguous() or dst2src_map.numel() < output_tensor.shape[0]:
+        raise RuntimeError("shuffle_rows: dst2src_map must be contiguous int32 with one entry per output row")
+    check(lib.fp8k_shuffle_rows(input_tensor.data_ptr(), dst2src_map.data_ptr(), output_tensor.data_ptr(), input_tensor.shape[0],
+                                output_tensor.shape[0], input_tensor.shape[1] * input_tensor.element_size(),
+                                stream_ptr(input_tensor.device)))
+
+
+def shuffle_rows(input_tensor: torch.Tensor, dst2src_map: torch.Tensor, output_tensor_shape) -> torch.Tensor:
+    """Reference: sgl-kernel/python/sgl_kernel/gemm.py:302-309."""
+    output_tensor = torch.empty(output_tensor_shape, device=input_tensor.device, dtype=input_tensor.dtype)
+    shuffle_rows_out(input_tensor, dst2src_map, output_tensor)
+    return output_tensor
+
+
+def apply_shuffle_mul_sum(input: torch.Tensor, output: torch.Tensor, permutation: torch.Tensor,
+                          factors: Optional[torch.Tensor]) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:243-251:
+    output = (input[permutation].view(m, topk, k) * factors.view(m, topk, 1)).sum(dim=1), summed in float32."""
+    require_cuda(input, output, permutation, factors)
+    if input.dim() != 2 or output.dim() != 2 or permutation.dim() != 1:
+        raise RuntimeError("apply_shuffle_mul_sum: input [m * topk, k], output [m, k], permutation [m * topk]")
+    if input.dtype != output.dtype or not (input.is_contiguous() and output.is_contiguous()) or input.shape[1] != output.shape[1]:
+        raise RuntimeError("apply_shuffle_mul_sum: input and output must be contiguous, of one dtype and row length")
+    m = output.shape[0]
+    topk = permutation.numel() // m if m else 0
+    if permutation.numel() != m * topk or permutation.dtype != torch.int32 or not permutation.is_contiguous():
+        raise RuntimeError("apply_shuffle_mul_sum: permutation size must match m * topk (contiguous int32)")
+    if factors is not None:
+        if factors.dtype != output.dtype:
+            raise RuntimeError("apply_shuffle_mul_sum: factors must match output dtype")
+        if factors.numel() != m * topk or not factors.is_contiguous():
+            raise RuntimeError("apply_shuffle_mul_sum: factors must have shape [m * topk]")
+    check(lib.fp8k_apply_shuffle_mul_sum(input.data_ptr(), output.data_ptr(), permutation.data_ptr(),
+                                         None if factors is None else factors.data_ptr(), m, topk, output.shape[1], input.shape[0],
+                                         dtype_code(output.dtype), stream_ptr(output.device)))
+
+
+def _expert_major_block_m(rows: int, num_experts: int) -> int:
+    """Slots per block of the grouped GEMM from the mean rows per expert; the thresholds are the measured ones of
+    fused_moe.get_default_config."""
+    per_expert = (rows + num_experts - 1) // max(num_experts, 1)
+    for limit, bm in ((4, 16), (22, 32), (48, 64), (96, 128)):
+        if per_expert <= limit:
+            return bm
+    return 256
+
+
+def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b,
+                                    stride_a, stride_b, stride_c, layout_sfa, layout_sfb, problem_sizes, expert_offsets,
+                                    workspace) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:175-214 (csrc/moe/fp8_blockwise_moe_kernel.cu).  For every expert e:
+    output[rows_e] = a[rows_e] @ b[e] with 1x128 scales on a and 128x128 scales on b, rows_e = expert_offsets[e] ..
+    + problem_sizes[e, 0].  a e4m3fn [rows, K]; b e4m3fn [E, K, N] column-major per expert (a [E, N, K] weight
+    transposed); scales_a float32 [rows, K/128]; scales_b float32 [E, K/128, N/128] (the [E, N/128, K/128] checkpoint
+    tensor transposed) or [E, N/128, K/128] contiguous; output bf16 / fp16 [rows, N].  The pointer arrays, stride
+    vectors, scale-layout buffers and the workspace serve the reference's CUTLASS launcher and are ignored here:
+    the grouped kernel takes a block table built on the device from expert_offsets and problem_sizes."""
+    require_cuda(output, a, b, scales_a, scales_b, problem_sizes, expert_offsets)
+    if a.dim() != 2 or b.dim() != 3 or output.dim() != 2:
+        raise RuntimeError("fp8_blockwise_scaled_grouped_mm: a [rows, K], b [E, K, N], output [rows, N]")
+    E, K, N = b.shape
+    if b.stride(1) != 1 and K > 1:
+        raise RuntimeError("fp8_blockwise_scaled_grouped_mm: b must be column-major per expert (K contiguous)")
+    kb, nb = (K + 127) // 128, (N + 127) // 128
+    if scales_b.dim() != 3 or scales_b.shape[0] != E:
+        raise RuntimeError("fp8_blockwise_scaled_grouped_mm: scales_b must be [E, K/128, N/128]")
+    if tuple(scales_b.shape[1:]) == (kb, nb) and (scales_b.stride(1) == 1 or kb == 1):
+        bs = scales_b.transpose(1, 2)
+    elif tuple(scales_b.shape[1:]) == (nb, kb) and (scales_b.stride(2) == 1 or kb == 1):
+        bs = scales_b
+    else:
+        raise RuntimeError("fp8_blockwise_scaled_grouped_mm: scales_b must be the [E, N/128, K/128] tensor or its transpose")
+    if problem_sizes.dtype != torch.int32 or problem_sizes.shape != (E, 3) or not problem_sizes.is_contiguous():
+        raise RuntimeError("fp8_blockwise_scaled_grouped_mm: problem_sizes must be contiguous int32 [E, 3]")
+    if expert_offsets.dtype != torch.int32 or expert_offsets.numel() < E or not expert_offsets.is_contiguous():
+        raise RuntimeError("fp8_blockwise_scaled_grouped_mm: expert_offsets must be contiguous int32 with E entries")
+    rows = a.shape[0]
+    if rows == 0:
+        return
+    block_m = _expert_major_block_m(rows, E)
+    cap = (rows + min(rows, E) * (block_m - 1)) // block_m * block_m
+    table = torch.empty((cap + cap // block_m + 1,), device=a.device, dtype=torch.int32)
+    sorted_ids, expert_ids, post_pad = table[:cap], table[cap:cap + cap // block_m], table[cap + cap // block_m:]
+    check(lib.fp8k_moe_blocks_from_offsets(expert_offsets.data_ptr(), problem_sizes.data_ptr(), E, rows, block_m,
+                                           sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), cap // block_m, post_pad.data_ptr(),
+                                           stream_ptr(a.device)))
+    moe_block_gemm(a, b.transpose(1, 2), output, scales_a, bs, None, sorted_ids, expert_ids, post_pad, False, 1, block_m, rows)
+
+
 def moe_fused_gate(
     input_tensor: torch.Tensor,
     bias: torch.Tensor,

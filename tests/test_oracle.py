@@ -527,3 +527,79 @@ def test_bmm_fp8_against_torch_bmm_and_brute_force():
                 brute[i, r, c] = sum(a_f[i, r, t] * b_f[i, c, t] for t in range(k)) * float(sa) * float(sb)
     assert np.allclose(got, brute, rtol=1e-6, atol=0)
     assert np.array_equal(O.bmm_fp8(aq, bq, sa, sb, "bf16"), O.to_bf16(got))
+
+
+def test_prepare_moe_input_against_stable_argsort_and_bincount():
+    """The expert-major sort restated with numpy library routines: bincount for the row counts, a stable argsort for
+    the order; c_map must invert a_map's placement, and ids outside [0, E) take no row."""
+    rng = np.random.default_rng(4)
+    m, topk, E, n, k = 37, 4, 9, 256, 384
+    ids = rng.integers(0, E, (m, topk)).astype(np.int32)
+    ids[5, 2] = -1
+    ids[6, 0] = E
+    off, bso, ps1, ps2, a_map, c_map = O.prepare_moe_input(ids, E, n, k)
+    flat = ids.reshape(-1)
+    valid = (flat >= 0) & (flat < E)
+    counts = np.bincount(flat[valid], minlength=E)
+    assert np.array_equal(off, np.concatenate([[0], np.cumsum(counts)]))
+    assert np.array_equal(bso, np.concatenate([[0], np.cumsum((counts + 127) // 128 * 128)]))
+    assert np.array_equal(ps1, np.stack([counts, np.full(E, 2 * n), np.full(E, k)], 1))
+    assert np.array_equal(ps2, np.stack([counts, np.full(E, k), np.full(E, n)], 1))
+    order = np.argsort(np.where(valid, flat, E), kind="stable")[: valid.sum()]  # slots by expert, ties in slot order
+    assert np.array_equal(a_map[: valid.sum()], order // topk)
+    assert np.array_equal(c_map[order], np.arange(valid.sum()))
+
+
+def test_apply_shuffle_mul_sum_against_the_torch_expression():
+    """The reference documents the op as (c2[c_map].view(m, topk, k) * topk_weights.view(m, topk, 1)).sum(dim=1)
+    (prepare_moe_input.cu:369-386), computed in float32 and rounded once: in float64 here, one bf16 ulp of slack."""
+    g = torch.Generator().manual_seed(8)
+    m, topk, k = 13, 6, 40
+    c2 = torch.randn(m * topk, k, generator=g).to(torch.bfloat16)
+    w = torch.rand(m, topk, generator=g).to(torch.bfloat16)
+    c_map = torch.randperm(m * topk, generator=g)
+    ref = (c2.double()[c_map].view(m, topk, k) * w.double().view(m, topk, 1)).sum(dim=1)
+    got = O.apply_shuffle_mul_sum(c2.float().numpy(), c_map.view(m, topk).numpy(), w.float().numpy(), "bf16")
+    assert np.array_equal(got, O.to_bf16(got))
+    err = np.abs(got - ref.numpy())
+    assert (err <= np.abs(ref.numpy()) * 2.0 ** -8 + 1e-30).all()
+    # no factors: a plain gather-sum, exact in float32 for small integers
+    ints = torch.randint(-8, 8, (m * topk, k), generator=g).float()
+    got2 = O.apply_shuffle_mul_sum(ints.numpy(), c_map.view(m, topk).numpy(), None, "f32")
+    assert np.array_equal(got2, ints[c_map].view(m, topk, k).sum(1).numpy())
+
+
+def test_grouped_mm_and_cutlass_composite():
+    """The grouped GEMM against torch.mm of the de-quantised operands per expert (the check of sgl-kernel/tests/
+    test_fp8_blockwise_moe.py:66-91), and the expert-major fused experts against the Triton-ordered composite: the
+    same mathematics with the routed weight applied at a different rounding point."""
+    rng = np.random.default_rng(6)
+    E, N, K = 3, 256, 384
+    sizes = [5, 0, 9]
+    rows = sum(sizes)
+    aq = rng.integers(0, 0x60, (rows, K), dtype=np.uint8) | (rng.integers(0, 2, (rows, K), dtype=np.uint8) << 7)
+    bq = rng.integers(0, 0x60, (E, N, K), dtype=np.uint8) | (rng.integers(0, 2, (E, N, K), dtype=np.uint8) << 7)
+    a_s = rng.uniform(0.5, 2.0, (rows, K // 128)).astype(np.float32) * 1e-2
+    b_s = rng.uniform(0.5, 2.0, (E, N // 128, K // 128)).astype(np.float32) * 1e-2
+    off = np.concatenate([[0], np.cumsum(sizes)]).astype(np.int32)
+    ps = np.array([[c, N, K] for c in sizes], dtype=np.int32)
+    got = O.fp8_blockwise_scaled_grouped_mm(aq, bq, a_s, b_s, off, ps, "f32", acc=np.float64)
+    A = torch.from_numpy(aq).view(torch.float8_e4m3fn).double() * torch.from_numpy(a_s).double().repeat_interleave(128, 1)
+    for e in range(E):
+        B = torch.from_numpy(bq[e]).view(torch.float8_e4m3fn).double() * \
+            torch.from_numpy(b_s[e]).double().repeat_interleave(128, 0).repeat_interleave(128, 1)
+        ref = torch.mm(A[off[e]:off[e + 1]], B.t()).numpy()
+        assert np.allclose(got[off[e]:off[e + 1]], ref, rtol=1e-5, atol=1e-7)
+
+    T, E, H, I, topk = 24, 6, 256, 128, 2
+    x = O.make_activation(T, H, 3)
+    w13q = np.empty((E, 2 * I, H), np.uint8); w13s = np.empty((E, 2 * I // 128, H // 128), np.float32)
+    w2q = np.empty((E, H, I), np.uint8); w2s = np.empty((E, H // 128, I // 128), np.float32)
+    for e in range(E):
+        w13q[e], w13s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((2 * I, H)).astype(np.float32) * 0.05))
+        w2q[e], w2s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((H, I)).astype(np.float32) * 0.05))
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    tw = O.to_bf16(rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32))
+    a = O.cutlass_fused_experts_fp8(x, w13q, w13s, w2q, w2s, tw, ids)
+    b = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0)
+    assert np.abs(a - b).max() <= 2e-2 * np.abs(b).max()
