@@ -15,6 +15,7 @@ namespace fp8k {
 // ---------------------------------------------------------------- host: errors
 int fail(int code, const char* fmt, ...);
 void clear_error();
+int num_cu();  // compute units of the current device (256 when no device is visible)
 
 #define FP8K_REQUIRE(cond, ...)                                   \
   do {                                                            \

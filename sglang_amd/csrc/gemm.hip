@@ -20,26 +20,6 @@ struct Plan {
   int64_t ws_bytes; // float workspace the plan needs
 };
 
-// Compute units of the current device, read once per device (a read-only cache; 256 on MI355X, which is also the
-// answer when no device is visible, so that the workspace queries work on a machine without a GPU).
-static int num_cu() {
-  constexpr int kMaxDev = 64;
-  static std::atomic<int> cache[kMaxDev];
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDev) {
-    (void)hipGetLastError();
-    return 256;
-  }
-  int n = cache[dev].load(std::memory_order_relaxed);
-  if (n > 0) return n;
-  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) {
-    (void)hipGetLastError();
-    n = 256;
-  }
-  cache[dev].store(n, std::memory_order_relaxed);
-  return n;
-}
-
 // tuning aid: force the kernel family (and the K split of the uniform-split families) of later calls made by the
 // calling thread; other threads keep the automatic choice
 static thread_local int g_force_kind = -1, g_force_splits = 0;
@@ -356,8 +336,8 @@ static int block_gemm_impl(const void* A, const void* B, const float* As, const 
   FP8K_REQUIRE(As && Bs, "fp8_blockwise_scaled_mm: null scale pointer");
   FP8K_REQUIRE(as_stride_m >= 0 && as_stride_k >= 0 && bs_stride_n >= 0 && bs_stride_k >= 0,
                "fp8_blockwise_scaled_mm: negative scale stride");
-  FP8K_REQUIRE((M - 1) * as_stride_m + ((K + kTileK - 1) / kTileK - 1) * as_stride_k < (1LL << 31),
-               "fp8_blockwise_scaled_mm: scales_a spans more than 2^31 elements");
+  FP8K_REQUIRE((M - 1) * as_stride_m + ((K + kTileK - 1) / kTileK - 1) * as_stride_k < 0x38000000LL,
+               "fp8_blockwise_scaled_mm: scales_a spans more than 3.5 GiB");
   const Plan pl = make_plan(M, N, K);
   const int64_t kb = (K + kTileK - 1) / kTileK;
   const int64_t need = wants_scale_copy(pl, M) ? align256(pl.ws_bytes) + M * kb * 4 : pl.ws_bytes;

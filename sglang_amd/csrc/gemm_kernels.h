@@ -125,6 +125,10 @@ __device__ __forceinline__ rsrc_t make_rsrc(const void* p, uint32_t bytes) {
 __device__ __forceinline__ void buf_load16_to_lds(rsrc_t r, uint32_t voff, uint32_t soff, uint8_t* lds_base) {
   __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)lds_base, 16, (int)voff, (int)soff, 0, 0);
 }
+// 4 bytes per lane into LDS at lds_base + lane*4 (inactive lanes write nothing)
+__device__ __forceinline__ void buf_load4_to_lds(rsrc_t r, uint32_t voff, uint32_t soff, uint8_t* lds_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(r, (lds_ptr_t)lds_base, 4, (int)voff, (int)soff, 0, 0);
+}
 __device__ __forceinline__ void wait_vm0_lgkm0() { __builtin_amdgcn_s_waitcnt(0x0070); }  // vmcnt(0) lgkmcnt(0)
 
 // Workgroup barrier that orders LDS traffic only.  __syncthreads() carries a release fence, and on this family
@@ -623,10 +627,11 @@ struct MoeItem {
   int tile_n;
   int expert;
 };
-__device__ __forceinline__ MoeItem moe_work_item(const GemmArgs& p, int bid) {
+// blocks in use (a device-side count: the host sizes the grid for the worst case)
+__device__ __forceinline__ int moe_blocks_used(const GemmArgs& p) { return min(p.num_post_pad[0] / p.block_m, p.m_blocks); }
+__device__ __forceinline__ MoeItem moe_work_item(const GemmArgs& p, int bid, int used) {
   constexpr int kWin = 4;
   MoeItem it{-1, 0, -1};
-  const int used = min(p.num_post_pad[0] / p.block_m, p.m_blocks);
   const int per_xcd = (used + 7) >> 3;
   const int j = bid >> 3;
   const int pos = j / p.tiles_n;                      // block position inside the XCD's run, before regrouping
@@ -653,6 +658,7 @@ __device__ __forceinline__ MoeItem moe_work_item(const GemmArgs& p, int bid) {
   it.expert = ex;
   return it;
 }
+__device__ __forceinline__ MoeItem moe_work_item(const GemmArgs& p, int bid) { return moe_work_item(p, bid, moe_blocks_used(p)); }
 
 // ------------------------------------------------------------------------------------------------
 // Weight-streaming kernel for 33..128 activation rows: 256(n) x TM(m) x 128(k) tile, TM in {64, 128}.
@@ -675,7 +681,9 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   constexpr int XL = (XG + NW - 1) / NW;         // X wave-loads per wave per stage
   constexpr int LPW = WL + XL;                   // LDS-DMA loads per wave per stage
   constexpr int WBYTES = kTileN * kTileK;
-  constexpr int STAGE = WBYTES + TM * kTileK;
+  // block mode: the scales of a K block travel with its stage (TM activation scales, then one weight scale per wave)
+  constexpr int SOFF = WBYTES + TM * kTileK;
+  constexpr int STAGE = SOFF + (MODE == kModeBlock ? 1024 : 0);
   __shared__ __attribute__((aligned(1024))) uint8_t smem[NSTAGE * STAGE + 1024];
   uint8_t* const dummy = smem + NSTAGE * STAGE;  // landing zone of padding loads
 
@@ -767,7 +775,21 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
     for (int j = 0; j < XL; ++j)
       buf_load16_to_lds(rX, voX[j] + ko, 0, xload[j] ? base + WBYTES + (w * XL + j) * 1024 : dummy);
   };
-  auto issue = [&](int kstep) { issue_w(kstep); issue_x(kstep); };
+  // Scales (block mode) go through the stage as well: two 4-byte LDS loads per wave and K block - lanes 0..TM/NW-1
+  // fetch the activation scales of the wave's share of the rows, lane 0 the wave's weight scale.  As part of the
+  // stage they are covered by the stage's wait; held in registers across trips instead, the compiler's copies
+  // between the trips wait for loads of the running trip, and with loads returning in order that drains the
+  // stage requested before them.
+  constexpr int SR = TM / NW;  // activation scale rows per wave
+  rsrc_t rSx, rSw;
+  uint32_t voS = 0xF0000000u;
+  auto issue_s = [&](int kstep) {
+    if (MODE != kModeBlock) return;
+    uint8_t* base = smem + (kstep % NSTAGE) * STAGE + SOFF;
+    if (lane < SR) buf_load4_to_lds(rSx, voS, (uint32_t)kstep * (uint32_t)(p.sx_k * 4), base + w * (SR * 4));
+    if (lane == 0) buf_load4_to_lds(rSw, 0u, (uint32_t)kstep * (uint32_t)(p.sw_k * 4), base + TM * 4 + w * 4);
+  };
+  auto issue = [&](int kstep) { issue_s(kstep); issue_w(kstep); issue_x(kstep); };
   // Grouped: the slot table is fetched first and the weights of the first stages behind it (loads retire in order:
   // the table arrives without waiting for the weights, and the weights do not wait for the table).
   int sid[XL];
@@ -813,15 +835,22 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   };
 
   // ---- scales (block mode): activation scale rows follow the activation rows
-  const float* sxp[MS];
-#pragma unroll
-  for (int ms = 0; ms < MS; ++ms) {
-    int64_t xr = out_ok[ms] ? (MOE ? out_slot[ms] / p.top_k : out_slot[ms]) : 0;
-    if (MOE && p.sx_sorted) xr = slot0 + mrow0 + ms * 32 + lr;
-    sxp[ms] = p.sx + xr * p.sx_m + (int64_t)kb_begin * p.sx_k;
+  if (MODE == kModeBlock) {
+    const int row = w * SR + lane;  // the lane's row of the block (lanes 0..SR-1)
+    int64_t xr = -1;
+    if (lane < SR && row < block_m) {
+      const int s = MOE ? p.sorted_ids[slot0 + row] : slot0 + row;
+      if (s < nrows) xr = (MOE && p.sx_sorted) ? slot0 + row : (MOE ? s / p.top_k : s);
+    }
+    const int64_t srows = (MOE && p.sx_sorted) ? (int64_t)p.m_blocks * block_m : xrows;
+    const int kb_all = p.K / kTileK;
+    // rows past the range (padding) read zeros; the host keeps the tensor below the marker offset
+    rSx = make_rsrc(p.sx + (int64_t)kb_begin * p.sx_k, (uint32_t)(((srows - 1) * p.sx_m + (int64_t)(kb_all - 1 - kb_begin) * p.sx_k + 1) * 4));
+    voS = xr >= 0 ? (uint32_t)(xr * p.sx_m * 4) : 0xF0000000u;
+    const int nb = min(n0 + wn * 32, p.N - 1) >> 7;
+    const float* swp = p.sw + (MOE ? (int64_t)expert * p.sw_expert_stride : 0) + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
+    rSw = make_rsrc(swp, (uint32_t)(((int64_t)(kb_all - 1 - kb_begin) * p.sw_k + 1) * 4));
   }
-  const int nb = min(n0 + wn * 32, p.N - 1) >> 7;
-  const float* swp = p.sw + (MOE ? (int64_t)expert * p.sw_expert_stride : 0) + (int64_t)nb * p.sw_n + (int64_t)kb_begin * p.sw_k;
 
   v16f acc[MS];
 #pragma unroll
@@ -831,42 +860,29 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
 
 #pragma unroll
   for (int s = 0; s < NSTAGE - 1; ++s) {
-    if (MOE) issue_x(s);  // the weights of these stages are on their way already
+    if (MOE) { issue_s(s); issue_x(s); }  // the weights of these stages are on their way already
     else issue(s);
   }
-  // Scales travel two K blocks ahead, and the loads of block it+2 are issued BEFORE the stage loads of the same
-  // trip: memory operations retire in order, so a scale that is younger than a stage load could only be waited
-  // for by draining that stage load too, which would serialise the whole pipeline on HBM latency.
-  constexpr int SL = MODE == kModeBlock ? MS + 1 : 0;  // scale loads per trip
-  float sxa[MS], sxb[MS], sba = 0.f, sbb = 0.f;         // scales of the even / odd K blocks in flight
-  auto load_scales = [&](float (&sx)[MS], float& sb, int kb) {
-    const int kn = min(kb, nkb - 1);
-#pragma unroll
-    for (int ms = 0; ms < MS; ++ms) sx[ms] = sxp[ms][(int64_t)kn * p.sx_k];
-    sb = swp[(int64_t)kn * p.sw_k];
-  };
-  if (MODE == kModeBlock && nkb > 0) {
-    load_scales(sxa, sba, 0);
-    load_scales(sxb, sbb, 1);
-  }
+  constexpr int SL = MODE == kModeBlock ? 2 : 0;  // scale loads per wave and trip
   if (MOE) wait_vm0();  // the grouped prologue issues its loads in another order than the trips' partial waits assume
 
-  // one K block; (sx, sb) hold its scales on entry and are reloaded with those of block it+2
-  auto trip = [&](auto na, int it, float (&sx)[MS], float& sb) {
+  // one K block
+  auto trip = [&](auto na, int it) {
     constexpr int NA = decltype(na)::value;  // 32-row groups of the wave that hold real rows (grouped form)
     // stage `it` has landed once at most NSTAGE-2 younger trips (stage + scale loads each) are still in flight
     constexpr int kInFlight = (NSTAGE - 2) * (LPW + SL);
     lds_barrier<kInFlight>();
-    float sc[MS];
-    if (MODE == kModeBlock) {
-#pragma unroll
-      for (int ms = 0; ms < MS; ++ms) sc[ms] = sx[ms] * sb;
-      load_scales(sx, sb, it + 2);
-      __builtin_amdgcn_sched_barrier(0);  // keep the scale loads ahead of the stage loads
-    }
+    __builtin_amdgcn_sched_barrier(0);  // nothing of this trip in front of the barrier
     issue(it + NSTAGE - 1);  // refills the stage every wave finished before this barrier
     if (NA == 0) return;
     const uint8_t* st = smem + (it % NSTAGE) * STAGE;
+    float sc[MS];
+    if (MODE == kModeBlock) {
+      const float* ss = reinterpret_cast<const float*>(st + SOFF);
+      const float sb = ss[TM + w];
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms) sc[ms] = ss[mrow0 + ms * 32 + lr] * sb;
+    }
     v8i wf[2];
     wf[0] = frag(st, rdW, 0);
     wf[1] = frag(st, rdW, 1);
@@ -891,10 +907,10 @@ __global__ __launch_bounds__(NW * 64, 1) void gemm_stream_kernel(const GemmArgs 
   auto run = [&](auto na) {
     int it = 0;
     for (; it + 1 < nkb; it += 2) {
-      trip(na, it, sxa, sba);
-      trip(na, it + 1, sxb, sbb);
+      trip(na, it);
+      trip(na, it + 1);
     }
-    if (it < nkb) trip(na, it, sxa, sba);
+    if (it < nkb) trip(na, it);
   };
   // Grouped form: the 32-row groups past an expert's last slot are padding (real slots come first in a block) and
   // skip their MFMAs; one straight-line copy of the loop per group count.

@@ -1,4 +1,4 @@
-// Grouped (MoE) block-FP8 GEMM for experts with 129..256 token slots: 256(n) x 256(m) x 128(k) tile,
+// Grouped (MoE) block-FP8 GEMM for experts with about a hundred and more token slots: 256(n) x 256(m) x 128(k) tile,
 // 8 wavefronts, weights streamed three K blocks deep.
 //
 // With a few hundred token slots per expert the grouped GEMM is bound by streaming each expert's weights
@@ -8,8 +8,12 @@
 // the streaming kernel's depth on the weights and pairs both 128-row halves on one weight stage:
 //   LDS = 3 weight stages (32 KB each) + 2 activation stages (32 KB each) = 160 KB, the whole CU.
 //   Activation tiles are re-read by every n tile of the block and come from L2; one stage ahead is enough.
-//   Waves: 4 along n (64 weight rows) x 2 along m (128 slots), 2 x 4 MFMA tiles of 32x32 each (24 KB of LDS
-//   operands per 16 MFMAs); 32-slot groups without real slots skip their MFMAs.
+//   Waves: 4 along n (64 weight rows) x 2 along m; the 32-slot groups of a block alternate between the two wave rows
+//   (groups wm, wm + 2, wm + 4, wm + 6), so that a block that is half padding still loads both rows of waves evenly;
+//   2 x 4 MFMA tiles of 32x32 each (24 KB of LDS operands per 16 MFMAs); groups without real slots skip their MFMAs.
+//   A workgroup can walk several items: the two stage rings run on across items, the last two trips of an item
+//   request the first two weight blocks of the next one, and the item is written out through the stages its last
+//   block used while the next item's first blocks travel.
 // Load order inside a K block is scales, activations, weights, so that at the next barrier only the four
 // youngest weight loads of each wave may still be in flight (memory operations retire in order).
 #pragma once
@@ -31,275 +35,349 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   constexpr int XBASE = WST * WBYTES;
   __shared__ __attribute__((aligned(1024))) uint8_t smem[WST * WBYTES + XST * XBYTES];
 
-  const int lane = threadIdx.x & 63;
   const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int wn = w & 3, wm = w >> 2;
-
-  // ---- work item (moe_work_item(): contiguous run of blocks per XCD, same-expert blocks of a window grouped)
-  const MoeItem item = moe_work_item(p, (int)blockIdx.x);
-  if (item.mb < 0) return;
-  const int mb = item.mb, tile_n = item.tile_n, expert = item.expert;
-  const int n0 = tile_n * kTileN;
-  const int slot0 = mb * TM;
   const int nrows = p.num_valid;
+  const int nkb = p.K / kTileK;
 
-  const int lr = lane & 31, h = lane >> 5;
-  if (expert < 0) {  // expert on another rank: the reference writes zeros
+  // ---- work items.  One workgroup per CU walks the items of its XCD (workgroup ids are dealt round-robin to the
+  // XCDs): item index j of XCD x is what workgroup 8 j + x of a one-item-per-workgroup launch would take
+  // (moe_work_item(): contiguous run of blocks per XCD, same-expert blocks of a window grouped), and the CUs of an
+  // XCD take consecutive j, so the tiles that run together share an expert's activation rows.  Items past the
+  // last block are empty, and so are all after them.
+  const int xcd = (int)blockIdx.x & 7, jstep = (int)gridDim.x >> 3;
+  int j = (int)blockIdx.x >> 3;
+  // an expert of another rank: the reference writes zeros; done here on the spot, and the walk goes on
+  auto zero_fill = [&](const MoeItem& it) {
+    const int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    const int lr = ln & 31, h = ln >> 5;
     for (int ms = 0; ms < MS; ++ms) {
-      const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
+      const int s = p.sorted_ids[it.mb * TM + wm * 128 + ms * 32 + lr];
       if (s >= nrows) continue;
       for (int q = 0; q < 4; ++q) {
         for (int ns = 0; ns < NS; ++ns) {
-          const int n = n0 + wn * 64 + ns * 32 + h * 16 + q * 4;
+          const int n = it.tile_n * kTileN + wn * 64 + ns * 32 + h * 16 + q * 4;
           if (n < p.N) store4<OUT_DT>(p.C, (int64_t)s * p.ldc + n, 0.f, 0.f, 0.f, 0.f);
         }
       }
     }
-    return;
-  }
-  // ---- global -> LDS: a wave load covers 8 rows (lane: row lane/8, 16-byte chunk lane%8, stored at chunk
-  // position c ^ ((row>>1)&7)); whole offsets travel in the bounds-checked per-lane operand
-  const uint8_t* Wb = p.W + (int64_t)expert * p.w_expert_stride;
-  const int rowsW = min(kTileN, p.N - n0);
-  const rsrc_t rW = make_rsrc(Wb + (int64_t)n0 * p.ldw, (uint32_t)((rowsW - 1) * p.ldw + p.K));
+  };
+  auto fetch_item = [&](int& jj) -> MoeItem {  // first item at or after jj that has a GEMM to do (or the end)
+    for (;;) {
+      const MoeItem it = moe_work_item(p, jj * 8 + xcd);
+      if (it.mb < 0 || it.expert >= 0) return it;
+      zero_fill(it);
+      jj += jstep;
+    }
+  };
+  MoeItem item = fetch_item(j);
+  if (item.mb < 0) return;
+
   const int64_t xrows = (int64_t)((p.num_valid + p.top_k - 1) / p.top_k);
   const rsrc_t rX = make_rsrc(p.X, (uint32_t)((xrows - 1) * p.ldx + p.K));
-  const int rl = lane >> 3, cp = lane & 7;
-  // the wave's 8-row groups g = 4w + q: groups q and q + 2 differ by 16 rows and share the chunk swizzle, so two
-  // lane offsets serve the four weight loads (the 16-row step is uniform and joins the K offset)
-  uint32_t voW[2], voX[LW];
+  const rsrc_t rS = make_rsrc(p.sx, (uint32_t)(((xrows - 1) * p.sx_m + nkb) * 4));  // used by the paired loads only
+  // through a buffer descriptor: a 32-bit lane offset and a uniform offset, no 64-bit address per lane and group
+  const rsrc_t rSall = make_rsrc(p.sx, 0xFFFFFFFFu);
+
+  // ---- global -> LDS: a wave load covers 8 rows (lane: row lane/8, 16-byte chunk lane%8, stored at chunk
+  // position c ^ ((row>>1)&7)); whole offsets travel in the bounds-checked per-lane operand
+  rsrc_t rW, rWn;  // weights of the item in work / of the item after it
+  uint32_t voW[2], voX[LW], w16;
+  int slot0 = 0, n0 = 0, expert = 0;
+  // The stages are two rings that run on across the items of a walk: block k of an item sits in weight stage
+  // (gw0 + k) % 3 and activation stage (gx0 + k) & 1, the next item's block 0 in the stage after its last block.
+  int gw0 = 0, gx0 = 0;
+  auto issue_w = [&](const rsrc_t& r, int kblk, int stage) {
+    uint8_t* base = smem + stage * WBYTES + w * (LW * 1024);
+    const uint32_t ko = (uint32_t)kblk * kTileK;
 #pragma unroll
-  for (int q = 0; q < 2; ++q) {
-    const int g = w * LW + q;  // 8-row group, 0..31, of both tiles
-    const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
-    voW[q] = (uint32_t)((g * 8 + rl) * p.ldw + c * 16);
-  }
-  const uint32_t w16 = (uint32_t)(16 * p.ldw);
-  auto issue_w = [&](int kstep) {
-    uint8_t* base = smem + (kstep % WST) * WBYTES + w * (LW * 1024);
-    const uint32_t ko = (uint32_t)kstep * kTileK;
-#pragma unroll
-    for (int q = 0; q < LW; ++q) buf_load16_to_lds(rW, voW[q & 1] + (ko + (q >> 1) * w16), 0, base + q * 1024);
+    for (int q = 0; q < LW; ++q) buf_load16_to_lds(r, voW[q & 1] + (ko + (q >> 1) * w16), 0, base + q * 1024);
   };
-  // slot table first, weights behind it: loads retire in order, so the table arrives without waiting for the
-  // weights, and the weights do not wait for the table
-  int sid[LW];
-#pragma unroll
-  for (int q = 0; q < LW; ++q) sid[q] = p.sorted_ids[slot0 + (w * LW + q) * 8 + rl];
-  __builtin_amdgcn_sched_barrier(0);
-  issue_w(0);
-  issue_w(1);
-  __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int q = 0; q < LW; ++q) {
-    const int g = w * LW + q;
-    const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
-    const int s = sid[q];
-    voX[q] = s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
-  }
-  auto issue_x = [&](int kstep) {
-    uint8_t* base = smem + XBASE + (kstep & 1) * XBYTES + w * (LW * 1024);
-    const uint32_t ko = (uint32_t)kstep * kTileK;
+  auto issue_x = [&](int kblk, int stage) {
+    uint8_t* base = smem + XBASE + stage * XBYTES + w * (LW * 1024);
+    const uint32_t ko = (uint32_t)kblk * kTileK;
 #pragma unroll
     for (int q = 0; q < LW; ++q) buf_load16_to_lds(rX, voX[q] + ko, 0, base + q * 1024);
   };
-
-  // ---- LDS -> MFMA operands
-  const int swz = (lr >> 1) & 7;
-  // lane part of an operand fetch address (row lr of a 32-row group, swizzled 16-byte chunk); stage, wave position
-  // and group are uniform, so weights and activations share these four registers
-  uint32_t fa[2][2];
-#pragma unroll
-  for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-    for (int q = 0; q < 2; ++q) fa[ks][q] = (uint32_t)(lr * kTileK + (((ks * 4 + h * 2 + q) ^ swz) << 4));
-  auto frag = [&](const uint8_t* grp, int ks) -> v8i {  // grp: first row of the 32-row group inside its stage (uniform)
-    const v4i lo = *reinterpret_cast<const v4i*>(grp + fa[ks][0]);
-    const v4i hi = *reinterpret_cast<const v4i*>(grp + fa[ks][1]);
-    v8i r;
-    r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
-    r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
-    return r;
+  auto weights_of = [&](const MoeItem& it) -> rsrc_t {
+    if (it.mb < 0) return make_rsrc(p.W, 0u);  // no item: every load is out of range and moves nothing
+    const uint8_t* Wb = p.W + (int64_t)it.expert * p.w_expert_stride;
+    const int nn = it.tile_n * kTileN;
+    const int rowsW = min(kTileN, p.N - nn);
+    return make_rsrc(Wb + (int64_t)nn * p.ldw, (uint32_t)((rowsW - 1) * p.ldw + p.K));
   };
-
-  // ---- scales: activation scale rows follow the activation rows
-  uint32_t sxo[MS];  // element offsets into the activation scales (the host checks they fit 32 bits)
-  int nact = 0;      // 32-slot groups of the wave's half that hold real slots (a prefix: real slots come first)
+  // Entering an item: its activation block 0 goes into its first activation stage (the weights of its blocks 0 and 1
+  // were requested in the last two trips of the item before it, or below for a workgroup's first item).  For every
+  // item but the first this runs in front of the previous item's write-out, which keeps to the weight and
+  // activation stages that item used last - the ones no request in flight points at.  The lane id is taken anew
+  // (from the execution mask): lane-derived values that stayed live across the K loops would be parked in scratch
+  // and reloaded inside them, and scratch reloads count against the partial vmcnt waits.
+  auto start_item = [&](const MoeItem& it, bool first) {
+    int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(ln));
+    const int rl = ln >> 3, cp = ln & 7;
+    slot0 = it.mb * TM;
+    n0 = it.tile_n * kTileN;
+    expert = it.expert;
+    // slot table first, weights behind it: loads retire in order, so the table arrives without waiting for the
+    // weights, and the weights do not wait for the table
+    int sid[LW];
 #pragma unroll
-  for (int ms = 0; ms < MS; ++ms) {
-    const int s = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr];
-    nact += __builtin_amdgcn_readfirstlane(s) < nrows ? 1 : 0;
-    sxo[ms] = SORTED ? (uint32_t)((int64_t)(slot0 + wm * 128 + lr) * p.sx_m)  // + ms * 32 rows, added as a uniform
-                     : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
-  }
-  const uint32_t sx32 = SORTED ? (uint32_t)(32 * p.sx_m) : 0u;  // step between the scale rows of two 32-slot groups
-  const int nb = min(n0 + wn * 64, p.N - 1) >> 7;  // the wave's 64 weight rows lie inside one 128-row block
-  const float* swp = p.sw + (int64_t)expert * p.sw_expert_stride + (int64_t)nb * p.sw_n;
-  const int nkb = p.K / kTileK;
-
-  v16f acc[NS][MS];
+    for (int q = 0; q < LW; ++q) sid[q] = p.sorted_ids[slot0 + (w * LW + q) * 8 + rl];
+    if (first) {
+      // the wave's 8-row groups g = 4w + q: groups q and q + 2 differ by 16 rows and share the chunk swizzle, so two
+      // lane offsets serve the four weight loads (the 16-row step is uniform and joins the K offset)
 #pragma unroll
-  for (int ns = 0; ns < NS; ++ns)
-#pragma unroll
-    for (int ms = 0; ms < MS; ++ms)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
-
-  // Scales.  PAIRS: sxp[ms] holds the activation scales of an even K block and the odd one after it, fetched with
-  // one 8-byte load every other trip; with row-major scales the rows of a block are gathered, so every lane's load is
-  // a cache line of its own whatever the layout, and what counts is the number of load instructions and that a
-  // row's line is met again on the following trips.  Otherwise sxn[ms] / sbn hold the scales of the NEXT K block,
-  // requested one trip ahead in front of that trip's stage loads: at the next barrier everything older than the
-  // four youngest weight loads has landed, the scales among it.
-  constexpr bool pairs = PAIRS;
-  v2f sxp[MS];
-  float sxn[MS], sbn = 0.f;
-  float sba = 0.f, sbb = 0.f;  // PAIRS: weight scales of the even / odd block in flight
-  const rsrc_t rS = make_rsrc(p.sx, (uint32_t)(((xrows - 1) * p.sx_m + nkb) * 4));  // used by the paired loads only
-  auto load_sb = [&](float& sb, int kb) { sb = swp[(int64_t)min(kb, nkb - 1) * p.sw_k]; };
-  // through a buffer descriptor: a 32-bit lane offset and a uniform offset, no 64-bit address per lane and group
-  const rsrc_t rSall = make_rsrc(p.sx, 0xFFFFFFFFu);
-  auto load_sx = [&](int kb) {
-    const uint32_t ko = (uint32_t)(min(kb, nkb - 1) * (int)p.sx_k);
-#pragma unroll
-    for (int ms = 0; ms < MS; ++ms)
-      sxn[ms] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rSall, (int)(sxo[SORTED ? 0 : ms] * 4u),
-                                                                              (int)((ko + (uint32_t)ms * sx32) * 4u), 0));
-  };
-  auto load_sx_pair = [&](int kb) {  // kb even: blocks kb and kb+1 (past the tensor: zero)
-#pragma unroll
-    for (int ms = 0; ms < MS; ++ms)
-      sxp[ms] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rS, (int)((sxo[ms] + (uint32_t)kb) * 4u), 0, 0));
-  };
-  if (pairs) { load_sx_pair(0); load_sb(sba, 0); load_sb(sbb, 1); }
-  else { load_sx(0); load_sb(sbn, 0); }
-  __builtin_amdgcn_sched_barrier(0);
-  issue_x(0);
-  wait_vm0();  // the first trip's partial wait assumes the in-loop order of loads
-
-  // one K block; its scales sit in sxp[.][parity] and sb on entry; the odd trips reload both blocks' activation
-  // scales in the paired form
-  auto trip = [&](auto na, int it, int parity, float& sb) {
-    constexpr int NA = decltype(na)::value;  // 32-slot groups of the wave's half with real slots
-    lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
-    float sc[MS];
-    if (pairs) {
-#pragma unroll
-      for (int ms = 0; ms < MS; ++ms) sc[ms] = sxp[ms][parity] * sb;
-      if (parity) load_sx_pair(it + 1);
-      load_sb(sb, it + 2);
-    } else {
-#pragma unroll
-      for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
-      load_sx(it + 1);
-      load_sb(sbn, it + 1);
-    }
-    __builtin_amdgcn_sched_barrier(0);  // scales, then activations, then weights
-    issue_x(it + 1);                    // into the stage of block it-1, which every wave has left
-    issue_w(it + 2);
-    if (NA == 0) return;
-    const uint8_t* sw_ = smem + (it % WST) * WBYTES;
-    const uint8_t* sx_ = smem + XBASE + (it & 1) * XBYTES;
-    v8i wf[NS][2];
-#pragma unroll
-    for (int ns = 0; ns < NS; ++ns) {
-      wf[ns][0] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 0);
-      wf[ns][1] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 1);
+      for (int q = 0; q < 2; ++q) {
+        const int g = w * LW + q;  // 8-row group, 0..31, of both tiles
+        const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
+        voW[q] = (uint32_t)((g * 8 + rl) * p.ldw + c * 16);
+      }
+      w16 = (uint32_t)(16 * p.ldw);
+      rW = weights_of(it);
+      __builtin_amdgcn_sched_barrier(0);
+      issue_w(rW, 0, 0);
+      issue_w(rW, 1, 1);
+      __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int ms = 0; ms < NA; ++ms) {  // groups past the expert's last slot are padding
-      const v8i x0 = frag(sx_ + (wm * 128 + ms * 32) * kTileK, 0);
-      const v8i x1 = frag(sx_ + (wm * 128 + ms * 32) * kTileK, 1);
+    for (int q = 0; q < LW; ++q) {
+      const int g = w * LW + q;
+      const int c = cp ^ (((g & 1) << 2) + (rl >> 1));
+      const int sd = sid[q];
+      voX[q] = sd < nrows ? (uint32_t)((int64_t)(sd / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
+    }
+    issue_x(0, gx0);
+  };
+  start_item(item, true);
+
+  for (;;) {
+    int ln = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(ln));
+    const int lr = ln & 31, h = ln >> 5;
+
+    // ---- LDS -> MFMA operands
+    const int swz = (lr >> 1) & 7;
+    // lane part of an operand fetch address (row lr of a 32-row group, swizzled 16-byte chunk); stage, wave position
+    // and group are uniform, so weights and activations share these four registers
+    uint32_t fa[2][2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+      for (int q = 0; q < 2; ++q) fa[ks][q] = (uint32_t)(lr * kTileK + (((ks * 4 + h * 2 + q) ^ swz) << 4));
+    auto frag = [&](const uint8_t* grp, int ks) -> v8i {  // grp: first row of the 32-row group inside its stage (uniform)
+      const v4i lo = *reinterpret_cast<const v4i*>(grp + fa[ks][0]);
+      const v4i hi = *reinterpret_cast<const v4i*>(grp + fa[ks][1]);
+      v8i r;
+      r[0] = lo[0]; r[1] = lo[1]; r[2] = lo[2]; r[3] = lo[3];
+      r[4] = hi[0]; r[5] = hi[1]; r[6] = hi[2]; r[7] = hi[3];
+      return r;
+    };
+
+    // ---- scales: activation scale rows follow the activation rows
+    uint32_t sxo[MS];  // element offsets into the activation scales (the host checks they fit 32 bits)
+    int nact = 0;      // the wave's 32-slot groups (wm, wm + 2, wm + 4, wm + 6) that hold real slots: a prefix, real slots come first
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) {
+      const int s = p.sorted_ids[slot0 + (ms * 2 + wm) * 32 + lr];
+      nact += __builtin_amdgcn_readfirstlane(s) < nrows ? 1 : 0;
+      sxo[ms] = SORTED ? (uint32_t)((int64_t)(slot0 + wm * 32 + lr) * p.sx_m)  // + ms * 64 rows, added as a uniform
+                       : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
+    }
+    const uint32_t sx32 = SORTED ? (uint32_t)(64 * p.sx_m) : 0u;  // step between the scale rows of two of the wave's groups
+    const int nb = min(n0 + wn * 64, p.N - 1) >> 7;  // the wave's 64 weight rows lie inside one 128-row block
+    const float* swp = p.sw + (int64_t)expert * p.sw_expert_stride + (int64_t)nb * p.sw_n;
+
+    v16f acc[NS][MS];
+#pragma unroll
+    for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[ns][ms][r] = 0.f;
+
+    // Scales.  PAIRS: sxp[ms] holds the activation scales of an even K block and the odd one after it, fetched with
+    // one 8-byte load every other trip; with row-major scales the rows of a block are gathered, so every lane's load is
+    // a cache line of its own whatever the layout, and what counts is the number of load instructions and that a
+    // row's line is met again on the following trips.  Otherwise sxn[ms] / sbn hold the scales of the NEXT K block,
+    // requested one trip ahead in front of that trip's stage loads: at the next barrier everything older than the
+    // four youngest weight loads has landed, the scales among it.
+    constexpr bool pairs = PAIRS;
+    v2f sxp[MS];
+    float sxn[MS], sbn = 0.f;
+    float sba = 0.f, sbb = 0.f;  // PAIRS: weight scales of the even / odd block in flight
+    auto load_sb = [&](float& sb, int kb) { sb = swp[(int64_t)min(kb, nkb - 1) * p.sw_k]; };
+    auto load_sx = [&](int kb) {
+      const uint32_t ko = (uint32_t)(min(kb, nkb - 1) * (int)p.sx_k);
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms)
+        sxn[ms] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rSall, (int)(sxo[SORTED ? 0 : ms] * 4u),
+                                                                                (int)((ko + (uint32_t)ms * sx32) * 4u), 0));
+    };
+    auto load_sx_pair = [&](int kb) {  // kb even: blocks kb and kb+1 (past the tensor: zero)
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms)
+        sxp[ms] = __builtin_bit_cast(v2f, __builtin_amdgcn_raw_buffer_load_b64(rS, (int)((sxo[ms] + (uint32_t)kb) * 4u), 0, 0));
+    };
+    if (pairs) { load_sx_pair(0); load_sb(sba, 0); load_sb(sbb, 1); }
+    else { load_sx(0); load_sb(sbn, 0); }
+    // the item after this one, looked up while the first blocks arrive
+    int jn = j + jstep;
+    const MoeItem next = fetch_item(jn);
+    rWn = weights_of(next);
+    wait_vm0();  // the first trip's partial wait assumes the in-loop order of loads; the previous item's stores are out
+
+    // one K block; its scales sit in sxp[.][parity] and sb on entry; the odd trips reload both blocks' activation
+    // scales in the paired form
+    auto trip = [&](auto na, int it, int parity, float& sb) {
+      constexpr int NA = decltype(na)::value;  // 32-slot groups of the wave's half with real slots
+      lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
+      // nothing of this trip may move in front of the barrier: the scale products below would drag a wait for
+      // the scale loads of the previous trip with them, and loads return in order - that wait would also be one for
+      // the weight block requested before those scales
+      __builtin_amdgcn_sched_barrier(0);
+      float sc[MS];
+      if (pairs) {
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) sc[ms] = sxp[ms][parity] * sb;
+        if (parity) load_sx_pair(it + 1);
+        load_sb(sb, it + 2);
+      } else {
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
+        load_sx(it + 1);
+        load_sb(sbn, it + 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // scales, then activations, then weights
+      issue_x(it + 1, (gx0 + it + 1) & 1);  // into the stage of block it-1, which every wave has left (past the item's
+                                            // last block the offsets are out of range: nothing moves)
+      {
+        // block it+2 of this item, or block 0 / 1 of the next one: the weight stream does not stop between items
+        const int k2 = it + 2;
+        const bool nx = k2 >= nkb;
+        issue_w(nx ? rWn : rW, nx ? k2 - nkb : k2, (gw0 + k2) % WST);
+      }
+      if (NA == 0) return;
+      const uint8_t* sw_ = smem + ((gw0 + it) % WST) * WBYTES;
+      const uint8_t* sx_ = smem + XBASE + ((gx0 + it) & 1) * XBYTES;
+      v8i wf[NS][2];
 #pragma unroll
       for (int ns = 0; ns < NS; ++ns) {
-        v16f z;
-#pragma unroll
-        for (int r = 0; r < 16; ++r) z[r] = 0.f;
-        v16f tq = mfma_32x32x64(wf[ns][0], x0, z);
-        tq = mfma_32x32x64(wf[ns][1], x1, tq);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[ns][ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ns][ms][r]);
+        wf[ns][0] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 0);
+        wf[ns][1] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 1);
       }
-    }
-  };
-  auto run = [&](auto na) {
-    int it = 0;
-    for (; it + 1 < nkb; it += 2) {
-      trip(na, it, 0, sba);
-      trip(na, it + 1, 1, sbb);
-    }
-    if (it < nkb) trip(na, it, 0, sba);
-  };
-  // one copy of the loop per group count keeps every copy straight-line.  (The four-group copy needs all 256
-  // registers; the compiler parks a few epilogue values in scratch around it, outside the loops, where those
-  // accesses are older than every load the partial waits count.)
-  switch (nact) {  // wave-uniform
-    case 4: run(std::integral_constant<int, 4>{}); break;
-    case 3: run(std::integral_constant<int, 3>{}); break;
-    case 2: run(std::integral_constant<int, 2>{}); break;
-    case 1: run(std::integral_constant<int, 1>{}); break;
-    default: run(std::integral_constant<int, 0>{}); break;
-  }
-  // output rows and routed weights, fetched while the stages drain.  The lane id is taken anew (from the execution
-  // mask, no register kept for it): lane-derived values that stayed live across the K loops would be parked in scratch
-  // and reloaded inside them, and scratch reloads count against the partial vmcnt waits.
-  const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
-  const int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
-  const int lr_e = lane_e & 31, h_e = lane_e >> 5;
-  const int er = lane_e >> 3, ec = lane_e & 7;  // store loop: row inside a group of 8, 16-byte chunk of the wave's 128 bytes
-  int oslots[MS], srow[16];
-  float rsw[MS];
 #pragma unroll
-  for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[slot0 + wm * 128 + ms * 32 + lr_e];
+      for (int ms = 0; ms < NA; ++ms) {  // groups past the expert's last slot are padding
+        const v8i x0 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 0);
+        const v8i x1 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 1);
 #pragma unroll
-  for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[slot0 + wm * 128 + i * 8 + er] : 0;
+        for (int ns = 0; ns < NS; ++ns) {
+          v16f z;
 #pragma unroll
-  for (int ms = 0; ms < MS; ++ms) rsw[ms] = (p.topk_w && oslots[ms] < nrows) ? p.topk_w[oslots[ms]] : 1.f;
-  wait_vm0();     // the loads past the last K block still target the stages
-  lds_barrier();  // every wave has left the stages: they become the output staging area
-
-  // ---- epilogue through LDS.  A wave re-lays its own 128 slots x 64 n block out in a private 16 KB slot (128 B per
-  // row, 16-byte chunk c of row r at position c ^ ((r >> 1) & 7), so that the accumulator-shaped 8-byte writes and
-  // the 16-byte reads spread over all banks): no second workgroup barrier, and every store instruction writes eight
-  // whole 128-byte lines.
-  uint8_t* const ep = smem + w * 16384;
+          for (int r = 0; r < 16; ++r) z[r] = 0.f;
+          v16f tq = mfma_32x32x64(wf[ns][0], x0, z);
+          tq = mfma_32x32x64(wf[ns][1], x1, tq);
 #pragma unroll
-  for (int ms = 0; ms < MS; ++ms) {
-    const int row = ms * 32 + lr_e;  // inside the wave's 128 slots
-    const int oslot = oslots[ms];
-    const bool ok = oslot < nrows;
-    const float rs = rsw[ms];
-#pragma unroll
-    for (int nr = 0; nr < NS * 4; ++nr) {
-      const int ns = nr >> 2, rg = nr & 3;
-      float v[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) v[r] = acc[ns][ms][rg * 4 + r] * rs;
-      if (wide) {
-        uint2 o;
-        if (OUT_DT == FP8K_BF16) {
-          o.x = pack_bf16x2(v[0], v[1]);
-          o.y = pack_bf16x2(v[2], v[3]);
-        } else {
-          o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
-          o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+          for (int r = 0; r < 16; ++r) acc[ns][ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ns][ms][r]);
         }
-        *reinterpret_cast<uint2*>(ep + row * 128 + ((nr ^ ((row >> 1) & 7)) << 4) + h_e * 8) = o;
-      } else {
-        const int n = n0 + wn * 64 + nr * 8 + h_e * 4;
-        if (ok && n < p.N) store4<OUT_DT>(p.C, (int64_t)oslot * p.ldc + n, v[0], v[1], v[2], v[3]);
+      }
+    };
+    auto run = [&](auto na) {
+      int it = 0;
+      for (; it + 1 < nkb; it += 2) {
+        trip(na, it, 0, sba);
+        trip(na, it + 1, 1, sbb);
+      }
+      if (it < nkb) trip(na, it, 0, sba);
+    };
+    // one copy of the loop per group count keeps every copy straight-line
+    switch (nact) {  // wave-uniform
+      case 4: run(std::integral_constant<int, 4>{}); break;
+      case 3: run(std::integral_constant<int, 3>{}); break;
+      case 2: run(std::integral_constant<int, 2>{}); break;
+      case 1: run(std::integral_constant<int, 1>{}); break;
+      default: run(std::integral_constant<int, 0>{}); break;
+    }
+    // output rows and routed weights, fetched while the stages drain (lane id taken anew, as above)
+    const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
+    int lane_e = (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u));
+    asm volatile("" : "+v"(lane_e));
+    const int lr_e = lane_e & 31, h_e = lane_e >> 5;
+    const int er = lane_e >> 3, ec = lane_e & 7;  // store loop: row inside a group of 8, 16-byte chunk of the wave's 128 bytes
+    const int eslot0 = slot0, en0 = n0;
+    int oslots[MS], srow[16];
+    float rsw[MS];
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[eslot0 + (ms * 2 + wm) * 32 + lr_e];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[eslot0 + ((i >> 2) * 2 + wm) * 32 + (i & 3) * 8 + er] : 0;
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) rsw[ms] = (p.topk_w && oslots[ms] < nrows) ? p.topk_w[oslots[ms]] : 1.f;
+    lds_barrier();  // every wave has left the item's last stages; the requests in flight point at the other ones
+    const int ews = (gw0 + nkb - 1) % WST, exs = (gx0 + nkb - 1) & 1;  // the stages of the item's last block
+    gw0 = (gw0 + nkb) % WST;
+    gx0 = (gx0 + nkb) & 1;
+    const bool has_next = next.mb >= 0;
+    if (has_next) {
+      rW = rWn;
+      start_item(next, false);  // its first activation block travels while this item is written out
+    }
+
+    // ---- write-out through LDS, in two passes of 64 slots.  A wave re-lays 64 slots x 64 n of its block out in a
+    // private 8 KB slot inside the weight / activation stage of the item's last block (128 B per row, 16-byte chunk c
+    // of row r at position c ^ ((r >> 1) & 7), so that the accumulator-shaped 8-byte writes and the 16-byte reads
+    // spread over all banks): no workgroup barrier, and every store instruction writes eight whole 128-byte lines.
+    uint8_t* const ep = smem + (w < 4 ? ews * WBYTES + w * 8192 : XBASE + exs * XBYTES + (w - 4) * 8192);
+#pragma unroll
+    for (int ph = 0; ph < 2; ++ph) {
+#pragma unroll
+      for (int mh = 0; mh < 2; ++mh) {
+        const int ms = ph * 2 + mh;
+        const int row = mh * 32 + lr_e;  // inside the pass's 64 slots
+        const int oslot = oslots[ms];
+        const bool ok = oslot < nrows;
+        const float rs = rsw[ms];
+#pragma unroll
+        for (int nr = 0; nr < NS * 4; ++nr) {
+          const int ns = nr >> 2, rg = nr & 3;
+          float v[4];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) v[r] = acc[ns][ms][rg * 4 + r] * rs;
+          if (wide) {
+            uint2 o;
+            if (OUT_DT == FP8K_BF16) {
+              o.x = pack_bf16x2(v[0], v[1]);
+              o.y = pack_bf16x2(v[2], v[3]);
+            } else {
+              o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16);
+              o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16);
+            }
+            *reinterpret_cast<uint2*>(ep + row * 128 + ((nr ^ ((row >> 1) & 7)) << 4) + h_e * 8) = o;
+          } else {
+            const int n = en0 + wn * 64 + nr * 8 + h_e * 4;
+            if (ok && n < p.N) store4<OUT_DT>(p.C, (int64_t)oslot * p.ldc + n, v[0], v[1], v[2], v[3]);
+          }
+        }
+      }
+      if (wide) {
+        __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int row = i * 8 + er;
+          const int s = srow[ph * 8 + i];
+          const int n = en0 + wn * 64 + (ec << 3);
+          const uint4 o = *reinterpret_cast<const uint4*>(ep + row * 128 + ((ec ^ ((row >> 1) & 7)) << 4));
+          if (s < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)s * p.ldc + n) = o;
+        }
+        __builtin_amdgcn_wave_barrier();
       }
     }
-  }
-  if (!wide) return;
-  __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
-#pragma unroll
-  for (int i = 0; i < 16; ++i) {
-    const int row = i * 8 + er;
-    const int s = srow[i];
-    const int n = n0 + wn * 64 + (ec << 3);
-    const uint4 o = *reinterpret_cast<const uint4*>(ep + row * 128 + ((ec ^ ((row >> 1) & 7)) << 4));
-    if (s < nrows && n < p.N) *reinterpret_cast<uint4*>((u16*)p.C + (int64_t)s * p.ldc + n) = o;
+    if (!has_next) {
+      wait_vm0();  // the out-of-range requests of the last trips still point at the stages: let them retire before the LDS goes back
+      return;
+    }
+    item = next;
+    j = jn;
   }
 }
 
