@@ -215,6 +215,28 @@ def run_quant_roofline(torch, dev, iters=30):
     return out
 
 
+def hbm_stream_read_gbs(torch, dev, gib=4, runs=5):
+    """Read rate (GB/s) of the library's LDS-staged load path on a plain contiguous buffer of `gib` GiB - the ceiling
+    the weight-streaming kernels can reach on this machine (fp8k_tune_stream_read, timed with HIP events; best of
+    `runs`, each run reads the whole buffer once, far more than the 256 MB last-level cache holds)."""
+    from sglang_amd._lib import check, lib, stream_ptr
+
+    buf = torch.empty(gib << 30, dtype=torch.uint8, device=dev)
+    buf.view(torch.int32).random_(0, 1 << 30)
+    best = float("inf")
+    for _ in range(runs + 1):
+        a, b = _events(torch, 2)
+        a.record()
+        check(lib.fp8k_tune_stream_read(buf.data_ptr(), buf.numel(), stream_ptr(dev)))
+        b.record()
+        torch.cuda.synchronize()
+        best = min(best, a.elapsed_time(b))
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    read = buf.numel() // ncu // 65536 * 65536 * ncu
+    del buf
+    return read / best / 1e6
+
+
 def run_cpu_baseline(seconds_target=12.0):
     """C restatement of quant + block GEMM (oracle/, OpenMP) on M_cpu rows of the headline workload."""
     import numpy as np
@@ -352,8 +374,11 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=Fals
     return lines
 
 
-def gemm_lines(torch, dev, shapes):
-    """Block-FP8 GEMM alone at the given (M, N, K): device time, TFLOP/s and algorithmic GB/s."""
+def gemm_lines(torch, dev, shapes, data="random"):
+    """Block-FP8 GEMM alone at the given (M, N, K): device time, TFLOP/s and algorithmic GB/s.  data = "zeros" runs
+    the same launches on all-zero operands (and unit scales): the same instructions and memory traffic, but no bit of
+    the matrix-core data paths toggles - the time difference against "random" is what the chip's power management
+    takes (it lowers the clock under the random-data load)."""
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8, w8a8_block_fp8_matmul
 
     lines = ["| M | N | K | us | TFLOP/s | % of 5 PFLOP/s | GB/s (algorithmic) |", "|---|---|---|---|---|---|---|"]
@@ -362,6 +387,10 @@ def gemm_lines(torch, dev, shapes):
         ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
         qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True)
               for s in range(nbuf)]
+        if data == "zeros":
+            for q, sc in ws + qs:
+                q.view(torch.uint8).zero_()
+                sc.fill_(1.0)
         us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
                                                                 ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
         tf = 2.0 * M * N * K / us / 1e6
@@ -384,6 +413,7 @@ def write_table(torch, dev, path, cpu=True):
     from sglang_amd.fp8_utils import w8a8_block_fp8_linear
     from sglang_amd.sgl_kernel import fp8_scaled_mm, mark_ue8m0
 
+    stream_gbs = hbm_stream_read_gbs(torch, dev)
     lines = ["# Per-shape report (one MI355X, synthetic data, rotating buffers)", "",
              "GPU: device time by HIP events around a HIP graph that replays the launches back to back (host launch cost excluded).",
              "Roofline: the binding one of dense-FP8 MFMA peak (5 PFLOP/s) and HBM peak (8 TB/s) for the shape's algorithmic",
@@ -392,7 +422,9 @@ def write_table(torch, dev, path, cpu=True):
              "n_tiles block-tile float32 matmul loop), median of 5 runs after one warm-up, at most %d rows of the shape" % CPU_ROW_CAP,
              "(the loop is interpreter-bound); host: torch.get_num_threads() = %d, os.cpu_count() = %d." % (
                  torch.get_num_threads(), os.cpu_count()),
-             "`err` = max |gpu - cpu| / max |cpu| on the rows the CPU computed (quant: bytes and scales compared for equality).", ""]
+             "`err` = max |gpu - cpu| / max |cpu| on the rows the CPU computed (quant: bytes and scales compared for equality).",
+             "HBM read rate that the library's LDS-staged load path reaches on a plain 4 GiB buffer on this machine "
+             "(fp8k_tune_stream_read): %.0f GB/s = %.2f of the 8 TB/s that `frac` is priced against." % (stream_gbs, stream_gbs / PEAK_HBM_GBS), ""]
 
     # ---- configs[0]
     lines += ["## configs[0] single W8A8 block-FP8 linear (x bf16 [32,4096], W [4096,4096], seed 0), quant + GEMM", "",
@@ -530,6 +562,10 @@ def main() -> int:
                     help="only time the fused MoE layer at these token counts (comma separated) and print its table")
     ap.add_argument("--gemm", type=str, default=None,
                     help="only time the block-FP8 GEMM at these shapes (MxNxK, comma separated) and print its table")
+    ap.add_argument("--gemm-data", choices=("random", "zeros"), default="random",
+                    help="operands of the --gemm runs: synthetic random data (default) or all zeros (same work, no "
+                         "toggling in the matrix cores: shows what the power management takes)")
+    ap.add_argument("--stream-read", action="store_true", help="only measure the HBM read rate of the LDS-staged load path")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no cross-GPU step); --gpus %d is not "
@@ -549,7 +585,10 @@ def main() -> int:
         return 0
     if args.gemm:
         shapes = [tuple(int(v) for v in t.split("x")) for t in args.gemm.split(",")]
-        print("\n".join(gemm_lines(torch, dev, shapes)))
+        print("\n".join(gemm_lines(torch, dev, shapes, args.gemm_data)))
+        return 0
+    if args.stream_read:
+        print("HBM stream read (4 GiB buffer, LDS-staged loads, one workgroup per CU): %.0f GB/s" % hbm_stream_read_gbs(torch, dev))
         return 0
     ms_per_step, gemm_us = run_headline(torch, dev, args.steps, args.warmup)
     M, N, K = HEADLINE["M"], HEADLINE["N"], HEADLINE["K"]
@@ -608,6 +647,7 @@ def main() -> int:
             "avg_launch_us": round(q_us, 2),
             "other_layouts_GBps": {k: round(v[1], 1) for k, v in quant.items()},
         },
+        "hbm_stream_read_GBps": round(hbm_stream_read_gbs(torch, dev), 1),
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

@@ -161,6 +161,15 @@ int fp8k_block_gemm_noalloc(const void* A, const void* B, const float* As, const
 void fp8k_tune_force_gemm_plan(int kind, int splits);
 
 /*
+ * Measurement aid (no counterpart in the reference): streams `bytes` of device memory at `src` once through the load
+ * path of the weight-streaming kernels - one workgroup of 8 wavefronts per CU, 32 KB stages of 16-byte-per-lane loads
+ * straight into LDS, two stages in flight, a workgroup barrier per stage - and drops the data.  Timed by the caller, it
+ * gives the read rate this load path reaches on the machine at hand, the practical ceiling under the 8 TB/s of the
+ * data sheet.  `bytes` is rounded down to a multiple of 64 KB per CU; src 16-byte aligned; bytes < 2^40.
+ */
+int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream);
+
+/*
  * Per-token x per-channel FP8 GEMM:  C = (A . B^T) * sa[m] * sb[n] (+ bias[n]), fp32 accumulate.
  * Replaces torch.ops.sgl_kernel.fp8_scaled_mm
  *   (sgl-kernel/python/sgl_kernel/gemm.py:35-43, sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532).

@@ -316,6 +316,43 @@ static int common_checks(const char* op, const void* A, const void* B, void* C, 
 
 using namespace fp8k;
 
+namespace fp8k {
+// every workgroup reads its own contiguous share, a 32 KB stage per trip, two stages in flight
+__global__ __launch_bounds__(512, 1) void stream_read_kernel(const uint8_t* __restrict__ src, int64_t share) {
+  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint8_t* base = src + (int64_t)blockIdx.x * share;
+  const int trips = (int)(share >> 15);
+  auto issue = [&](int t) {
+    // the descriptor moves with the trip: a share may exceed the 4 GB a descriptor can span
+    const rsrc_t r = make_rsrc(base + (int64_t)t * 32768, 32768u);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      buf_load16_to_lds(r, (uint32_t)((w * 4 + q) * 1024 + lane * 16), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
+  };
+  issue(0);
+  if (trips > 1) issue(1);
+  for (int t = 0; t < trips; ++t) {
+    if (t + 1 < trips) lds_barrier<4>();
+    else lds_barrier<0>();
+    if (t + 2 < trips) issue(t + 2);
+  }
+  wait_vm0();
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read: bad size");
+  FP8K_REQUIRE(src && aligned(src, 16), "tune_stream_read: src must be a 16-byte aligned device pointer");
+  const int ncu = num_cu();
+  const int64_t share = bytes / ncu / 65536 * 65536;
+  if (share == 0) return FP8K_OK;
+  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src, share);
+  return check_launch("tune_stream_read");
+}
+
 extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) {
   g_tail_halves = kind != -2;  // -2: automatic choice with the last round of 256x256 tiles kept whole
   g_force_kind = kind == -2 ? -1 : kind;
