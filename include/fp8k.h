@@ -289,6 +289,28 @@ int fp8k_moe_blocks_from_offsets(const int32_t* expert_starts, const int32_t* pr
                                  int64_t expert_capacity, int32_t* num_tokens_post_pad, void* stream);
 
 /*
+ * Grouped GEMM 1 of the fused MoE layer with silu_and_mul and the per-token-group requantisation inside its write-out
+ * (256-slot blocks): what fp8k_moe_block_gemm into a 16-bit [slots, 2 I] tensor followed by
+ * fp8k_silu_mul_group_quant would produce, bit for bit, without that tensor ever being written.
+ * Replaces the sequence invoke_fused_moe_kernel -> silu_and_mul -> per_token_group_quant_fp8 of fused_experts_impl
+ *   (python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:498-600); the reference has the activation + quant
+ *   fusion as its own kernel (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:336-341), not inside the GEMM.
+ * B e4m3fn [E, 2 I, K]: gate rows, then up rows (the checkpoint layout, no re-ordering); I % 128 == 0.
+ * As_sorted: activation scales in the order of sorted_token_ids (fp8k_moe_sort_scales), as_stride_k floats between
+ * K blocks.  q_out e4m3fn [slots, I] (ldq bytes between rows, row = token slot); qs_out float, the scale of
+ * activation column block g of the slot at position i of sorted_token_ids at qs_out[g * qs_stride_g + i] (0 for
+ * padding) - the layout fp8k_moe_block_gemm takes with as_sorted = 1.  act_dtype: the 16-bit type whose roundings
+ * the write-out reproduces (the dtype the layer runs in).  eps as for fp8k_group_quant.
+ */
+int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, const float* As_sorted, const float* Bs, void* q_out,
+                                   float* qs_out, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                   const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t num_valid_tokens,
+                                   int64_t top_k, int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_k,
+                                   int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e, int64_t bs_stride_n,
+                                   int64_t bs_stride_k, int64_t ldq, int64_t qs_stride_g, float eps, int act_dtype,
+                                   void* stream);
+
+/*
  * Activation scales in the order of sorted_token_ids (no counterpart in the reference, whose Triton kernel gathers
  * them per K block): out[kb * sorted_capacity + i] = As[sorted_token_ids[i] / top_k, kb] for i below
  * num_tokens_post_padded[0], 0 for padding entries.  Passing `out` to fp8k_moe_block_gemm with as_stride_m = 1,

@@ -50,6 +50,7 @@ SIGNATURES = {
     "fp8k_shuffle_rows": (_c_int, [_c_ptr] * 3 + [_c_i64] * 3 + [_c_ptr]),
     "fp8k_apply_shuffle_mul_sum": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int, _c_ptr]),
     "fp8k_moe_blocks_from_offsets": (_c_int, [_c_ptr] * 2 + [_c_i64] * 3 + [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
+    "fp8k_moe_block_gemm_silu_quant": (_c_int, [_c_ptr] * 9 + [_c_i64] * 15 + [_c_f32, _c_int, _c_ptr]),
     "fp8k_block_gemm": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 10 + [_c_int, _c_ptr, _c_i64, _c_ptr],

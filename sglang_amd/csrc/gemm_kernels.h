@@ -42,6 +42,13 @@ struct GemmArgs {
   int block_m;                  // grouped: slots per block in sorted_ids (<= TM)
   int sx_sorted;                // grouped: sx holds one row per position of sorted_ids (row = position), not per token
   int64_t w_expert_stride;      // bytes between experts in W
+  // grouped GEMM 1 with the activation and the requantisation in its write-out (moe_stream256_kernel<..., FUSE>):
+  // N = 2 I weight rows (gate rows, then up rows); q_out [slots, I] e4m3fn, qs_out [I/128][capacity of sorted_ids] float
+  uint8_t* q_out;
+  float* qs_out;
+  int64_t ldq;
+  int64_t qs_ld;                // floats between the scale rows of two activation column blocks (>= capacity)
+  float q_eps;                  // lower clamp of the group maximum (already rounded to the element type)
   int64_t sw_expert_stride;     // floats between experts in sw
   // batched form of the 128x128 tile kernel (grid y = batch entry); zero for a single GEMM
   int64_t batch_x, batch_w;     // bytes between batch entries of X and W

@@ -21,6 +21,7 @@
 #include <type_traits>
 
 #include "gemm_kernels.h"
+#include "quant_math.h"
 
 namespace fp8k {
 
@@ -28,8 +29,14 @@ namespace fp8k {
 // 8 bytes; the host checks), and a lane fetches two K blocks per load.  SORTED: one scale row per position of
 // sorted_token_ids (what the layer passes): the rows of a wave's four 32-slot groups are a uniform step apart, so one
 // offset register serves them.
-template <int OUT_DT, bool PAIRS, bool SORTED>
+// FUSE (GEMM 1 of the layer, sorted scales only): the tile's 256 weight rows are 128 gate rows and the 128 up rows of
+// the same activation columns (rows n0 .. n0+127 and I + n0 .. I + n0+127 of the [2 I, K] weight, I = N / 2), and the
+// write-out produces what silu_and_mul followed by the group quantisation would have made of the 16-bit GEMM result,
+// bit for bit: q_out[slot, n0 .. n0+127] and one scale per slot in the sorted order GEMM 2 reads.  The [slots, 2 I]
+// intermediate is never written.
+template <int OUT_DT, bool PAIRS, bool SORTED, bool FUSE = false>
 __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p) {
+  static_assert(!FUSE || (SORTED && !PAIRS), "the fused write-out is built for sorted activation scales");
   constexpr int TM = 256, WST = 3, XST = 2, MS = 4, NS = 2, LW = 4;  // LW: wave loads per tile per stage
   constexpr int WBYTES = kTileN * kTileK, XBYTES = TM * kTileK;
   constexpr int XBASE = WST * WBYTES;
@@ -53,6 +60,13 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     const int lr = ln & 31, h = ln >> 5;
     for (int ms = 0; ms < MS; ++ms) {
       const int s = p.sorted_ids[it.mb * TM + wm * 128 + ms * 32 + lr];
+      if (FUSE) {  // zero bytes and a zero scale: the slot contributes nothing to GEMM 2
+        if (wn == 0 && h == 0) p.qs_out[(int64_t)it.tile_n * p.qs_ld + it.mb * TM + wm * 128 + ms * 32 + lr] = 0.f;
+        if (s < nrows && h == 0)
+          *reinterpret_cast<uint4*>(p.q_out + (int64_t)s * p.ldq + it.tile_n * 128 + wn * 32) = make_uint4(0, 0, 0, 0),
+          *reinterpret_cast<uint4*>(p.q_out + (int64_t)s * p.ldq + it.tile_n * 128 + wn * 32 + 16) = make_uint4(0, 0, 0, 0);
+        continue;
+      }
       if (s >= nrows) continue;
       for (int q = 0; q < 4; ++q) {
         for (int ns = 0; ns < NS; ++ns) {
@@ -87,11 +101,14 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   // The stages are two rings that run on across the items of a walk: block k of an item sits in weight stage
   // (gw0 + k) % 3 and activation stage (gx0 + k) & 1, the next item's block 0 in the stage after its last block.
   int gw0 = 0, gx0 = 0;
+  // FUSE: the waves that load tile rows 128..255 (w >= 4) take them from the up rows, I - 128 rows further on
+  const int half_n = p.N >> 1;
+  const uint32_t wsoff = (FUSE && w >= 4) ? (uint32_t)((int64_t)(half_n - 128) * p.ldw) : 0u;
   auto issue_w = [&](const rsrc_t& r, int kblk, int stage) {
     uint8_t* base = smem + stage * WBYTES + w * (LW * 1024);
     const uint32_t ko = (uint32_t)kblk * kTileK;
 #pragma unroll
-    for (int q = 0; q < LW; ++q) buf_load16_to_lds(r, voW[q & 1] + (ko + (q >> 1) * w16), 0, base + q * 1024);
+    for (int q = 0; q < LW; ++q) buf_load16_to_lds(r, voW[q & 1] + (ko + (q >> 1) * w16), wsoff, base + q * 1024);
   };
   auto issue_x = [&](int kblk, int stage) {
     uint8_t* base = smem + XBASE + stage * XBYTES + w * (LW * 1024);
@@ -102,6 +119,10 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   auto weights_of = [&](const MoeItem& it) -> rsrc_t {
     if (it.mb < 0) return make_rsrc(p.W, 0u);  // no item: every load is out of range and moves nothing
     const uint8_t* Wb = p.W + (int64_t)it.expert * p.w_expert_stride;
+    if (FUSE) {  // gate rows from n0 on; the range reaches the last up row of the tile
+      const int nn = it.tile_n * 128;
+      return make_rsrc(Wb + (int64_t)nn * p.ldw, (uint32_t)((int64_t)(half_n + 127) * p.ldw + p.K));
+    }
     const int nn = it.tile_n * kTileN;
     const int rowsW = min(kTileN, p.N - nn);
     return make_rsrc(Wb + (int64_t)nn * p.ldw, (uint32_t)((rowsW - 1) * p.ldw + p.K));
@@ -117,7 +138,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     asm volatile("" : "+v"(ln));
     const int rl = ln >> 3, cp = ln & 7;
     slot0 = it.mb * TM;
-    n0 = it.tile_n * kTileN;
+    n0 = it.tile_n * (FUSE ? 128 : kTileN);
     expert = it.expert;
     // slot table first, weights behind it: loads retire in order, so the table arrives without waiting for the
     // weights, and the weights do not wait for the table
@@ -185,7 +206,8 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
                        : (s < nrows ? (uint32_t)((int64_t)(s / p.top_k) * p.sx_m) : 0u);
     }
     const uint32_t sx32 = SORTED ? (uint32_t)(64 * p.sx_m) : 0u;  // step between the scale rows of two of the wave's groups
-    const int nb = min(n0 + wn * 64, p.N - 1) >> 7;  // the wave's 64 weight rows lie inside one 128-row block
+    // the wave's 64 weight rows lie inside one 128-row block (FUSE: gate rows for wn 0, 1, up rows for wn 2, 3)
+    const int nb = FUSE ? ((wn < 2 ? n0 : half_n + n0) >> 7) : (min(n0 + wn * 64, p.N - 1) >> 7);
     const float* swp = p.sw + (int64_t)expert * p.sw_expert_stride + (int64_t)nb * p.sw_n;
 
     v16f acc[NS][MS];
@@ -310,7 +332,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
     for (int ms = 0; ms < MS; ++ms) oslots[ms] = p.sorted_ids[eslot0 + (ms * 2 + wm) * 32 + lr_e];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) srow[i] = wide ? p.sorted_ids[eslot0 + ((i >> 2) * 2 + wm) * 32 + (i & 3) * 8 + er] : 0;
+    for (int i = 0; i < 16; ++i) srow[i] = (wide && !FUSE) ? p.sorted_ids[eslot0 + ((i >> 2) * 2 + wm) * 32 + (i & 3) * 8 + er] : 0;
 #pragma unroll
     for (int ms = 0; ms < MS; ++ms) rsw[ms] = (p.topk_w && oslots[ms] < nrows) ? p.topk_w[oslots[ms]] : 1.f;
     lds_barrier();  // every wave has left the item's last stages; the requests in flight point at the other ones
@@ -321,6 +343,110 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     if (has_next) {
       rW = rWn;
       start_item(next, false);  // its first activation block travels while this item is written out
+    }
+
+    if constexpr (FUSE) {
+      // ---- activation and requantisation of the finished tile.  The waves wn = 2, 3 hold the up columns of the
+      // activation columns whose gate values the waves wn = 0, 1 (same wm) hold in the same lanes and registers:
+      // they hand their 16-bit values over through LDS (16 KB per pair, inside the stages of the item's last block),
+      // the gate waves form a = T(T(silu(T(gate))) * T(up)), exchange the row maxima of their two 64-column halves,
+      // quantise and store bytes (re-laid out through LDS for 16-byte stores) and the scale of every slot.
+      const int pr = wn & 1;
+      uint8_t* const xr = smem + (wm == 0 ? ews * WBYTES : XBASE + exs * XBYTES) + pr * 16384;
+      int qrow[8];  // store loop: lane -> row it * 16 + lane / 4 of the wave's 128 slots, 16-byte chunk lane % 4
+#pragma unroll
+      for (int it8 = 0; it8 < 8; ++it8) {
+        const int r = it8 * 16 + (lane_e >> 2);
+        qrow[it8] = wn < 2 ? p.sorted_ids[eslot0 + ((r >> 5) * 2 + wm) * 32 + (r & 31)] : nrows;
+      }
+      if (wn >= 2) {
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms)
+#pragma unroll
+          for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+              uint2 o;
+              const float v[4] = {acc[ns][ms][rg * 4], acc[ns][ms][rg * 4 + 1], acc[ns][ms][rg * 4 + 2], acc[ns][ms][rg * 4 + 3]};
+              if (OUT_DT == FP8K_BF16) { o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]); }
+              else { o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16); o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16); }
+              *reinterpret_cast<uint2*>(xr + ((ms * 2 + ns) * 4 + rg) * 512 + lane_e * 8) = o;
+            }
+      }
+      lds_barrier();
+      float amx[MS];
+      if (wn < 2) {
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) {
+          float m = 0.f;
+#pragma unroll
+          for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+            for (int rg = 0; rg < 4; ++rg) {
+              const uint2 u = *reinterpret_cast<const uint2*>(xr + ((ms * 2 + ns) * 4 + rg) * 512 + lane_e * 8);
+              float uf[4];
+              if (OUT_DT == FP8K_BF16) { uf[0] = bf16_lo(u.x); uf[1] = bf16_hi(u.x); uf[2] = bf16_lo(u.y); uf[3] = bf16_hi(u.y); }
+              else { uf[0] = f16_bits_to_f32(u.x & 0xffff); uf[1] = f16_bits_to_f32(u.x >> 16); uf[2] = f16_bits_to_f32(u.y & 0xffff); uf[3] = f16_bits_to_f32(u.y >> 16); }
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const float g = round_to<OUT_DT>(acc[ns][ms][rg * 4 + r]);
+                const float a = round_to<OUT_DT>(round_to<OUT_DT>(silu_f32(g)) * uf[r]);
+                acc[ns][ms][rg * 4 + r] = a;
+                m = fmaxf(m, fabsf(a));
+              }
+            }
+          m = fmaxf(m, __shfl_xor(m, 32));  // the other 16 columns of every tile of the row
+          amx[ms] = m;
+        }
+        // own pair area is read: the maxima of the wave's 64 columns go to its start for the other gate wave
+        if (h_e == 0) {
+#pragma unroll
+          for (int ms = 0; ms < MS; ++ms) reinterpret_cast<float*>(xr)[ms * 32 + lr_e] = amx[ms];
+        }
+      }
+      lds_barrier();
+      if (wn < 2) {
+        const float* other = reinterpret_cast<const float*>(xr + (pr ? -16384 : 16384));
+        uint8_t* const st = xr + 1024;  // 128 rows x 64 B of bytes, behind the maxima
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) {
+          const float amax = fmaxf(fmaxf(amx[ms], other[ms * 32 + lr_e]), p.q_eps);
+          const float sc = div448<true>(amax);
+          const int row = ms * 32 + lr_e;
+#pragma unroll
+          for (int ns = 0; ns < NS; ++ns)
+#pragma unroll
+            for (int rp = 0; rp < 2; ++rp) {
+              float a8[8];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) { a8[r] = acc[ns][ms][(rp * 2) * 4 + r]; a8[4 + r] = acc[ns][ms][(rp * 2 + 1) * 4 + r]; }
+              bool redo;
+              uint2 o = quant8_bracket<true>(a8, sc, amax, redo);
+              if (redo) o = quant8_divide(a8, sc);
+              *reinterpret_cast<uint32_t*>(st + row * 64 + ns * 32 + (rp * 2) * 8 + h_e * 4) = o.x;
+              *reinterpret_cast<uint32_t*>(st + row * 64 + ns * 32 + (rp * 2 + 1) * 8 + h_e * 4) = o.y;
+            }
+          if (pr == 0 && h_e == 0) {
+            const int pos = eslot0 + (ms * 2 + wm) * 32 + lr_e;
+            p.qs_out[(int64_t)(en0 >> 7) * p.qs_ld + pos] = oslots[ms] < nrows ? sc : 0.f;
+          }
+        }
+        __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order
+#pragma unroll
+        for (int it8 = 0; it8 < 8; ++it8) {
+          const int r = it8 * 16 + (lane_e >> 2), c = lane_e & 3;
+          const uint4 o = *reinterpret_cast<const uint4*>(st + r * 64 + c * 16);
+          const int sdst = qrow[it8];
+          if (sdst < nrows) *reinterpret_cast<uint4*>(p.q_out + (int64_t)sdst * p.ldq + en0 + pr * 64 + c * 16) = o;
+        }
+      }
+      if (!has_next) {
+        wait_vm0();
+        return;
+      }
+      item = next;
+      j = jn;
+      continue;
     }
 
     // ---- write-out through LDS, in two passes of 64 slots.  A wave re-lays 64 slots x 64 n of its block out in a

@@ -373,6 +373,69 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
   return check_launch(op);
 }
 
+extern "C" int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, const float* As_sorted, const float* Bs, void* q_out,
+                                              float* qs_out, const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                              const int32_t* num_tokens_post_padded, int64_t sorted_capacity,
+                                              int64_t num_valid_tokens, int64_t top_k, int64_t num_experts, int64_t N,
+                                              int64_t K, int64_t lda, int64_t as_stride_k, int64_t b_stride_e, int64_t ldb,
+                                              int64_t bs_stride_e, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldq,
+                                              int64_t qs_stride_g, float eps, int act_dtype, void* stream) {
+  clear_error();
+  const char* op = "moe_block_gemm_silu_quant";
+  constexpr int64_t block_m = 256;
+  FP8K_REQUIRE(N > 0 && K > 0 && num_experts > 0 && top_k > 0, "%s: bad shape", op);
+  FP8K_REQUIRE(N <= 0x7fffffffLL && K <= 0x7fffffffLL && num_valid_tokens >= 0 && num_valid_tokens < 0x7fffffffLL,
+               "%s: shape too large", op);
+  FP8K_REQUIRE(act_dtype == FP8K_F16 || act_dtype == FP8K_BF16, "%s: the activation type must be Half or BFloat16", op);
+  FP8K_REQUIRE(K % kTileK == 0, "%s: K (%lld) must be a multiple of 128", op, (long long)K);
+  FP8K_REQUIRE(N % 256 == 0, "%s: N = 2 I with I a multiple of 128 (got N = %lld)", op, (long long)N);
+  const int64_t I = N / 2;
+  FP8K_REQUIRE(sorted_capacity >= 0 && sorted_capacity < 0x7fffffffLL, "%s: bad sorted_token_ids length", op);
+  FP8K_REQUIRE(lda >= K && ldb >= K && ldq >= I, "%s: leading dimension smaller than the row length", op);
+  FP8K_REQUIRE(lda % 16 == 0 && ldb % 16 == 0 && ldq % 16 == 0, "%s: rows must be 16-byte aligned", op);
+  FP8K_REQUIRE(qs_stride_g >= sorted_capacity, "%s: the scale rows must hold one float per position of sorted_token_ids", op);
+  if (num_valid_tokens == 0 || sorted_capacity < block_m) return FP8K_OK;
+  FP8K_REQUIRE(A && B && As_sorted && Bs && q_out && qs_out && sorted_token_ids && expert_ids && num_tokens_post_padded,
+               "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(A, 16) && aligned(B, 16) && aligned(q_out, 16) && b_stride_e % 16 == 0, "%s: operands must be 16-byte aligned", op);
+  const int64_t xrows = (num_valid_tokens + top_k - 1) / top_k;
+  FP8K_REQUIRE(xrows * lda < 0xE0000000LL, "%s: activation matrix exceeds 3.5 GiB, split the token batch", op);
+  FP8K_REQUIRE(ldb < (1LL << 23) && lda < (1LL << 23), "%s: rows longer than 8 MiB are not supported", op);
+  FP8K_REQUIRE((I + 128) * ldb + K < 0xF0000000LL, "%s: an expert's weight exceeds 3.75 GiB", op);
+  FP8K_REQUIRE(as_stride_k >= sorted_capacity && bs_stride_n >= 0 && bs_stride_k >= 0 && bs_stride_e >= 0, "%s: bad scale stride", op);
+  FP8K_REQUIRE(sorted_capacity + (K / kTileK) * as_stride_k < 0x38000000LL, "%s: activation scale tensor too large", op);
+
+  GemmArgs a{};
+  a.X = (const uint8_t*)A; a.W = (const uint8_t*)B; a.sx = As_sorted; a.sw = Bs; a.C = nullptr;
+  a.M = (int)num_valid_tokens; a.N = (int)N; a.K = (int)K; a.ldx = lda; a.ldw = ldb; a.ldc = 0;
+  a.sx_m = 1; a.sx_k = as_stride_k; a.sw_n = bs_stride_n; a.sw_k = bs_stride_k;
+  a.tiles_m = 0; a.tiles_n = (int)(I / 128);
+  a.splits = 1; a.kb_per_split = (int)(K / kTileK);
+  a.sorted_ids = sorted_token_ids; a.expert_ids = expert_ids; a.num_post_pad = num_tokens_post_padded;
+  a.topk_w = nullptr; a.top_k = (int)top_k; a.num_valid = (int)num_valid_tokens;
+  a.m_blocks = (int)(sorted_capacity / block_m);
+  a.block_m = (int)block_m;
+  a.w_expert_stride = b_stride_e; a.sw_expert_stride = bs_stride_e;
+  a.sx_sorted = 1;
+  a.q_out = (uint8_t*)q_out; a.qs_out = qs_out; a.ldq = ldq; a.qs_ld = qs_stride_g;
+  // the group maximum is clamped in the activation type, as the quantisation kernels do
+  a.q_eps = eps;
+  if (act_dtype == FP8K_BF16) {
+    uint32_t u;
+    memcpy(&u, &eps, 4);
+    u = ((u + 0x7fffu + ((u >> 16) & 1u)) >> 16) << 16;
+    memcpy(&a.q_eps, &u, 4);
+  }
+  const int64_t per_xcd = (a.m_blocks + 7) / 8;
+  const bool walk = num_valid_tokens <= num_experts * 192 && K >= 2 * kTileK;
+  const int64_t nwg = walk ? std::min<int64_t>(per_xcd * 8 * a.tiles_n, std::max(8, num_cu() / 8 * 8)) : per_xcd * 8 * a.tiles_n;
+  FP8K_REQUIRE(nwg < 0x7fffffffLL, "%s: grid too large", op);
+  hipStream_t st = (hipStream_t)stream;
+  if (act_dtype == FP8K_BF16) hipLaunchKernelGGL((moe_stream256_kernel<FP8K_BF16, false, true, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+  else hipLaunchKernelGGL((moe_stream256_kernel<FP8K_F16, false, true, true>), dim3((unsigned)nwg), dim3(512), 0, st, a);
+  return check_launch(op);
+}
+
 extern "C" int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
                                  void* stream) {
   clear_error();

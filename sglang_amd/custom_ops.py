@@ -120,6 +120,14 @@ _register(
 )
 
 
+_register(
+    "moe_block_gemm_silu_quant(Tensor A, Tensor B, Tensor A_scale_sorted, Tensor B_scale, Tensor(a!) out_q, Tensor(b!) out_s, "
+    "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, int top_k, int num_valid_tokens, "
+    "ScalarType act_dtype, float eps=1e-10) -> ()",
+    _k.moe_block_gemm_silu_quant, _none,
+)
+
+
 def _gate_fake(input, bias, num_expert_group, topk_group, topk, num_fused_shared_experts=0, routed_scaling_factor=0.0,
                apply_routed_scaling_factor_on_output=False):
     rows = input.shape[0]
@@ -232,6 +240,12 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
                    mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int, scales_sorted: bool = False) -> None:
     _ops.moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                         mul_routed_weight, top_k, block_m, num_valid_tokens, scales_sorted)
+
+
+def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,
+                              num_tokens_post_padded, top_k: int, num_valid_tokens: int, act_dtype, eps: float = 1e-10) -> None:
+    _ops.moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,
+                                   num_tokens_post_padded, top_k, num_valid_tokens, act_dtype, float(eps))
 
 
 def moe_fused_gate(input_tensor, bias, num_expert_group, topk_group, topk, num_fused_shared_experts=0,

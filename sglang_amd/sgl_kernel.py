@@ -746,6 +746,50 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
     moe_block_gemm(a, b.transpose(1, 2), output, scales_a, bs, None, sorted_ids, expert_ids, post_pad, False, 1, block_m, rows)
 
 
+def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,
+                              num_tokens_post_padded, top_k: int, num_valid_tokens: int, act_dtype: torch.dtype,
+                              eps: float = 1e-10) -> None:
+    """Grouped GEMM 1 of the fused MoE layer (256-slot blocks) with silu_and_mul and the group requantisation inside its
+    write-out (include/fp8k.h: fp8k_moe_block_gemm_silu_quant).  A e4m3fn [rows, K]; B e4m3fn [E, 2 I, K] (gate rows,
+    then up rows); A_scale_sorted float32 [len(sorted_token_ids), K/128] as moe_sort_scales returns it; B_scale float32
+    [E, 2 I/128, K/128]; out_q e4m3fn [num_valid_tokens, I]; out_s float32 [len(sorted_token_ids), I/128] in the same
+    sorted layout (column-major: one row of the underlying [I/128, len] buffer per column block)."""
+    require_cuda(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE or out_q.dtype != FP8_DTYPE:
+        raise RuntimeError("moe_block_gemm_silu_quant: A, B and out_q must be Float8_e4m3fn")
+    if A_scale_sorted.dtype != torch.float32 or B_scale.dtype != torch.float32 or out_s.dtype != torch.float32:
+        raise RuntimeError("moe_block_gemm_silu_quant: scales must be Float32")
+    if B.dim() != 3 or A.dim() != 2 or out_q.dim() != 2:
+        raise RuntimeError("moe_block_gemm_silu_quant: A [rows,K], B [E,2I,K], out_q [slots,I]")
+    E, N, K = B.shape
+    I = N // 2
+    cap = sorted_token_ids.numel()
+    kb = (K + 127) // 128
+    if N % 256 != 0 or A.shape[1] != K or A.stride(1) != 1 or B.stride(2) != 1:
+        raise RuntimeError("moe_block_gemm_silu_quant: N must be 2 I with I a multiple of 128, K contiguous")
+    if tuple(A_scale_sorted.shape) != (cap, kb) or A_scale_sorted.stride(0) != 1:
+        raise RuntimeError("moe_block_gemm_silu_quant: A_scale_sorted must be the [len(sorted_token_ids), K/128] view of moe_sort_scales")
+    if tuple(out_s.shape) != (cap, I // 128) or out_s.stride(0) != 1 or (I // 128 > 1 and out_s.stride(1) < cap):
+        raise RuntimeError("moe_block_gemm_silu_quant: out_s must be a [len(sorted_token_ids), I/128] view with the slots contiguous")
+    if tuple(out_q.shape) != (num_valid_tokens, I) or out_q.stride(1) != 1:
+        raise RuntimeError("moe_block_gemm_silu_quant: out_q must be [num_valid_tokens, I] with I contiguous")
+    if tuple(B_scale.shape) != (E, N // 128, kb):
+        raise RuntimeError("moe_block_gemm_silu_quant: B_scale shape does not match B")
+    if A.shape[0] * top_k < num_valid_tokens:
+        raise RuntimeError("moe_block_gemm_silu_quant: A has too few rows for num_valid_tokens / top_k")
+    for t in (sorted_token_ids, expert_ids, num_tokens_post_padded):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("moe_block_gemm_silu_quant: index tensors must be contiguous int32")
+    if expert_ids.numel() * 256 < cap - (cap % 256):
+        raise RuntimeError("moe_block_gemm_silu_quant: expert_ids is shorter than sorted_token_ids / 256")
+    check(lib.fp8k_moe_block_gemm_silu_quant(
+        A.data_ptr(), B.data_ptr(), A_scale_sorted.data_ptr(), B_scale.data_ptr(), out_q.data_ptr(), out_s.data_ptr(),
+        sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(), cap, num_valid_tokens, top_k, E,
+        N, K, A.stride(0), A_scale_sorted.stride(1) if kb > 1 else cap, B.stride(0), B.stride(1), B_scale.stride(0),
+        B_scale.stride(1), B_scale.stride(2), out_q.stride(0), out_s.stride(1) if I // 128 > 1 else cap, float(eps),
+        dtype_code(act_dtype), stream_ptr(A.device)))
+
+
 def moe_fused_gate(
     input_tensor: torch.Tensor,
     bias: torch.Tensor,

@@ -13,7 +13,7 @@ import torch
 from torch._subclasses.fake_tensor import FakeTensorMode
 
 OPS = ["sgl_per_token_group_quant_8bit", "sgl_per_token_quant_fp8", "sgl_per_tensor_quant_fp8", "fp8_blockwise_scaled_mm",
-       "fp8_scaled_mm", "block_gemm_nk", "block_gemm_nk_ue8m0", "tensor_quant_mla", "bmm_fp8", "prepare_moe_input", "shuffle_rows", "apply_shuffle_mul_sum", "fp8_blockwise_scaled_grouped_mm", "moe_align_block_size", "silu_and_mul", "moe_sum_reduce",
+       "fp8_scaled_mm", "block_gemm_nk", "block_gemm_nk_ue8m0", "tensor_quant_mla", "bmm_fp8", "prepare_moe_input", "shuffle_rows", "apply_shuffle_mul_sum", "fp8_blockwise_scaled_grouped_mm", "moe_block_gemm_silu_quant", "moe_align_block_size", "silu_and_mul", "moe_sum_reduce",
        "moe_sort_scales", "moe_block_gemm", "moe_fused_gate"]
 
 

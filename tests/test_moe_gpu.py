@@ -534,3 +534,60 @@ def test_moe_fused_gate_errors(dev):
         moe_fused_gate(x, torch.zeros((256,), device=dev), 4, 2, 4)
     with pytest.raises(RuntimeError, match="same dtype"):
         moe_fused_gate(x, torch.zeros((256,), device=dev, dtype=torch.bfloat16), 8, 4, 8)
+
+
+@pytest.mark.parametrize("T,E,H,I,topk", [(1024, 8, 512, 256, 2), (700, 4, 256, 128, 4), (2100, 8, 384, 384, 3)])
+@pytest.mark.parametrize("dt", [torch.bfloat16, torch.float16])
+def test_gemm1_with_fused_activation_quant_is_the_three_step_sequence(dev, T, E, H, I, topk, dt):
+    """256-slot blocks: the first grouped GEMM with silu_and_mul and the requantisation in its write-out against the same
+    GEMM into a 16-bit tensor followed by the fused silu + group quant kernel - bytes and scales of every real slot bit
+    for bit, and the whole layer with and without the fusion bit for bit."""
+    import sglang_amd.fused_moe as fm
+    from sglang_amd import custom_ops as ops
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+
+    rng = np.random.default_rng(T + I)
+    x = torch.from_numpy(O.make_activation(T, H, T)).to(dev).to(dt)
+    w13q = np.empty((E, 2 * I, H), np.uint8); w13s = np.empty((E, 2 * I // 128, H // 128), np.float32)
+    w2q = np.empty((E, H, I), np.uint8); w2s = np.empty((E, H // 128, I // 128), np.float32)
+    for e in range(E):
+        w13q[e], w13s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((2 * I, H)).astype(np.float32) * 0.05))
+        w2q[e], w2s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((H, I)).astype(np.float32) * 0.05))
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    if E > 4:
+        ids[ids == 1] = 0  # one expert without tokens, one with twice the share (more than one block)
+    tw = rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32)
+    w1, w2 = fp8_tensor(w13q, dev), fp8_tensor(w2q, dev)
+    s1, s2 = torch.from_numpy(w13s).to(dev), torch.from_numpy(w2s).to(dev)
+    idt, twt = torch.from_numpy(ids).to(dev), torch.from_numpy(tw).to(dev)
+    slots = T * topk
+
+    sorted_ids, expert_ids, post_pad = fm.moe_align_block_size(idt, 256, E)
+    a1_q, a1_s = sglang_per_token_group_quant_fp8(x, 128)
+    a1_ss = ops.moe_sort_scales(a1_s, sorted_ids, post_pad, topk, slots)
+    c1 = torch.empty((slots, 2 * I), device=dev, dtype=dt)
+    ops.moe_block_gemm(a1_q, w1, c1, a1_ss, s1, None, sorted_ids, expert_ids, post_pad, False, topk, 256, slots, scales_sorted=True)
+    ref_q, ref_s = sglang_per_token_group_quant_fp8(c1, 128, fuse_silu_and_mul=True)
+    got_q = torch.zeros((slots, I), device=dev, dtype=torch.float8_e4m3fn)
+    got_s = torch.full((I // 128, sorted_ids.numel()), -1.0, device=dev, dtype=torch.float32).t()
+    ops.moe_block_gemm_silu_quant(a1_q, w1, a1_ss, s1, got_q, got_s, sorted_ids, expert_ids, post_pad, topk, slots, dt)
+    torch.cuda.synchronize()
+    assert torch.equal(got_q.view(torch.uint8), ref_q.view(torch.uint8))
+    sid = sorted_ids[: int(post_pad.item())].long()
+    real = sid < slots
+    assert torch.equal(got_s[: sid.numel()][real], ref_s[sid[real]])
+    assert bool((got_s[: sid.numel()][~real] == 0).all())
+
+    kw = dict(use_fp8_w8a8=True, w1_scale=s1, w2_scale=s2, block_shape=[128, 128])
+    old = fm.get_default_config
+    fm.get_default_config = lambda M_, E_, t_: {"BLOCK_SIZE_M": 256, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}
+    keep = fm.FUSE_ACT_QUANT_INTO_GEMM1
+    try:
+        fm.FUSE_ACT_QUANT_INTO_GEMM1 = True
+        fused = fm.fused_experts_impl(x, w1, w2, twt, idt, **kw)
+        fm.FUSE_ACT_QUANT_INTO_GEMM1 = False
+        plain = fm.fused_experts_impl(x, w1, w2, twt, idt, **kw)
+    finally:
+        fm.FUSE_ACT_QUANT_INTO_GEMM1 = keep
+        fm.get_default_config = old
+    assert torch.equal(fused, plain)
