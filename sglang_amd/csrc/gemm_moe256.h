@@ -288,19 +288,49 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
         wf[ns][0] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 0);
         wf[ns][1] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 1);
       }
+      v16f z;
 #pragma unroll
-      for (int ms = 0; ms < NA; ++ms) {  // groups past the expert's last slot are padding
-        const v8i x0 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 0);
-        const v8i x1 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 1);
+      for (int r = 0; r < 16; ++r) z[r] = 0.f;
+      if constexpr (NA <= 3) {
+        // two products in flight: the 16 scale-FMAs of one 32x32 product issue while the matrix core works on the
+        // next (with one product at a time the wave sits out the matrix core's latency in front of every group of
+        // FMAs, and with two waves per SIMD nobody else fills it).  The four-group copy has no registers for it.
+        v16f tq[2];
+        v8i x0 = frag(sx_ + (wm * 32) * kTileK, 0);
+        v8i x1 = frag(sx_ + (wm * 32) * kTileK, 1);
+        tq[0] = mfma_32x32x64(wf[0][0], x0, z);
+        tq[0] = mfma_32x32x64(wf[0][1], x1, tq[0]);
 #pragma unroll
-        for (int ns = 0; ns < NS; ++ns) {
-          v16f z;
+        for (int i = 1; i < NA * NS; ++i) {
+          const int ms = i >> 1, ns = i & 1;
+          if (ns == 0) {
+            x0 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 0);
+            x1 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 1);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          tq[i & 1] = mfma_32x32x64(wf[ns][0], x0, z);
+          tq[i & 1] = mfma_32x32x64(wf[ns][1], x1, tq[i & 1]);
+          __builtin_amdgcn_sched_barrier(0);
+          const int pm = (i - 1) >> 1, pn = (i - 1) & 1;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) z[r] = 0.f;
-          v16f tq = mfma_32x32x64(wf[ns][0], x0, z);
-          tq = mfma_32x32x64(wf[ns][1], x1, tq);
+          for (int r = 0; r < 16; ++r) acc[pn][pm][r] = __builtin_fmaf(tq[(i - 1) & 1][r], sc[pm], acc[pn][pm][r]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        constexpr int L = NA * NS - 1;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) acc[ns][ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ns][ms][r]);
+        for (int r = 0; r < 16; ++r) acc[L & 1][L >> 1][r] = __builtin_fmaf(tq[L & 1][r], sc[L >> 1], acc[L & 1][L >> 1][r]);
+      } else {
+#pragma unroll
+        for (int ms = 0; ms < NA; ++ms) {  // groups past the expert's last slot are padding
+          const v8i x0 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 0);
+          const v8i x1 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 1);
+#pragma unroll
+          for (int ns = 0; ns < NS; ++ns) {
+            v16f tq = mfma_32x32x64(wf[ns][0], x0, z);
+            tq = mfma_32x32x64(wf[ns][1], x1, tq);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[ns][ms][r] = __builtin_fmaf(tq[r], sc[ms], acc[ns][ms][r]);
+          }
         }
       }
     };
