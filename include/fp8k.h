@@ -244,6 +244,24 @@ int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const flo
                         int out_dtype, int as_sorted, void* stream);
 
 /*
+ * fp8k_moe_block_gemm for scale tensors that hold only powers of two (UE8M0 checkpoints, activations quantised with
+ * scale_ue8m0): same arguments, same result up to the rounding of the accumulation.  With block_m == 256 and
+ * as_sorted != 0 the matrix cores apply both scales themselves (v_mfma_scale_f32_32x32x64_f8f6f4 with the exponent
+ * byte of each float) and the products accumulate in place; every other block size runs the kernels of
+ * fp8k_moe_block_gemm.  A scale that is not a power of two is truncated to one (its mantissa is ignored): the caller
+ * vouches for the tensors, as SGLang does when DEEPGEMM_SCALE_UE8M0 is set
+ *   (python/sglang/srt/layers/deep_gemm_wrapper/configurer.py, python/sglang/srt/layers/quantization/fp8_utils.py:229-268);
+ * the grouped entry points this serves are python/sglang/srt/layers/deep_gemm_wrapper/entrypoint.py:26-67.
+ */
+int fp8k_moe_block_gemm_ue8m0(const void* A, const void* B, const float* As, const float* Bs, void* C,
+                              const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                              const int32_t* num_tokens_post_padded, const float* topk_weights, int64_t sorted_capacity,
+                              int64_t block_m, int64_t num_valid_tokens, int64_t top_k, int64_t num_experts, int64_t N,
+                              int64_t K, int64_t lda, int64_t as_stride_m, int64_t as_stride_k, int64_t b_stride_e,
+                              int64_t ldb, int64_t bs_stride_e, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc,
+                              int out_dtype, int as_sorted, void* stream);
+
+/*
  * Expert-major row layout for the grouped GEMM (integer work): the (token, k) slots of topk_ids int32 [numel] sorted by
  * expert into contiguous, un-padded row ranges.
  * Replaces torch.ops.sgl_kernel.prepare_moe_input (sgl-kernel/python/sgl_kernel/moe.py:217-240,

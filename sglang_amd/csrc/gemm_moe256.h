@@ -34,9 +34,13 @@ namespace fp8k {
 // write-out produces what silu_and_mul followed by the group quantisation would have made of the 16-bit GEMM result,
 // bit for bit: q_out[slot, n0 .. n0+127] and one scale per slot in the sorted order GEMM 2 reads.  The [slots, 2 I]
 // intermediate is never written.
-template <int OUT_DT, bool PAIRS, bool SORTED, bool FUSE = false>
+// SCALED (sorted scales only): both scale tensors hold powers of two (UE8M0 checkpoints with UE8M0-rounded activation
+// scales) and the matrix core applies them itself (v_mfma_scale_f32_32x32x64_f8f6f4 takes the two exponent bytes):
+// the products accumulate in place, the float promote and its second accumulator disappear.
+template <int OUT_DT, bool PAIRS, bool SORTED, bool FUSE = false, bool SCALED = false>
 __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p) {
   static_assert(!FUSE || (SORTED && !PAIRS), "the fused write-out is built for sorted activation scales");
+  static_assert(!SCALED || (SORTED && !PAIRS && !FUSE), "hardware scaling is built for sorted activation scales");
   constexpr int TM = 256, WST = 3, XST = 2, MS = 4, NS = 2, LW = 4;  // LW: wave loads per tile per stage
   constexpr int WBYTES = kTileN * kTileK, XBYTES = TM * kTileK;
   constexpr int XBASE = WST * WBYTES;
@@ -258,7 +262,8 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       // the scale loads of the previous trip with them, and loads return in order - that wait would also be one for
       // the weight block requested before those scales
       __builtin_amdgcn_sched_barrier(0);
-      float sc[MS];
+      float sc[MS];  // SCALED: the exponent byte of the activation scale, as bits
+      int sc_w = 127;  // SCALED: exponent byte of the weight scale
       if (pairs) {
 #pragma unroll
         for (int ms = 0; ms < MS; ++ms) sc[ms] = sxp[ms][parity] * sb;
@@ -266,7 +271,8 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
         load_sb(sb, it + 2);
       } else {
 #pragma unroll
-        for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
+        for (int ms = 0; ms < MS; ++ms) sc[ms] = SCALED ? __uint_as_float(__float_as_uint(sxn[ms]) >> 23) : sxn[ms] * sbn;
+        if (SCALED) sc_w = (int)(__float_as_uint(sbn) >> 23);
         load_sx(it + 1);
         load_sb(sbn, it + 1);
       }
@@ -291,7 +297,19 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       v16f z;
 #pragma unroll
       for (int r = 0; r < 16; ++r) z[r] = 0.f;
-      if constexpr (NA <= 3) {
+      if constexpr (SCALED) {
+#pragma unroll
+        for (int ms = 0; ms < NA; ++ms) {
+          const v8i x0 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 0);
+          const v8i x1 = frag(sx_ + ((ms * 2 + wm) * 32) * kTileK, 1);
+          const int ex = (int)__float_as_uint(sc[ms]);
+#pragma unroll
+          for (int ns = 0; ns < NS; ++ns) {
+            acc[ns][ms] = mfma_32x32x64_scaled(wf[ns][0], x0, acc[ns][ms], sc_w, ex);
+            acc[ns][ms] = mfma_32x32x64_scaled(wf[ns][1], x1, acc[ns][ms], sc_w, ex);
+          }
+        }
+      } else if constexpr (NA <= 3) {
         // two products in flight: the 16 scale-FMAs of one 32x32 product issue while the matrix core works on the
         // next (with one product at a time the wave sits out the matrix core's latency in front of every group of
         // FMAs, and with two waves per SIMD nobody else fills it).  The four-group copy has no registers for it.

@@ -288,16 +288,16 @@ extern "C" int fp8k_moe_sort_scales(const float* As, float* out, const int32_t* 
   return check_launch(op);
 }
 
-extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
-                                   const int32_t* sorted_token_ids, const int32_t* expert_ids,
-                                   const int32_t* num_tokens_post_padded, const float* topk_weights,
-                                   int64_t sorted_capacity, int64_t block_m, int64_t num_valid_tokens, int64_t top_k,
-                                   int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_m,
-                                   int64_t as_stride_k, int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e,
-                                   int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, int as_sorted,
-                                   void* stream) {
+static int moe_block_gemm_impl(const void* A, const void* B, const float* As, const float* Bs, void* C,
+                               const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                               const int32_t* num_tokens_post_padded, const float* topk_weights,
+                               int64_t sorted_capacity, int64_t block_m, int64_t num_valid_tokens, int64_t top_k,
+                               int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_m,
+                               int64_t as_stride_k, int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e,
+                               int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, int as_sorted,
+                               bool pow2_scales, void* stream) {
   clear_error();
-  const char* op = "moe_block_gemm";
+  const char* op = pow2_scales ? "moe_block_gemm_ue8m0" : "moe_block_gemm";
   FP8K_REQUIRE(N > 0 && K > 0 && num_experts > 0 && top_k > 0, "%s: bad shape", op);
   FP8K_REQUIRE(N <= 0x7fffffffLL && K <= 0x7fffffffLL && num_valid_tokens >= 0 && num_valid_tokens < 0x7fffffffLL,
                "%s: shape too large", op);
@@ -367,6 +367,7 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
 #define FP8K_MOE256(O) \
   do { \
     if (pairs) hipLaunchKernelGGL((moe_stream256_kernel<O, true, false>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
+    else if (as_sorted && pow2_scales) hipLaunchKernelGGL((moe_stream256_kernel<O, false, true, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
     else if (as_sorted) hipLaunchKernelGGL((moe_stream256_kernel<O, false, true>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
     else hipLaunchKernelGGL((moe_stream256_kernel<O, false, false>), dim3((unsigned)nwg), dim3(512), 0, st, a); \
   } while (0)
@@ -386,6 +387,34 @@ extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As
   }
 #undef FP8K_MOE
   return check_launch(op);
+}
+
+extern "C" int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
+                                   const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                   const int32_t* num_tokens_post_padded, const float* topk_weights,
+                                   int64_t sorted_capacity, int64_t block_m, int64_t num_valid_tokens, int64_t top_k,
+                                   int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_m,
+                                   int64_t as_stride_k, int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e,
+                                   int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, int as_sorted,
+                                   void* stream) {
+  return moe_block_gemm_impl(A, B, As, Bs, C, sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights,
+                             sorted_capacity, block_m, num_valid_tokens, top_k, num_experts, N, K, lda, as_stride_m,
+                             as_stride_k, b_stride_e, ldb, bs_stride_e, bs_stride_n, bs_stride_k, ldc, out_dtype, as_sorted,
+                             false, stream);
+}
+
+extern "C" int fp8k_moe_block_gemm_ue8m0(const void* A, const void* B, const float* As, const float* Bs, void* C,
+                                         const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                         const int32_t* num_tokens_post_padded, const float* topk_weights,
+                                         int64_t sorted_capacity, int64_t block_m, int64_t num_valid_tokens, int64_t top_k,
+                                         int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_m,
+                                         int64_t as_stride_k, int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e,
+                                         int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype,
+                                         int as_sorted, void* stream) {
+  return moe_block_gemm_impl(A, B, As, Bs, C, sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights,
+                             sorted_capacity, block_m, num_valid_tokens, top_k, num_experts, N, K, lda, as_stride_m,
+                             as_stride_k, b_stride_e, ldb, bs_stride_e, bs_stride_n, bs_stride_k, ldc, out_dtype, as_sorted,
+                             true, stream);
 }
 
 extern "C" int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, const float* As_sorted, const float* Bs, void* q_out,

@@ -115,7 +115,7 @@ _register("moe_sort_scales(Tensor A_scale, Tensor sorted_token_ids, Tensor num_t
 _register(
     "moe_block_gemm(Tensor A, Tensor B, Tensor(a!) C, Tensor A_scale, Tensor B_scale, Tensor? topk_weights, "
     "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, bool mul_routed_weight, int top_k, "
-    "int block_m, int num_valid_tokens, bool scales_sorted=False) -> ()",
+    "int block_m, int num_valid_tokens, bool scales_sorted=False, bool pow2_scales=False) -> ()",
     _k.moe_block_gemm, _none,
 )
 
@@ -237,9 +237,10 @@ def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: in
 
 
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                   mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int, scales_sorted: bool = False) -> None:
+                   mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int, scales_sorted: bool = False,
+                   pow2_scales: bool = False) -> None:
     _ops.moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                        mul_routed_weight, top_k, block_m, num_valid_tokens, scales_sorted)
+                        mul_routed_weight, top_k, block_m, num_valid_tokens, scales_sorted, pow2_scales)
 
 
 def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,

@@ -13,7 +13,9 @@ accumulation.  The grouped forms run on the grouped MoE GEMM: the group of every
 sorts the rows into per-group blocks, and each row is its own token slot (top_k = 1, no routed weight).
 Scales are float32, or packed UE8M0 words (int32: [.., m, ceil(k/128/4)] for the activations, one row per weight row
 [.., n, ceil(k/128/4)] for the weights, the layout the reference prepares for DeepGEMM on Blackwell, fp8_kernel.py:
-1018-1043); the grouped kernels take float scales, so packed words are expanded to powers of two first.
+1018-1043); the grouped kernels take float scales, so packed words are expanded to powers of two first.  When BOTH
+tensors arrive packed every scale is a power of two, and 256-row blocks let the matrix cores apply them
+(fp8k_moe_block_gemm_ue8m0) instead of the float promote.
 """
 from typing import Tuple
 
@@ -36,13 +38,15 @@ def _check_pair(name: str, x: Tuple[torch.Tensor, torch.Tensor]) -> None:
 
 
 def _float_scales(a, a_s, b, b_s):
-    """Packed UE8M0 words -> float32 powers of two (activations per row, weights per 128-row block)."""
+    """Packed UE8M0 words -> float32 powers of two (activations per row, weights per 128-row block); the third
+    result says whether both tensors came packed (then every scale is a power of two by construction)."""
     k = a.shape[-1]
+    pow2 = a_s.dtype == torch.int32 and b_s.dtype == torch.int32
     if a_s.dtype == torch.int32:
         a_s = unpack_ue8m0_scales(a_s, (k + 127) // 128)
     if b_s.dtype == torch.int32:
         b_s = unpack_ue8m0_weight_scales(b_s, k)
-    return a_s, b_s
+    return a_s, b_s, pow2
 
 
 def gemm_nt_f8f8bf16(lhs: Tuple[torch.Tensor, torch.Tensor], rhs: Tuple[torch.Tensor, torch.Tensor], out: torch.Tensor):
@@ -55,13 +59,18 @@ def gemm_nt_f8f8bf16(lhs: Tuple[torch.Tensor, torch.Tensor], rhs: Tuple[torch.Te
     out.copy_(res)
 
 
-def _grouped(a, a_s, b, b_s, out, row_group: torch.Tensor, rows_per_group: int) -> None:
+def _grouped(a, a_s, b, b_s, out, row_group: torch.Tensor, rows_per_group: int, pow2: bool) -> None:
     G = b.shape[0]
     rows = a.shape[0]
     if rows == 0:
         return
     block_m = get_default_config(max(rows_per_group, 1) * G, G, 1)["BLOCK_SIZE_M"]
     sorted_ids, expert_ids, num_post_pad = moe_align_block_size(row_group, block_m, G)
+    if pow2 and block_m == 256:
+        a_s = _ops.moe_sort_scales(a_s, sorted_ids, num_post_pad, 1, rows)
+        _ops.moe_block_gemm(a, b, out, a_s, b_s, None, sorted_ids, expert_ids, num_post_pad, False, 1, block_m, rows,
+                            True, True)
+        return
     _ops.moe_block_gemm(a, b, out, a_s, b_s, None, sorted_ids, expert_ids, num_post_pad, False, 1, block_m, rows)
 
 
@@ -75,12 +84,12 @@ def grouped_gemm_nt_f8f8bf16_contig(
     _check_pair("rhs", rhs)
     a, a_s = lhs
     b, b_s = rhs
-    a_s, b_s = _float_scales(a, a_s, b, b_s)
+    a_s, b_s, pow2 = _float_scales(a, a_s, b, b_s)
     if a.dim() != 2 or b.dim() != 3 or m_indices.numel() != a.shape[0]:
         raise RuntimeError("grouped_gemm_nt_f8f8bf16_contig: lhs [m,k], rhs [G,n,k], m_indices [m]")
     idx = m_indices.to(torch.int32)
     idx = torch.where(idx < 0, torch.full_like(idx, _IGNORED), idx)
-    _grouped(a, a_s, b, b_s, out, idx, (a.shape[0] + b.shape[0] - 1) // b.shape[0])
+    _grouped(a, a_s, b, b_s, out, idx, (a.shape[0] + b.shape[0] - 1) // b.shape[0], pow2)
 
 
 def grouped_gemm_nt_f8f8bf16_masked(
@@ -93,7 +102,7 @@ def grouped_gemm_nt_f8f8bf16_masked(
     _check_pair("rhs", rhs)
     a, a_s = lhs
     b, b_s = rhs
-    a_s, b_s = _float_scales(a, a_s, b, b_s)
+    a_s, b_s, pow2 = _float_scales(a, a_s, b, b_s)
     if a.dim() != 3 or b.dim() != 3 or a.shape[0] != b.shape[0] or masked_m.numel() != a.shape[0]:
         raise RuntimeError("grouped_gemm_nt_f8f8bf16_masked: lhs [G,m_max,k], rhs [G,n,k], masked_m [G]")
     G, m_max, k = a.shape
@@ -103,4 +112,4 @@ def grouped_gemm_nt_f8f8bf16_masked(
     row = torch.arange(m_max, device=dev, dtype=torch.int32)[None, :]
     grp = torch.arange(G, device=dev, dtype=torch.int32)[:, None]
     idx = torch.where(row < masked_m.to(torch.int32)[:, None], grp, torch.full_like(grp, _IGNORED)).reshape(-1)
-    _grouped(a.view(G * m_max, k), a_s.reshape(G * m_max, -1), b, b_s, out.view(G * m_max, -1), idx, max(int(expected_m), 1))
+    _grouped(a.view(G * m_max, k), a_s.reshape(G * m_max, -1), b, b_s, out.view(G * m_max, -1), idx, max(int(expected_m), 1), pow2)

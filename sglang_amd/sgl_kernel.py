@@ -580,11 +580,13 @@ def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: in
 
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                    mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int,
-                   scales_sorted: bool = False) -> None:
+                   scales_sorted: bool = False, pow2_scales: bool = False) -> None:
     """Grouped block-FP8 GEMM behind invoke_fused_moe_kernel (see include/fp8k.h: fp8k_moe_block_gemm).
     A e4m3fn [rows, K]; B e4m3fn [E, N, K]; A_scale float32 [rows, K/128] (scales_sorted: one row per entry of
     sorted_token_ids, from moe_sort_scales); B_scale float32 [E, N/128, K/128];
-    C [num_valid_tokens, N] (any leading shape, flattened) bf16/fp16, written in place."""
+    C [num_valid_tokens, N] (any leading shape, flattened) bf16/fp16, written in place.
+    pow2_scales: the caller vouches that every scale is a power of two (UE8M0); 256-slot blocks with sorted scales
+    then let the matrix cores apply the scales (fp8k_moe_block_gemm_ue8m0)."""
     require_cuda(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded)
     if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
         raise RuntimeError("moe_block_gemm: A and B must be Float8_e4m3fn")
@@ -613,7 +615,7 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
     if expert_ids.numel() * block_m < sorted_token_ids.numel() - (sorted_token_ids.numel() % block_m):
         raise RuntimeError("moe_block_gemm: expert_ids is shorter than sorted_token_ids / block_m")
     check(
-        lib.fp8k_moe_block_gemm(
+        (lib.fp8k_moe_block_gemm_ue8m0 if pow2_scales else lib.fp8k_moe_block_gemm)(
             A.data_ptr(), B.data_ptr(), A_scale.data_ptr(), B_scale.data_ptr(), C2.data_ptr(),
             sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(),
             topk_weights.data_ptr() if mul_routed_weight else None, sorted_token_ids.numel(), block_m,

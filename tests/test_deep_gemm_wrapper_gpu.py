@@ -121,3 +121,68 @@ def test_grouped_masked_with_packed_ue8m0_scales(dev):
             ref = O.w8a8_block_fp8_matmul(aq[g, :m], bq[g], a_s[g, :m], b_s[g], acc=np.float64)
             assert _rel(got[g, :m], ref) <= REL_TOL
         assert (got[g, m:] == 7.0).all()
+
+
+@pytest.mark.parametrize("G,m_max,masked,N,K,expected_m", [
+    (4, 320, [320, 0, 131, 257], 256, 640, 300),      # 256-row blocks, ragged tails, an empty group
+    (2, 512, [512, 100], 384, 256, 512),              # two trips of K only; N not a multiple of 256
+    (3, 200, [200, 199, 1], 128, 2048, 128),          # one 128-column tile, long K
+])
+def test_grouped_masked_packed_scales_on_the_hardware_scaled_kernel(dev, G, m_max, masked, N, K, expected_m):
+    """Both scale tensors packed and enough rows per group for 256-row blocks: the matrix cores apply the exponents
+    (fp8k_moe_block_gemm_ue8m0).  Oracle parity to the tolerance of the other GEMMs, untouched rows stay untouched,
+    and the result agrees with the float-scale kernels on the same powers of two to bf16 rounding."""
+    from sglang_amd.deep_gemm_wrapper import grouped_gemm_nt_f8f8bf16_masked
+    from sglang_amd.fused_moe import get_default_config
+
+    assert get_default_config(expected_m * G, G, 1)["BLOCK_SIZE_M"] == 256
+    rng = np.random.default_rng(G * 1000 + K)
+    masked = np.array(masked, dtype=np.int32)
+    aq, bq = _codes(rng, (G, m_max, K)), _codes(rng, (G, N, K))
+    a_s = (2.0 ** rng.integers(-12, 3, (G, m_max, K // 128))).astype(np.float32)
+    b_s = (2.0 ** rng.integers(-12, 3, (G, N // 128, K // 128))).astype(np.float32)
+    a_p = torch.from_numpy(np.stack([O.pack_ue8m0_scales(x) for x in a_s])).to(dev)
+    b_p = torch.from_numpy(np.stack([O.pack_ue8m0_scales(np.repeat(x, 128, axis=0)) for x in b_s])).to(dev)
+    A, B = fp8_tensor(aq, dev), fp8_tensor(bq, dev)
+    mm = torch.from_numpy(masked).to(dev)
+    out = torch.full((G, m_max, N), 7.0, device=dev, dtype=torch.bfloat16)
+    grouped_gemm_nt_f8f8bf16_masked((A, a_p), (B, b_p), out, mm, expected_m)
+    out_f = torch.full((G, m_max, N), 7.0, device=dev, dtype=torch.bfloat16)
+    grouped_gemm_nt_f8f8bf16_masked((A, torch.from_numpy(a_s).to(dev)), (B, torch.from_numpy(b_s).to(dev)), out_f, mm, expected_m)
+    got, got_f = out.float().cpu().numpy(), out_f.float().cpu().numpy()
+    for g in range(G):
+        m = int(masked[g])
+        if m:
+            ref = O.w8a8_block_fp8_matmul(aq[g, :m], bq[g], a_s[g, :m], b_s[g], acc=np.float64)
+            assert _rel(got[g, :m], ref) <= REL_TOL
+            assert _rel(got[g, :m], got_f[g, :m]) <= 2.0 ** -7
+        assert (got[g, m:] == 7.0).all()
+
+
+def test_grouped_contiguous_packed_scales_on_the_hardware_scaled_kernel(dev):
+    """The contiguous layout with packed scales and 256-row blocks; rows marked -1 stay untouched."""
+    from sglang_amd.deep_gemm_wrapper import grouped_gemm_nt_f8f8bf16_contig
+
+    rng = np.random.default_rng(77)
+    G, N, K = 3, 512, 1024
+    rows = [384, 256, 640]
+    real = [300, 256, 513]
+    M = sum(rows)
+    idx = np.full(M, -1, dtype=np.int32)
+    start = 0
+    for g in range(G):
+        idx[start:start + real[g]] = g
+        start += rows[g]
+    aq, bq = _codes(rng, (M, K)), _codes(rng, (G, N, K))
+    a_s = (2.0 ** rng.integers(-10, 0, (M, K // 128))).astype(np.float32)
+    b_s = (2.0 ** rng.integers(-10, 0, (G, N // 128, K // 128))).astype(np.float32)
+    a_p = torch.from_numpy(O.pack_ue8m0_scales(a_s)).to(dev)
+    b_p = torch.from_numpy(np.stack([O.pack_ue8m0_scales(np.repeat(x, 128, axis=0)) for x in b_s])).to(dev)
+    out = torch.full((M, N), 7.0, device=dev, dtype=torch.bfloat16)
+    grouped_gemm_nt_f8f8bf16_contig((fp8_tensor(aq, dev), a_p), (fp8_tensor(bq, dev), b_p), out, torch.from_numpy(idx).to(dev))
+    got = out.float().cpu().numpy()
+    for g in range(G):
+        sel = np.nonzero(idx == g)[0]
+        ref = O.w8a8_block_fp8_matmul(aq[sel], bq[g], a_s[sel], b_s[g], acc=np.float64)
+        assert _rel(got[sel], ref) <= REL_TOL
+    assert (got[idx < 0] == 7.0).all()
