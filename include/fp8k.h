@@ -213,7 +213,8 @@ int fp8k_bmm_fp8(const void* A, const void* B, const float* sa, const float* sb,
  * Outputs: sorted_token_ids - for every bucket in use, its flat id positions (order inside a bucket is
  *   unspecified) followed, when pad_sorted_token_ids, by the value numel up to a multiple of block_size;
  *   expert_ids[b] = bucket-1 of block b for b < post_pad/block_size; num_tokens_post_pad[0] = slots in use.
- * cumsum_buffer: num_buckets+1 ints of scratch (start offsets; consumed), may be NULL when numel <= 65536.
+ * cumsum_buffer: num_buckets+1 ints of scratch (consumed); with it more than 8192 ids are counted and placed by one
+ *   workgroup per 4096 ids (four launches); NULL: a single workgroup does all the work whatever numel is.
  * Capacities are checked against the worst case numel + min(numel, num_buckets)*(block_size-1).
  */
 int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64, int64_t numel, int64_t num_buckets,

@@ -13,11 +13,11 @@ namespace fp8k {
 // id -1) with LDS atomics, an exclusive scan of the counts rounded up to the block size by the first
 // wavefront, then per-block expert ids by binary search, the scatter of token slots through LDS
 // cursors and the padding tail of every bucket.  Ids outside [-1, buckets-1) are ignored.
-// With SCATTER = false the kernel stops after writing the start offsets to `cumsum`, and
-// moe_scatter_kernel (many workgroups, global atomics on `cumsum`) places the slots.
+// With SCATTER = false the kernel stops after writing the start offsets to `cumsum` (the many-id path below).
 // ------------------------------------------------------------------------------------------------
 constexpr int kAlignThreads = 1024;
 constexpr int kAlignMaxBuckets = 4096;
+constexpr int64_t kAlignFusedMax = 8192;  // ids up to which one workgroup does the whole job
 
 template <typename IdT>
 __device__ __forceinline__ int bucket_of(const IdT* ids, int64_t i, int nb) {
@@ -25,7 +25,78 @@ __device__ __forceinline__ int bucket_of(const IdT* ids, int64_t i, int nb) {
   return (b >= 0 && b < nb) ? (int)b : -1;
 }
 
-template <typename IdT, bool SCATTER>
+// histogram of ids[first, last) into an LDS table (zeroed by the caller, barriers around the call are the caller's):
+// eight ids per lane and trip, eight loads in flight instead of one load latency per id
+template <typename IdT>
+__device__ __forceinline__ void count_ids(const IdT* __restrict__ ids, int64_t first, int64_t last, int nb, int32_t* counts) {
+  for (int64_t i0 = first + threadIdx.x; i0 < last; i0 += 8 * kAlignThreads) {
+    int b8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t i = i0 + (int64_t)u * kAlignThreads;
+      b8[u] = i < last ? bucket_of(ids, i, nb) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (b8[u] >= 0) atomicAdd(&counts[b8[u]], 1);
+  }
+}
+// ids[first, last) to their places: cursor[b] (LDS) is the next free position of bucket b
+template <typename IdT>
+__device__ __forceinline__ void place_ids(const IdT* __restrict__ ids, int64_t first, int64_t last, int nb, int32_t* cursor,
+                                          int32_t* __restrict__ sorted) {
+  for (int64_t i0 = first + threadIdx.x; i0 < last; i0 += 8 * kAlignThreads) {
+    int b8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int64_t i = i0 + (int64_t)u * kAlignThreads;
+      b8[u] = i < last ? bucket_of(ids, i, nb) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (b8[u] >= 0) sorted[atomicAdd(&cursor[b8[u]], 1)] = (int32_t)(i0 + (int64_t)u * kAlignThreads);
+  }
+}
+
+// Many ids: the histogram and the placement are spread over workgroups that each take a contiguous run of
+// kAlignChunk ids.  moe_count_kernel adds every workgroup's LDS histogram to the (zeroed) global table, the single
+// workgroup of moe_align_kernel<PRECOUNTED> turns the table into start offsets, and moe_place_kernel reserves a
+// workgroup's share of every bucket with one global atomic per bucket in use and places its ids through LDS cursors.
+constexpr int kAlignChunk = 4096;
+__global__ __launch_bounds__(256) void zero_ints_kernel(int32_t* __restrict__ p, int n) {
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+template <typename IdT>
+__global__ __launch_bounds__(kAlignThreads) void moe_count_kernel(const IdT* __restrict__ ids, int64_t numel, int nb,
+                                                                  int32_t* __restrict__ table) {
+  __shared__ int32_t counts[kAlignMaxBuckets];
+  for (int b = threadIdx.x; b < nb; b += kAlignThreads) counts[b] = 0;
+  __syncthreads();
+  const int64_t first = (int64_t)blockIdx.x * kAlignChunk;
+  count_ids(ids, first, min(numel, first + kAlignChunk), nb, counts);
+  __syncthreads();
+  for (int b = threadIdx.x; b < nb; b += kAlignThreads)
+    if (counts[b]) atomicAdd(&table[b], counts[b]);
+}
+template <typename IdT>
+__global__ __launch_bounds__(kAlignThreads) void moe_place_kernel(const IdT* __restrict__ ids, int64_t numel, int nb,
+                                                                  int32_t* __restrict__ sorted, int32_t* __restrict__ cumsum) {
+  __shared__ int32_t counts[kAlignMaxBuckets];
+  for (int b = threadIdx.x; b < nb; b += kAlignThreads) counts[b] = 0;
+  __syncthreads();
+  const int64_t first = (int64_t)blockIdx.x * kAlignChunk, last = min(numel, first + kAlignChunk);
+  count_ids(ids, first, last, nb, counts);
+  __syncthreads();
+  for (int b = threadIdx.x; b < nb; b += kAlignThreads) {
+    const int c = counts[b];
+    counts[b] = c ? atomicAdd(&cumsum[b], c) : 0;  // from here on the workgroup's cursor inside bucket b
+  }
+  __syncthreads();
+  place_ids(ids, first, last, nb, counts, sorted);
+}
+
+template <typename IdT, bool SCATTER, bool PRECOUNTED = false>
 __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const IdT* __restrict__ ids, int64_t numel, int nb,
                                                                   int block, int32_t* __restrict__ sorted,
                                                                   int32_t* __restrict__ expert_ids,
@@ -35,19 +106,12 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const IdT* __r
   __shared__ int32_t prefix[kAlignMaxBuckets + 1];
   __shared__ int32_t cursor[kAlignMaxBuckets];
   const int tid = threadIdx.x;
-  for (int b = tid; b < nb; b += kAlignThreads) counts[b] = 0;
-  __syncthreads();
-  // eight ids per lane and trip: eight loads in flight instead of one load latency per id
-  for (int64_t i0 = tid; i0 < numel; i0 += 8 * kAlignThreads) {
-    int b8[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) {
-      const int64_t i = i0 + (int64_t)u * kAlignThreads;
-      b8[u] = i < numel ? bucket_of(ids, i, nb) : -1;
-    }
-#pragma unroll
-    for (int u = 0; u < 8; ++u)
-      if (b8[u] >= 0) atomicAdd(&counts[b8[u]], 1);
+  if (PRECOUNTED) {  // cumsum holds the histogram (moe_count_kernel)
+    for (int b = tid; b < nb; b += kAlignThreads) counts[b] = cumsum[b];
+  } else {
+    for (int b = tid; b < nb; b += kAlignThreads) counts[b] = 0;
+    __syncthreads();
+    count_ids(ids, 0, numel, nb, counts);
   }
   __syncthreads();
   if (tid < 64) {
@@ -89,32 +153,13 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const IdT* __r
     expert_ids[i] = lo - 1;
   }
   if (pad_ids) {
-    for (int b = tid; b < nb; b += kAlignThreads)
-      for (int j = prefix[b] + counts[b]; j < prefix[b + 1]; ++j) sorted[j] = (int32_t)numel;
+    // a wavefront per bucket, a lane per slot: up to block-1 slots per bucket, far too many for one lane each
+    for (int b = tid >> 6; b < nb; b += kAlignThreads / 64)
+      for (int j = prefix[b] + counts[b] + (tid & 63); j < prefix[b + 1]; j += 64) sorted[j] = (int32_t)numel;
   }
   if (SCATTER) {
     __syncthreads();
-    for (int64_t i0 = tid; i0 < numel; i0 += 8 * kAlignThreads) {
-      int b8[8];
-#pragma unroll
-      for (int u = 0; u < 8; ++u) {
-        const int64_t i = i0 + (int64_t)u * kAlignThreads;
-        b8[u] = i < numel ? bucket_of(ids, i, nb) : -1;
-      }
-#pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (b8[u] >= 0) sorted[atomicAdd(&cursor[b8[u]], 1)] = (int32_t)(i0 + (int64_t)u * kAlignThreads);
-    }
-  }
-}
-
-template <typename IdT>
-__global__ __launch_bounds__(256) void moe_scatter_kernel(const IdT* __restrict__ ids, int64_t numel, int nb,
-                                                          int32_t* __restrict__ sorted, int32_t* __restrict__ cumsum) {
-  const int64_t stride = (int64_t)gridDim.x * 256;
-  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < numel; i += stride) {
-    const int b = bucket_of(ids, i, nb);
-    if (b >= 0) sorted[atomicAdd(&cumsum[b], 1)] = (int32_t)i;
+    place_ids(ids, 0, numel, nb, cursor, sorted);
   }
 }
 
@@ -232,7 +277,10 @@ extern "C" int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64
   FP8K_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_pad, "moe_align_block_size: null output pointer");
   FP8K_REQUIRE(numel == 0 || topk_ids, "moe_align_block_size: null topk_ids");
   hipStream_t st = (hipStream_t)stream;
-  const bool fused = numel <= 65536 || !cumsum_buffer;
+  // one workgroup does everything up to kAlignFusedMax ids (and whenever the caller gives no scratch table); more ids
+  // are counted and placed by one workgroup per kAlignChunk ids
+  const bool fused = numel <= kAlignFusedMax || !cumsum_buffer;
+  const unsigned chunks = (unsigned)((numel + kAlignChunk - 1) / kAlignChunk);
 #define FP8K_ALIGN(T)                                                                                                \
   do {                                                                                                               \
     if (fused) {                                                                                                     \
@@ -240,11 +288,15 @@ extern "C" int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64
                          (int)num_buckets, (int)block_size, sorted_token_ids, expert_ids, num_tokens_post_pad,        \
                          cumsum_buffer, pad_sorted_token_ids);                                                        \
     } else {                                                                                                         \
-      hipLaunchKernelGGL((moe_align_kernel<T, false>), dim3(1), dim3(kAlignThreads), 0, st, (const T*)topk_ids, numel, \
-                         (int)num_buckets, (int)block_size, sorted_token_ids, expert_ids, num_tokens_post_pad,        \
+      hipLaunchKernelGGL(zero_ints_kernel, dim3((unsigned)((num_buckets + 1 + 255) / 256)), dim3(256), 0, st,         \
+                         cumsum_buffer, (int)num_buckets + 1);                                                        \
+      hipLaunchKernelGGL((moe_count_kernel<T>), dim3(chunks), dim3(kAlignThreads), 0, st, (const T*)topk_ids, numel,  \
+                         (int)num_buckets, cumsum_buffer);                                                            \
+      hipLaunchKernelGGL((moe_align_kernel<T, false, true>), dim3(1), dim3(kAlignThreads), 0, st, (const T*)topk_ids, \
+                         numel, (int)num_buckets, (int)block_size, sorted_token_ids, expert_ids, num_tokens_post_pad, \
                          cumsum_buffer, pad_sorted_token_ids);                                                        \
-      hipLaunchKernelGGL((moe_scatter_kernel<T>), dim3(stream_grid(numel)), dim3(256), 0, st, (const T*)topk_ids,     \
-                         numel, (int)num_buckets, sorted_token_ids, cumsum_buffer);                                   \
+      hipLaunchKernelGGL((moe_place_kernel<T>), dim3(chunks), dim3(kAlignThreads), 0, st, (const T*)topk_ids, numel,  \
+                         (int)num_buckets, sorted_token_ids, cumsum_buffer);                                          \
     }                                                                                                                \
   } while (0)
   if (ids_are_int64) FP8K_ALIGN(int64_t);
