@@ -335,10 +335,11 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=Fals
     bias = torch.randn((E,), generator=g, device=dev) * 0.01  # near-balanced routing, as a trained router gives
     lines = ["", "## configs[4] block-FP8 fused MoE layer (E=256, H=7168, I=2048, top-8 of 8 groups / top-4 groups)", "",
              "whole layer: align + quant + grouped GEMM w13 + silu_and_mul + quant + grouped GEMM w2 + top-k sum; "
-             "bytes = fp8 weights of the experts hit (44.04 MB each); roofline = those bytes at 8 TB/s (HBM-bound at every M);",
+             "bytes = fp8 weights of the experts hit (44.04 MB each); roofline = the binding one of those bytes at 8 TB/s and the "
+             "layer's FLOPs (2 x M x 8 x 3 I H) at the 5 PFLOP/s dense-FP8 peak;",
              "CPU: the same layer in torch-CPU ops, expert by expert, on the first token only (8 experts) - us per token", "",
-             "| M | experts hit | us | TFLOP/s | weight GB/s | fraction of HBM roofline | max rel err vs CPU (token 0) | CPU us / token |",
-             "|---|---|---|---|---|---|---|---|"]
+             "| M | experts hit | us | TFLOP/s | weight GB/s | bound | frac | max rel err vs CPU (token 0) | CPU us / token |",
+             "|---|---|---|---|---|---|---|---|---|"]
     for M in token_counts:
         print("[table] configs[4] M=%d" % M, file=sys.stderr, flush=True)
         x = _activation(torch, M, H, M, dev)
@@ -369,8 +370,10 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=Fals
             t = _median_time(layer_cpu, runs=1)
             err = "%.1e" % _rel_err(torch, out, layer_cpu()[0])
             cpu_us = "%.0f" % (t * 1e6)
-        lines.append("| %d | %d | %.1f | %.1f | %.0f | %.2f | %s | %s |" % (
-            M, hit, us, flops / us / 1e6, wbytes / us / 1e3, wbytes / us / 1e3 / PEAK_HBM_GBS, err, cpu_us))
+        t_hbm, t_mfma = wbytes / (PEAK_HBM_GBS * 1e3), flops / (PEAK_FP8_TFLOPS * 1e6)  # microseconds
+        lines.append("| %d | %d | %.1f | %.1f | %.0f | %s | %.2f | %s | %s |" % (
+            M, hit, us, flops / us / 1e6, wbytes / us / 1e3, "hbm" if t_hbm >= t_mfma else "mfma", max(t_hbm, t_mfma) / us,
+            err, cpu_us))
     return lines
 
 
