@@ -377,6 +377,38 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=Fals
     return lines
 
 
+def grouped_lines(torch, dev, shapes):
+    """The masked grouped GEMM of the DeepGEMM-shaped entry points (G groups of m rows each, [G, N, K] weights) with
+    power-of-two scales: once handed over as float32 tensors (float-scale grouped kernel) and once as packed UE8M0 words
+    (256-row blocks: the matrix cores apply the exponents)."""
+    from sglang_amd.deep_gemm_wrapper import grouped_gemm_nt_f8f8bf16_masked
+
+    def pack(e):  # exponent bytes [.., kb] -> int32 words [.., ceil(kb / 4)], K block 4 j + i in byte i of word j
+        kb = e.shape[-1]
+        pad = (-kb) % 4
+        if pad:
+            e = torch.cat([e, torch.zeros(e.shape[:-1] + (pad,), dtype=e.dtype, device=e.device)], dim=-1)
+        e = e.view(e.shape[:-1] + (-1, 4))
+        return (e[..., 0] | (e[..., 1] << 8) | (e[..., 2] << 16) | (e[..., 3] << 24)).contiguous()
+
+    lines = ["| groups | rows / group | N | K | float scales us | packed UE8M0 us | TFLOP/s (packed) |", "|---|---|---|---|---|---|---|"]
+    g = torch.Generator(device=dev)
+    g.manual_seed(0)
+    for (G, m, N, K) in shapes:
+        a = _rand_fp8(torch, (G, m, K), g, dev)
+        b = _rand_fp8(torch, (G, N, K), g, dev)
+        ea = torch.randint(115, 125, (G, m, K // 128), device=dev, dtype=torch.int32, generator=g)
+        eb = torch.randint(115, 125, (G, N // 128, K // 128), device=dev, dtype=torch.int32, generator=g)
+        a_s, b_s = (ea << 23).view(torch.float32), (eb << 23).view(torch.float32)
+        a_p, b_p = pack(ea), pack(eb.repeat_interleave(128, dim=1))
+        masked = torch.full((G,), m, device=dev, dtype=torch.int32)
+        out = torch.empty((G, m, N), device=dev, dtype=torch.bfloat16)
+        t_f = _time_graph(torch, lambda i: grouped_gemm_nt_f8f8bf16_masked((a, a_s), (b, b_s), out, masked, m), 5)
+        t_p = _time_graph(torch, lambda i: grouped_gemm_nt_f8f8bf16_masked((a, a_p), (b, b_p), out, masked, m), 5)
+        lines.append("| %d | %d | %d | %d | %.0f | %.0f | %.0f |" % (G, m, N, K, t_f, t_p, 2.0 * G * m * N * K / t_p / 1e6))
+    return lines
+
+
 def gemm_lines(torch, dev, shapes, data="random"):
     """Block-FP8 GEMM alone at the given (M, N, K): device time, TFLOP/s and algorithmic GB/s.  data = "zeros" runs
     the same launches on all-zero operands (and unit scales): the same instructions and memory traffic, but no bit of
@@ -568,6 +600,9 @@ def main() -> int:
     ap.add_argument("--gemm-data", choices=("random", "zeros"), default="random",
                     help="operands of the --gemm runs: synthetic random data (default) or all zeros (same work, no "
                          "toggling in the matrix cores: shows what the power management takes)")
+    ap.add_argument("--grouped", type=str, default=None,
+                    help="only time the masked grouped GEMM (groups x rows x N x K, comma separated) with float and "
+                         "with packed UE8M0 scales")
     ap.add_argument("--stream-read", action="store_true", help="only measure the HBM read rate of the LDS-staged load path")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -589,6 +624,10 @@ def main() -> int:
     if args.gemm:
         shapes = [tuple(int(v) for v in t.split("x")) for t in args.gemm.split(",")]
         print("\n".join(gemm_lines(torch, dev, shapes, args.gemm_data)))
+        return 0
+    if args.grouped:
+        shapes = [tuple(int(v) for v in t.split("x")) for t in args.grouped.split(",")]
+        print("\n".join(grouped_lines(torch, dev, shapes)))
         return 0
     if args.stream_read:
         print("HBM stream read (4 GiB buffer, LDS-staged loads, one workgroup per CU): %.0f GB/s" % hbm_stream_read_gbs(torch, dev))

@@ -23,7 +23,7 @@ import torch
 
 from . import custom_ops as _ops
 from .fp8_kernel import w8a8_block_fp8_matmul
-from .fused_moe import get_default_config, moe_align_block_size
+from .fused_moe import SORT_SCALES_MIN_BLOCK, get_default_config, moe_align_block_size
 from .sgl_kernel import unpack_ue8m0_scales, unpack_ue8m0_weight_scales
 
 _IGNORED = -2  # moe_align_block_size drops ids below -1
@@ -66,10 +66,12 @@ def _grouped(a, a_s, b, b_s, out, row_group: torch.Tensor, rows_per_group: int, 
         return
     block_m = get_default_config(max(rows_per_group, 1) * G, G, 1)["BLOCK_SIZE_M"]
     sorted_ids, expert_ids, num_post_pad = moe_align_block_size(row_group, block_m, G)
-    if pow2 and block_m == 256:
+    if block_m >= SORT_SCALES_MIN_BLOCK:
+        # as in the fused-MoE layer: the activation scales first go into the order of the sorted rows; with both tensors
+        # packed and 256-row blocks the matrix cores then apply the exponents themselves
         a_s = _ops.moe_sort_scales(a_s, sorted_ids, num_post_pad, 1, rows)
         _ops.moe_block_gemm(a, b, out, a_s, b_s, None, sorted_ids, expert_ids, num_post_pad, False, 1, block_m, rows,
-                            True, True)
+                            True, pow2 and block_m == 256)
         return
     _ops.moe_block_gemm(a, b, out, a_s, b_s, None, sorted_ids, expert_ids, num_post_pad, False, 1, block_m, rows)
 
