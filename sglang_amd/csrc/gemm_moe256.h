@@ -362,13 +362,120 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       }
       if (it < nkb) trip(na, it, 0, sba);
     };
+    // The hardware-scaled form keeps the matrix core fed across the barrier of a trip: the products of a block's LAST
+    // slot group are formed behind the NEXT barrier, from registers, and the fragments of the new block are fetched
+    // from LDS in their shadow - each weight fragment refilled in place right behind the MFMA that used it last, the
+    // first activation fragments of the new block behind the MFMAs that used the old ones.  (Otherwise every wave of
+    // the workgroup opens a trip with the same ten LDS fetches and the matrix cores idle until they are back.)  The
+    // float-scale forms have no registers for it: their second accumulator set takes the room.
+    auto run_scaled = [&](auto na) {
+      constexpr int NA = decltype(na)::value;
+      using yes = std::integral_constant<bool, true>;
+      using no = std::integral_constant<bool, false>;
+      v8i wf[NS][2], xa, xb;
+      int ex[MS], ew = 127;      // exponent bytes of the block in work
+      int exd = 127, ewd = 127;  // ... of the deferred group
+      // barrier of trip `it`, the exponents of its block, the next scales and the stage loads
+      auto open = [&](int it) {
+        lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
+        SB();
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) ex[ms] = (int)(__float_as_uint(sxn[ms]) >> 23);
+        ew = (int)(__float_as_uint(sbn) >> 23);
+        load_sx(it + 1);
+        load_sb(sbn, it + 1);
+        SB();  // scales, then activations, then weights
+        issue_x(it + 1, (gx0 + it + 1) & 1);
+        const int k2 = it + 2;
+        const bool nx = k2 >= nkb;
+        issue_w(nx ? rWn : rW, nx ? k2 - nkb : k2, (gw0 + k2) % WST);
+        SB();
+      };
+      // the last group of the previous block (fragments xa / xb, exponents exd / ewd); REFILL: the fragments of block
+      // `it` take the registers over as they fall free
+      auto deferred = [&](auto refill, const uint8_t* sw_, const uint8_t* sx_) {
+        constexpr bool RF = decltype(refill)::value;
+        constexpr int L = NA > 0 ? NA - 1 : 0;
+        const uint8_t* w0 = sw_ + (wn * 64) * kTileK;
+        const uint8_t* w1 = sw_ + (wn * 64 + 32) * kTileK;
+        const uint8_t* xg = sx_ + (wm * 32) * kTileK;
+        acc[0][L] = mfma_32x32x64_scaled(wf[0][0], xa, acc[0][L], ewd, exd); SB();
+        if (RF) wf[0][0] = frag(w0, 0);
+        SB();
+        acc[1][L] = mfma_32x32x64_scaled(wf[1][0], xa, acc[1][L], ewd, exd); SB();
+        if (RF) { wf[1][0] = frag(w1, 0); xa = frag(xg, 0); }
+        SB();
+        acc[0][L] = mfma_32x32x64_scaled(wf[0][1], xb, acc[0][L], ewd, exd); SB();
+        if (RF) wf[0][1] = frag(w0, 1);
+        SB();
+        acc[1][L] = mfma_32x32x64_scaled(wf[1][1], xb, acc[1][L], ewd, exd); SB();
+        if (RF) { wf[1][1] = frag(w1, 1); xb = frag(xg, 1); }
+        SB();
+      };
+      // groups 0 .. NA-2 of the block whose fragments sit in wf / xa / xb; leaves the last group's fragments in xa / xb
+      auto groups = [&](const uint8_t* sx_) {
+#pragma unroll
+        for (int ms = 0; ms + 1 < NA; ++ms) {
+          acc[0][ms] = mfma_32x32x64_scaled(wf[0][0], xa, acc[0][ms], ew, ex[ms]);
+          acc[1][ms] = mfma_32x32x64_scaled(wf[1][0], xa, acc[1][ms], ew, ex[ms]);
+          acc[0][ms] = mfma_32x32x64_scaled(wf[0][1], xb, acc[0][ms], ew, ex[ms]);
+          acc[1][ms] = mfma_32x32x64_scaled(wf[1][1], xb, acc[1][ms], ew, ex[ms]);
+          SB();
+          xa = frag(sx_ + (((ms + 1) * 2 + wm) * 32) * kTileK, 0);
+          xb = frag(sx_ + (((ms + 1) * 2 + wm) * 32) * kTileK, 1);
+          SB();
+        }
+        exd = ex[NA > 0 ? NA - 1 : 0];
+        ewd = ew;
+      };
+      open(0);
+      if constexpr (NA > 0) {
+        const uint8_t* sw_ = smem + (gw0 % WST) * WBYTES;
+        const uint8_t* sx_ = smem + XBASE + (gx0 & 1) * XBYTES;
+#pragma unroll
+        for (int ns = 0; ns < NS; ++ns) {
+          wf[ns][0] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 0);
+          wf[ns][1] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 1);
+        }
+        xa = frag(sx_ + (wm * 32) * kTileK, 0);
+        xb = frag(sx_ + (wm * 32) * kTileK, 1);
+        SB();
+        groups(sx_);
+      }
+      auto trip = [&](int it) {
+        open(it);
+        if constexpr (NA > 0) {
+          const uint8_t* sw_ = smem + ((gw0 + it) % WST) * WBYTES;
+          const uint8_t* sx_ = smem + XBASE + ((gx0 + it) & 1) * XBYTES;
+          deferred(yes{}, sw_, sx_);
+          groups(sx_);
+        }
+      };
+      int it = 1;
+      for (; it + 1 < nkb; it += 2) {  // two trips per round: the scale registers then need no copies between rounds
+        trip(it);
+        trip(it + 1);
+      }
+      if (it < nkb) trip(it);
+      if constexpr (NA > 0) deferred(no{}, smem, smem);
+    };
     // one copy of the loop per group count keeps every copy straight-line
-    switch (nact) {  // wave-uniform
-      case 4: run(std::integral_constant<int, 4>{}); break;
-      case 3: run(std::integral_constant<int, 3>{}); break;
-      case 2: run(std::integral_constant<int, 2>{}); break;
-      case 1: run(std::integral_constant<int, 1>{}); break;
-      default: run(std::integral_constant<int, 0>{}); break;
+    if constexpr (SCALED) {
+      switch (nact) {  // wave-uniform
+        case 4: run_scaled(std::integral_constant<int, 4>{}); break;
+        case 3: run_scaled(std::integral_constant<int, 3>{}); break;
+        case 2: run_scaled(std::integral_constant<int, 2>{}); break;
+        case 1: run_scaled(std::integral_constant<int, 1>{}); break;
+        default: run_scaled(std::integral_constant<int, 0>{}); break;
+      }
+    } else {
+      switch (nact) {  // wave-uniform
+        case 4: run(std::integral_constant<int, 4>{}); break;
+        case 3: run(std::integral_constant<int, 3>{}); break;
+        case 2: run(std::integral_constant<int, 2>{}); break;
+        case 1: run(std::integral_constant<int, 1>{}); break;
+        default: run(std::integral_constant<int, 0>{}); break;
+      }
     }
     // output rows and routed weights, fetched while the stages drain (lane id taken anew, as above)
     const bool wide = (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
