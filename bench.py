@@ -578,6 +578,10 @@ def write_table(torch, dev, path, cpu=True):
             lines.append("| %d | %d | %d | %.1f | %.1f | %s | %.3f | %s | %s | %s |" % (M, N, K, us, tf, bname, floor / us, err, cpu_us, cpu_gf))
         del bs
     lines += moe_table(torch, dev, cpu=cpu)
+    print("[table] masked grouped GEMM", file=sys.stderr, flush=True)
+    lines += ["", "## masked grouped block-FP8 GEMM of the DeepGEMM-shaped entry points (align + scale sort + grouped GEMM; every row "
+              "valid; power-of-two scales handed over as float32 tensors / as packed UE8M0 words)", ""]
+    lines += grouped_lines(torch, dev, [(256, 128, 4096, 7168), (256, 128, 7168, 2048), (32, 1024, 4096, 7168), (32, 1024, 7168, 2048)])
     os.makedirs(os.path.dirname(os.path.abspath(path)), exist_ok=True)
     with open(path, "w") as f:
         f.write("\n".join(lines) + "\n")
