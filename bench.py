@@ -237,6 +237,50 @@ def hbm_stream_read_gbs(torch, dev, gib=4, runs=5):
     return read / best / 1e6
 
 
+def stream_mix_lines(torch, dev, gib=4):
+    """What stores inside a read stream cost on this machine: fp8k_tune_stream_read_write (one workgroup per CU reads its
+    share in 32 KB stages, two in flight, and after every `tile` of stages writes 8 KB x n to a place of its own) against
+    the same stream without stores, next to a plain fill and a plain copy (torch kernels) of the same size."""
+    from sglang_amd._lib import check, lib, stream_ptr
+
+    def best_ms(fn, runs=4):
+        best = float("inf")
+        for _ in range(runs + 1):
+            a, b = _events(torch, 2)
+            a.record()
+            fn()
+            b.record()
+            torch.cuda.synchronize()
+            best = min(best, a.elapsed_time(b))
+        return best
+
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    src = torch.empty(gib << 30, dtype=torch.uint8, device=dev)
+    src.view(torch.int32).random_(0, 1 << 30)
+    dst = torch.empty(gib << 29, dtype=torch.uint8, device=dev)
+    lines = ["| stages of 32 KB per tile | stores per tile and CU | us | read GB/s | us added per tile | time of a stored byte / time of a read byte |",
+             "|---|---|---|---|---|---|"]
+    for spt in (56, 16):
+        share = src.numel() // ncu // (32768 * spt) * (32768 * spt)
+        tiles = share // (32768 * spt)
+        base = None
+        for spw in (0, 1, 2, 4, 8, 16):
+            ms = best_ms(lambda: check(lib.fp8k_tune_stream_read_write(src.data_ptr(), src.numel(), dst.data_ptr(), dst.numel(),
+                                                                        spt, spw, stream_ptr(dev))))
+            if spw == 0:
+                base = ms
+            added = (ms - base) * 1e3 / tiles
+            rel = "" if spw == 0 else "%.1f" % ((ms - base) / base * (spt * 32768) / (spw * 8192))
+            lines.append("| %d | %d KB | %.0f | %.0f | %.1f | %s |" % (spt, spw * 8, ms * 1e3, share * ncu / ms / 1e6, added, rel))
+    n = dst.numel()
+    ms = best_ms(lambda: dst.fill_(1))
+    lines += ["", "plain fill of %.1f GiB (torch): %.0f us = %.0f GB/s written" % (n / 2**30, ms * 1e3, n / ms / 1e6)]
+    ms = best_ms(lambda: dst.copy_(src[:n]))
+    lines.append("plain copy of %.1f GiB (torch): %.0f us = %.0f GB/s read + the same written" % (n / 2**30, ms * 1e3, n / ms / 1e6))
+    del src, dst
+    return lines
+
+
 def run_cpu_baseline(seconds_target=12.0):
     """C restatement of quant + block GEMM (oracle/, OpenMP) on M_cpu rows of the headline workload."""
     import numpy as np
@@ -608,6 +652,8 @@ def main() -> int:
                     help="only time the masked grouped GEMM (groups x rows x N x K, comma separated) with float and "
                          "with packed UE8M0 scales")
     ap.add_argument("--stream-read", action="store_true", help="only measure the HBM read rate of the LDS-staged load path")
+    ap.add_argument("--stream-mix", action="store_true",
+                    help="only measure what small write-outs inside the read stream cost (read stream with stores, fill, copy)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (the path has no cross-GPU step); --gpus %d is not "
@@ -632,6 +678,9 @@ def main() -> int:
     if args.grouped:
         shapes = [tuple(int(v) for v in t.split("x")) for t in args.grouped.split(",")]
         print("\n".join(grouped_lines(torch, dev, shapes)))
+        return 0
+    if args.stream_mix:
+        print("\n".join(stream_mix_lines(torch, dev)))
         return 0
     if args.stream_read:
         print("HBM stream read (4 GiB buffer, LDS-staged loads, one workgroup per CU): %.0f GB/s" % hbm_stream_read_gbs(torch, dev))

@@ -170,6 +170,17 @@ void fp8k_tune_force_gemm_plan(int kind, int splits);
 int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream);
 
 /*
+ * Measurement aid (no counterpart in the reference): fp8k_tune_stream_read with a write-out inside the stream.  After
+ * every stages_per_tile stages of 32 KB ("a weight tile") each of the workgroup's 8 wavefronts stores stores_per_wave
+ * times 1 KB (16 bytes a lane) to a place of its own in dst: 8 KB x stores_per_wave per tile and workgroup, the shape of
+ * a weight-streaming GEMM that writes a small output tile per weight tile.  Timed by the caller against
+ * stores_per_wave = 0 it shows what the stores cost the read stream.  `bytes` is rounded down to whole tiles per CU;
+ * dst must hold CUs x tiles x 8 KB x stores_per_wave; both pointers 16-byte aligned.
+ */
+int fp8k_tune_stream_read_write(const void* src, int64_t bytes, void* dst, int64_t dst_bytes, int64_t stages_per_tile,
+                                int64_t stores_per_wave, void* stream);
+
+/*
  * Per-token x per-channel FP8 GEMM:  C = (A . B^T) * sa[m] * sb[n] (+ bias[n]), fp32 accumulate.
  * Replaces torch.ops.sgl_kernel.fp8_scaled_mm
  *   (sgl-kernel/python/sgl_kernel/gemm.py:35-43, sgl-kernel/csrc/gemm/fp8_gemm_kernel.cu:1450-1532).

@@ -353,6 +353,62 @@ extern "C" int fp8k_tune_stream_read(const void* src, int64_t bytes, void* strea
   return check_launch("tune_stream_read");
 }
 
+namespace fp8k {
+// stream_read_kernel with a write-out after every `spt` stages ("a tile"): each wave stores `spw` times 1 KB (16 bytes a
+// lane), the workgroup 8 KB x spw, to a place of its own in dst - the shape of a GEMM that streams weights and writes
+// a small output tile per weight tile
+__global__ __launch_bounds__(512, 1) void stream_read_write_kernel(const uint8_t* __restrict__ src, int64_t share,
+                                                                   uint8_t* __restrict__ dst, int spt, int spw) {
+  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint8_t* base = src + (int64_t)blockIdx.x * share;
+  const int trips = (int)(share >> 15);
+  const int tiles = trips / spt;
+  auto issue = [&](int t) {
+    const rsrc_t r = make_rsrc(base + (int64_t)t * 32768, 32768u);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      buf_load16_to_lds(r, (uint32_t)((w * 4 + q) * 1024 + lane * 16), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
+  };
+  issue(0);
+  if (trips > 1) issue(1);
+  int t = 0;
+  for (int ti = 0; ti < tiles; ++ti) {
+    for (int k = 0; k < spt; ++k, ++t) {
+      // stores and loads retire in order: a wait that leaves this wave's four youngest loads in flight has seen every
+      // store issued before them complete
+      if (t + 1 < trips) lds_barrier<4>();
+      else lds_barrier<0>();
+      if (t + 2 < trips) issue(t + 2);
+    }
+    uint4* o = reinterpret_cast<uint4*>(dst + ((((int64_t)blockIdx.x * tiles + ti) * 8 + w) * spw) * 1024) + lane;
+    const uint4 v = make_uint4(1u, 2u, 3u, (unsigned)ti);
+    for (int i = 0; i < spw; ++i) o[i * 64] = v;
+  }
+  wait_vm0();
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_stream_read_write(const void* src, int64_t bytes, void* dst, int64_t dst_bytes, int64_t stages_per_tile,
+                                           int64_t stores_per_wave, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read_write: bad size");
+  FP8K_REQUIRE(src && aligned(src, 16) && dst && aligned(dst, 16), "tune_stream_read_write: src and dst must be 16-byte aligned device pointers");
+  FP8K_REQUIRE(stages_per_tile >= 1 && stages_per_tile <= 4096 && stores_per_wave >= 0 && stores_per_wave <= 64,
+               "tune_stream_read_write: stages_per_tile in [1, 4096], stores_per_wave in [0, 64]");
+  const int ncu = num_cu();
+  const int64_t share = bytes / ncu / (32768 * stages_per_tile) * (32768 * stages_per_tile);  // whole tiles per workgroup
+  if (share == 0) return FP8K_OK;
+  const int64_t tiles = share / (32768 * stages_per_tile);
+  FP8K_REQUIRE(dst_bytes >= (int64_t)ncu * tiles * 8 * stores_per_wave * 1024,
+               "tune_stream_read_write: dst holds %lld bytes, %lld are written", (long long)dst_bytes,
+               (long long)((int64_t)ncu * tiles * 8 * stores_per_wave * 1024));
+  hipLaunchKernelGGL(stream_read_write_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src,
+                     share, (uint8_t*)dst, (int)stages_per_tile, (int)stores_per_wave);
+  return check_launch("tune_stream_read_write");
+}
+
 extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) {
   g_tail_halves = kind != -2;  // -2: automatic choice with the last round of 256x256 tiles kept whole
   g_force_kind = kind == -2 ? -1 : kind;
