@@ -382,3 +382,27 @@ def test_linear_path_against_golden_vectors(dev, case):
                                   [128, 128], torch.bfloat16)
         torch.cuda.synchronize()
         assert _rel_err(y.float().cpu().numpy(), G[case + "_y"]) <= REL_TOL
+
+
+def test_stream_read_write_probe_writes_its_pattern_and_checks_its_arguments(dev):
+    """The measurement aid fp8k_tune_stream_read_write: every workgroup writes 8 KB x stores_per_wave after each tile of
+    stages, all of it inside the caller's buffer (words 1, 2, 3, tile index), nothing beyond; too small a destination
+    is refused."""
+    from sglang_amd._lib import lib, stream_ptr
+
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    spt, spw, tiles = 3, 2, 4
+    share = 32768 * spt * tiles
+    src = torch.zeros(ncu * share + 4096, dtype=torch.uint8, device=dev)
+    written = ncu * tiles * 8 * spw * 1024
+    dst = torch.full((written // 4 + 1024,), -1, dtype=torch.int32, device=dev)
+    rc = lib.fp8k_tune_stream_read_write(src.data_ptr(), src.numel(), dst.data_ptr(), written, spt, spw, stream_ptr(dev))
+    assert rc == 0, lib.fp8k_last_error()
+    torch.cuda.synchronize()
+    got = dst.cpu().numpy()
+    body = got[: written // 4].reshape(ncu, tiles, 8 * spw * 64, 4)
+    assert (body[..., 0] == 1).all() and (body[..., 1] == 2).all() and (body[..., 2] == 3).all()
+    assert (body[..., 3] == np.arange(tiles)[None, :, None]).all()
+    assert (got[written // 4:] == -1).all()
+    rc = lib.fp8k_tune_stream_read_write(src.data_ptr(), src.numel(), dst.data_ptr(), written - 1, spt, spw, stream_ptr(dev))
+    assert rc != 0 and b"dst holds" in lib.fp8k_last_error()
