@@ -308,10 +308,21 @@ def run_cpu_baseline(seconds_target=12.0):
     M = int(min(HEADLINE["M"], max(64, rows // 64 * 64)))
     reps = int(max(1, min(8, rows // HEADLINE["M"])))
     dt = sum(once(M) for _ in range(reps))
+    # the algorithm of the reference's own CPU kernel (fp8_scaled_mm_cpu: W8A16 - bf16 activations, weight blocks
+    # dequantised to bf16), restated in C/OpenMP, on a quarter of the same sample
+    Mt = max(64, M // 4 // 64 * 64)
+    xt = O.bf16_bits(O.make_activation(Mt, K, 0))
+    t0 = time.perf_counter()
+    c_oracle.w8a16_block_gemm(lib, xt, wq, wsc)
+    dtt = time.perf_counter() - t0
     return dict(value=2.0 * M * reps * N * K / dt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
                 sample="C/OpenMP restatement of per-token-group quant + block-FP8 matmul, %d pass(es) over M=%d rows "
                        "of the headline workload (N=%d, K=%d), %.1f s of CPU time on %d threads"
-                       % (reps, M, N, K, dt, cores))
+                       % (reps, M, N, K, dt, cores),
+                w8a16_twin=dict(value=2.0 * Mt * N * K / dtt / 1e12, unit="TFLOP/s", cores=cores, kind="port",
+                                sample="C/OpenMP restatement of the algorithm of the reference's CPU kernel "
+                                       "fp8_scaled_mm_cpu (W8A16: bf16 activations, weight blocks dequantised to bf16, "
+                                       "float accumulation), M=%d rows of the same workload, %.1f s" % (Mt, dtt)))
 
 
 def _rand_fp8(torch, shape, gen, dev):

@@ -28,6 +28,7 @@ def load() -> ctypes.CDLL:
     lib.oracle_group_quant_bf16.argtypes = [p, p, p, i64, i64, ctypes.c_int, ctypes.c_float, ctypes.c_int]
     lib.oracle_block_gemm.argtypes = [p, p, p, p, p, i64, i64, i64]
     lib.oracle_scaled_mm.argtypes = [p, p, p, p, p, p, i64, i64, i64]
+    lib.oracle_w8a16_block_gemm.argtypes = [p, p, p, p, p, i64, i64, i64]
     return lib
 
 
@@ -64,4 +65,17 @@ def scaled_mm(lib, A, B, sa, sb, bias=None):
     C = np.empty((M, N), dtype=np.uint16)
     b = None if bias is None else np.ascontiguousarray(bias, np.float32)
     lib.oracle_scaled_mm(_ptr(A), _ptr(B), _ptr(sa), _ptr(sb), None if b is None else _ptr(b), _ptr(C), M, N, K)
+    return C
+
+
+def w8a16_block_gemm(lib, A_bits, B, Bs, bias=None):
+    """The reference CPU twin's algorithm (W8A16, see fp8_oracle.c): A_bits uint16 [M,K] bf16 patterns, B uint8 [N,K],
+    Bs float32 [ceil(N/128), K/128] -> bf16 bit patterns uint16 [M,N]."""
+    A_bits = np.ascontiguousarray(A_bits, np.uint16); B = np.ascontiguousarray(B, np.uint8)
+    Bs = np.ascontiguousarray(Bs, np.float32)
+    M, K = A_bits.shape
+    N = B.shape[0]
+    C = np.empty((M, N), dtype=np.uint16)
+    b = None if bias is None else np.ascontiguousarray(bias, np.float32)
+    lib.oracle_w8a16_block_gemm(_ptr(A_bits), _ptr(B), _ptr(Bs), None if b is None else _ptr(b), _ptr(C), M, N, K)
     return C

@@ -10,6 +10,7 @@
  *   group quant   python/sglang/test/test_block_fp8.py:23-48
  *   block matmul  python/sglang/test/test_block_fp8.py:273-325
  *   scaled_mm     sgl-kernel/tests/test_fp8_gemm.py:6-14
+ *   W8A16 twin    sgl-kernel/csrc/cpu/gemm_fp8.cpp:46-100 (weight block -> bf16 with its scale), :256-298, :356-424
  */
 #include <math.h>
 #ifdef _OPENMP
@@ -154,6 +155,41 @@ void oracle_scaled_mm(const uint8_t* A, const uint8_t* B, const float* sa, const
         float acc = ((lane[0] + lane[4]) + (lane[2] + lane[6])) + ((lane[1] + lane[5]) + (lane[3] + lane[7]));
         for (; k < K; ++k) acc += a[k] * brow[k];
         acc = acc * sb[n] * sa[m];
+        if (bias) acc += bias[n];
+        C[m * N + n] = f32_to_bf16(acc);
+      }
+    }
+    free(brow);
+  }
+  free(Af);
+}
+
+/* The ALGORITHM of the reference's CPU kernel fp8_scaled_mm_cpu for more than four rows (W8A16, not the W8A8 path of
+ * the rest of this file; a timing baseline and a sanity check, never a bit oracle): the bf16 activations are used as
+ * they are, every weight element becomes bf16(float(bf16(w8)) * Bs[n/128, k/128]) (gemm_fp8.cpp:46-100: e4m3 -> bf16 is
+ * exact, the product with the block scale is rounded to bf16), the dot products accumulate in float over the whole K,
+ * the result (+ float bias) is rounded to bf16.  A bf16 bits [M,K]; B e4m3fn bytes [N,K]; Bs [ceil(N/128), K/128]. */
+void oracle_w8a16_block_gemm(const uint16_t* A, const uint8_t* B, const float* Bs, const float* bias, uint16_t* C, int64_t M,
+                             int64_t N, int64_t K) {
+  if (!g_lut_ready) build_lut();
+  const int64_t KB = (K + 127) / 128;
+  float* Af = (float*)malloc((size_t)M * K * sizeof(float));
+  for (int64_t i = 0; i < M * K; ++i) Af[i] = bf16_to_f32(A[i]);
+#pragma omp parallel
+  {
+    float* brow = (float*)malloc((size_t)K * sizeof(float));
+#pragma omp for schedule(dynamic, 8)
+    for (int64_t n = 0; n < N; ++n) {
+      const float* bs = Bs + (n / 128) * KB;
+      for (int64_t k = 0; k < K; ++k) brow[k] = bf16_to_f32(f32_to_bf16(g_lut[B[n * K + k]] * bs[k / 128]));
+      for (int64_t m = 0; m < M; ++m) {
+        const float* a = Af + m * K;
+        float lane[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int64_t k = 0;
+        for (; k + 8 <= K; k += 8)
+          for (int j = 0; j < 8; ++j) lane[j] += a[k + j] * brow[k + j];
+        float acc = ((lane[0] + lane[4]) + (lane[2] + lane[6])) + ((lane[1] + lane[5]) + (lane[3] + lane[7]));
+        for (; k < K; ++k) acc += a[k] * brow[k];
         if (bias) acc += bias[n];
         C[m * N + n] = f32_to_bf16(acc);
       }

@@ -292,6 +292,23 @@ def w8a8_block_fp8_matmul(Aq, Bq, As, Bs, block_size=(128, 128), out_dtype="bf16
     return _cast_out(C, out_dtype)
 
 
+def w8a16_block_fp8_matmul_cpu_twin(A, Bq, Bs, bias=None, block_size=(128, 128), acc=np.float32):
+    """The ALGORITHM of the reference's CPU kernel fp8_scaled_mm_cpu for more than four rows
+    (sgl-kernel/csrc/cpu/gemm_fp8.cpp:46-100, 256-298, 356-424).  W8A16 - NOT the W8A8 path of the rest of this
+    file: a timing baseline and a sanity check, no bit oracle.  The bf16 activations A [M,K] are used unquantised;
+    every weight element becomes bf16(float(w8) * Bs[n/bn, k/bk]); float accumulation over the whole K; + float
+    bias; one rounding to bf16."""
+    bn, bk = block_size
+    A = to_bf16(np.asarray(A, dtype=np.float32))
+    N, K = Bq.shape
+    W = e4m3fn_to_f32(Bq)
+    W = to_bf16(W * np.repeat(np.repeat(Bs, bn, axis=0)[:N], bk, axis=1)[:, :K])
+    C = A.astype(acc) @ W.astype(acc).T
+    if bias is not None:
+        C = C + np.asarray(bias, dtype=np.float32).astype(acc)[None, :]
+    return to_bf16(C.astype(np.float32))
+
+
 def _cast_out(C, out_dtype):
     if out_dtype == "bf16":
         return to_bf16(C.astype(np.float32))

@@ -221,6 +221,48 @@ def test_c_oracle_matches_numpy_oracle():
     assert np.abs(c2 - ref2).max() <= 2**-7 * np.abs(ref2).max()
 
 
+def test_w8a16_cpu_twin_restatement():
+    """The W8A16 algorithm of the reference's CPU kernel (sgl-kernel/csrc/cpu/gemm_fp8.cpp:46-100, 356-424), restated in
+    numpy and in C.  Pins: (1) on weights whose block scale is 1 and activations that are exact e4m3 values it IS the
+    W8A8 block matmul with unit scales (no rounding anywhere: integers); (2) the weight dequantisation is the torch
+    expression bf16(w8.to(bf16).float() * scale); (3) C == numpy to float-accumulation noise; (4) on realistic data it
+    stays within 2e-2 of the W8A8 result (the activations are not quantised: that is the whole difference)."""
+    import torch
+
+    lib = c_oracle.load()
+    rng = np.random.default_rng(5)
+    M, N, K = 9, 256, 384
+    # (1) exact case: small integers, unit scales
+    a_int = rng.integers(-3, 4, (M, K)).astype(np.float32)
+    aq = O.f32_to_e4m3fn(a_int)
+    bq = O.f32_to_e4m3fn(rng.integers(-2, 3, (N, K)).astype(np.float32))
+    ones_a = np.ones((M, K // 128), np.float32)
+    ones_b = np.ones((N // 128, K // 128), np.float32)
+    w8a8 = O.w8a8_block_fp8_matmul(aq, bq, ones_a, ones_b)
+    twin = O.w8a16_block_fp8_matmul_cpu_twin(a_int, bq, ones_b)
+    assert np.array_equal(w8a8, twin)
+    assert np.array_equal(O.bf16_from_bits(c_oracle.w8a16_block_gemm(lib, O.bf16_bits(a_int), bq, ones_b)), twin)
+    # (2) the dequantised weight against torch's own conversions
+    wq, ws = O.block_quant_weight(O.make_weight(N, K, 3))
+    wt = torch.from_numpy(wq).view(torch.float8_e4m3fn).to(torch.bfloat16).float()
+    st = torch.from_numpy(np.repeat(np.repeat(ws, 128, axis=0), 128, axis=1))
+    w_ref = (wt * st).to(torch.bfloat16).float().numpy()
+    x = O.make_activation(M, K, 4)
+    eye = np.eye(K, dtype=np.float32)[:M]  # rows of the identity pick weight columns out
+    picked = O.w8a16_block_fp8_matmul_cpu_twin(eye, wq, ws)
+    assert np.array_equal(picked, w_ref[:, :M].T)
+    # (3) C against numpy, with bias
+    bias = rng.normal(size=N).astype(np.float32)
+    ref = O.w8a16_block_fp8_matmul_cpu_twin(x, wq, ws, bias, acc=np.float64)
+    c = O.bf16_from_bits(c_oracle.w8a16_block_gemm(lib, O.bf16_bits(x), wq, ws, bias))
+    assert np.abs(c - ref).max() <= 2**-7 * np.abs(ref).max()
+    # (4) next to the W8A8 path on the same data
+    q, s = O.per_token_group_quant_fp8(x, 128)
+    w8 = O.w8a8_block_fp8_matmul(q, wq, s, ws, acc=np.float64)
+    no_bias = O.w8a16_block_fp8_matmul_cpu_twin(x, wq, ws, acc=np.float64)
+    assert np.abs(no_bias - w8).max() <= 2e-2 * np.abs(w8).max()
+
+
 # ---------------------------------------------------------------- MoE helpers
 @pytest.mark.parametrize("E,topk,block", [(8, 2, 16), (64, 6, 64), (256, 8, 64), (257, 8, 128)])
 def test_moe_align_invariants(E, topk, block):
