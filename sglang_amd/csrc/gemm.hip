@@ -49,6 +49,13 @@ static Plan plan_direct(int64_t M, int64_t N, int64_t K) {
   // 128 and more n tiles keep half the CUs streaming on their own: no K cut and no reduction launch (18432 x 7168:
   // 26.6 us against 28.6 us with three cuts; two cuts, 288 workgroups, leave the CUs unevenly loaded: 33 us)
   if (tiles_n >= 128) splits = 1;
+  // a share of 9 or 10 K blocks is one full prefetch round of 8 and a round for the one or two left over: one more cut
+  // gives every workgroup a single shorter round (7168 x 2304, 18 K blocks: 10.2 -> 8.5 us at M = 1 with three cuts)
+  while (splits > 1 && splits < kb) {
+    const int64_t per = (kb + splits - 1) / splits;
+    if (per > kDirDepth && per % kDirDepth >= 1 && per % kDirDepth <= 2 && (kb + splits) / (splits + 1) >= 4) ++splits;
+    else break;
+  }
   if (g_force_kind == 3 && g_force_splits > 0) splits = std::min<int64_t>(g_force_splits, kb);  // tuning aid
   const int kbps = (int)((kb + splits - 1) / splits);
   pl.kb_per_split = kbps;
