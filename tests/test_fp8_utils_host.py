@@ -93,3 +93,23 @@ def test_ue8m0_unpack_and_marking():
         mark_ue8m0(torch.tensor([[1.0, 3.0]]))
     with pytest.raises(RuntimeError, match="powers of two"):
         mark_ue8m0(torch.tensor([[1.0, 0.0]]))
+
+
+def test_cast_to_e8m0_with_rounding_up_host():
+    """deep_gemm_moe_runner.cast_to_e8m0_with_rounding_up on CPU tensors (reference: moe_runner/deep_gemm.py:48-58):
+    equal to the oracle's ceil-to-power-of-two + word packing on ordinary scales, and the reference's corner cases."""
+    import numpy as np
+    import torch
+
+    from oracle import fp8_oracle as O
+    from sglang_amd.deep_gemm_moe_runner import cast_to_e8m0_with_rounding_up
+
+    rng = np.random.default_rng(8)
+    s = (rng.uniform(1.0, 2.0, (2, 5, 7)) * 2.0 ** rng.integers(-20, 10, (2, 5, 7))).astype(np.float32)
+    s[0, 0, :3] = [1.0, 0.25, 3.0]
+    got = cast_to_e8m0_with_rounding_up(torch.from_numpy(s)).numpy()
+    ref = np.stack([O.pack_ue8m0_scales(O.ceil_to_ue8m0(x)) for x in s])
+    assert got.shape == (2, 5, 2) and np.array_equal(got, ref)
+    edge = np.array([[3.0e38, 1e-45, 8e-39, 0.0]], dtype=np.float32)
+    b = cast_to_e8m0_with_rounding_up(torch.from_numpy(edge)).numpy().view(np.uint8).reshape(-1)
+    assert list(b[:4]) == [0xFE, 0, 1, 0]
