@@ -142,6 +142,60 @@ def scaled_fp8_quant(
     return output, scale
 
 
+def static_quant_fp8(x: torch.Tensor, x_s: torch.Tensor, repeat_scale: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:639-692 (a Triton kernel there): q = cast(clamp(x * (1 / x_s), -448, 448)) with the
+    given per-tensor scale - the arithmetic of the static branch of sgl_per_tensor_quant_fp8, which runs it here.
+    repeat_scale: the scale is returned once per row ([rows, 1]) instead of as given."""
+    assert x.is_contiguous(), "`x` is not contiguous"
+    assert x_s.numel() == 1, "only supports per-tensor scale"
+    x_q = torch.empty_like(x, device=x.device, dtype=fp8_dtype)
+    scale = x_s.reshape(1).to(torch.float32)
+    if x.numel() > 0:
+        _ops.sgl_per_tensor_quant_fp8(x.view(-1, x.shape[-1]), x_q.view(-1, x.shape[-1]), scale, is_static=True)
+    if repeat_scale:
+        return x_q, scale.expand(x.numel() // max(x.shape[-1], 1)).reshape(-1, 1).contiguous()
+    return x_q, x_s
+
+
+def sglang_per_token_group_quant_8bit(
+    x: torch.Tensor,
+    group_size: int,
+    dst_dtype: torch.dtype,
+    eps: float = 1e-10,
+    column_major_scales: bool = False,
+    scale_tma_aligned: bool = False,
+    scale_ue8m0: bool = False,
+    fuse_silu_and_mul: bool = False,
+    masked_m: Optional[torch.Tensor] = None,
+    enable_v2: Optional[bool] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:535-574.  The int8 destination of the reference is another quantisation path and is not
+    built here."""
+    if dst_dtype != fp8_dtype:
+        raise RuntimeError("sglang_per_token_group_quant_8bit: only float8_e4m3fn is built on gfx950")
+    return sglang_per_token_group_quant_fp8(
+        x, group_size, eps, column_major_scales=column_major_scales, scale_tma_aligned=scale_tma_aligned,
+        scale_ue8m0=scale_ue8m0, fuse_silu_and_mul=fuse_silu_and_mul, masked_m=masked_m, enable_v2=enable_v2,
+    )
+
+
+def per_token_group_quant_8bit(
+    x: torch.Tensor,
+    group_size: int,
+    dst_dtype: torch.dtype,
+    eps: float = 1e-10,
+    column_major_scales: bool = False,
+    scale_tma_aligned: bool = False,
+    scale_ue8m0: bool = False,
+    fuse_silu_and_mul: bool = False,
+    masked_m: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Reference: fp8_kernel.py:404-434 (the Triton entry point, with its fused silu_and_mul branch :330-401); the same
+    kernel as the sgl-kernel entry point here."""
+    return sglang_per_token_group_quant_8bit(x, group_size, dst_dtype, eps, column_major_scales, scale_tma_aligned,
+                                             scale_ue8m0, fuse_silu_and_mul, masked_m)
+
+
 def per_tensor_quant_mla_fp8(x: torch.Tensor, x_s_out: torch.Tensor, eps: float = 1e-12) -> Tuple[torch.Tensor, torch.Tensor]:
     """Reference: fp8_kernel.py:1221-1266 - tensor-wise quantisation specialised for the MLA absorbed products: x is a
     (possibly transposed) [num_head, num_seq, head_size] view, the result is contiguous.  x_s_out: one float32 that
@@ -240,3 +294,9 @@ def w8a8_block_fp8_matmul(
         raise RuntimeError("w8a8_block_fp8_matmul: scales must be float32 (or packed int32 UE8M0 scales)")
     out = _ops.block_gemm_nk(A2, B, As2, Bs, output_dtype)
     return out.reshape(C_shape)
+
+
+# the reference dispatches between a Triton and a DeepGEMM implementation of the same op (fp8_kernel.py:1051-1169); one
+# implementation here
+w8a8_block_fp8_matmul_triton = w8a8_block_fp8_matmul
+w8a8_block_fp8_matmul_deepgemm = w8a8_block_fp8_matmul

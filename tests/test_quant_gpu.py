@@ -273,6 +273,39 @@ def test_per_tensor_quant(dev, numel):
     np.testing.assert_array_equal(u8(q2), q2_ref)
 
 
+@pytest.mark.parametrize("shape", [(5, 7, 64), (300, 2048), (1, 8)])
+def test_static_quant_fp8(dev, shape):
+    """static_quant_fp8 (reference: fp8_kernel.py:639-692): bytes of the oracle's static per-tensor quant, the scale handed
+    back as given or once per row."""
+    from sglang_amd.fp8_kernel import static_quant_fp8
+
+    rng = np.random.default_rng(sum(shape))
+    x = O.to_bf16(rng.standard_normal(shape).astype(np.float32) * 6)
+    st = torch.tensor([0.037], dtype=torch.float32, device=dev)
+    q, s = static_quant_fp8(bf16_tensor(x, dev), st)
+    q_ref, _ = O.per_tensor_quant_fp8(x.reshape(-1, shape[-1]), 0.037)
+    np.testing.assert_array_equal(u8(q).reshape(-1, shape[-1]), q_ref)
+    assert s is st
+    q2, s2 = static_quant_fp8(bf16_tensor(x, dev), st, repeat_scale=True)
+    np.testing.assert_array_equal(u8(q2).reshape(-1, shape[-1]), q_ref)
+    rows = int(np.prod(shape[:-1]))
+    assert s2.shape == (rows, 1) and bool((s2 == st).all())
+
+
+def test_group_quant_8bit_entry_points(dev):
+    """sglang_per_token_group_quant_8bit / per_token_group_quant_8bit (reference: fp8_kernel.py:404-434, 535-574) are the
+    FP8 group quant under the 8-bit names; the int8 destination is refused."""
+    from sglang_amd.fp8_kernel import per_token_group_quant_8bit, sglang_per_token_group_quant_8bit, sglang_per_token_group_quant_fp8
+
+    x = bf16_tensor(O.make_activation(33, 512, 2), dev)
+    q0, s0 = sglang_per_token_group_quant_fp8(x, 128, column_major_scales=True)
+    for fn in (sglang_per_token_group_quant_8bit, per_token_group_quant_8bit):
+        q, s = fn(x, 128, torch.float8_e4m3fn, column_major_scales=True)
+        assert torch.equal(q.view(torch.uint8), q0.view(torch.uint8)) and torch.equal(s, s0) and s.stride() == s0.stride()
+        with pytest.raises(RuntimeError, match="float8_e4m3fn"):
+            fn(x, 128, torch.int8)
+
+
 @pytest.mark.parametrize("layout", _layouts())
 @pytest.mark.parametrize("M,K", [(1, 128), (37, 2048), (512, 2048), (4096, 2048)])
 def test_silu_mul_group_quant_equals_the_two_step_pipeline(dev, M, K, layout):
