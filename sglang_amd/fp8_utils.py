@@ -178,3 +178,51 @@ def requant_weight_ue8m0(weight: torch.Tensor, weight_scale_inv: torch.Tensor, w
     assert list(weight_block_size) == [128, 128]
     deq = block_quant_dequant(weight, weight_scale_inv, weight_block_size, torch.bfloat16)
     return quant_weight_ue8m0(deq, weight_block_size)
+
+
+def requant_weight_ue8m0_inplace(weight: torch.nn.Parameter, weight_scale_inv: torch.nn.Parameter,
+                                 weight_block_size: List[int]) -> None:
+    """Reference: fp8_utils.py:441-450 - requant_weight_ue8m0 written back into the two parameters."""
+    assert isinstance(weight, torch.nn.Parameter)
+    assert isinstance(weight_scale_inv, torch.nn.Parameter)
+    q, s = requant_weight_ue8m0(weight.data.to(weight_scale_inv.device), weight_scale_inv.data, weight_block_size)
+    weight.data = q
+    weight_scale_inv.data = s
+    mark_ue8m0(weight_scale_inv.data, check=False)
+
+
+def transform_scale_ue8m0(sf: torch.Tensor, mn: int) -> torch.Tensor:
+    """Power-of-two block scales float32 [.., ceil(mn/128), kb] -> the packed layout DeepGEMM is handed: one row per weight
+    row, four exponent bytes to an int32 word (K block 4j+i in byte i of word j), [.., mn, ceil(kb/4)] with the mn
+    dimension contiguous and padded to a multiple of 4.  Reference: fp8_utils.py:510-515 (which calls the DeepGEMM
+    layout helper for the second half).  Accepted as weight scales by w8a8_block_fp8_matmul and the grouped entry points."""
+    if sf.dtype != torch.float32:
+        raise RuntimeError("transform_scale_ue8m0: float32 scales expected")
+    rows = sf.index_select(-2, torch.arange(mn, device=sf.device) // 128)
+    exp = (rows.contiguous().view(torch.int32) >> 23) & 0xFF
+    kb = exp.shape[-1]
+    if kb % 4:
+        exp = torch.cat([exp, exp.new_zeros(exp.shape[:-1] + (4 - kb % 4,))], dim=-1)
+    exp = exp.view(exp.shape[:-1] + (-1, 4))
+    words = exp[..., 0] | (exp[..., 1] << 8) | (exp[..., 2] << 16) | (exp[..., 3] << 24)  # [.., mn, kb4]
+    aligned = (mn + 3) // 4 * 4
+    out = torch.zeros(words.shape[:-2] + (words.shape[-1], aligned), dtype=torch.int32, device=sf.device)
+    out[..., :mn] = words.transpose(-1, -2)
+    return out.transpose(-1, -2)[..., :mn, :]
+
+
+def transform_scale_ue8m0_inplace(param: torch.nn.Parameter, mn: int) -> None:
+    """Reference: fp8_utils.py:505-507."""
+    param.data = transform_scale_ue8m0(param.data, mn=mn)
+
+
+def inverse_transform_scale_ue8m0(sf_packed: torch.Tensor, mn: int) -> torch.Tensor:
+    """Packed weight scales [.., mn, ceil(kb/4)] back to float32 powers of two [.., mn/128, 4 ceil(kb/4)], with the
+    reference's consistency check (the 128 rows of a block must carry the same words, and packing the result again
+    must give the input).  Reference: fp8_utils.py:518-565."""
+    if sf_packed.dtype != torch.int32 or mn % 128 != 0 or sf_packed.shape[-2] != mn:
+        raise RuntimeError("inverse_transform_scale_ue8m0: int32 [.., mn, k/4] with mn a multiple of 128 expected")
+    k = sf_packed.shape[-1] * 4
+    sf = unpack_ue8m0_weight_scales(sf_packed, k * 128)
+    assert torch.equal(transform_scale_ue8m0(sf, mn), sf_packed), "packed scales are not uniform over their 128-row blocks"
+    return sf

@@ -113,3 +113,26 @@ def test_cast_to_e8m0_with_rounding_up_host():
     edge = np.array([[3.0e38, 1e-45, 8e-39, 0.0]], dtype=np.float32)
     b = cast_to_e8m0_with_rounding_up(torch.from_numpy(edge)).numpy().view(np.uint8).reshape(-1)
     assert list(b[:4]) == [0xFE, 0, 1, 0]
+
+
+def test_transform_scale_ue8m0_round_trip():
+    """transform_scale_ue8m0 / inverse_transform_scale_ue8m0 (reference: fp8_utils.py:505-565): words equal to the
+    oracle's packing of the row-repeated scales, mn-major storage padded to 4 rows, exact round trip, 2-D and 3-D."""
+    import numpy as np
+    import torch
+
+    from oracle import fp8_oracle as O
+    from sglang_amd.fp8_utils import inverse_transform_scale_ue8m0, transform_scale_ue8m0
+
+    rng = np.random.default_rng(12)
+    for shape, mn in (((3, 6), 384), ((2, 2, 5), 256)):
+        sf = (2.0 ** rng.integers(-14, 3, shape)).astype(np.float32)
+        packed = transform_scale_ue8m0(torch.from_numpy(sf), mn)
+        kb4 = (shape[-1] + 3) // 4
+        assert packed.shape == shape[:-2] + (mn, kb4) and packed.dtype == torch.int32
+        assert packed.stride(-2) == 1 and packed.stride(-1) == (mn + 3) // 4 * 4
+        rep = np.repeat(sf, 128, axis=-2)
+        ref = O.pack_ue8m0_scales(rep) if sf.ndim == 2 else np.stack([O.pack_ue8m0_scales(x) for x in rep])
+        assert np.array_equal(packed.numpy(), ref)
+        back = inverse_transform_scale_ue8m0(packed, mn)
+        assert np.array_equal(back.numpy()[..., : shape[-1]], sf)

@@ -359,6 +359,12 @@ def test_packed_ue8m0_weight_scales(dev, M):
     c = w8a8_block_fp8_matmul(xq, B, xs_packed, packed_rows, [128, 128], torch.bfloat16)
     c_float = w8a8_block_fp8_matmul(xq, B, xs_packed, mark_ue8m0(torch.from_numpy(ws2).to(dev)), [128, 128], torch.bfloat16)
     assert torch.equal(c, c_float)
+    # the same words in the mn-major storage transform_scale_ue8m0 produces (reference: fp8_utils.py:505-515)
+    from sglang_amd.fp8_utils import transform_scale_ue8m0
+
+    mn_major = transform_scale_ue8m0(torch.from_numpy(ws2).to(dev), N)
+    assert mn_major.stride(0) == 1 and torch.equal(mn_major, packed_rows)
+    assert torch.equal(w8a8_block_fp8_matmul(xq, B, xs_packed, mn_major, [128, 128], torch.bfloat16), c)
     ref = O.w8a8_block_fp8_matmul(xq.view(torch.uint8).cpu().numpy(), wq,
                                   unpack_ue8m0_scales(xs_packed, K // 128).cpu().numpy(), ws2, acc=np.float64)
     assert _rel_err(c.float().cpu().numpy(), ref) <= REL_TOL
