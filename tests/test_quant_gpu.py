@@ -409,3 +409,28 @@ def test_silu_and_mul_masked_post_quant_fwd(dev):
             np.testing.assert_array_equal(u8(out).reshape(E, m_max, K)[e, :m], u8(q2).reshape(m, K))
             assert torch.equal(sc[e, :m], s2)
         assert torch.all(sc[e, m:] == 0)
+
+
+def test_silu_and_mul_masked_post_quant_fwd_ue8m0_scales_as_floats(dev):
+    """scale_ue8m0=True (reference: ep_moe/kernels.py:348-350): the scale is 2^ceil(log2(amax/448)) stored as float32;
+    bytes and scales equal the oracle's fused activation quant with UE8M0 scales, rows past masked_m keep their values."""
+    from sglang_amd.ep_moe_kernels import silu_and_mul_masked_post_quant_fwd, tma_align_input_scale
+
+    rng = np.random.default_rng(31)
+    E, m_max, K = 3, 70, 384
+    masked = np.array([70, 0, 33], dtype=np.int32)
+    x = O.to_bf16(rng.standard_normal((E, m_max, 2 * K)).astype(np.float32) * 2)
+    out = torch.full((E, m_max, K), 0x55, device=dev, dtype=torch.uint8).view(torch.float8_e4m3fn)
+    sc = torch.full((E, m_max, K // 128), 7.0, device=dev, dtype=torch.float32)
+    silu_and_mul_masked_post_quant_fwd(bf16_tensor(x, dev), out, sc, 128, torch.from_numpy(masked).to(dev), scale_ue8m0=True)
+    qn, sn = u8(out).reshape(E, m_max, K), sc.cpu().numpy()
+    for e, m in enumerate(masked.tolist()):
+        if m:
+            q_ref, s_ref = O.silu_mul_per_token_group_quant_fp8(x[e, :m], 128, scale_ue8m0=True)
+            np.testing.assert_array_equal(qn[e, :m], q_ref)
+            np.testing.assert_array_equal(sn[e, :m], s_ref)
+        assert np.all(qn[e, m:] == 0x55) and np.all(sn[e, m:] == 7.0)
+    # the column-major copy of a scale matrix
+    s2 = torch.from_numpy(rng.standard_normal((37, 5)).astype(np.float32)).to(dev)
+    al = tma_align_input_scale(s2)
+    assert al.shape == s2.shape and al.stride() == (1, 40) and torch.equal(al, s2)
