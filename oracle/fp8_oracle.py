@@ -415,6 +415,20 @@ def moe_sum_reduce(x, routed_scaling_factor=1.0):
     return to_bf16((acc * np.float32(routed_scaling_factor)).astype(np.float32))
 
 
+def moe_sum(x):
+    """Reference: sgl-kernel/csrc/moe/moe_sum.cu:11-69.  x float32-of-bf16 [T, topk, H] -> [T, H]: for 2, 3 and 4
+    experts per token the sum runs in the element type (a bf16 rounding after every addition, ascending k, starting from
+    zero), otherwise at::sum_out (float accumulation, one rounding)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    topk = x.shape[1]
+    if topk in (2, 3, 4):
+        acc = np.zeros((x.shape[0], x.shape[2]), dtype=np.float32)
+        for k in range(topk):
+            acc = to_bf16(acc + x[:, k])
+        return acc
+    return to_bf16(x.astype(np.float64).sum(axis=1).astype(np.float32))
+
+
 def biased_grouped_topk(logits, bias, num_expert_group, topk_group, topk, renormalize=True):
     """Reference: biased_grouped_topk_impl, python/sglang/srt/layers/moe/topk.py:665-738.
 

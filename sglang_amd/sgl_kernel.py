@@ -560,6 +560,22 @@ def moe_sum_reduce(input_tensor: torch.Tensor, output_tensor: torch.Tensor, rout
                                   dtype_code(input_tensor.dtype), stream_ptr(input_tensor.device)))
 
 
+def moe_sum(input_tensor: torch.Tensor, output_tensor: torch.Tensor) -> None:
+    """Reference: sgl-kernel/python/sgl_kernel/moe.py:95-102; csrc/moe/moe_sum.cu:11-69.  input [tokens, topk, hidden],
+    output [tokens, hidden].  As in the reference, 2, 3 and 4 experts per token are summed in the element type, one
+    rounding per addition (the elementwise adds of torch do exactly that); any other count is the float-accumulated sum
+    of moe_sum_reduce with factor 1."""
+    if input_tensor.dim() != 3 or input_tensor.shape[1] == 0:
+        raise RuntimeError("moe_sum: input must be [tokens, topk, hidden] with topk >= 1")
+    topk = input_tensor.shape[1]
+    if topk in (2, 3, 4):
+        torch.add(input_tensor[:, 0], input_tensor[:, 1], out=output_tensor)
+        for k in range(2, topk):
+            output_tensor.add_(input_tensor[:, k])
+        return
+    moe_sum_reduce(input_tensor, output_tensor, 1.0)
+
+
 def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: int, num_valid_tokens: int) -> torch.Tensor:
     """Activation scales gathered into the order of sorted_token_ids (see include/fp8k.h: fp8k_moe_sort_scales):
     returns a [len(sorted_token_ids), K/128] view with strides (1, len): row i holds the scales of slot

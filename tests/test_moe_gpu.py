@@ -157,6 +157,17 @@ def test_moe_sum_reduce_exact(dev, T, topk, H, scale):
     np.testing.assert_array_equal(out.float().cpu().numpy(), O.moe_sum_reduce(x, scale))
 
 
+@pytest.mark.parametrize("topk", [1, 2, 3, 4, 8])
+def test_moe_sum_exact(dev, topk):
+    from sglang_amd.sgl_kernel import moe_sum
+
+    rng = np.random.default_rng(topk)
+    x = O.to_bf16(rng.standard_normal((37, topk, 256)).astype(np.float32) * 3)
+    out = torch.empty((37, 256), dtype=torch.bfloat16, device=dev)
+    moe_sum(bf16_tensor(x, dev), out)
+    np.testing.assert_array_equal(out.float().cpu().numpy(), O.moe_sum(x))
+
+
 def _expert_weights(rng, E, N, K):
     wq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((E, N, K)).astype(np.float32) * 100, -448, 448))
     ws = (rng.uniform(0.5, 2.0, (E, (N + 127) // 128, K // 128)) * 1e-3).astype(np.float32)

@@ -263,6 +263,27 @@ def test_w8a16_cpu_twin_restatement():
     assert np.abs(no_bias - w8).max() <= 2e-2 * np.abs(w8).max()
 
 
+def test_moe_sum_rounding_orders():
+    """moe_sum (sgl-kernel/csrc/moe/moe_sum.cu): element-type accumulation for 2-4 experts per token against torch's
+    bf16 adds, float accumulation otherwise against torch.sum."""
+    import torch
+
+    rng = np.random.default_rng(4)
+    for topk in (2, 3, 4, 8):
+        x = O.to_bf16(rng.standard_normal((19, topk, 64)).astype(np.float32) * 3)
+        xt = torch.from_numpy(x).to(torch.bfloat16)
+        if topk <= 4:
+            ref = torch.zeros((19, 64), dtype=torch.bfloat16)
+            for k in range(topk):
+                ref = ref + xt[:, k]
+        else:
+            ref = torch.sum(xt, dim=1)
+        assert np.array_equal(O.moe_sum(x), ref.float().numpy())
+    # the two orders differ: the pin above is not vacuous
+    x = O.to_bf16(rng.standard_normal((200, 3, 64)).astype(np.float32) * 3)
+    assert not np.array_equal(O.moe_sum(x), O.to_bf16(x.sum(axis=1)))
+
+
 # ---------------------------------------------------------------- MoE helpers
 @pytest.mark.parametrize("E,topk,block", [(8, 2, 16), (64, 6, 64), (256, 8, 64), (257, 8, 128)])
 def test_moe_align_invariants(E, topk, block):
