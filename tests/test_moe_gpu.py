@@ -168,6 +168,42 @@ def test_moe_sum_exact(dev, topk):
     np.testing.assert_array_equal(out.float().cpu().numpy(), O.moe_sum(x))
 
 
+@pytest.mark.parametrize("seed", [0, 1, 2])
+def test_grouped_gemm_hardware_scaled_is_exact_on_integer_data(dev, seed):
+    """fp8k_moe_block_gemm_ue8m0 (256-slot blocks, sorted power-of-two scales): on small integers with power-of-two
+    scales every product and sum is exact, so the matrix cores' own scaling must give the oracle's bf16 values bit
+    for bit, and so must the float-scale kernel."""
+    from sglang_amd.fused_moe import moe_align_block_size
+    from sglang_amd.sgl_kernel import moe_block_gemm, moe_sort_scales
+
+    rng = np.random.default_rng(seed)
+    T, E, topk = int(rng.integers(200, 900)), int(rng.integers(2, 9)), 2
+    N, K = int(rng.integers(1, 6)) * 128, int(rng.integers(2, 7)) * 128
+    ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
+    ids[rng.random(ids.shape) < 0.05] = -1
+    wq = O.f32_to_e4m3fn(rng.integers(-4, 5, (E, N, K)).astype(np.float32))
+    ws = (2.0 ** rng.integers(-3, 3, (E, N // 128, K // 128))).astype(np.float32)
+    xq = O.f32_to_e4m3fn(rng.integers(-4, 5, (T, K)).astype(np.float32))
+    xs = (2.0 ** rng.integers(-3, 3, (T, K // 128))).astype(np.float32)
+    sorted_ids, expert_ids, npad = moe_align_block_size(torch.from_numpy(ids).to(dev), 256, E)
+    A, B = fp8_tensor(xq, dev), fp8_tensor(wq, dev)
+    As, Bs = torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev)
+    sc = moe_sort_scales(As, sorted_ids, npad, topk, ids.size)
+    tw = torch.ones((T, topk), device=dev)
+    flat = ids.reshape(-1)
+    for pow2 in (False, True):
+        C = torch.full((T * topk, N), float("nan"), dtype=torch.bfloat16, device=dev)
+        moe_block_gemm(A, B, C, sc, Bs, tw, sorted_ids, expert_ids, npad, False, topk, 256, ids.size, scales_sorted=True,
+                       pow2_scales=pow2)
+        got = C.float().cpu().numpy()
+        assert (got[flat == -1] == 0).all()
+        for e in range(E):
+            slots = np.nonzero(flat == e)[0]
+            if slots.size:
+                ref = O.w8a8_block_fp8_matmul(xq[slots // topk], wq[e], xs[slots // topk], ws[e], acc=np.float64)
+                np.testing.assert_array_equal(got[slots], ref)
+
+
 def _expert_weights(rng, E, N, K):
     wq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((E, N, K)).astype(np.float32) * 100, -448, 448))
     ws = (rng.uniform(0.5, 2.0, (E, (N + 127) // 128, K // 128)) * 1e-3).astype(np.float32)
