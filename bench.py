@@ -237,6 +237,52 @@ def hbm_stream_read_gbs(torch, dev, gib=4, runs=5):
     return read / best / 1e6
 
 
+def mfma_ceiling_tflops(torch, dev, iters=40000, runs=3):
+    """Rate of a bare v_mfma_f32_32x32x64 (e4m3) loop on this machine (fp8k_tune_mfma_peak: 8 waves per CU, operands in
+    registers, nothing else in the loop) on operand bytes taken from a quantised headline weight ("random") and on
+    all-zero bytes ("zeros"); best of `runs` after a settling launch.  The power management clocks the chip by what the
+    data toggles: the random-data figure is the practical ceiling of any FP8 GEMM on real data here, and its ratio to
+    the zero-data figure separates that limit from kernel quality."""
+    import ctypes
+
+    from sglang_amd._lib import check, lib, stream_ptr
+
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    wq, _ = _block_quant_weight(torch, 4096, 4096, 0, dev)
+    sink = torch.empty(ncu * 512, dtype=torch.float32, device=dev)
+    out = {}
+    for name, ops in (("random", wq.view(torch.uint8)), ("zeros", torch.zeros_like(wq.view(torch.uint8)))):
+        flops = ctypes.c_int64(0)
+        best = float("inf")
+        for r in range(runs + 1):
+            a, b = _events(torch, 2)
+            a.record()
+            check(lib.fp8k_tune_mfma_peak(ops.data_ptr(), ops.numel(), iters, sink.data_ptr(), sink.numel(),
+                                          ctypes.byref(flops), stream_ptr(dev)))
+            b.record()
+            torch.cuda.synchronize()
+            if r:
+                best = min(best, a.elapsed_time(b))
+        out[name] = round(flops.value / best / 1e9, 1)
+    return out
+
+
+def headline_zero_data_us(torch, dev):
+    """The headline GEMM launch on all-zero operands and unit scales: the same instructions and memory traffic with no
+    bit toggling in the matrix cores.  Reported next to the random-data time so that a slower box (or a lower power
+    cap) can be told from a slower kernel."""
+    from sglang_amd.fp8_kernel import w8a8_block_fp8_matmul
+
+    M, N, K = HEADLINE["M"], HEADLINE["N"], HEADLINE["K"]
+    nbuf = 3
+    ws = [(torch.zeros((N, K), device=dev, dtype=torch.uint8).view(torch.float8_e4m3fn),
+           torch.ones((N // 128, K // 128), device=dev)) for _ in range(nbuf)]
+    qs = [(torch.zeros((M, K), device=dev, dtype=torch.uint8).view(torch.float8_e4m3fn),
+           torch.ones((K // 128, M), device=dev).t()) for _ in range(nbuf)]
+    return _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
+                                                              ws[i % nbuf][1], [128, 128], torch.bfloat16), 12)
+
+
 def stream_mix_lines(torch, dev, gib=4):
     """What stores inside a read stream cost on this machine: fp8k_tune_stream_read_write (one workgroup per CU reads its
     share in 32 KB stages, two in flight, and after every `tile` of stages writes 8 KB x n to a place of its own) against
@@ -378,7 +424,7 @@ def _rel_err(torch, got, ref):
 
 def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=False):
     """BASELINE configs[4]: 256 experts, hidden 7168, intermediate 2048, top-8 grouped-sigmoid routing."""
-    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl
+    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl
 
     E, H, I, topk = 256, 7168, 2048, 8
     g = torch.Generator(device=dev)
@@ -399,7 +445,7 @@ def moe_table(torch, dev, token_counts=(1, 32, 256, 1024, 4096, 16384), cpu=Fals
         print("[table] configs[4] M=%d" % M, file=sys.stderr, flush=True)
         x = _activation(torch, M, H, M, dev)
         logits = torch.randn((M, E), generator=g, device=dev)
-        tw, ids = biased_grouped_topk_impl(x, logits, bias, topk, True, 8, 4)
+        tw, ids = biased_grouped_topk(x, logits, bias, topk, True, 8, 4)
         hit = int(torch.unique(ids).numel())
         kw = dict(use_fp8_w8a8=True, w1_scale=w1s, w2_scale=w2s, block_shape=[128, 128], routed_scaling_factor=2.5)
         us = _time_graph(torch, lambda i: fused_experts_impl(x, w1, w2, tw, ids, **kw), 10 if M < 4096 else 5)
@@ -663,6 +709,8 @@ def main() -> int:
                     help="only time the masked grouped GEMM (groups x rows x N x K, comma separated) with float and "
                          "with packed UE8M0 scales")
     ap.add_argument("--stream-read", action="store_true", help="only measure the HBM read rate of the LDS-staged load path")
+    ap.add_argument("--mfma-ceiling", action="store_true",
+                    help="only measure the bare matrix-core rate on random and on all-zero FP8 operands")
     ap.add_argument("--stream-mix", action="store_true",
                     help="only measure what small write-outs inside the read stream cost (read stream with stores, fill, copy)")
     args = ap.parse_args()
@@ -692,6 +740,12 @@ def main() -> int:
         return 0
     if args.stream_mix:
         print("\n".join(stream_mix_lines(torch, dev)))
+        return 0
+    if args.mfma_ceiling:
+        c = mfma_ceiling_tflops(torch, dev)
+        print("bare v_mfma_f32_32x32x64 e4m3 loop, 8 waves per CU: %.0f TFLOP/s on quantised-weight bytes (%.2f of 5 PFLOP/s), "
+              "%.0f TFLOP/s on all-zero bytes (%.2f)" % (c["random"], c["random"] / PEAK_FP8_TFLOPS, c["zeros"],
+                                                        c["zeros"] / PEAK_FP8_TFLOPS))
         return 0
     if args.stream_read:
         print("HBM stream read (4 GiB buffer, LDS-staged loads, one workgroup per CU): %.0f GB/s" % hbm_stream_read_gbs(torch, dev))
@@ -754,6 +808,8 @@ def main() -> int:
             "other_layouts_GBps": {k: round(v[1], 1) for k, v in quant.items()},
         },
         "hbm_stream_read_GBps": round(hbm_stream_read_gbs(torch, dev), 1),
+        "mfma_ceiling_TFLOPs": mfma_ceiling_tflops(torch, dev),
+        "headline_zero_data_us": round(headline_zero_data_us(torch, dev), 2),
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))

@@ -31,7 +31,9 @@ typedef enum { FP8K_F32 = 0, FP8K_F16 = 1, FP8K_BF16 = 2 } fp8k_dtype;
 
 typedef enum {
   FP8K_SCALE_F32 = 0,         /* one float per group, addressed by (stride_m, stride_g) */
-  FP8K_SCALE_UE8M0_PACKED = 1 /* int32 words, 4 exponent bytes each, word (g/4) byte (g%4) */
+  FP8K_SCALE_UE8M0_PACKED = 1, /* int32 words, 4 exponent bytes each, word (g/4) byte (g%4) */
+  FP8K_SCALE_UE8M0_F32 = 2     /* the power of two 2^ceil(log2 scale) stored as a float, addressed like FP8K_SCALE_F32
+                                  (fp8k_group_quant_masked only) */
 } fp8k_scale_kind;
 
 /* Message of the last failed call on this thread ("" if none). */
@@ -74,7 +76,9 @@ int fp8k_silu_mul_group_quant(const void* x, void* q, void* s, int64_t M, int64_
  *   (sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu, wrapper fp8_kernel.py:481-531) and the Triton
  *   silu_and_mul_masked_post_quant_fwd (python/sglang/srt/layers/moe/ep_moe/kernels.py:364-429).
  * Scales as in fp8k_group_quant with one more stride: row i of expert e, group g at
- *   s[e*s_stride_e + i*s_stride_m + g*s_stride_g] (packed UE8M0: word g/4 at (g/4)*s_stride_g).
+ *   s[e*s_stride_e + i*s_stride_m + g*s_stride_g] (packed UE8M0: word g/4 at (g/4)*s_stride_g); FP8K_SCALE_UE8M0_F32
+ *   writes the rounded-up power of two as a float at the float position (the Triton kernel's SCALE_UE8M0 branch,
+ *   ep_moe/kernels.py:348-350).
  * masked_m: int32[E] on the device.  group_size must be 128.
  */
 int fp8k_group_quant_masked(const void* x, void* q, void* s, int64_t E, int64_t m_max, int64_t K, int64_t group_size,
@@ -139,46 +143,14 @@ int64_t fp8k_block_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
  * launches, the column-major copy of row-major activation scales) is a fixed 80 MiB array in device memory that is
  * part of this library - one copy on every GPU that loads it, held until the process ends.  The call allocates and
  * frees nothing.  The first call on a device looks up the array's device address (hipGetSymbolAddress) and keeps it;
- * make that call outside a graph capture.  A shape whose fp8k_block_gemm_workspace_bytes exceeds 80 MiB is refused
+ * make that call outside a graph capture (inside one it is refused with FP8K_ERR_UNSUPPORTED).  The stream's device
+ * must be the calling thread's current device (FP8K_ERR_INVALID otherwise): each GPU has its own copy of the array.  A shape whose fp8k_block_gemm_workspace_bytes exceeds 80 MiB is refused
  * with FP8K_ERR_WORKSPACE.  All calls on one GPU share the one array: calls that overlap in time on the same GPU
  * (two streams, two threads) race; nothing in the array has to be cleared between calls.
  */
 int fp8k_block_gemm_noalloc(const void* A, const void* B, const float* As, const float* Bs, void* C, int64_t M,
                             int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t as_stride_m, int64_t as_stride_k,
                             int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldc, int out_dtype, void* stream);
-
-/*
- * Tuning and test aid (no counterpart in the reference): pins the kernel family that the dense GEMM entry points
- * pick for later calls made by the calling thread (the setting is thread-local; other threads keep the automatic
- * choice).  kind -1: automatic (the default).  kind 4: the 128x128 tile kernel with K
- * cut into `splits` runs (0 or 1: none).  kind 0: the choice by the number of rows alone, without the 128x128
- * kernel.  kind 1: 256x256 tiles; kind 2: the streaming kernel (up to 128 rows); kind 3: the direct kernel (up to 32
- * rows, `splits` > 0 pins its K cut too); where a pinned family cannot take the shape, the choice by rows stands.
- * `splits` is ignored for kinds 0..2.
- * kind -2: automatic, but the last round of 256x256 tiles is kept whole instead of being computed in 128-row halves.
- * fp8k_*_workspace_bytes, called from the same thread, follows the pinned choice.
- */
-void fp8k_tune_force_gemm_plan(int kind, int splits);
-
-/*
- * Measurement aid (no counterpart in the reference): streams `bytes` of device memory at `src` once through the load
- * path of the weight-streaming kernels - one workgroup of 8 wavefronts per CU, 32 KB stages of 16-byte-per-lane loads
- * straight into LDS, two stages in flight, a workgroup barrier per stage - and drops the data.  Timed by the caller, it
- * gives the read rate this load path reaches on the machine at hand, the practical ceiling under the 8 TB/s of the
- * data sheet.  `bytes` is rounded down to a multiple of 64 KB per CU; src 16-byte aligned; bytes < 2^40.
- */
-int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream);
-
-/*
- * Measurement aid (no counterpart in the reference): fp8k_tune_stream_read with a write-out inside the stream.  After
- * every stages_per_tile stages of 32 KB ("a weight tile") each of the workgroup's 8 wavefronts stores stores_per_wave
- * times 1 KB (16 bytes a lane) to a place of its own in dst: 8 KB x stores_per_wave per tile and workgroup, the shape of
- * a weight-streaming GEMM that writes a small output tile per weight tile.  Timed by the caller against
- * stores_per_wave = 0 it shows what the stores cost the read stream.  `bytes` is rounded down to whole tiles per CU;
- * dst must hold CUs x tiles x 8 KB x stores_per_wave; both pointers 16-byte aligned.
- */
-int fp8k_tune_stream_read_write(const void* src, int64_t bytes, void* dst, int64_t dst_bytes, int64_t stages_per_tile,
-                                int64_t stores_per_wave, void* stream);
 
 /*
  * Per-token x per-channel FP8 GEMM:  C = (A . B^T) * sa[m] * sb[n] (+ bias[n]), fp32 accumulate.
@@ -301,7 +273,8 @@ int fp8k_shuffle_rows(const void* input, const int32_t* dst2src_map, void* outpu
  * output[t, :] = sum_j factors[t * topk + j] * input[permutation[t * topk + j], :], float32 sum in ascending j, one
  * rounding to the element type; factors (same element type as the data) may be null (= 1).
  * Replaces torch.ops.sgl_kernel.apply_shuffle_mul_sum (sgl-kernel/python/sgl_kernel/moe.py:243-251,
- * prepare_moe_input.cu:252-392).  cols % 8 == 0; rows whose permutation entry is outside [0, input_rows) are skipped.
+ * prepare_moe_input.cu:252-392).  cols % 8 == 0; rows whose permutation entry is outside [0, input_rows) are skipped;
+ * permutation NULL = the identity (input rows already in slot order).
  */
 int fp8k_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* permutation, const void* factors, int64_t m,
                                int64_t topk, int64_t cols, int64_t input_rows, int dtype, void* stream);
@@ -317,6 +290,19 @@ int fp8k_apply_shuffle_mul_sum(const void* input, void* output, const int32_t* p
 int fp8k_moe_blocks_from_offsets(const int32_t* expert_starts, const int32_t* problem_sizes, int64_t num_experts, int64_t rows,
                                  int64_t block_m, int32_t* sorted_token_ids, int64_t sorted_capacity, int32_t* expert_ids,
                                  int64_t expert_capacity, int32_t* num_tokens_post_pad, void* stream);
+
+/*
+ * The same block table holding token SLOTS (slot = token * topk + j, padded with num_slots) at the positions of their
+ * expert-major rows: from what fp8k_moe_prepare_input wrote (expert_starts, problem_sizes, slot_rows = its
+ * output_permutation) and the routed ids themselves (slots whose id is outside [0, num_experts) take no place).  With it
+ * fp8k_moe_block_gemm (top_k = topk, num_valid_tokens = num_slots) gathers token slot / topk from the un-shuffled
+ * activations and writes its rows in slot order: the two shuffle_rows copies that cutlass_fused_experts_fp8 makes in
+ * front of its grouped GEMM (python/sglang/srt/layers/moe/cutlass_moe.py:152-154) are not needed.
+ */
+int fp8k_moe_slot_blocks_from_offsets(const int32_t* expert_starts, const int32_t* problem_sizes, int64_t num_experts,
+                                      const int32_t* topk_ids, const int32_t* slot_rows, int64_t num_slots, int64_t block_m,
+                                      int32_t* sorted_token_ids, int64_t sorted_capacity, int32_t* expert_ids,
+                                      int64_t expert_capacity, int32_t* num_tokens_post_pad, void* stream);
 
 /*
  * Grouped GEMM 1 of the fused MoE layer with silu_and_mul and the per-token-group requantisation inside its write-out
@@ -370,6 +356,15 @@ int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t
  */
 int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,
                         int64_t stride_topk, int64_t out_stride_token, float scale, int dtype, void* stream);
+
+/*
+ * out[t, :] = sum_k x[t, k, :] as torch.ops.sgl_kernel.moe_sum computes it (sgl-kernel/python/sgl_kernel/moe.py:95-102,
+ * sgl-kernel/csrc/moe/moe_sum.cu:11-69): for topk 2, 3 and 4 the sum runs in the element type, one rounding per
+ * addition in ascending k; any other topk is the float32-accumulated sum of fp8k_moe_sum_reduce with scale 1.
+ * Strides in elements; hidden % 8 == 0.
+ */
+int fp8k_moe_sum(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,
+                 int64_t stride_topk, int64_t out_stride_token, int dtype, void* stream);
 
 /*
  * Grouped top-k routing with a selection bias (DeepSeek-V3 style gate).

@@ -1,4 +1,4 @@
-"""ctypes binding of libfp8k.so (the C ABI declared in include/fp8k.h).
+"""ctypes binding of libfp8k.so (the C ABI declared in include/fp8k.h and include/fp8k_tune.h).
 
 There is one code path: if the shared library is missing or fails to load, importing this
 module raises; nothing falls back to torch or CPU code.
@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "csrc", "libfp8k.so")
 ABI_VERSION = 2
 
 F32, F16, BF16 = 0, 1, 2
-SCALE_F32, SCALE_UE8M0_PACKED = 0, 1
+SCALE_F32, SCALE_UE8M0_PACKED, SCALE_UE8M0_F32 = 0, 1, 2
 
 _DTYPE_CODE = {torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16}
 
@@ -25,7 +25,7 @@ _c_int = ctypes.c_int
 _c_f32 = ctypes.c_float
 _c_ptr = ctypes.c_void_p
 
-# name -> (restype, argtypes); kept in the order of include/fp8k.h
+# name -> (restype, argtypes)
 SIGNATURES = {
     "fp8k_last_error": (ctypes.c_char_p, []),
     "fp8k_abi_version": (_c_int, []),
@@ -50,6 +50,7 @@ SIGNATURES = {
     "fp8k_shuffle_rows": (_c_int, [_c_ptr] * 3 + [_c_i64] * 3 + [_c_ptr]),
     "fp8k_apply_shuffle_mul_sum": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int, _c_ptr]),
     "fp8k_moe_blocks_from_offsets": (_c_int, [_c_ptr] * 2 + [_c_i64] * 3 + [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
+    "fp8k_moe_slot_blocks_from_offsets": (_c_int, [_c_ptr] * 2 + [_c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
     "fp8k_moe_block_gemm_silu_quant": (_c_int, [_c_ptr] * 9 + [_c_i64] * 15 + [_c_f32, _c_int, _c_ptr]),
     "fp8k_block_gemm": (
         _c_int,
@@ -69,6 +70,7 @@ SIGNATURES = {
     "fp8k_tune_force_gemm_plan": (None, [_c_int, _c_int]),
     "fp8k_tune_stream_read": (_c_int, [_c_ptr, _c_i64, _c_ptr]),
     "fp8k_tune_stream_read_write": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr]),
+    "fp8k_tune_mfma_peak": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
     "fp8k_moe_align_block_size": (
         _c_int,
         [_c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr],
@@ -78,6 +80,7 @@ SIGNATURES = {
     "fp8k_moe_sort_scales": (_c_int, [_c_ptr] * 4 + [_c_i64] * 6 + [_c_ptr]),
     "fp8k_silu_and_mul": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr]),
     "fp8k_moe_sum_reduce": (_c_int, [_c_ptr, _c_ptr] + [_c_i64] * 6 + [_c_f32, _c_int, _c_ptr]),
+    "fp8k_moe_sum": (_c_int, [_c_ptr, _c_ptr] + [_c_i64] * 6 + [_c_int, _c_ptr]),
     "fp8k_moe_fused_gate": (
         _c_int, [_c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 6 + [ctypes.c_double, _c_int, _c_int, _c_ptr],
     ),

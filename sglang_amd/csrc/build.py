@@ -14,8 +14,9 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB = os.path.join(HERE, "libfp8k.so")
-SOURCES = ["api.hip", "quant.hip", "gemm.hip", "moe.hip"]
-HEADERS = ["fp8k_common.h", "quant_math.h", "gemm_kernels.h", "gemm_direct.h", "gemm_moe256.h", "gemm_tile128.h", os.path.join("..", "..", "include", "fp8k.h")]
+SOURCES = ["api.hip", "quant.hip", "gemm.hip", "moe.hip", "tune.hip"]
+HEADERS = ["fp8k_common.h", "quant_math.h", "gemm_kernels.h", "gemm_direct.h", "gemm_moe256.h", "gemm_tile128.h", os.path.join("..", "..", "include", "fp8k.h"),
+           os.path.join("..", "..", "include", "fp8k_tune.h")]
 
 # -packed-fp32-ops off: packed float32 VALU forms are not used on this hardware pool.
 FLAGS = [

@@ -7,6 +7,8 @@
 #include "gemm_direct.h"
 #include "gemm_tile128.h"
 
+#include "../../include/fp8k_tune.h"
+
 namespace fp8k {
 
 struct Plan {
@@ -323,99 +325,6 @@ static int common_checks(const char* op, const void* A, const void* B, void* C, 
 
 using namespace fp8k;
 
-namespace fp8k {
-// every workgroup reads its own contiguous share, a 32 KB stage per trip, two stages in flight
-__global__ __launch_bounds__(512, 1) void stream_read_kernel(const uint8_t* __restrict__ src, int64_t share) {
-  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
-  const int lane = threadIdx.x & 63;
-  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const uint8_t* base = src + (int64_t)blockIdx.x * share;
-  const int trips = (int)(share >> 15);
-  auto issue = [&](int t) {
-    // the descriptor moves with the trip: a share may exceed the 4 GB a descriptor can span
-    const rsrc_t r = make_rsrc(base + (int64_t)t * 32768, 32768u);
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      buf_load16_to_lds(r, (uint32_t)((w * 4 + q) * 1024 + lane * 16), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
-  };
-  issue(0);
-  if (trips > 1) issue(1);
-  for (int t = 0; t < trips; ++t) {
-    if (t + 1 < trips) lds_barrier<4>();
-    else lds_barrier<0>();
-    if (t + 2 < trips) issue(t + 2);
-  }
-  wait_vm0();
-}
-}  // namespace fp8k
-
-extern "C" int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream) {
-  clear_error();
-  FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read: bad size");
-  FP8K_REQUIRE(src && aligned(src, 16), "tune_stream_read: src must be a 16-byte aligned device pointer");
-  const int ncu = num_cu();
-  const int64_t share = bytes / ncu / 65536 * 65536;
-  if (share == 0) return FP8K_OK;
-  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src, share);
-  return check_launch("tune_stream_read");
-}
-
-namespace fp8k {
-// stream_read_kernel with a write-out after every `spt` stages ("a tile"): each wave stores `spw` times 1 KB (16 bytes a
-// lane), the workgroup 8 KB x spw, to a place of its own in dst - the shape of a GEMM that streams weights and writes
-// a small output tile per weight tile
-__global__ __launch_bounds__(512, 1) void stream_read_write_kernel(const uint8_t* __restrict__ src, int64_t share,
-                                                                   uint8_t* __restrict__ dst, int spt, int spw) {
-  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
-  const int lane = threadIdx.x & 63;
-  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
-  const uint8_t* base = src + (int64_t)blockIdx.x * share;
-  const int trips = (int)(share >> 15);
-  const int tiles = trips / spt;
-  auto issue = [&](int t) {
-    const rsrc_t r = make_rsrc(base + (int64_t)t * 32768, 32768u);
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      buf_load16_to_lds(r, (uint32_t)((w * 4 + q) * 1024 + lane * 16), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
-  };
-  issue(0);
-  if (trips > 1) issue(1);
-  int t = 0;
-  for (int ti = 0; ti < tiles; ++ti) {
-    for (int k = 0; k < spt; ++k, ++t) {
-      // stores and loads retire in order: a wait that leaves this wave's four youngest loads in flight has seen every
-      // store issued before them complete
-      if (t + 1 < trips) lds_barrier<4>();
-      else lds_barrier<0>();
-      if (t + 2 < trips) issue(t + 2);
-    }
-    uint4* o = reinterpret_cast<uint4*>(dst + ((((int64_t)blockIdx.x * tiles + ti) * 8 + w) * spw) * 1024) + lane;
-    const uint4 v = make_uint4(1u, 2u, 3u, (unsigned)ti);
-    for (int i = 0; i < spw; ++i) o[i * 64] = v;
-  }
-  wait_vm0();
-}
-}  // namespace fp8k
-
-extern "C" int fp8k_tune_stream_read_write(const void* src, int64_t bytes, void* dst, int64_t dst_bytes, int64_t stages_per_tile,
-                                           int64_t stores_per_wave, void* stream) {
-  clear_error();
-  FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read_write: bad size");
-  FP8K_REQUIRE(src && aligned(src, 16) && dst && aligned(dst, 16), "tune_stream_read_write: src and dst must be 16-byte aligned device pointers");
-  FP8K_REQUIRE(stages_per_tile >= 1 && stages_per_tile <= 4096 && stores_per_wave >= 0 && stores_per_wave <= 64,
-               "tune_stream_read_write: stages_per_tile in [1, 4096], stores_per_wave in [0, 64]");
-  const int ncu = num_cu();
-  const int64_t share = bytes / ncu / (32768 * stages_per_tile) * (32768 * stages_per_tile);  // whole tiles per workgroup
-  if (share == 0) return FP8K_OK;
-  const int64_t tiles = share / (32768 * stages_per_tile);
-  FP8K_REQUIRE(dst_bytes >= (int64_t)ncu * tiles * 8 * stores_per_wave * 1024,
-               "tune_stream_read_write: dst holds %lld bytes, %lld are written", (long long)dst_bytes,
-               (long long)((int64_t)ncu * tiles * 8 * stores_per_wave * 1024));
-  hipLaunchKernelGGL(stream_read_write_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src,
-                     share, (uint8_t*)dst, (int)stages_per_tile, (int)stores_per_wave);
-  return check_launch("tune_stream_read_write");
-}
-
 extern "C" void fp8k_tune_force_gemm_plan(int kind, int splits) {
   g_tail_halves = kind != -2;  // -2: automatic choice with the last round of 256x256 tiles kept whole
   g_force_kind = kind == -2 ? -1 : kind;
@@ -477,7 +386,7 @@ extern "C" int fp8k_block_gemm(const void* A, const void* B, const float* As, co
 constexpr int64_t kStaticScratchBytes = 80ll << 20;  // 64 MiB of float partials (one 256x256 tile per CU) + 16 MiB of copied scales
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
-static int static_scratch(void** out) {
+static int static_scratch(void** out, hipStream_t stream) {
   constexpr int kMaxDev = 64;
   static std::mutex mu;
   static void* ptrs[kMaxDev];  // device address of `scratch` on each device, resolved on the first call there
@@ -485,8 +394,22 @@ static int static_scratch(void** out) {
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return fail(FP8K_ERR_LAUNCH, "fp8k_block_gemm_noalloc: hipGetDevice: %s", hipGetErrorString(e));
   if (dev < 0 || dev >= kMaxDev) return fail(FP8K_ERR_UNSUPPORTED, "fp8k_block_gemm_noalloc: device index %d not supported", dev);
+  // every GPU holds its own copy of the array: the copy used must be the one of the GPU the launches go to
+  if (stream) {
+    int sdev = -1;
+    e = hipStreamGetDevice(stream, &sdev);
+    if (e != hipSuccess) return fail(FP8K_ERR_LAUNCH, "fp8k_block_gemm_noalloc: hipStreamGetDevice: %s", hipGetErrorString(e));
+    if (sdev != dev)
+      return fail(FP8K_ERR_INVALID, "fp8k_block_gemm_noalloc: the stream belongs to device %d but device %d is current; make the "
+                  "stream's device current before the call", sdev, dev);
+  }
   std::lock_guard<std::mutex> lock(mu);
   if (!ptrs[dev]) {
+    // the look-up is not a stream operation; under a capture it would break the capture, so it is refused there
+    hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+    if (stream && hipStreamIsCapturing(stream, &cs) == hipSuccess && cs != hipStreamCaptureStatusNone)
+      return fail(FP8K_ERR_UNSUPPORTED, "fp8k_block_gemm_noalloc: the first call on a device resolves the scratch address and "
+                  "cannot run while the stream is capturing; make one call outside the capture first");
     void* p = nullptr;
     e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !p)
@@ -509,7 +432,7 @@ extern "C" int fp8k_block_gemm_noalloc(const void* A, const void* B, const float
                 (long long)K, (long long)need, (long long)kStaticScratchBytes);
   void* ws = nullptr;
   if (need > 0) {
-    const int rc = static_scratch(&ws);
+    const int rc = static_scratch(&ws, (hipStream_t)stream);
     if (rc) return rc;
   }
   // nothing in the buffer has to start at zero: every float partial and every copied scale that a launch reads was

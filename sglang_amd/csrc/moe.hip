@@ -223,7 +223,8 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const void* __restric
 // ------------------------------------------------------------------------------------------------
 // moe_sum_reduce: out[t, :] = T( scale * sum_k float(x[t, k, :]) ), k ascending, float32 accumulate
 // ------------------------------------------------------------------------------------------------
-template <int DT>
+// ELEM (moe_sum with 2..4 experts per token): the running sum is rounded to the element type after every addition
+template <int DT, bool ELEM = false>
 __global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const void* __restrict__ x, void* __restrict__ out,
                                                              int64_t tokens, int topk, int hidden, int64_t stride_t,
                                                              int64_t stride_k, int64_t out_stride_t, float scale) {
@@ -240,10 +241,12 @@ __global__ __launch_bounds__(256) void moe_sum_reduce_kernel(const void* __restr
       float v[8];
       load8<DT>(x, t * stride_t + (int64_t)k * stride_k + c, v);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) acc[j] += v[j];
+      for (int j = 0; j < 8; ++j) acc[j] = (ELEM && k > 0) ? round_to<DT>(acc[j] + v[j]) : acc[j] + v[j];
     }
+    if (!ELEM) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc[j] *= scale;
+      for (int j = 0; j < 8; ++j) acc[j] *= scale;
+    }
     store8<DT>(out, t * out_stride_t + c, acc);
   }
 }
@@ -552,10 +555,8 @@ extern "C" int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t
   return check_launch("silu_and_mul");
 }
 
-extern "C" int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden,
-                                   int64_t stride_token, int64_t stride_topk, int64_t out_stride_token, float scale,
-                                   int dtype, void* stream) {
-  clear_error();
+static int moe_sum_impl(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,
+                        int64_t stride_topk, int64_t out_stride_token, float scale, int dtype, bool elem, void* stream) {
   FP8K_REQUIRE(tokens >= 0 && topk >= 0 && hidden >= 0, "moe_sum_reduce: negative shape");
   FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "moe_sum_reduce: bad dtype %d", dtype);
   FP8K_REQUIRE(hidden % 8 == 0 && hidden <= 0x7fffffffLL && topk <= 0x7fffffffLL,
@@ -568,8 +569,15 @@ extern "C" int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int
   FP8K_REQUIRE(aligned(x, 16) && aligned(out, 16), "moe_sum_reduce: pointers must be 16-byte aligned");
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(stream_grid(tokens * (hidden / 8))), block(256);
-#define FP8K_SR(DT) \
-  hipLaunchKernelGGL(moe_sum_reduce_kernel<DT>, grid, block, 0, st, x, out, tokens, (int)topk, (int)hidden, stride_token, stride_topk, out_stride_token, scale)
+#define FP8K_SR(DT)                                                                                                         \
+  do {                                                                                                                      \
+    if (elem)                                                                                                               \
+      hipLaunchKernelGGL((moe_sum_reduce_kernel<DT, true>), grid, block, 0, st, x, out, tokens, (int)topk, (int)hidden,     \
+                         stride_token, stride_topk, out_stride_token, scale);                                               \
+    else                                                                                                                    \
+      hipLaunchKernelGGL((moe_sum_reduce_kernel<DT, false>), grid, block, 0, st, x, out, tokens, (int)topk, (int)hidden,    \
+                         stride_token, stride_topk, out_stride_token, scale);                                               \
+  } while (0)
   switch (dtype) {
     case FP8K_BF16: FP8K_SR(FP8K_BF16); break;
     case FP8K_F16: FP8K_SR(FP8K_F16); break;
@@ -577,6 +585,21 @@ extern "C" int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int
   }
 #undef FP8K_SR
   return check_launch("moe_sum_reduce");
+}
+
+extern "C" int fp8k_moe_sum_reduce(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden,
+                                   int64_t stride_token, int64_t stride_topk, int64_t out_stride_token, float scale,
+                                   int dtype, void* stream) {
+  clear_error();
+  return moe_sum_impl(x, out, tokens, topk, hidden, stride_token, stride_topk, out_stride_token, scale, dtype, false, stream);
+}
+
+extern "C" int fp8k_moe_sum(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,
+                            int64_t stride_topk, int64_t out_stride_token, int dtype, void* stream) {
+  clear_error();
+  // 2, 3 and 4 experts per token: one rounding to the element type per addition; otherwise the float-accumulated sum
+  return moe_sum_impl(x, out, tokens, topk, hidden, stride_token, stride_topk, out_stride_token, 1.0f, dtype,
+                      topk >= 2 && topk <= 4, stream);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -884,7 +907,7 @@ __global__ __launch_bounds__(256) void shuffle_mul_sum_kernel(const void* __rest
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     for (int j = 0; j < topk; ++j) {
       const int64_t slot = t * topk + j;
-      const int64_t r = perm[slot];
+      const int64_t r = perm ? perm[slot] : slot;
       if (r < 0 || r >= in_rows) continue;
       float f = 1.0f;
       if (factors) {
@@ -904,11 +927,17 @@ __global__ __launch_bounds__(256) void shuffle_mul_sum_kernel(const void* __rest
 // Block table of the grouped GEMM for the expert-major layout: expert e owns rows [starts[e], starts[e] + sizes[3e]).
 // Every expert's rows are cut into blocks of `block` slots (the last one padded with the id `rows`), experts in
 // ascending order.  One workgroup: scan of the block counts by the first wavefront, then one pass over the slots.
+// With slot_expert / slot_row given (the routed expert of every (token, k) slot and the expert-major row that
+// moe_prepare_kernel gave it) the table holds the SLOT at the position of its row, padded with num_slots: the grouped
+// GEMM then gathers token slot / top_k straight from the un-shuffled activations and writes its rows in slot order.
 __global__ __launch_bounds__(kAlignThreads) void moe_offset_blocks_kernel(const int32_t* __restrict__ starts,
                                                                           const int32_t* __restrict__ sizes, int E, int rows,
                                                                           int block, int32_t* __restrict__ sorted,
                                                                           int32_t* __restrict__ expert_ids,
-                                                                          int32_t* __restrict__ post_pad, int max_blocks) {
+                                                                          int32_t* __restrict__ post_pad, int max_blocks,
+                                                                          const int32_t* __restrict__ slot_expert,
+                                                                          const int32_t* __restrict__ slot_row,
+                                                                          int num_slots) {
   __shared__ int32_t first_block[kAlignMaxBuckets + 1];
   const int tid = threadIdx.x;
   if (tid < 64) {
@@ -953,7 +982,18 @@ __global__ __launch_bounds__(kAlignThreads) void moe_offset_blocks_kernel(const 
     }
     const int within = i - first_block[lo] * block;
     const int row = starts[lo] + within;
-    sorted[i] = (within < sizes[lo * 3] && row >= 0 && row < rows) ? row : rows;
+    if (slot_row) sorted[i] = num_slots;
+    else sorted[i] = (within < sizes[lo * 3] && row >= 0 && row < rows) ? row : rows;
+  }
+  if (!slot_row) return;
+  __syncthreads();  // the padding values are in place before any slot lands on one of them
+  for (int i = tid; i < num_slots; i += kAlignThreads) {
+    const int e = slot_expert[i];
+    if (e < 0 || e >= E) continue;
+    const int within = slot_row[i] - starts[e];
+    if (within < 0 || within >= sizes[e * 3]) continue;
+    const int64_t pos = (int64_t)first_block[e] * block + within;
+    if (pos < total) sorted[pos] = i;
   }
 }
 
@@ -1006,7 +1046,7 @@ extern "C" int fp8k_apply_shuffle_mul_sum(const void* input, void* output, const
   FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "%s: bad dtype %d", op, dtype);
   FP8K_REQUIRE(cols % 8 == 0 && cols <= 0x7fffffffLL, "%s: the row length (%lld) must be a multiple of 8", op, (long long)cols);
   if (m == 0 || cols == 0) return FP8K_OK;
-  FP8K_REQUIRE(output && (topk == 0 || (input && permutation)), "%s: null pointer", op);
+  FP8K_REQUIRE(output && (topk == 0 || input), "%s: null pointer", op);
   FP8K_REQUIRE(aligned(input, 16) && aligned(output, 16), "%s: pointers must be 16-byte aligned", op);
   const dim3 grid(stream_grid(m * (cols / 8))), block(256);
   hipStream_t st = (hipStream_t)stream;
@@ -1040,6 +1080,33 @@ extern "C" int fp8k_moe_blocks_from_offsets(const int32_t* expert_starts, const 
   const int64_t max_blocks = sorted_capacity / block_m < expert_capacity ? sorted_capacity / block_m : expert_capacity;
   hipLaunchKernelGGL(moe_offset_blocks_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, expert_starts,
                      problem_sizes, (int)num_experts, (int)rows, (int)block_m, sorted_token_ids, expert_ids,
-                     num_tokens_post_pad, (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks));
+                     num_tokens_post_pad, (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks),
+                     (const int32_t*)nullptr, (const int32_t*)nullptr, 0);
+  return check_launch(op);
+}
+
+extern "C" int fp8k_moe_slot_blocks_from_offsets(const int32_t* expert_starts, const int32_t* problem_sizes,
+                                                 int64_t num_experts, const int32_t* topk_ids, const int32_t* slot_rows,
+                                                 int64_t num_slots, int64_t block_m, int32_t* sorted_token_ids,
+                                                 int64_t sorted_capacity, int32_t* expert_ids, int64_t expert_capacity,
+                                                 int32_t* num_tokens_post_pad, void* stream) {
+  clear_error();
+  const char* op = "moe_slot_blocks_from_offsets";
+  FP8K_REQUIRE(num_experts >= 1 && num_experts <= kAlignMaxBuckets, "%s: num_experts must be in [1, %d] (got %lld)", op,
+               kAlignMaxBuckets, (long long)num_experts);
+  FP8K_REQUIRE(num_slots >= 0 && num_slots < 0x7fffffffLL && block_m >= 1 && block_m <= 1024, "%s: bad slot count / block size", op);
+  FP8K_REQUIRE(expert_starts && problem_sizes && sorted_token_ids && expert_ids && num_tokens_post_pad, "%s: null pointer", op);
+  FP8K_REQUIRE(num_slots == 0 || (topk_ids && slot_rows), "%s: null pointer", op);
+  const int64_t used = num_slots < num_experts ? num_slots : num_experts;
+  const int64_t worst = num_slots + used * (block_m - 1);
+  FP8K_REQUIRE(sorted_capacity >= worst / block_m * block_m && expert_capacity >= worst / block_m,
+               "%s: block table too small (%lld slots, %lld blocks; %lld slots may be needed)", op, (long long)sorted_capacity,
+               (long long)expert_capacity, (long long)(worst / block_m * block_m));
+  const int64_t max_blocks = sorted_capacity / block_m < expert_capacity ? sorted_capacity / block_m : expert_capacity;
+  // slot_rows of an empty problem is never read: any non-null pointer keeps the kernel on its slot path
+  hipLaunchKernelGGL(moe_offset_blocks_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, expert_starts,
+                     problem_sizes, (int)num_experts, (int)num_slots, (int)block_m, sorted_token_ids, expert_ids,
+                     num_tokens_post_pad, (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks), topk_ids,
+                     slot_rows ? slot_rows : expert_starts, (int)num_slots);
   return check_launch(op);
 }

@@ -116,7 +116,7 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
   };
   constexpr int LPG = GROUP / 8;
   constexpr int GPW = 64 / LPG;
-  static_assert(KIND == FP8K_SCALE_F32 || GROUP == 128, "packed UE8M0 scales need 128-element groups");
+  static_assert(KIND != FP8K_SCALE_UE8M0_PACKED || GROUP == 128, "packed UE8M0 scales need 128-element groups");
 
   const int lane = threadIdx.x & 63;
   const int lg = lane / LPG, li = lane % LPG;
@@ -189,6 +189,14 @@ __global__ __launch_bounds__(256) void group_quant_kernel(const void* __restrict
                            ((uint32_t)__builtin_amdgcn_readlane((int)eb, 32) << 16) |
                            ((uint32_t)__builtin_amdgcn_readlane((int)eb, 48) << 24);
         if (lane == 0) reinterpret_cast<uint32_t*>(s)[(int64_t)segs[j] * sg + scale_row(rows[j])] = w;
+      } else if (KIND == FP8K_SCALE_UE8M0_F32) {
+        // the same power of two, stored as a float at the place of a float scale
+        const uint32_t b = __float_as_uint(fmaxf(sc, 1e-10f));
+        const uint32_t e = (b >> 23) + ((b & 0x7fffffu) != 0u);
+        const float rinv = __uint_as_float((254u - e) << 23);
+        out.x = cvt4_fp8(a[0] * rinv, a[1] * rinv, a[2] * rinv, a[3] * rinv);
+        out.y = cvt4_fp8(a[4] * rinv, a[5] * rinv, a[6] * rinv, a[7] * rinv);
+        if (valid && li == 0) reinterpret_cast<float*>(s)[scale_row(rows[j]) + (int64_t)g * sg] = __uint_as_float(e << 23);
       } else {
         bool redo;
         out = quant8_bracket<DT != FP8K_F32>(a, sc, amax, redo);
@@ -536,7 +544,8 @@ extern "C" int fp8k_group_quant_masked(const void* x, void* q, void* s, int64_t 
                (long long)K, (long long)group_size);
   FP8K_REQUIRE(fp8_max == 448.0f && fp8_min == -448.0f, "%s: fp8_min/fp8_max must be -448/448 (OCP e4m3fn)", op);
   FP8K_REQUIRE(in_dtype == FP8K_F32 || in_dtype == FP8K_F16 || in_dtype == FP8K_BF16, "%s: bad input dtype %d", op, in_dtype);
-  FP8K_REQUIRE(scale_kind == FP8K_SCALE_F32 || scale_kind == FP8K_SCALE_UE8M0_PACKED, "%s: bad scale kind %d", op, scale_kind);
+  FP8K_REQUIRE(scale_kind == FP8K_SCALE_F32 || scale_kind == FP8K_SCALE_UE8M0_PACKED || scale_kind == FP8K_SCALE_UE8M0_F32,
+               "%s: bad scale kind %d", op, scale_kind);
   FP8K_REQUIRE(E * m_max <= 0x7fffffffLL && m_max <= 0x7fffffffLL && K / group_size <= 0x3fffffffLL, "%s: shape too large", op);
   if (E == 0 || m_max == 0 || K == 0) return FP8K_OK;
   FP8K_REQUIRE(x && q && s && masked_m, "%s: null pointer", op);
@@ -554,7 +563,10 @@ extern "C" int fp8k_group_quant_masked(const void* x, void* q, void* s, int64_t 
 #define FP8K_MQ3(DT, KIND, FUSE) \
   launch_group_quant<DT, 128, KIND, FUSE, true>(x, q, s, M, K, eps_eff, s_stride_m, s_stride_g, st, masked_m, (int)m_max, s_stride_e)
 #define FP8K_MQ2(DT, KIND) (fuse_silu_and_mul ? FP8K_MQ3(DT, KIND, true) : FP8K_MQ3(DT, KIND, false))
-#define FP8K_MQ(DT) (scale_kind == FP8K_SCALE_F32 ? FP8K_MQ2(DT, FP8K_SCALE_F32) : FP8K_MQ2(DT, FP8K_SCALE_UE8M0_PACKED))
+#define FP8K_MQ(DT)                                                  \
+  (scale_kind == FP8K_SCALE_F32            ? FP8K_MQ2(DT, FP8K_SCALE_F32) \
+   : scale_kind == FP8K_SCALE_UE8M0_PACKED ? FP8K_MQ2(DT, FP8K_SCALE_UE8M0_PACKED) \
+                                           : FP8K_MQ2(DT, FP8K_SCALE_UE8M0_F32))
   switch (in_dtype) {
     case FP8K_BF16: return FP8K_MQ(FP8K_BF16);
     case FP8K_F16: return FP8K_MQ(FP8K_F16);

@@ -1,0 +1,157 @@
+// Measurement aids of the fp8k library (declared in include/fp8k_tune.h): probes of what this machine gives the load
+// path and the matrix cores, with none of a GEMM's other work around them.  Timed by the caller.
+#include "gemm_kernels.h"
+
+#include "../../include/fp8k_tune.h"
+
+using namespace fp8k;
+
+namespace fp8k {
+// every workgroup reads its own contiguous share, a 32 KB stage per trip, two stages in flight
+__global__ __launch_bounds__(512, 1) void stream_read_kernel(const uint8_t* __restrict__ src, int64_t share) {
+  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint8_t* base = src + (int64_t)blockIdx.x * share;
+  const int trips = (int)(share >> 15);
+  auto issue = [&](int t) {
+    // the descriptor moves with the trip: a share may exceed the 4 GB a descriptor can span
+    const rsrc_t r = make_rsrc(base + (int64_t)t * 32768, 32768u);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      buf_load16_to_lds(r, (uint32_t)((w * 4 + q) * 1024 + lane * 16), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
+  };
+  issue(0);
+  if (trips > 1) issue(1);
+  for (int t = 0; t < trips; ++t) {
+    if (t + 1 < trips) lds_barrier<4>();
+    else lds_barrier<0>();
+    if (t + 2 < trips) issue(t + 2);
+  }
+  wait_vm0();
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read: bad size");
+  FP8K_REQUIRE(src && aligned(src, 16), "tune_stream_read: src must be a 16-byte aligned device pointer");
+  const int ncu = num_cu();
+  const int64_t share = bytes / ncu / 65536 * 65536;
+  if (share == 0) return FP8K_OK;
+  hipLaunchKernelGGL(stream_read_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src, share);
+  return check_launch("tune_stream_read");
+}
+
+namespace fp8k {
+// stream_read_kernel with a write-out after every `spt` stages ("a tile"): each wave stores `spw` times 1 KB (16 bytes a
+// lane), the workgroup 8 KB x spw, to a place of its own in dst - the shape of a GEMM that streams weights and writes
+// a small output tile per weight tile
+__global__ __launch_bounds__(512, 1) void stream_read_write_kernel(const uint8_t* __restrict__ src, int64_t share,
+                                                                   uint8_t* __restrict__ dst, int spt, int spw) {
+  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const uint8_t* base = src + (int64_t)blockIdx.x * share;
+  const int trips = (int)(share >> 15);
+  const int tiles = trips / spt;
+  auto issue = [&](int t) {
+    const rsrc_t r = make_rsrc(base + (int64_t)t * 32768, 32768u);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      buf_load16_to_lds(r, (uint32_t)((w * 4 + q) * 1024 + lane * 16), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
+  };
+  issue(0);
+  if (trips > 1) issue(1);
+  int t = 0;
+  for (int ti = 0; ti < tiles; ++ti) {
+    for (int k = 0; k < spt; ++k, ++t) {
+      // stores and loads retire in order: a wait that leaves this wave's four youngest loads in flight has seen every
+      // store issued before them complete
+      if (t + 1 < trips) lds_barrier<4>();
+      else lds_barrier<0>();
+      if (t + 2 < trips) issue(t + 2);
+    }
+    uint4* o = reinterpret_cast<uint4*>(dst + ((((int64_t)blockIdx.x * tiles + ti) * 8 + w) * spw) * 1024) + lane;
+    const uint4 v = make_uint4(1u, 2u, 3u, (unsigned)ti);
+    for (int i = 0; i < spw; ++i) o[i * 64] = v;
+  }
+  wait_vm0();
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_stream_read_write(const void* src, int64_t bytes, void* dst, int64_t dst_bytes, int64_t stages_per_tile,
+                                           int64_t stores_per_wave, void* stream) {
+  clear_error();
+  FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read_write: bad size");
+  FP8K_REQUIRE(src && aligned(src, 16) && dst && aligned(dst, 16), "tune_stream_read_write: src and dst must be 16-byte aligned device pointers");
+  FP8K_REQUIRE(stages_per_tile >= 1 && stages_per_tile <= 4096 && stores_per_wave >= 0 && stores_per_wave <= 64,
+               "tune_stream_read_write: stages_per_tile in [1, 4096], stores_per_wave in [0, 64]");
+  const int ncu = num_cu();
+  const int64_t share = bytes / ncu / (32768 * stages_per_tile) * (32768 * stages_per_tile);  // whole tiles per workgroup
+  if (share == 0) return FP8K_OK;
+  const int64_t tiles = share / (32768 * stages_per_tile);
+  FP8K_REQUIRE(dst_bytes >= (int64_t)ncu * tiles * 8 * stores_per_wave * 1024,
+               "tune_stream_read_write: dst holds %lld bytes, %lld are written", (long long)dst_bytes,
+               (long long)((int64_t)ncu * tiles * 8 * stores_per_wave * 1024));
+  hipLaunchKernelGGL(stream_read_write_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src,
+                     share, (uint8_t*)dst, (int)stages_per_tile, (int)stores_per_wave);
+  return check_launch("tune_stream_read_write");
+}
+
+
+namespace fp8k {
+// Bare matrix-core loop: every wave keeps two weight-side and four activation-side operand fragments of the caller's
+// bytes in registers and issues the eight independent products of them, `iters` times over, into eight accumulators -
+// no loads, no LDS, no barriers inside the loop.  One workgroup of 8 waves per CU (two waves per SIMD, the occupancy
+// of the tile kernels).  The accumulators are folded into `sink` at the end so that the loop stays.
+__global__ __launch_bounds__(512, 1) void mfma_peak_kernel(const uint8_t* __restrict__ operands, int64_t bytes, int iters,
+                                                           float* __restrict__ sink) {
+  const int lane = threadIdx.x & 63;
+  const int64_t frag0 = ((int64_t)blockIdx.x * 8 + (threadIdx.x >> 6)) * 6;  // 6 fragments of 64 lanes x 32 bytes per wave
+  const int64_t nfrag = bytes / 2048;
+  v8i a[2], b[4];
+#pragma unroll
+  for (int i = 0; i < 6; ++i) {
+    const v8i v = *reinterpret_cast<const v8i*>(operands + ((frag0 + i) % nfrag) * 2048 + lane * 32);
+    if (i < 2) a[i] = v;
+    else b[i - 2] = v;
+  }
+  v16f acc[2][4];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma_32x32x64(a[i], b[j], acc[i][j]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s += acc[i][j][r];
+  sink[(int64_t)blockIdx.x * 512 + threadIdx.x] = s;
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_mfma_peak(const void* operands, int64_t bytes, int64_t iters, float* sink, int64_t sink_floats,
+                                   int64_t* flops, void* stream) {
+  clear_error();
+  const char* op = "tune_mfma_peak";
+  FP8K_REQUIRE(operands && aligned(operands, 32), "%s: operands must be a 32-byte aligned device pointer", op);
+  FP8K_REQUIRE(bytes >= 2048 && bytes < (1LL << 40), "%s: at least 2048 operand bytes are needed", op);
+  FP8K_REQUIRE(iters >= 1 && iters <= (1 << 24), "%s: iters must be in [1, 2^24]", op);
+  const int ncu = num_cu();
+  FP8K_REQUIRE(sink && sink_floats >= (int64_t)ncu * 512, "%s: sink must hold %lld floats", op, (long long)ncu * 512);
+  if (flops) *flops = (int64_t)ncu * 8 * iters * 8 * (2LL * 32 * 32 * 64);
+  hipLaunchKernelGGL(mfma_peak_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)operands, bytes,
+                     (int)iters, sink);
+  return check_launch(op);
+}

@@ -83,7 +83,7 @@ _register(
     _none,
 )
 _register("shuffle_rows(Tensor input, Tensor dst2src_map, Tensor(a!) output) -> ()", _k.shuffle_rows_out, _none)
-_register("apply_shuffle_mul_sum(Tensor input, Tensor(a!) output, Tensor permutation, Tensor? factors) -> ()",
+_register("apply_shuffle_mul_sum(Tensor input, Tensor(a!) output, Tensor? permutation, Tensor? factors) -> ()",
           _k.apply_shuffle_mul_sum, _none)
 _register(
     "fp8_blockwise_scaled_grouped_mm(Tensor(a!) output, Tensor a_ptrs, Tensor b_ptrs, Tensor out_ptrs, Tensor a_scales_ptrs, "
@@ -91,6 +91,18 @@ _register(
     "Tensor stride_c, Tensor layout_sfa, Tensor layout_sfb, Tensor problem_sizes, Tensor expert_offsets, Tensor workspace) -> ()",
     _k.fp8_blockwise_scaled_grouped_mm, _none,
 )
+
+
+
+def _slot_blocks_fake(topk_ids, expert_offsets, problem_sizes, output_permutation, block_m):
+    slots, E = topk_ids.numel(), problem_sizes.shape[0]
+    cap = max((slots + min(slots, E) * (block_m - 1)) // block_m * block_m, block_m)
+    i32 = lambda n: topk_ids.new_empty((n,), dtype=torch.int32)  # noqa: E731
+    return i32(cap), i32(cap // block_m), i32(1)
+
+
+_register("moe_slot_blocks(Tensor topk_ids, Tensor expert_offsets, Tensor problem_sizes, Tensor output_permutation, "
+          "int block_m) -> (Tensor, Tensor, Tensor)", _k.moe_slot_blocks, _slot_blocks_fake)
 
 # ---- fused-MoE stages
 _register(
@@ -205,6 +217,10 @@ def shuffle_rows(input_tensor, dst2src_map, output_tensor_shape) -> torch.Tensor
 
 def apply_shuffle_mul_sum(input, output, permutation, factors) -> None:
     _ops.apply_shuffle_mul_sum(input, output, permutation, factors)
+
+
+def moe_slot_blocks(topk_ids, expert_offsets, problem_sizes, output_permutation, block_m: int):
+    return _ops.moe_slot_blocks(topk_ids, expert_offsets, problem_sizes, output_permutation, block_m)
 
 
 def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_ptrs, b_scales_ptrs, a, b, scales_a, scales_b,

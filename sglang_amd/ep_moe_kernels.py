@@ -8,7 +8,6 @@ import torch
 
 from . import custom_ops as _ops
 from .fp8_kernel import fp8_max, fp8_min
-from .sgl_kernel import unpack_ue8m0_scales
 
 
 def silu_and_mul_masked_post_quant_fwd(
@@ -30,20 +29,12 @@ def silu_and_mul_masked_post_quant_fwd(
     assert input.shape[0] == masked_m.shape[0]
     assert input.shape[-1] % 2 == 0
     assert (input.shape[-1] // 2) % quant_group_size == 0
-    mm = masked_m.to(torch.int32)
-    if scale_ue8m0:
-        # scale = 2^ceil(log2(amax / 448)) stored as float32 (reference kernel :348-350).  The kernel writes such scales
-        # as packed exponent bytes: they are written to a temporary and expanded into the valid rows of output_scale.
-        if quant_group_size != 128:
-            raise RuntimeError("silu_and_mul_masked_post_quant_fwd: UE8M0 scales are built for groups of 128")
-        e, m, h = output.shape
-        kb = h // quant_group_size
-        packed = torch.zeros((e, (kb + 3) // 4, (m + 3) // 4 * 4), device=input.device, dtype=torch.int32).transpose(-1, -2)[:, :m, :]
-        _ops.sgl_per_token_group_quant_8bit(input, output, packed, quant_group_size, 1e-10, fp8_min, fp8_max, True, True, mm)
-        valid = torch.arange(m, device=input.device, dtype=torch.int32)[None, :, None] < mm[:, None, None]
-        output_scale.copy_(torch.where(valid, unpack_ue8m0_scales(packed, kb), output_scale))
-        return
-    _ops.sgl_per_token_group_quant_8bit(input, output, output_scale, quant_group_size, 1e-10, fp8_min, fp8_max, False, True, mm)
+    if scale_ue8m0 and quant_group_size != 128:
+        raise RuntimeError("silu_and_mul_masked_post_quant_fwd: UE8M0 scales are built for groups of 128")
+    # scale_ue8m0 with a float32 output_scale: the kernel stores 2^ceil(log2(amax / 448)) as a float (reference kernel
+    # :348-350)
+    _ops.sgl_per_token_group_quant_8bit(input, output, output_scale, quant_group_size, 1e-10, fp8_min, fp8_max, scale_ue8m0,
+                                        True, masked_m.to(torch.int32))
 
 
 def tma_align_input_scale(input_scale: torch.Tensor) -> torch.Tensor:

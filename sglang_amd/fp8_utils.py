@@ -188,7 +188,7 @@ def requant_weight_ue8m0_inplace(weight: torch.nn.Parameter, weight_scale_inv: t
     q, s = requant_weight_ue8m0(weight.data.to(weight_scale_inv.device), weight_scale_inv.data, weight_block_size)
     weight.data = q
     weight_scale_inv.data = s
-    mark_ue8m0(weight_scale_inv.data, check=False)
+    mark_ue8m0(weight_scale_inv, check=False)  # the parameter object: it lives as long as the layer does
 
 
 def transform_scale_ue8m0(sf: torch.Tensor, mn: int) -> torch.Tensor:

@@ -251,41 +251,6 @@ def fused_experts(hidden_states, w1, w2, topk_weights, topk_ids, **kwargs) -> to
     return fused_experts_impl(hidden_states, w1, w2, topk_weights, topk_ids, inplace=False, **kwargs)
 
 
-def biased_grouped_topk_impl(
-    hidden_states: torch.Tensor,
-    gating_output: torch.Tensor,
-    correction_bias: torch.Tensor,
-    topk: int,
-    renormalize: bool,
-    num_expert_group: Optional[int] = None,
-    topk_group: Optional[int] = None,
-    routed_scaling_factor: Optional[float] = None,
-    apply_routed_scaling_factor_on_output: bool = False,
-) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Grouped top-k routing with a selection bias in plain tensor ops, for the shapes the fused gate kernel does not
-    take (same interface and selection rule as python/sglang/srt/layers/moe/topk.py:665-738): an expert's choice value
-    is sigmoid(logit) + bias; a group is worth the sum of its two best choice values; only experts of the
-    `topk_group` best groups compete for the `topk` places; the routing weights are the un-biased sigmoid values of
-    the winners, normalised to sum 1 when `renormalize`."""
-    tokens, experts = gating_output.shape
-    assert hidden_states.shape[0] == tokens, "Number of tokens mismatch"
-    per_group = experts // num_expert_group
-    prob = torch.sigmoid(gating_output)
-    choice = (prob + correction_bias).view(tokens, num_expert_group, per_group)
-    group_worth = torch.topk(choice, 2, dim=2).values.sum(dim=2)                      # [tokens, groups]
-    kept_groups = torch.topk(group_worth, topk_group, dim=1, sorted=False).indices     # [tokens, topk_group]
-    group_open = torch.zeros((tokens, num_expert_group), dtype=torch.bool, device=choice.device)
-    group_open.scatter_(1, kept_groups, True)
-    candidates = torch.where(group_open.unsqueeze(2), choice, choice.new_full((), float("-inf"))).view(tokens, experts)
-    winners = torch.topk(candidates, topk, dim=1, sorted=False).indices
-    weights = torch.gather(prob, 1, winners)
-    if renormalize:
-        weights = weights / weights.sum(dim=1, keepdim=True)
-        if apply_routed_scaling_factor_on_output:
-            weights = weights * routed_scaling_factor
-    return weights.float(), winners.int()
-
-
 def biased_grouped_topk(
     hidden_states: torch.Tensor,
     gating_output: torch.Tensor,
@@ -298,23 +263,22 @@ def biased_grouped_topk(
     routed_scaling_factor: Optional[float] = None,
     apply_routed_scaling_factor_on_output: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Reference: biased_grouped_topk_gpu, python/sglang/srt/layers/moe/topk.py:762-850: the fused gate kernel
-    where its shape limits hold (power-of-two expert count, at most 32 experts per group, renormalised weights),
-    the torch restatement otherwise."""
+    """Reference: biased_grouped_topk_gpu, python/sglang/srt/layers/moe/topk.py:762-850, on the fused gate kernel.
+    Its shape limits are the reference kernel's (power-of-two expert count, at most 32 experts per group, at most 64
+    groups, renormalised weights); where the reference falls back to tensor ops for other shapes, this path has no
+    second implementation and raises."""
     experts = gating_output.shape[1]
     fits = (
         renormalize and num_expert_group and topk_group and experts & (experts - 1) == 0
         and experts % num_expert_group == 0 and experts // num_expert_group <= 32 and num_expert_group <= 64
     )
-    if fits:
-        return _ops.moe_fused_gate(
-            gating_output.contiguous(), correction_bias.to(gating_output.dtype).contiguous(), num_expert_group, topk_group,
-            topk, num_fused_shared_experts, routed_scaling_factor if routed_scaling_factor is not None else 0.0,
-            apply_routed_scaling_factor_on_output,
-        )
-    if num_fused_shared_experts:
-        raise RuntimeError("biased_grouped_topk: shared-expert fusion needs the fused gate kernel's shapes")
-    return biased_grouped_topk_impl(
-        hidden_states, gating_output, correction_bias, topk, renormalize, num_expert_group, topk_group,
-        routed_scaling_factor, apply_routed_scaling_factor_on_output,
+    if not fits:
+        raise RuntimeError(
+            "biased_grouped_topk: built for renormalised weights, a power-of-two expert count, at most 32 experts per "
+            "group and at most 64 groups (got %d experts, %s groups, renormalize=%s)" % (experts, num_expert_group, renormalize))
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    return _ops.moe_fused_gate(
+        gating_output.contiguous(), correction_bias.to(gating_output.dtype).contiguous(), num_expert_group, topk_group,
+        topk, num_fused_shared_experts, routed_scaling_factor if routed_scaling_factor is not None else 0.0,
+        apply_routed_scaling_factor_on_output,
     )

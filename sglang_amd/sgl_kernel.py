@@ -7,7 +7,9 @@ on the current torch stream of the tensor's device and never synchronises.
 """
 from __future__ import annotations
 
+import weakref
 from typing import Optional
+
 
 import torch
 
@@ -125,8 +127,9 @@ def sgl_per_token_group_quant_8bit(
 def _group_quant_masked(input, output_q, output_s, group_size, eps, fp8_min, fp8_max, scale_ue8m0, fuse_silu_and_mul,
                         masked_m) -> None:
     """Masked expert layout of the v2 op (gemm.py:118-133): input [E, m_max, K] (or 2K with fuse_silu_and_mul),
-    output_q [E, m_max, K], output_s [E, m_max, K/g] float32 in any strides or int32 [E, m_max, ceil(K/g/4)] packed;
-    masked_m int32 [E] - rows at or past masked_m[e] are neither read nor written."""
+    output_q [E, m_max, K], output_s [E, m_max, K/g] float32 in any strides or int32 [E, m_max, ceil(K/g/4)] packed
+    (scale_ue8m0 with a float32 output_s stores the powers of two as floats); masked_m int32 [E] - rows at or past
+    masked_m[e] are neither read nor written."""
     if input.dim() != 3 or output_q.dim() != 3 or output_s.dim() != 3:
         raise RuntimeError("masked_m needs 3-D input, output_q and output_s ([num_experts, max_tokens, hidden])")
     if not (input.is_contiguous() and output_q.is_contiguous()):
@@ -144,7 +147,12 @@ def _group_quant_masked(input, output_q, output_s, group_size, eps, fp8_min, fp8
         raise RuntimeError("output_q must be [num_experts, max_tokens, hidden]")
     if masked_m.dtype != torch.int32 or masked_m.numel() != E or not masked_m.is_contiguous():
         raise RuntimeError("masked_m must be contiguous int32 [num_experts]")
-    if scale_ue8m0:
+    if scale_ue8m0 and output_s.dtype == torch.float32:
+        # the rounded-up power of two as a float at the place of a float scale (ep_moe/kernels.py:348-350)
+        if tuple(output_s.shape) != (E, m_max, G):
+            raise RuntimeError("output_s must be float32 [num_experts, max_tokens, K/group_size]")
+        kind = _lib.SCALE_UE8M0_F32
+    elif scale_ue8m0:
         if output_s.dtype != torch.int32 or tuple(output_s.shape) != (E, m_max, (G + 3) // 4):
             raise RuntimeError("packed output_s must be int32 [num_experts, max_tokens, ceil(K/group/4)]")
         kind = _lib.SCALE_UE8M0_PACKED
@@ -424,21 +432,49 @@ def unpack_ue8m0_weight_scales(packed: torch.Tensor, K: int) -> torch.Tensor:
     return unpack_ue8m0_scales(packed[..., ::128, :], kb)
 
 
+# Tensors declared to hold powers of two, by the memory they describe: (device, address of the first element, shape,
+# strides) -> weak reference to the tensor object that was marked.  A Python attribute on the tensor object alone would
+# be lost by every `.data`, `nn.Parameter(t)` or view that describes the same memory with a new object; an entry lives
+# only as long as the marked object does (so the memory cannot have been handed to another tensor meanwhile).
+_UE8M0_MARKED: dict = {}
+
+
+def _memory_key(t: torch.Tensor):
+    return (str(t.device), t.data_ptr(), tuple(t.shape), tuple(t.stride()))
+
+
 def is_ue8m0(scales: torch.Tensor) -> bool:
-    """True for a float32 scale tensor that has been declared to hold powers of two only (mark_ue8m0)."""
-    return bool(getattr(scales, "_fp8k_ue8m0", False))
+    """True for a float32 scale tensor whose memory has been declared to hold powers of two only (mark_ue8m0): the
+    marked tensor itself, its `.data`, a Parameter wrapped around it, or any other tensor object of the same device,
+    address, shape and strides, for as long as the marked object is alive."""
+    if scales.dtype != torch.float32:
+        return False
+    if getattr(scales, "_fp8k_ue8m0", False):  # the marked object itself (also what a graph tracer can see)
+        return True
+    if torch.compiler.is_compiling():  # no addresses while tracing: unmarked objects take the float-scale kernels
+        return False
+    ref = _UE8M0_MARKED.get(_memory_key(scales))
+    return ref is not None and ref() is not None
 
 
 def mark_ue8m0(scales: torch.Tensor, check: bool = True) -> torch.Tensor:
     """Declare a float32 weight-scale tensor to hold positive powers of two only, which lets the block GEMM hand the
     exponents to the matrix core instead of multiplying.  With `check` (the default; one device synchronisation, meant
-    for weight-loading time) every mantissa is verified to be zero first.  Returns the same tensor."""
+    for weight-loading time) every mantissa is verified to be zero first.  The declaration is about the contents: mark
+    again after overwriting them.  Returns the same tensor."""
     if scales.dtype != torch.float32:
         raise RuntimeError("mark_ue8m0: float32 scales expected")
     if check:
         bits = scales.contiguous().view(torch.int32)
         if bool(((bits & 0x7FFFFF) != 0).any()) or bool((bits <= 0).any()):
             raise RuntimeError("mark_ue8m0: the scales are not all positive powers of two")
+    key = _memory_key(scales)
+
+    def _forget(ref, key=key):
+        if _UE8M0_MARKED.get(key) is ref:
+            del _UE8M0_MARKED[key]
+
+    _UE8M0_MARKED[key] = weakref.ref(scales, _forget)
     scales._fp8k_ue8m0 = True
     return scales
 
@@ -545,35 +581,36 @@ def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
 def moe_sum_reduce(input_tensor: torch.Tensor, output_tensor: torch.Tensor, routed_scaling_factor: float = 0) -> None:
     """Reference: sgl-kernel/python/sgl_kernel/moe.py:83-92; csrc/moe/moe_sum_reduce.cu:227-.
     input [tokens, topk, hidden] (hidden contiguous), output [tokens, hidden]."""
-    require_cuda(input_tensor, output_tensor)
-    if input_tensor.dim() != 3 or output_tensor.dim() != 2:
-        raise RuntimeError("moe_sum_reduce: input must be [tokens, topk, hidden] and output [tokens, hidden]")
-    T, topk, H = input_tensor.shape
-    if output_tensor.shape[0] != T or output_tensor.shape[1] != H:
-        raise RuntimeError("moe_sum_reduce: output shape does not match the input")
-    if input_tensor.dtype != output_tensor.dtype:
-        raise RuntimeError("moe_sum_reduce: input and output dtypes differ")
-    if (H > 1 and input_tensor.stride(2) != 1) or (H > 1 and output_tensor.stride(1) != 1):
-        raise RuntimeError("moe_sum_reduce: the hidden dimension must be contiguous")
+    T, topk, H = _sum_args("moe_sum_reduce", input_tensor, output_tensor)
     check(lib.fp8k_moe_sum_reduce(input_tensor.data_ptr(), output_tensor.data_ptr(), T, topk, H, input_tensor.stride(0),
                                   input_tensor.stride(1), output_tensor.stride(0), float(routed_scaling_factor),
                                   dtype_code(input_tensor.dtype), stream_ptr(input_tensor.device)))
 
 
+def _sum_args(op: str, input_tensor: torch.Tensor, output_tensor: torch.Tensor):
+    require_cuda(input_tensor, output_tensor)
+    if input_tensor.dim() != 3 or output_tensor.dim() != 2:
+        raise RuntimeError("%s: input must be [tokens, topk, hidden] and output [tokens, hidden]" % op)
+    T, topk, H = input_tensor.shape
+    if output_tensor.shape[0] != T or output_tensor.shape[1] != H:
+        raise RuntimeError("%s: output shape does not match the input" % op)
+    if input_tensor.dtype != output_tensor.dtype:
+        raise RuntimeError("%s: input and output dtypes differ" % op)
+    if (H > 1 and input_tensor.stride(2) != 1) or (H > 1 and output_tensor.stride(1) != 1):
+        raise RuntimeError("%s: the hidden dimension must be contiguous" % op)
+    return T, topk, H
+
+
 def moe_sum(input_tensor: torch.Tensor, output_tensor: torch.Tensor) -> None:
     """Reference: sgl-kernel/python/sgl_kernel/moe.py:95-102; csrc/moe/moe_sum.cu:11-69.  input [tokens, topk, hidden],
     output [tokens, hidden].  As in the reference, 2, 3 and 4 experts per token are summed in the element type, one
-    rounding per addition (the elementwise adds of torch do exactly that); any other count is the float-accumulated sum
-    of moe_sum_reduce with factor 1."""
-    if input_tensor.dim() != 3 or input_tensor.shape[1] == 0:
+    rounding per addition; any other count is the float-accumulated sum of moe_sum_reduce with factor 1."""
+    T, topk, H = _sum_args("moe_sum", input_tensor, output_tensor)
+    if topk == 0:
         raise RuntimeError("moe_sum: input must be [tokens, topk, hidden] with topk >= 1")
-    topk = input_tensor.shape[1]
-    if topk in (2, 3, 4):
-        torch.add(input_tensor[:, 0], input_tensor[:, 1], out=output_tensor)
-        for k in range(2, topk):
-            output_tensor.add_(input_tensor[:, k])
-        return
-    moe_sum_reduce(input_tensor, output_tensor, 1.0)
+    check(lib.fp8k_moe_sum(input_tensor.data_ptr(), output_tensor.data_ptr(), T, topk, H, input_tensor.stride(0),
+                           input_tensor.stride(1), output_tensor.stride(0), dtype_code(input_tensor.dtype),
+                           stream_ptr(input_tensor.device)))
 
 
 def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: int, num_valid_tokens: int) -> torch.Tensor:
@@ -694,20 +731,25 @@ def apply_shuffle_mul_sum(input: torch.Tensor, output: torch.Tensor, permutation
     """Reference: sgl-kernel/python/sgl_kernel/moe.py:243-251:
     output = (input[permutation].view(m, topk, k) * factors.view(m, topk, 1)).sum(dim=1), summed in float32."""
     require_cuda(input, output, permutation, factors)
-    if input.dim() != 2 or output.dim() != 2 or permutation.dim() != 1:
+    if input.dim() != 2 or output.dim() != 2 or (permutation is not None and permutation.dim() != 1):
         raise RuntimeError("apply_shuffle_mul_sum: input [m * topk, k], output [m, k], permutation [m * topk]")
     if input.dtype != output.dtype or not (input.is_contiguous() and output.is_contiguous()) or input.shape[1] != output.shape[1]:
         raise RuntimeError("apply_shuffle_mul_sum: input and output must be contiguous, of one dtype and row length")
     m = output.shape[0]
-    topk = permutation.numel() // m if m else 0
-    if permutation.numel() != m * topk or permutation.dtype != torch.int32 or not permutation.is_contiguous():
-        raise RuntimeError("apply_shuffle_mul_sum: permutation size must match m * topk (contiguous int32)")
+    if permutation is None:  # rows already in slot order: output[t] sums input[t * topk .. t * topk + topk - 1]
+        topk = input.shape[0] // m if m else 0
+        if input.shape[0] != m * topk:
+            raise RuntimeError("apply_shuffle_mul_sum: without a permutation input must hold m * topk rows")
+    else:
+        topk = permutation.numel() // m if m else 0
+        if permutation.numel() != m * topk or permutation.dtype != torch.int32 or not permutation.is_contiguous():
+            raise RuntimeError("apply_shuffle_mul_sum: permutation size must match m * topk (contiguous int32)")
     if factors is not None:
         if factors.dtype != output.dtype:
             raise RuntimeError("apply_shuffle_mul_sum: factors must match output dtype")
         if factors.numel() != m * topk or not factors.is_contiguous():
             raise RuntimeError("apply_shuffle_mul_sum: factors must have shape [m * topk]")
-    check(lib.fp8k_apply_shuffle_mul_sum(input.data_ptr(), output.data_ptr(), permutation.data_ptr(),
+    check(lib.fp8k_apply_shuffle_mul_sum(input.data_ptr(), output.data_ptr(), None if permutation is None else permutation.data_ptr(),
                                          None if factors is None else factors.data_ptr(), m, topk, output.shape[1], input.shape[0],
                                          dtype_code(output.dtype), stream_ptr(output.device)))
 
@@ -728,8 +770,9 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
     """Reference: sgl-kernel/python/sgl_kernel/moe.py:175-214 (csrc/moe/fp8_blockwise_moe_kernel.cu).  For every expert e:
     output[rows_e] = a[rows_e] @ b[e] with 1x128 scales on a and 128x128 scales on b, rows_e = expert_offsets[e] ..
     + problem_sizes[e, 0].  a e4m3fn [rows, K]; b e4m3fn [E, K, N] column-major per expert (a [E, N, K] weight
-    transposed); scales_a float32 [rows, K/128]; scales_b float32 [E, K/128, N/128] (the [E, N/128, K/128] checkpoint
-    tensor transposed) or [E, N/128, K/128] contiguous; output bf16 / fp16 [rows, N].  The pointer arrays, stride
+    transposed); scales_a float32 [rows, K/128]; scales_b float32 [E, K/128, N/128] with any strides (the reference
+    passes the [E, N/128, K/128] checkpoint tensor transposed), or, when N/128 != K/128 makes the shape unambiguous, the
+    un-transposed [E, N/128, K/128] tensor; output bf16 / fp16 [rows, N].  The pointer arrays, stride
     vectors, scale-layout buffers and the workspace serve the reference's CUTLASS launcher and are ignored here:
     the grouped kernel takes a block table built on the device from expert_offsets and problem_sizes."""
     require_cuda(output, a, b, scales_a, scales_b, problem_sizes, expert_offsets)
@@ -741,9 +784,11 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
     kb, nb = (K + 127) // 128, (N + 127) // 128
     if scales_b.dim() != 3 or scales_b.shape[0] != E:
         raise RuntimeError("fp8_blockwise_scaled_grouped_mm: scales_b must be [E, K/128, N/128]")
-    if tuple(scales_b.shape[1:]) == (kb, nb) and (scales_b.stride(1) == 1 or kb == 1):
+    # the op's own layout is [E, K/128, N/128] whatever the strides (a square tensor is always read that way); a tensor
+    # whose shape can only be the un-transposed [E, N/128, K/128] checkpoint tensor is taken as that
+    if tuple(scales_b.shape[1:]) == (kb, nb):
         bs = scales_b.transpose(1, 2)
-    elif tuple(scales_b.shape[1:]) == (nb, kb) and (scales_b.stride(2) == 1 or kb == 1):
+    elif tuple(scales_b.shape[1:]) == (nb, kb):
         bs = scales_b
     else:
         raise RuntimeError("fp8_blockwise_scaled_grouped_mm: scales_b must be the [E, N/128, K/128] tensor or its transpose")
@@ -762,6 +807,29 @@ def fp8_blockwise_scaled_grouped_mm(output, a_ptrs, b_ptrs, out_ptrs, a_scales_p
                                            sorted_ids.data_ptr(), cap, expert_ids.data_ptr(), cap // block_m, post_pad.data_ptr(),
                                            stream_ptr(a.device)))
     moe_block_gemm(a, b.transpose(1, 2), output, scales_a, bs, None, sorted_ids, expert_ids, post_pad, False, 1, block_m, rows)
+
+
+def moe_slot_blocks(topk_ids: torch.Tensor, expert_offsets: torch.Tensor, problem_sizes: torch.Tensor,
+                    output_permutation: torch.Tensor, block_m: int):
+    """Block table of the grouped GEMM for the expert-major layout, holding token SLOTS (include/fp8k.h:
+    fp8k_moe_slot_blocks_from_offsets): from what prepare_moe_input wrote (expert_offsets, problem_sizes,
+    output_permutation = slot -> row) returns (sorted_token_ids, expert_ids, num_tokens_post_padded) in the form
+    moe_align_block_size produces, so moe_block_gemm gathers token slot // topk from the un-shuffled activations."""
+    require_cuda(topk_ids, expert_offsets, problem_sizes, output_permutation)
+    E = problem_sizes.shape[0]
+    slots = topk_ids.numel()
+    for t, name, need in ((topk_ids, "topk_ids", slots), (expert_offsets, "expert_offsets", E),
+                          (problem_sizes, "problem_sizes", 3 * E), (output_permutation, "output_permutation", slots)):
+        if t.dtype != torch.int32 or not t.is_contiguous() or t.numel() < need:
+            raise RuntimeError("moe_slot_blocks: %s must be contiguous int32 with at least %d entries" % (name, need))
+    cap = max((slots + min(slots, E) * (block_m - 1)) // block_m * block_m, block_m)
+    table = torch.empty((cap + cap // block_m + 1,), device=topk_ids.device, dtype=torch.int32)
+    sorted_ids, expert_ids, post_pad = table[:cap], table[cap:cap + cap // block_m], table[cap + cap // block_m:]
+    check(lib.fp8k_moe_slot_blocks_from_offsets(expert_offsets.data_ptr(), problem_sizes.data_ptr(), E, topk_ids.data_ptr(),
+                                                output_permutation.data_ptr(), slots, block_m, sorted_ids.data_ptr(), cap,
+                                                expert_ids.data_ptr(), cap // block_m, post_pad.data_ptr(),
+                                                stream_ptr(topk_ids.device)))
+    return sorted_ids, expert_ids, post_pad
 
 
 def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,

@@ -1,19 +1,22 @@
-"""C-ABI checks that need no GPU: the library loads, exports every symbol include/fp8k.h declares,
+"""C-ABI checks that need no GPU: the library loads, exports every symbol the headers under include/ declare,
 and rejects bad arguments with a status and a message before touching the device."""
 import ctypes
+import glob
 import os
 import re
 
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-HEADER = os.path.join(ROOT, "include", "fp8k.h")
+HEADERS = sorted(glob.glob(os.path.join(ROOT, "include", "*.h")))
 
 
 def _declared_symbols():
-    text = open(HEADER).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(fp8k_[a-z0-9_]+)\s*\(", text)))
+    syms = set()
+    for header in HEADERS:
+        text = re.sub(r"/\*.*?\*/", "", open(header).read(), flags=re.S)
+        syms.update(re.findall(r"\b(fp8k_[a-z0-9_]+)\s*\(", text))
+    return sorted(syms)
 
 
 def test_library_exports_every_declared_symbol():

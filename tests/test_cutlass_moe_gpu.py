@@ -101,6 +101,51 @@ def test_apply_shuffle_mul_sum(dev, dtype, name, m, topk, k, with_factors):
     assert np.array_equal(out.float().cpu().numpy(), ref)
 
 
+def test_apply_shuffle_mul_sum_without_permutation_is_the_identity_map(dev):
+    from sglang_amd.sgl_kernel import apply_shuffle_mul_sum
+
+    g = torch.Generator().manual_seed(5)
+    m, topk, k = 77, 8, 512
+    c2 = torch.randn(m * topk, k, generator=g).to(torch.bfloat16)
+    w = torch.rand(m, topk, generator=g).to(torch.bfloat16)
+    out = torch.empty((m, k), device=dev, dtype=torch.bfloat16)
+    apply_shuffle_mul_sum(c2.to(dev), out, None, w.to(dev).reshape(-1))
+    ref = O.apply_shuffle_mul_sum(c2.float().numpy(), np.arange(m * topk, dtype=np.int32).reshape(m, topk), w.float().numpy(), "bf16")
+    assert np.array_equal(out.float().cpu().numpy(), ref)
+    with pytest.raises(RuntimeError, match="without a permutation"):
+        apply_shuffle_mul_sum(c2[:-1].to(dev), out, None, None)
+
+
+@pytest.mark.parametrize("m,topk,E,block", [(1, 8, 256, 16), (37, 4, 9, 32), (512, 8, 256, 64), (700, 8, 8, 256), (4096, 8, 256, 128)])
+def test_moe_slot_blocks(dev, m, topk, E, block):
+    """The slot table built from prepare_moe_input's outputs: integer invariants of the reference's aligner
+    (python/sglang/srt/layers/moe/fused_moe_triton/moe_align_block_size.py:17-82) - every expert's slots, as a set, in
+    blocks of its own, padded with the slot count - without the leading bucket for ids outside [0, E)."""
+    from sglang_amd.sgl_kernel import moe_slot_blocks
+
+    rng = np.random.default_rng(m * 7 + E)
+    ids = np.stack([rng.permutation(E)[:topk] if E >= topk else rng.integers(0, E, topk) for _ in range(m)]).astype(np.int32)
+    if m > 8:
+        ids[3, 0] = -1
+        ids[4, topk - 1] = E
+    off, _, ps1, _, _, c_map = _prepare(dev, ids, E, 256, 512)
+    sorted_ids, expert_ids, post_pad = moe_slot_blocks(torch.from_numpy(ids).to(dev), off, ps1, c_map, block)
+    torch.cuda.synchronize()
+    sorted_ids, expert_ids, used = sorted_ids.cpu().numpy(), expert_ids.cpu().numpy(), int(post_pad.cpu()[0])
+    flat = ids.reshape(-1)
+    counts = np.bincount(flat[(flat >= 0) & (flat < E)], minlength=E)
+    assert used == int(((counts + block - 1) // block * block).sum())
+    pos = 0
+    for e in range(E):
+        nblk = (counts[e] + block - 1) // block
+        assert (expert_ids[pos // block:pos // block + nblk] == e).all()
+        seg = sorted_ids[pos:pos + nblk * block]
+        assert np.array_equal(np.sort(seg[:counts[e]]), np.nonzero(flat == e)[0])
+        assert (seg[counts[e]:] == flat.size).all()
+        pos += nblk * block
+    assert pos == used
+
+
 def test_apply_shuffle_mul_sum_errors(dev):
     from sglang_amd.sgl_kernel import apply_shuffle_mul_sum
 
@@ -158,7 +203,7 @@ def test_grouped_mm_leaves_unowned_rows_untouched_and_takes_untransposed_scales(
     from sglang_amd.sgl_kernel import fp8_blockwise_scaled_grouped_mm
 
     rng = np.random.default_rng(12)
-    E, N, K = 4, 256, 256
+    E, N, K = 4, 256, 384  # N/128 != K/128: the shape alone says the scales are the un-transposed checkpoint tensor
     sizes = np.array([10, 0, 20, 5])
     rows, aq, bq, a_s, b_s, off, ps = _grouped_case(rng, E, sizes, N, K)
     ps[2, 0] = 12  # expert 2 uses only 12 of its 20 rows
@@ -179,6 +224,29 @@ def test_grouped_mm_leaves_unowned_rows_untouched_and_takes_untransposed_scales(
                                         fp8_tensor(bq, dev).transpose(1, 2).contiguous(), torch.from_numpy(a_s).to(dev),
                                         torch.from_numpy(b_s).to(dev), dummy, dummy, dummy, dummy, dummy,
                                         torch.from_numpy(ps).to(dev), torch.from_numpy(off[:-1].copy()).to(dev), dummy)
+
+
+def test_grouped_mm_reads_square_scales_in_the_ops_own_layout(dev):
+    """N/128 == K/128: scales_b is [E, K/128, N/128] whatever its strides - the transposed view the reference passes and a
+    contiguous tensor of the same logical content give the same result (a contiguous square tensor is never taken for
+    the un-transposed checkpoint layout)."""
+    from sglang_amd.sgl_kernel import fp8_blockwise_scaled_grouped_mm
+
+    rng = np.random.default_rng(13)
+    E, N, K = 3, 256, 256
+    sizes = np.array([7, 40, 3])
+    rows, aq, bq, a_s, b_s, off, ps = _grouped_case(rng, E, sizes, N, K)
+    b_s = (b_s * rng.uniform(0.5, 2.0, b_s.shape)).astype(np.float32)  # make the block scales visibly non-symmetric
+    dummy = torch.empty((E,), device=dev, dtype=torch.int64)
+    ref = O.fp8_blockwise_scaled_grouped_mm(aq, bq, a_s, b_s, off, ps, "f32", acc=np.float64)
+    view = torch.from_numpy(b_s).to(dev).transpose(1, 2)                      # [E, K/128, N/128], stride(1) == 1
+    dense = torch.from_numpy(np.ascontiguousarray(b_s.transpose(0, 2, 1))).to(dev)  # same values, contiguous
+    for scales in (view, dense):
+        out = torch.empty((rows, N), device=dev, dtype=torch.bfloat16)
+        fp8_blockwise_scaled_grouped_mm(out, dummy, dummy, dummy, dummy, dummy, fp8_tensor(aq, dev), fp8_tensor(bq, dev).transpose(1, 2),
+                                        torch.from_numpy(a_s).to(dev), scales, dummy, dummy, dummy, dummy, dummy,
+                                        torch.from_numpy(ps).to(dev), torch.from_numpy(off[:-1].copy()).to(dev), dummy)
+        assert _rel(out.float().cpu().numpy(), ref) <= REL_TOL
 
 
 def _experts(rng, E, H, I, std=0.05):

@@ -93,6 +93,31 @@ def test_ue8m0_unpack_and_marking():
         mark_ue8m0(torch.tensor([[1.0, 3.0]]))
     with pytest.raises(RuntimeError, match="powers of two"):
         mark_ue8m0(torch.tensor([[1.0, 0.0]]))
+    # the mark belongs to the memory: other tensor objects over it see it, other memory does not, and it ends with
+    # the marked object
+    assert is_ue8m0(t.data) and is_ue8m0(torch.nn.Parameter(t, requires_grad=False)) and is_ue8m0(t.view(3, 10))
+    assert not is_ue8m0(t.clone()) and not is_ue8m0(t[1:]) and not is_ue8m0(t.t())
+    other = t.data
+    del t
+    assert not is_ue8m0(other)
+
+
+def test_requant_weight_ue8m0_inplace_marks_the_parameter():
+    """After the in-place requantisation of a float-scale checkpoint the scale parameter - the object a layer passes to
+    the GEMM - and its .data are known to hold powers of two, so the hardware-scaled route can be taken."""
+    from sglang_amd.fp8_utils import requant_weight_ue8m0_inplace
+    from sglang_amd.sgl_kernel import is_ue8m0
+
+    rng = np.random.default_rng(9)
+    wq, ws = O.block_quant_weight(O.make_weight(256, 384, 1))
+    ws = (ws * rng.uniform(0.6, 1.7, ws.shape)).astype(np.float32)
+    weight = torch.nn.Parameter(torch.from_numpy(wq).view(torch.float8_e4m3fn), requires_grad=False)
+    scale = torch.nn.Parameter(torch.from_numpy(ws), requires_grad=False)
+    assert not is_ue8m0(scale)
+    requant_weight_ue8m0_inplace(weight, scale, [128, 128])
+    assert is_ue8m0(scale) and is_ue8m0(scale.data)
+    bits = scale.data.view(torch.int32)
+    assert bool(((bits & 0x7FFFFF) == 0).all())
 
 
 def test_cast_to_e8m0_with_rounding_up_host():

@@ -463,7 +463,7 @@ def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
     tokens (all of them up to 3 tokens) with only the experts those tokens hit copied back; the whole output must
     be finite, and permuting the tokens must permute the result (exactly where the kernel choice per expert is
     unchanged, which holds for a permutation: every expert keeps its slot count)."""
-    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl, get_default_config
+    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl, get_default_config
 
     d = deepseek_experts
     E, H, topk = d["E"], d["H"], 8
@@ -472,7 +472,7 @@ def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
     x = O.make_activation(T, H, T)
     logits = torch.randn((T, E), generator=d["gen"], device=dev)
     xt = bf16_tensor(x, dev)
-    tw, ids = biased_grouped_topk_impl(xt, logits, d["bias"], topk, True, 8, 4)
+    tw, ids = biased_grouped_topk(xt, logits, d["bias"], topk, True, 8, 4)
     kw = dict(use_fp8_w8a8=True, w1_scale=d["w1s"], w2_scale=d["w2s"], block_shape=[128, 128], routed_scaling_factor=2.5)
     out = fused_experts_impl(xt, d["w1"], d["w2"], tw, ids, **kw)
     torch.cuda.synchronize()
@@ -500,7 +500,7 @@ def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
 def test_fused_experts_deepseek_dims_other_block_sizes(dev, deepseek_experts, T, block):
     """The 64- and 128-slot grouped streaming kernels at the full expert dimensions (the default choice takes them
     between 1024 and 3072 tokens): a sample of tokens against the oracle."""
-    from sglang_amd.fused_moe import biased_grouped_topk_impl, fused_experts_impl, get_default_config
+    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl, get_default_config
 
     d = deepseek_experts
     E, H, topk = d["E"], d["H"], 8
@@ -508,7 +508,7 @@ def test_fused_experts_deepseek_dims_other_block_sizes(dev, deepseek_experts, T,
     x = O.make_activation(T, H, T)
     logits = torch.randn((T, E), generator=d["gen"], device=dev)
     xt = bf16_tensor(x, dev)
-    tw, ids = biased_grouped_topk_impl(xt, logits, d["bias"], topk, True, 8, 4)
+    tw, ids = biased_grouped_topk(xt, logits, d["bias"], topk, True, 8, 4)
     out = fused_experts_impl(xt, d["w1"], d["w2"], tw, ids, use_fp8_w8a8=True, w1_scale=d["w1s"], w2_scale=d["w2s"],
                              block_shape=[128, 128], routed_scaling_factor=2.5)
     torch.cuda.synchronize()
@@ -568,6 +568,30 @@ def test_moe_fused_gate_bf16_and_ties(dev, dtype, name):
     w0, i0 = moe_fused_gate(z, torch.zeros((256,), device=dev, dtype=dtype), 8, 4, 8)
     assert i0.cpu().tolist() == [list(range(8))] * 3
     assert torch.allclose(w0, torch.full_like(w0, 0.125))
+
+
+def test_biased_grouped_topk_is_the_gate_kernel_and_matches_the_tensor_op_restatement(dev):
+    """The layer-level routing entry point runs the fused gate kernel; on well-separated float32 logits its expert sets
+    and weights are those of the tensor-op restatement of topk.py:665-738 kept with the tests.  Shapes the kernel does
+    not take are refused (the product path has no second implementation)."""
+    from sglang_amd.fused_moe import biased_grouped_topk
+    from tests.routing_torch import biased_grouped_topk_impl
+
+    g = torch.Generator(device=dev)
+    g.manual_seed(3)
+    logits = torch.randn((513, 256), generator=g, device=dev)
+    bias = torch.randn((256,), generator=g, device=dev) * 0.01
+    x = torch.empty((513, 16), device=dev, dtype=torch.bfloat16)
+    w, ids = biased_grouped_topk(x, logits, bias, 8, True, 8, 4)
+    w_t, ids_t = biased_grouped_topk_impl(x, logits, bias, 8, True, 8, 4)
+    order, order_t = ids.argsort(dim=1), ids_t.argsort(dim=1)
+    same = (ids.gather(1, order) == ids_t.gather(1, order_t)).all(dim=1)
+    assert float(same.float().mean()) >= 0.99  # a last-bit difference in the sigmoid can swap two near-equal choices
+    torch.testing.assert_close(w.gather(1, order)[same], w_t.gather(1, order_t)[same], rtol=1e-5, atol=1e-7)
+    with pytest.raises(RuntimeError, match="power-of-two expert count"):
+        biased_grouped_topk(x, logits[:, :96].contiguous(), bias[:96].contiguous(), 4, True, 4, 2)
+    with pytest.raises(RuntimeError, match="renormalised"):
+        biased_grouped_topk(x, logits, bias, 8, False, 8, 4)
 
 
 def test_moe_fused_gate_errors(dev):

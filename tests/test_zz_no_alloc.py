@@ -79,3 +79,39 @@ def test_noalloc_block_gemm_refuses_sizes_beyond_its_buffer(dev):
     assert rc == 4
     msg = lib.fp8k_last_error().decode()
     assert "needs" in msg and "built-in" in msg and "fp8k_block_gemm" in msg
+
+
+def test_noalloc_block_gemm_replayed_from_a_hip_graph(dev):
+    """Two calls recorded into one HIP graph after a warm-up call outside the capture (the address look-up is not a
+    stream operation), replayed three times with eager work and synchronisations in between: every replay must give the
+    workspace form's bits.  Both shapes use the built-in scratch (K-cut partials, scale copy)."""
+    from sglang_amd._lib import check, stream_ptr
+
+    lib, fn = _entry()
+    shapes = [(128, 7168, 16384), (1024, 4608, 7168)]
+    probs = [_problem(M, N, K, 7 + M, dev) for (M, N, K) in shapes]
+    refs = []
+    for (M, N, K), pr in zip(shapes, probs):
+        C, C_ref, need = _both(lib, fn, *pr[4:], M, N, K, dev)  # also the warm-up call on this device
+        assert need > 0 and torch.equal(C, C_ref)
+        refs.append(C_ref)
+    outs = [torch.empty_like(r) for r in refs]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        st = stream_ptr(dev)
+        for (M, N, K), pr, C in zip(shapes, probs, outs):
+            A, B, As, Bs = pr[4:]
+            check(fn(A.data_ptr(), B.data_ptr(), As.data_ptr(), Bs.data_ptr(), C.data_ptr(), M, N, K, K, K,
+                     As.stride(0), As.stride(1), Bs.stride(0), Bs.stride(1), N, 2, st))
+    for replay in range(3):
+        for C in outs:
+            C.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for C, r in zip(outs, refs):
+            assert torch.equal(C, r), replay
+        # eager work that uses the same built-in buffer between the replays
+        M, N, K = shapes[0]
+        C, C_ref, _ = _both(lib, fn, *probs[0][4:], M, N, K, dev)
+        assert torch.equal(C, C_ref)
