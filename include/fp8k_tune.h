@@ -19,7 +19,8 @@ extern "C" {
  * choice).  kind -1: automatic (the default).  kind 4: the 128x128 tile kernel with K
  * cut into `splits` runs (0 or 1: none).  kind 0: the choice by the number of rows alone, without the 128x128
  * kernel.  kind 1: 256x256 tiles; kind 2: the streaming kernel (up to 128 rows); kind 3: the direct kernel (up to 32
- * rows, `splits` > 0 pins its K cut too); where a pinned family cannot take the shape, the choice by rows stands.
+ * rows, `splits` > 0 pins its K cut too); kind 5: the direct kernel that cuts K across the waves of a workgroup (up to
+ * 32 rows); where a pinned family cannot take the shape, the choice by rows stands.
  * `splits` is ignored for kinds 0..2.
  * kind -2: automatic, but the last round of 256x256 tiles is kept whole instead of being computed in 128-row halves.
  * fp8k_*_workspace_bytes, called from the same thread, follows the pinned choice.

@@ -13,7 +13,7 @@ namespace fp8k {
 
 struct Plan {
   int kind;    // 0 = generic, 1 = tile256, 2 = weight-streaming through LDS (33..128 rows), 3 = direct (<= 32 rows),
-               // 4 = tile128
+               // 4 = tile128, 5 = direct with K cut across the waves of a workgroup (<= 32 rows, N below 16 K)
   int splits;  // >1: split-K through the float workspace
   int kb_per_split;
   int tm;      // rows per block of the streaming kernels
@@ -66,6 +66,43 @@ static Plan plan_direct(int64_t M, int64_t N, int64_t K) {
   return pl;
 }
 
+// decode-sized with fewer than 128 tiles of 128 weight rows: a workgroup owns 16 (or 32) weight rows and its waves cut
+// K between them, so that every CU streams without float partials in memory or a reduction launch.  `splits` stays 1
+// (nothing goes through the workspace); kb_per_split is the K range of one wave, tm reuses the row-count slot, and
+// the number of waves along n travels in `halves`.
+constexpr int64_t kWaveKMaxN = 16384;
+static Plan plan_wavek(int64_t M, int64_t N, int64_t K) {
+  Plan pl{5, 1, 0, 0, 0, 0};
+  const int kb = (int)(K / kTileK);
+  pl.tm = M <= 16 ? 16 : 32;
+  // waves along n: the choice that leaves the busiest CU the fewest weight rows (workgroups go two to a CU at most);
+  // among equals the widest workgroup whose waves still get at most 16 K blocks each (measured: wider workgroups
+  // re-read less of the activations, longer per-wave K ranges start to serialise)
+  int nw = 1;
+  int64_t best_rows = -1;
+  for (int cand = 1; cand <= 4; cand *= 2) {
+    const int64_t wgs = (N + 16 * cand - 1) / (16 * cand);
+    if (wgs > 2 * (int64_t)num_cu() && cand < 4) continue;
+    const int64_t rows = (wgs + num_cu() - 1) / num_cu() * 16 * cand;
+    const int per_wave = (kb + 8 / cand - 1) / (8 / cand);
+    if (best_rows < 0 || rows < best_rows || (rows == best_rows && per_wave <= 16)) { best_rows = rows; nw = cand; }
+  }
+  if (g_force_kind == 5 && (g_force_splits == 1 || g_force_splits == 2 || g_force_splits == 4 || g_force_splits == 8))
+    nw = g_force_splits;  // tuning aid
+  pl.halves = nw;
+  pl.kb_per_split = (kb + 8 / nw - 1) / (8 / nw);
+  return pl;
+}
+// Which of the two decode kernels: every workgroup of the wave-cut kernel reads all of the activations' K range for its
+// 16 * nw weight rows, so its traffic through the CUs' load path grows with the rows of the batch; the workgroup-cut
+// kernel shares the activations among 128 weight rows but pays float partials and a reduction launch.  Measured
+// (M = 1 .. 32 on the DeepSeek-V3 and Llama projection shapes): the wave cut wins for up to 8 rows, and for up to 32
+// rows while the weights are at most about 24 MB.
+static bool prefers_wavek(int64_t M, int64_t N, int64_t K) {
+  if (N >= kWaveKMaxN) return false;  // 128 and more tiles of 128 rows: the workgroup-cut kernel runs uncut
+  return M <= 8 || N * K <= (24LL << 20);
+}
+
 // up to 128 rows: stream the weights once, every CU takes a K slice of one 256-row weight tile
 static Plan plan_stream(int64_t M, int64_t N, int64_t K) {
   Plan pl{2, 1, 0, 0, 0, 0};
@@ -111,8 +148,10 @@ static Plan plan_tile256(int64_t M, int64_t N, int64_t K) {
 static Plan plan_base(int64_t M, int64_t N, int64_t K) {
   const bool fits32 = M * K < (1LL << 31);
   if (g_force_kind == 3 && M <= 32 && fits32) return plan_direct(M, N, K);
+  if (g_force_kind == 5 && M <= 32 && fits32) return plan_wavek(M, N, K);
   if (g_force_kind == 2 && M <= 128 && fits32) return plan_stream(M, N, K);
   if (g_force_kind == 1) return plan_tile256(M, N, K);
+  if (M <= 32 && fits32 && prefers_wavek(M, N, K)) return plan_wavek(M, N, K);
   if (M <= 32 && fits32) return plan_direct(M, N, K);
   if (M <= 128 && fits32) return plan_stream(M, N, K);
   return plan_tile256(M, N, K);
@@ -279,6 +318,13 @@ static int launch(const GemmArgs& a0, const Plan& pl, hipStream_t st) {
     hipLaunchKernelGGL((splitk_reduce_kernel<MODE, OUT_DT, BIAS_DT>), dim3((unsigned)((quads + 255) / 256)), dim3(256),
                        0, st, a);
     return check_launch("splitk_reduce");
+  }
+  if (pl.kind == 5) {
+    a.wk_nw = pl.halves;
+    const unsigned nwg = (unsigned)((a.N + 16 * a.wk_nw - 1) / (16 * a.wk_nw));
+    if (pl.tm == 16) hipLaunchKernelGGL((gemm_wavek_kernel<16, MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
+    else hipLaunchKernelGGL((gemm_wavek_kernel<32, MODE, OUT_DT, BIAS_DT>), dim3(nwg), dim3(512), 0, st, a);
+    return check_launch("gemm_wavek");
   }
   if (pl.kind == 2) {
     a.m_blocks = 1;

@@ -267,4 +267,148 @@ __global__ __launch_bounds__(512, 2) void gemm_direct_kernel(const GemmArgs p) {
   }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same weight stream for matrices with too few 128-row tiles to fill the chip (N below about 16 K rows): the K
+// range is cut across the WAVES of a workgroup instead of across workgroups, so the partial sums meet in LDS and
+// neither float partials in memory nor a reduction launch are needed.  A workgroup owns 16 * NW weight rows; its 8
+// waves are NW (along n) x KS (along k), NW * KS = 8; wave (nw, ks) streams rows nw*16.. of K blocks
+// [ks * kbw, (ks+1) * kbw).  No wave shares an activation K range with another (NW = 1) or only with NW - 1 others,
+// so the activations skip LDS: a lane fetches its 32 bytes of a row and K block in matrix-core operand form straight
+// from memory (they are L2 hits: every workgroup reads the same few rows).  The K loop has no barrier; each wave keeps
+// D K blocks of weights, activations and scales in flight.  At the end the 8 accumulator sets are summed through LDS
+// in ascending ks (a fixed order: results do not depend on timing) and the ks = 0 waves write the output.
+// ------------------------------------------------------------------------------------------------
+template <int TM, int MODE, int OUT_DT, int BIAS_DT>
+__global__ __launch_bounds__(512, 2) void gemm_wavek_kernel(const GemmArgs p) {
+  static_assert(TM == 16 || TM == 32, "gemm_wavek_kernel: 16 or 32 rows");
+  constexpr int MS = TM / 16;
+  constexpr int D = 4;  // K blocks in flight per wave
+  __shared__ __attribute__((aligned(16))) uint8_t wl[8][16 * kTileK];  // per wave: one K block of its 16 weight rows
+  __shared__ __attribute__((aligned(16))) float red[8][MS][64][4];
+
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int r = lane & 15, kq = lane >> 4;
+  const int NW = p.wk_nw, nw = w % NW, ks = w / NW;
+  const int n0w = (blockIdx.x * NW + nw) * 16;
+  const int kb_all = p.K / kTileK;
+  const int kb0 = ks * p.kb_per_split;
+  const int nkb = n0w < p.N ? max(min(kb_all, kb0 + p.kb_per_split) - kb0, 0) : 0;
+  const uint32_t kbytes = (uint32_t)nkb * kTileK;
+
+  // ---- weights: line-shaped loads, re-laid out through the wave's LDS slot (as in gemm_direct_kernel)
+  const int rowsW = min(16, p.N - n0w);
+  const rsrc_t rW = make_rsrc(p.W + (int64_t)n0w * p.ldw + (int64_t)kb0 * kTileK,
+                              (rowsW > 0 && nkb > 0) ? (uint32_t)((rowsW - 1) * p.ldw) + kbytes : 0u);
+  const int wrow = lane >> 3, wc = lane & 7;
+  const uint32_t voW0 = (uint32_t)(wrow * p.ldw + wc * 16), voW1 = (uint32_t)((wrow + 8) * p.ldw + wc * 16);
+  uint8_t* const wslot = wl[w];
+  const uint32_t wst0 = (uint32_t)(wrow * kTileK + ((wc ^ ((wrow >> 1) & 7)) << 4));
+  const uint32_t wst1 = (uint32_t)((wrow + 8) * kTileK + ((wc ^ (((wrow + 8) >> 1) & 7)) << 4));
+  const uint32_t wrd0 = (uint32_t)(r * kTileK + ((kq ^ ((r >> 1) & 7)) << 4));
+  const uint32_t wrd1 = (uint32_t)(r * kTileK + (((4 + kq) ^ ((r >> 1) & 7)) << 4));
+  // ---- activations: lane (r, kq) takes chunks kq and 4 + kq of row ms*16 + r, the K order the weight operand has
+  const rsrc_t rX = make_rsrc(p.X + (int64_t)kb0 * kTileK, nkb > 0 ? (uint32_t)((p.M - 1) * p.ldx) + kbytes : 0u);
+  uint32_t voX[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int m = ms * 16 + r;
+    voX[ms] = m < p.M ? (uint32_t)(m * p.ldx) + kq * 16 : kOutOfRange;
+  }
+  // ---- block scales: one activation scale per lane row and K block, one weight scale per K block
+  const float* sxp[MS];
+  const float* swp = p.sw;
+  if (MODE == kModeBlock) {
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) sxp[ms] = p.sx + (int64_t)min(ms * 16 + r, p.M - 1) * p.sx_m + (int64_t)kb0 * p.sx_k;
+    swp = p.sw + (int64_t)(min(n0w, p.N - 1) >> 7) * p.sw_n + (int64_t)kb0 * p.sw_k;
+  }
+
+  v4i wreg[D][2], xreg[D][MS][2];
+  float sxr[D][MS], swr[D];
+  auto issue = [&](int slot, int kb) {
+    const bool ok = kb < nkb;
+    const uint32_t ko = (uint32_t)kb * kTileK;
+    wreg[slot][0] = buf_load16_stream(rW, ok ? voW0 + ko : kOutOfRange);
+    wreg[slot][1] = buf_load16_stream(rW, ok ? voW1 + ko : kOutOfRange);
+#pragma unroll
+    for (int ms = 0; ms < MS; ++ms) {
+      const bool okx = ok && voX[ms] != kOutOfRange;
+      xreg[slot][ms][0] = buf_load16(rX, okx ? voX[ms] + ko : kOutOfRange);
+      xreg[slot][ms][1] = buf_load16(rX, okx ? voX[ms] + ko + 64 : kOutOfRange);
+    }
+    if (MODE == kModeBlock) {
+      const int kc = min(kb, max(nkb - 1, 0));  // past the range the products are zero: any finite scale will do
+#pragma unroll
+      for (int ms = 0; ms < MS; ++ms) sxr[slot][ms] = sxp[ms][(int64_t)kc * p.sx_k];
+      swr[slot] = swp[(int64_t)kc * p.sw_k];
+    }
+  };
+
+  v4f acc[MS];
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) acc[ms] = v4f{0.f, 0.f, 0.f, 0.f};
+
+  if (nkb > 0) {
+#pragma unroll
+    for (int d = 0; d < D; ++d) issue(d, d);
+    for (int k0 = 0; k0 < nkb; k0 += D) {
+#pragma unroll
+      for (int d = 0; d < D; ++d) {
+        *reinterpret_cast<v4i*>(wslot + wst0) = wreg[d][0];
+        *reinterpret_cast<v4i*>(wslot + wst1) = wreg[d][1];
+        const v8i wa = join(*reinterpret_cast<const v4i*>(wslot + wrd0), *reinterpret_cast<const v4i*>(wslot + wrd1));
+        v8i xa[MS];
+        float sc[MS];
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) {
+          xa[ms] = join(xreg[d][ms][0], xreg[d][ms][1]);
+          if (MODE == kModeBlock) sc[ms] = sxr[d][ms] * swr[d];
+        }
+        issue(d, k0 + d + D);
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) {
+          if (MODE == kModeBlock) {
+            const v4f t = mfma_16x16x128(wa, xa[ms], v4f{0.f, 0.f, 0.f, 0.f});
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc[ms][i] = __builtin_fmaf(t[i], sc[ms], acc[ms][i]);
+          } else {
+            acc[ms] = mfma_16x16x128(wa, xa[ms], acc[ms]);
+          }
+        }
+      }
+    }
+  }
+  // ---- the K ranges meet: every wave leaves its sums in LDS, the ks = 0 waves add them up in ascending ks
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) *reinterpret_cast<v4f*>(red[w][ms][lane]) = acc[ms];
+  __syncthreads();
+  if (ks != 0) return;
+  const int KS = 8 / NW;
+  const int n = n0w + kq * 4;
+  if (n >= p.N) return;
+#pragma unroll
+  for (int ms = 0; ms < MS; ++ms) {
+    const int m = ms * 16 + r;
+    if (m >= p.M) continue;
+    v4f s = acc[ms];
+    for (int k = 1; k < KS; ++k) {
+      const v4f o = *reinterpret_cast<const v4f*>(red[k * NW + nw][ms][lane]);
+      s[0] += o[0]; s[1] += o[1]; s[2] += o[2]; s[3] += o[3];
+    }
+    float v[4] = {s[0], s[1], s[2], s[3]};
+    if (MODE == kModeRow) {
+      const float sa = p.sx[m];
+      const float4 sb = *reinterpret_cast<const float4*>(p.sw + n);
+      v[0] = v[0] * sb.x * sa; v[1] = v[1] * sb.y * sa; v[2] = v[2] * sb.z * sa; v[3] = v[3] * sb.w * sa;
+      if (p.bias) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += load_scalar<BIAS_DT>(p.bias, n + i);
+      }
+    }
+    store4<OUT_DT>(p.C, (int64_t)m * p.ldc + n, v[0], v[1], v[2], v[3]);
+  }
+}
+
+
 }  // namespace fp8k

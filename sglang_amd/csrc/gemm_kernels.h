@@ -31,6 +31,7 @@ struct GemmArgs {
   int tail_halves;    // tile256 only: those tiles are computed as two 128-row halves, one workgroup each (no K cut)
   int walkers;        // tile256 only: workgroups [0, walkers) walk the whole tiles (a multiple of 8)
   int tail_shared;    // tile256 only: unit u of the tail belongs to workgroup u (after its walk), else to workgroup walkers + u
+  int wk_nw;          // gemm_wavek_kernel only: waves of a workgroup along n (1, 2, 4 or 8; the other 8 / wk_nw cut K)
   // grouped (MoE) form of the streaming kernel; all null / zero for a dense GEMM
   const int32_t* sorted_ids;    // [m_blocks * TM] token slots, padded with values >= num_valid
   const int32_t* expert_ids;    // [m_blocks] expert of each block of TM slots, -1 = not on this rank

@@ -32,19 +32,28 @@ def w8a8_block_fp8_linear(
     input_scale: Optional[torch.Tensor] = None,
     bias: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
-    """Reference: cutlass_/triton_w8a8_block_fp8_linear, fp8_utils.py:196-226,306-326.
+    """Reference: cutlass_/triton_w8a8_block_fp8_linear, fp8_utils.py:196-226,306-326, and the pre-quantised input of the
+    ROCm variant (:268-304; Fp8LinearMethod.apply hands over `(x_q, x_scale)` as input / input_scale, fp8.py:500-508).
 
     input [..., K] bf16/fp16; weight e4m3fn [N,K]; weight_scale float32 [ceil(N/128), ceil(K/128)].
     Flatten -> per-token-group quant (column-major scales) -> block GEMM -> + bias -> reshape.
+    With input_scale the input is e4m3fn already (quantised upstream in groups of block_size[1], scales float32
+    [tokens, K/128] in any strides); the result is bf16, as in the reference.
     """
-    assert input_scale is None
     input_2d = input.view(-1, input.shape[-1])
     output_shape = [*input.shape[:-1], weight.shape[0]]
-    q_input, x_scale = sglang_per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True)
-    output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=input_2d.dtype)
+    if input_scale is not None:
+        if input_2d.dtype != fp8_dtype:
+            raise RuntimeError("w8a8_block_fp8_linear: input_scale given, so input must be float8_e4m3fn already")
+        q_input, x_scale = input_2d, input_scale.view(-1, input_scale.shape[-1])
+        out_dtype = torch.bfloat16
+    else:
+        q_input, x_scale = sglang_per_token_group_quant_fp8(input_2d, block_size[1], column_major_scales=True)
+        out_dtype = input_2d.dtype
+    output = w8a8_block_fp8_matmul(q_input, weight, x_scale, weight_scale, block_size, output_dtype=out_dtype)
     if bias is not None:
         output = output + bias
-    return output.to(dtype=input_2d.dtype).view(*output_shape)
+    return output.to(dtype=out_dtype).view(*output_shape)
 
 
 def dispatch_w8a8_block_fp8_linear() -> Callable:

@@ -210,6 +210,40 @@ def test_block_gemm_random_shapes_every_plan(dev):
         assert np.array_equal(c, ref), "case %d: M=%d N=%d K=%d" % (case, M, N, K)
 
 
+@pytest.mark.parametrize("nw", [0, 1, 2, 4, 8])
+def test_decode_gemm_with_k_cut_across_waves_is_exact_on_integers(dev, nw):
+    """The decode kernel that cuts K across the waves of a workgroup (partial sums meet in LDS), pinned with every
+    wave layout (0 = the plan's own): K block counts that do not divide by the number of K ranges (waves with short or
+    empty ranges), N not a multiple of the 16 rows of a wave, 1 .. 32 rows, both scale layouts, bf16 and fp16 output -
+    integer data with power-of-two scales, so the sums are exact whatever their order - and the same through
+    fp8_scaled_mm with a bias."""
+    from sglang_amd._lib import lib
+    from sglang_amd.sgl_kernel import fp8_scaled_mm
+
+    rng = np.random.default_rng(77 + nw)
+    lib.fp8k_tune_force_gemm_plan(5, nw)
+    try:
+        for case, (M, N, K) in enumerate([(1, 4096, 4096), (7, 1000, 128 * 5), (16, 264, 128 * 19), (17, 4608, 128 * 9),
+                                          (32, 7168, 2304), (3, 8, 128), (29, 520, 128 * 33)]):
+            xq = O.f32_to_e4m3fn(rng.integers(-4, 5, (M, K)).astype(np.float32))
+            wq = O.f32_to_e4m3fn(rng.integers(-4, 5, (N, K)).astype(np.float32))
+            xs = (2.0 ** rng.integers(-3, 3, (M, K // 128))).astype(np.float32)
+            ws = (2.0 ** rng.integers(-3, 3, ((N + 127) // 128, K // 128))).astype(np.float32)
+            dt, name = (torch.bfloat16, "bf16") if case & 1 else (torch.float16, "f16")
+            ref = O.w8a8_block_fp8_matmul(xq, wq, xs, ws, out_dtype=name, acc=np.float64)
+            c = _run_block(xq, xs, wq, ws, dev, col_major_as=bool(case & 2), out_dtype=dt)
+            assert np.array_equal(c, ref), "nw=%d M=%d N=%d K=%d" % (nw, M, N, K)
+            sa = (2.0 ** rng.integers(-3, 3, (M,))).astype(np.float32)
+            sb = (2.0 ** rng.integers(-3, 3, (N,))).astype(np.float32)
+            bias = torch.from_numpy(rng.integers(-8, 9, (N,)).astype(np.float32))
+            got = fp8_scaled_mm(fp8_tensor(xq, dev), fp8_tensor(wq, dev).t(), torch.from_numpy(sa).to(dev),
+                                torch.from_numpy(sb).to(dev), torch.bfloat16, bias.to(dev)).float().cpu().numpy()
+            want = O.fp8_scaled_mm(xq, wq, sa, sb, out_dtype="bf16", bias=bias.numpy())
+            assert np.array_equal(got, want), "row mode nw=%d M=%d N=%d K=%d" % (nw, M, N, K)
+    finally:
+        lib.fp8k_tune_force_gemm_plan(-1, 0)
+
+
 def _run_scaled_mm(aq, bq, sa, sb, dev, out_dtype=torch.bfloat16, bias=None):
     from sglang_amd.sgl_kernel import fp8_scaled_mm
 

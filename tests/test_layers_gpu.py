@@ -109,6 +109,29 @@ def test_block_fp8_linear_bias_and_nd_input(dev, shape, with_bias):
         assert torch.equal(out, plain + bf16_tensor(bias, dev))
 
 
+@pytest.mark.parametrize("shape", [(5, 1024), (2, 37, 1024)])
+def test_block_fp8_linear_takes_a_prequantised_input(dev, shape):
+    """Fp8LinearMethod.apply hands an upstream-quantised `(x_q, x_scale)` pair over as input / input_scale
+    (fp8.py:500-508): the same bits as quantising here (bf16 out), and <= 1e-2 against the oracle."""
+    from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
+    from sglang_amd.fp8_utils import dispatch_w8a8_block_fp8_linear
+
+    N, K = 384, shape[-1]
+    rows = int(np.prod(shape[:-1]))
+    x = O.make_activation(rows, K, seed=rows)
+    wq, ws = O.block_quant_weight(O.make_weight(N, K, 6))
+    fn = dispatch_w8a8_block_fp8_linear()
+    xt = bf16_tensor(x, dev)
+    W, Ws = fp8_tensor(wq, dev), torch.from_numpy(ws).to(dev)
+    x_q, x_s = sglang_per_token_group_quant_fp8(xt, 128)  # row-major scales: any strides are taken
+    out = fn(x_q.view(*shape), W, [128, 128], Ws, x_s.view(*shape[:-1], K // 128))
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == tuple(shape[:-1]) + (N,)
+    assert torch.equal(out.view(rows, N), fn(xt, W, [128, 128], Ws))
+    assert _rel_err(out.float().cpu().numpy().reshape(rows, N), O.block_fp8_linear(x, wq, ws)) <= REL_TOL
+    with pytest.raises(RuntimeError, match="float8_e4m3fn already"):
+        fn(xt, W, [128, 128], Ws, x_s)
+
+
 def test_graph_capture_split_k_gemm_survives_workspace_growth(dev):
     """A K-cut GEMM (M=16, N=7168, K=16384: float partials in the workspace) captured in a graph; afterwards a GEMM
     that needs a larger workspace runs eagerly on the stream the capture used, which makes the wrapper hand out a
