@@ -503,80 +503,108 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     }
 
     if constexpr (FUSE) {
-      // ---- activation and requantisation of the finished tile.  The waves wn = 2, 3 hold the up columns of the
-      // activation columns whose gate values the waves wn = 0, 1 (same wm) hold in the same lanes and registers:
-      // they hand their 16-bit values over through LDS (16 KB per pair, inside the stages of the item's last block),
-      // the gate waves form a = T(T(silu(T(gate))) * T(up)), exchange the row maxima of their two 64-column halves,
-      // quantise and store bytes (re-laid out through LDS for 16-byte stores) and the scale of every slot.
+      // ---- activation and requantisation of the finished tile, spread over all eight waves.  A gate wave (wn = 0, 1)
+      // and the up wave of the same lanes and registers (wn + 2, same wm) hold the two factors of the same 128 slots x
+      // 64 activation columns.  They swap halves through LDS as 16-bit values (which is what the reference's
+      // intermediate holds): the up wave hands over its slot groups 0, 2, the gate wave its groups 1, 3; then the gate
+      // wave forms a = T(T(silu(T(gate))) * T(up)) for groups 0, 2 and the up wave for groups 1, 3 (real slots come
+      // first in a block, so a half-empty block leaves every wave one group of real slots; groups that are all
+      // padding are skipped, only their zero scales are written).  The two waves
+      // that hold the two 64-column halves of the same slots (wn ^ 1) exchange their row maxima, every wave quantises
+      // its 64 slots x 64 columns with the quant kernels' arithmetic and stores bytes (re-laid out through LDS for
+      // 16-byte stores) and, the lower half's wave, the scale of every slot.  Each pair works inside 16 KB of the
+      // stages of the item's last block: [0, 8 KB) belongs to the gate wave, [8 KB, 16 KB) to the up wave.
       const int pr = wn & 1;
-      uint8_t* const xr = smem + (wm == 0 ? ews * WBYTES : XBASE + exs * XBYTES) + pr * 16384;
-      int qrow[8];  // store loop: lane -> row it * 16 + lane / 4 of the wave's 128 slots, 16-byte chunk lane % 4
+      const bool upw = wn >= 2;
+      uint8_t* const pair = smem + (wm == 0 ? ews * WBYTES : XBASE + exs * XBYTES) + pr * 16384;
+      uint8_t* const own_area = pair + (upw ? 8192 : 0);
+      const uint8_t* const partner_area = pair + (upw ? 0 : 8192);
+      const float* const mate_max = reinterpret_cast<const float*>(pair + (pr ? -16384 : 16384) + (upw ? 8192 : 0));
+      auto pack4 = [&](const float (&v)[4]) -> uint2 {
+        uint2 o;
+        if (OUT_DT == FP8K_BF16) { o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]); }
+        else { o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16); o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16); }
+        return o;
+      };
+      // MINE: first of the wave's own two slot groups (MINE, MINE + 2); it hands over the other two; UP: the wave holds
+      // up values
+      auto finish = [&](auto mine_c, auto up_c) {
+        constexpr int MINE = decltype(mine_c)::value, SEND = 1 - MINE;
+        constexpr bool UP = decltype(up_c)::value;
+        int qrow[4];  // store loop: lane -> row it * 16 + lane / 4 of the wave's 64 slots, 16-byte chunk lane % 4
 #pragma unroll
-      for (int it8 = 0; it8 < 8; ++it8) {
-        const int r = it8 * 16 + (lane_e >> 2);
-        qrow[it8] = wn < 2 ? p.sorted_ids[eslot0 + ((r >> 5) * 2 + wm) * 32 + (r & 31)] : nrows;
-      }
-      if (wn >= 2) {
+        for (int it4 = 0; it4 < 4; ++it4) {
+          const int r = it4 * 16 + (lane_e >> 2);
+          qrow[it4] = p.sorted_ids[eslot0 + ((MINE + 2 * (r >> 5)) * 2 + wm) * 32 + (r & 31)];
+        }
+        // a group holds real slots iff its first slot is real (wave-uniform)
+        bool real_mine[2], real_send[2];
 #pragma unroll
-        for (int ms = 0; ms < MS; ++ms)
+        for (int i = 0; i < 2; ++i) {
+          real_mine[i] = __builtin_amdgcn_readfirstlane(oslots[MINE + 2 * i]) < nrows;
+          real_send[i] = __builtin_amdgcn_readfirstlane(oslots[SEND + 2 * i]) < nrows;
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+          if (!real_send[i]) continue;
 #pragma unroll
           for (int ns = 0; ns < NS; ++ns)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
-              uint2 o;
-              const float v[4] = {acc[ns][ms][rg * 4], acc[ns][ms][rg * 4 + 1], acc[ns][ms][rg * 4 + 2], acc[ns][ms][rg * 4 + 3]};
-              if (OUT_DT == FP8K_BF16) { o.x = pack_bf16x2(v[0], v[1]); o.y = pack_bf16x2(v[2], v[3]); }
-              else { o.x = f32_to_f16_bits(v[0]) | (f32_to_f16_bits(v[1]) << 16); o.y = f32_to_f16_bits(v[2]) | (f32_to_f16_bits(v[3]) << 16); }
-              *reinterpret_cast<uint2*>(xr + ((ms * 2 + ns) * 4 + rg) * 512 + lane_e * 8) = o;
+              const float v[4] = {acc[ns][SEND + 2 * i][rg * 4], acc[ns][SEND + 2 * i][rg * 4 + 1],
+                                  acc[ns][SEND + 2 * i][rg * 4 + 2], acc[ns][SEND + 2 * i][rg * 4 + 3]};
+              *reinterpret_cast<uint2*>(own_area + ((i * 2 + ns) * 4 + rg) * 512 + lane_e * 8) = pack4(v);
             }
-      }
-      lds_barrier();
-      float amx[MS];
-      if (wn < 2) {
+        }
+        lds_barrier();
+        float amx[2] = {0.f, 0.f};
 #pragma unroll
-        for (int ms = 0; ms < MS; ++ms) {
+        for (int i = 0; i < 2; ++i) {
+          if (!real_mine[i]) continue;
           float m = 0.f;
 #pragma unroll
           for (int ns = 0; ns < NS; ++ns)
 #pragma unroll
             for (int rg = 0; rg < 4; ++rg) {
-              const uint2 u = *reinterpret_cast<const uint2*>(xr + ((ms * 2 + ns) * 4 + rg) * 512 + lane_e * 8);
-              float uf[4];
-              if (OUT_DT == FP8K_BF16) { uf[0] = bf16_lo(u.x); uf[1] = bf16_hi(u.x); uf[2] = bf16_lo(u.y); uf[3] = bf16_hi(u.y); }
-              else { uf[0] = f16_bits_to_f32(u.x & 0xffff); uf[1] = f16_bits_to_f32(u.x >> 16); uf[2] = f16_bits_to_f32(u.y & 0xffff); uf[3] = f16_bits_to_f32(u.y >> 16); }
+              const uint2 u = *reinterpret_cast<const uint2*>(partner_area + ((i * 2 + ns) * 4 + rg) * 512 + lane_e * 8);
+              float pv[4];
+              if (OUT_DT == FP8K_BF16) { pv[0] = bf16_lo(u.x); pv[1] = bf16_hi(u.x); pv[2] = bf16_lo(u.y); pv[3] = bf16_hi(u.y); }
+              else { pv[0] = f16_bits_to_f32(u.x & 0xffff); pv[1] = f16_bits_to_f32(u.x >> 16); pv[2] = f16_bits_to_f32(u.y & 0xffff); pv[3] = f16_bits_to_f32(u.y >> 16); }
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
-                const float g = round_to<OUT_DT>(acc[ns][ms][rg * 4 + r]);
-                const float a = round_to<OUT_DT>(round_to<OUT_DT>(silu_f32(g)) * uf[r]);
-                acc[ns][ms][rg * 4 + r] = a;
+                const float own = round_to<OUT_DT>(acc[ns][MINE + 2 * i][rg * 4 + r]);
+                const float g = UP ? pv[r] : own, up = UP ? own : pv[r];
+                const float a = round_to<OUT_DT>(round_to<OUT_DT>(silu_f32(g)) * up);
+                acc[ns][MINE + 2 * i][rg * 4 + r] = a;
                 m = fmaxf(m, fabsf(a));
               }
             }
           m = fmaxf(m, __shfl_xor(m, 32));  // the other 16 columns of every tile of the row
-          amx[ms] = m;
+          amx[i] = m;
         }
-        // own pair area is read: the maxima of the wave's 64 columns go to its start for the other gate wave
+        lds_barrier();  // every wave has read what it was sent: the areas are free for the maxima and the bytes
         if (h_e == 0) {
 #pragma unroll
-          for (int ms = 0; ms < MS; ++ms) reinterpret_cast<float*>(xr)[ms * 32 + lr_e] = amx[ms];
+          for (int i = 0; i < 2; ++i) reinterpret_cast<float*>(own_area)[i * 32 + lr_e] = amx[i];
         }
-      }
-      lds_barrier();
-      if (wn < 2) {
-        const float* other = reinterpret_cast<const float*>(xr + (pr ? -16384 : 16384));
-        uint8_t* const st = xr + 1024;  // 128 rows x 64 B of bytes, behind the maxima
+        lds_barrier();
+        uint8_t* const st = own_area + 1024;  // 64 rows x 64 B of bytes, behind the maxima
 #pragma unroll
-        for (int ms = 0; ms < MS; ++ms) {
-          const float amax = fmaxf(fmaxf(amx[ms], other[ms * 32 + lr_e]), p.q_eps);
+        for (int i = 0; i < 2; ++i) {
+          if (!real_mine[i]) {  // all padding: nothing to store but the zero scales GEMM 2 reads for these positions
+            if (pr == 0 && h_e == 0) p.qs_out[(int64_t)(en0 >> 7) * p.qs_ld + eslot0 + ((MINE + 2 * i) * 2 + wm) * 32 + lr_e] = 0.f;
+            continue;
+          }
+          const float amax = fmaxf(fmaxf(amx[i], mate_max[i * 32 + lr_e]), p.q_eps);
           const float sc = div448<true>(amax);
-          const int row = ms * 32 + lr_e;
+          const int row = i * 32 + lr_e;
 #pragma unroll
           for (int ns = 0; ns < NS; ++ns)
 #pragma unroll
             for (int rp = 0; rp < 2; ++rp) {
               float a8[8];
 #pragma unroll
-              for (int r = 0; r < 4; ++r) { a8[r] = acc[ns][ms][(rp * 2) * 4 + r]; a8[4 + r] = acc[ns][ms][(rp * 2 + 1) * 4 + r]; }
+              for (int r = 0; r < 4; ++r) { a8[r] = acc[ns][MINE + 2 * i][(rp * 2) * 4 + r]; a8[4 + r] = acc[ns][MINE + 2 * i][(rp * 2 + 1) * 4 + r]; }
               bool redo;
               uint2 o = quant8_bracket<true>(a8, sc, amax, redo);
               if (redo) o = quant8_divide(a8, sc);
@@ -584,19 +612,22 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
               *reinterpret_cast<uint32_t*>(st + row * 64 + ns * 32 + (rp * 2 + 1) * 8 + h_e * 4) = o.y;
             }
           if (pr == 0 && h_e == 0) {
-            const int pos = eslot0 + (ms * 2 + wm) * 32 + lr_e;
-            p.qs_out[(int64_t)(en0 >> 7) * p.qs_ld + pos] = oslots[ms] < nrows ? sc : 0.f;
+            const int pos = eslot0 + ((MINE + 2 * i) * 2 + wm) * 32 + lr_e;
+            p.qs_out[(int64_t)(en0 >> 7) * p.qs_ld + pos] = oslots[MINE + 2 * i] < nrows ? sc : 0.f;
           }
         }
         __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order
 #pragma unroll
-        for (int it8 = 0; it8 < 8; ++it8) {
-          const int r = it8 * 16 + (lane_e >> 2), c = lane_e & 3;
+        for (int it4 = 0; it4 < 4; ++it4) {
+          if (!real_mine[it4 >> 1]) continue;
+          const int r = it4 * 16 + (lane_e >> 2), c = lane_e & 3;
           const uint4 o = *reinterpret_cast<const uint4*>(st + r * 64 + c * 16);
-          const int sdst = qrow[it8];
+          const int sdst = qrow[it4];
           if (sdst < nrows) *reinterpret_cast<uint4*>(p.q_out + (int64_t)sdst * p.ldq + en0 + pr * 64 + c * 16) = o;
         }
-      }
+      };
+      if (upw) finish(std::integral_constant<int, 1>{}, std::integral_constant<bool, true>{});
+      else finish(std::integral_constant<int, 0>{}, std::integral_constant<bool, false>{});
       if (!has_next) {
         wait_vm0();
         return;

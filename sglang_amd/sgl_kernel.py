@@ -451,7 +451,8 @@ def is_ue8m0(scales: torch.Tensor) -> bool:
         return False
     if getattr(scales, "_fp8k_ue8m0", False):  # the marked object itself (also what a graph tracer can see)
         return True
-    if torch.compiler.is_compiling():  # no addresses while tracing: unmarked objects take the float-scale kernels
+    # no addresses while tracing or under fake tensors: unmarked objects take the float-scale kernels
+    if torch.compiler.is_compiling() or isinstance(scales, torch._subclasses.fake_tensor.FakeTensor):
         return False
     ref = _UE8M0_MARKED.get(_memory_key(scales))
     return ref is not None and ref() is not None

@@ -612,7 +612,9 @@ def test_moe_fused_gate_errors(dev):
 def test_gemm1_with_fused_activation_quant_is_the_three_step_sequence(dev, T, E, H, I, topk, dt):
     """256-slot blocks: the first grouped GEMM with silu_and_mul and the requantisation in its write-out against the same
     GEMM into a 16-bit tensor followed by the fused silu + group quant kernel - bytes and scales of every real slot bit
-    for bit, and the whole layer with and without the fusion bit for bit."""
+    for bit, and the whole layer (fused by default at this block size) bit for bit the sequence continued by hand.  The
+    layer with the fusion on is held against the oracle at the full DeepSeek-V3 dimensions by
+    test_fused_experts_deepseek_dims (4096 tokens take 256-slot blocks)."""
     import sglang_amd.fused_moe as fm
     from sglang_amd import custom_ops as ops
     from sglang_amd.fp8_kernel import sglang_per_token_group_quant_fp8
@@ -649,16 +651,18 @@ def test_gemm1_with_fused_activation_quant_is_the_three_step_sequence(dev, T, E,
     assert torch.equal(got_s[: sid.numel()][real], ref_s[sid[real]])
     assert bool((got_s[: sid.numel()][~real] == 0).all())
 
+    # the whole layer (which takes the fused GEMM 1 with 256-slot blocks) against the three-step sequence continued by hand
+    a2_ss = ops.moe_sort_scales(ref_s, sorted_ids, post_pad, 1, slots)
+    c3 = torch.empty((T, topk, H), device=dev, dtype=dt)
+    ops.moe_block_gemm(ref_q, w2, c3, a2_ss, s2, twt, sorted_ids, expert_ids, post_pad, True, 1, 256, slots, scales_sorted=True)
+    plain = torch.empty((T, H), device=dev, dtype=dt)
+    ops.moe_sum_reduce(c3, plain, 1.0)
     kw = dict(use_fp8_w8a8=True, w1_scale=s1, w2_scale=s2, block_shape=[128, 128])
     old = fm.get_default_config
     fm.get_default_config = lambda M_, E_, t_: {"BLOCK_SIZE_M": 256, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}
-    keep = fm.FUSE_ACT_QUANT_INTO_GEMM1
     try:
-        fm.FUSE_ACT_QUANT_INTO_GEMM1 = True
+        assert fm.gemm1_fuses_activation(fm.get_default_config(T, E, topk), 2 * I)
         fused = fm.fused_experts_impl(x, w1, w2, twt, idt, **kw)
-        fm.FUSE_ACT_QUANT_INTO_GEMM1 = False
-        plain = fm.fused_experts_impl(x, w1, w2, twt, idt, **kw)
     finally:
-        fm.FUSE_ACT_QUANT_INTO_GEMM1 = keep
         fm.get_default_config = old
     assert torch.equal(fused, plain)
