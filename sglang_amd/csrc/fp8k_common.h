@@ -45,14 +45,15 @@ constexpr float kFp8Max = 448.0f;
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
 
-// float -> bf16 bits, round to nearest even (NaN kept quiet)
+// float -> bf16 bits, round to nearest even (NaN stays a quiet NaN): gfx950 converts in hardware, two values per
+// v_cvt_pk_bf16_f32 (the add / shift / select sequence it replaces was most of a GEMM tile's write-out time)
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  uint32_t r = (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
-  return (f != f) ? 0x7fc0u : r;
+  return (uint32_t)__builtin_bit_cast(unsigned short, (__bf16)f);
 }
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return f32_to_bf16_bits(lo) | (f32_to_bf16_bits(hi) << 16);
+  const v2f v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 __device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
   _Float16 h = (_Float16)f;

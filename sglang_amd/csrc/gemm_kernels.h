@@ -221,7 +221,12 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
   Item item;
   if (!next_item(item)) return;
 
-  bool first_item = true;  // no item before this one has requested its first K block
+  // The LDS stages are two rings that run on across the items of a walk: K block b of an item sits in weight stage
+  // (gw0 + b) % 3 and activation stage (gx0 + b) & 1, and the loads that would fall behind an item's last block fetch
+  // the first blocks of the next item instead (its activation block 0 and its weight blocks 0 and 1 - the three requests
+  // a fresh tile would otherwise wait for with nothing else to do).  `pref`: the item before requested them.
+  int gw0 = 0, gx0 = 0;
+  bool pref = false;
   for (;;) {
     const int t = item.t, split = item.split, half = item.half;
     const bool is_split = item.is_split, is_half = item.is_half;
@@ -262,30 +267,24 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     // ---- global -> LDS through buffer loads: descriptor at the tile's first row, rows past the matrix edge are out
     // of range and read as zero
     rsrc_t rW = make_rsrc(p.W, 0), rX = make_rsrc(p.X, 0);
-    auto tile_rsrcs = [&](int tile, int hf, bool halved, int kb0) {
+    rsrc_t rWn = make_rsrc(p.W, 0), rXn = make_rsrc(p.X, 0);  // the item after this one (empty: every load is a no-op)
+    auto tile_rsrcs = [&](rsrc_t& dW, rsrc_t& dX, int tile, int hf, bool halved, int kb0, int kb1) {
       int tm, tn;
       tile_coords(tile, p.tiles_m, p.tiles_n, tm, tn);
       const int mm = tm * kTileM + hf * (kTileM / 2), nn = tn * kTileN;
       const int rowsW = min(kTileN, p.N - nn), rowsX = min(halved ? kTileM / 2 : kTileM, p.M - mm);
-      const int kbytes = p.K - kb0 * kTileK;
-      rW = make_rsrc(p.W + (int64_t)nn * p.ldw + (int64_t)kb0 * kTileK, (uint32_t)((rowsW - 1) * p.ldw + kbytes));
-      rX = make_rsrc(p.X + (int64_t)mm * p.ldx + (int64_t)kb0 * kTileK, (uint32_t)((rowsX - 1) * p.ldx + kbytes));
-    };
-    // one 1 KB global->LDS load (slice j of the wave's 32 rows) of K block kstep into weight stage ws / activation
-    // stage xst.  The whole offset travels in the bounds-checked per-lane operand (a uniform offset operand is exempt
-    // from the range check, and rows past the matrix edge must read as zero, not touch memory).
-    auto LW = [&](int j, int kstep, int ws) {
-      buf_load16_to_lds(rW, voW[j & 1] + (soW + j * stepW + (uint32_t)kstep * kTileK), 0, smem + ws * kWStage + w * 4096 + j * 1024);
-    };
-    auto LX = [&](int j, int kstep, int xst) {
-      buf_load16_to_lds(rX, voX[j & 1] + (soX + j * stepX + (uint32_t)kstep * kTileK), 0,
-                        smem + kXBase + xst * kXStage + w * 4096 + j * 1024);
+      const int kbytes = (kb1 - kb0) * kTileK;  // the item's own K range: a request past it moves nothing
+      dW = make_rsrc(p.W + (int64_t)nn * p.ldw + (int64_t)kb0 * kTileK, rowsX > 0 ? (uint32_t)((rowsW - 1) * p.ldw + kbytes) : 0u);
+      dX = make_rsrc(p.X + (int64_t)mm * p.ldx + (int64_t)kb0 * kTileK, rowsX > 0 ? (uint32_t)((rowsX - 1) * p.ldx + kbytes) : 0u);
     };
 
     int tile_m, tile_n;
     tile_coords(t, p.tiles_m, p.tiles_n, tile_m, tile_n);
     const int m0 = tile_m * kTileM + half * (kTileM / 2), n0 = tile_n * kTileN;
-    if (m0 >= p.M) return;                                              // upper half of a tile past the last row
+    if (m0 >= p.M) {                                                    // upper half of a tile past the last row
+      wait_vm0();  // requests of the item before may still point at the stages
+      return;
+    }
     const int nrows = is_half ? min(p.M, m0 + kTileM / 2) : p.M;        // exclusive bound of a valid output row
 
     const int kb_begin = is_split ? split * p.kb_per_split : 0;
@@ -293,7 +292,34 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     const int nkb = kb_end - kb_begin;
 
     auto slot_at = [&](int i) -> int { return m0 + i; };
-    tile_rsrcs(t, half, is_half, kb_begin);
+    tile_rsrcs(rW, rX, t, half, is_half, kb_begin, kb_end);
+    // the item after this one: with three and more K blocks here its first blocks are requested by this item's last trips
+    Item next;
+    const bool has_next = next_item(next);
+    const bool stream = has_next && nkb >= 3;
+    if (has_next) {
+      const int nb0 = next.is_split ? next.split * p.kb_per_split : 0;
+      const int nb1 = next.is_split ? min(p.K / kTileK, nb0 + p.kb_per_split) : p.K / kTileK;
+      tile_rsrcs(rWn, rXn, next.t, next.half, next.is_half, nb0, nb1);
+    }
+    const rsrc_t rWs = stream ? rWn : make_rsrc(p.W, 0), rXs = stream ? rXn : make_rsrc(p.X, 0);
+    // one 1 KB global->LDS load (slice j of the wave's 32 rows) of K block kstep into weight stage ws / activation
+    // stage xst; a block behind the item's last one is the next item's block kstep - nkb.  The whole offset travels in
+    // the bounds-checked per-lane operand (a uniform offset operand is exempt from the range check, and rows past the
+    // matrix edge must read as zero, not touch memory).
+    auto LW = [&](int j, int kstep, int ws) {
+      const bool nx = kstep >= nkb;
+      buf_load16_to_lds(nx ? rWs : rW, voW[j & 1] + (soW + j * stepW + (uint32_t)(nx ? kstep - nkb : kstep) * kTileK), 0,
+                        smem + ws * kWStage + w * 4096 + j * 1024);
+    };
+    auto LX = [&](int j, int kstep, int xst) {
+      const bool nx = kstep >= nkb;
+      buf_load16_to_lds(nx ? rXs : rX, voX[j & 1] + (soX + j * stepX + (uint32_t)(nx ? kstep - nkb : kstep) * kTileK), 0,
+                        smem + kXBase + xst * kXStage + w * 4096 + j * 1024);
+    };
+    // stages of K block b of this item
+    auto wst = [&](int b) -> int { return (gw0 + b) % 3; };
+    auto xst = [&](int b) -> int { return (gx0 + b) & 1; };
 
     // ---- scales (block mode)
     // activation rows whose scales this lane applies (any valid row for padding lanes)
@@ -358,31 +384,34 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       }
     };
 
-    if (nkb <= 0) return;
+    if (nkb <= 0) {
+      wait_vm0();
+      return;
+    }
     if (is_half && wm >= 2) {
       // half tile (always a workgroup's last item): the waves of the upper 128 rows issue their share of the loads
       // (their activation rows are out of range and arrive as zeros) and keep the barriers, with the same order and
       // counts of loads as the others
-      if (first_item) {
+      if (!pref) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+        for (int j = 0; j < 4; ++j) LX(j, 0, xst(0));
 #pragma unroll
-        for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+        for (int j = 0; j < 4; ++j) LW(j, 0, wst(0));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) LW(j, 1, wst(1));
       }
       wait_vm0();
       __syncthreads();
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LX(j, 1, 1);
+      for (int j = 0; j < 4; ++j) LX(j, 1, xst(1));
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LW(j, 1, 1);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) LW(j, 2, 2);
-      int w_ld = 0, w_rd = 1;
+      for (int j = 0; j < 4; ++j) LW(j, 2, wst(2));
+      int w_ld = wst(0), w_rd = wst(1);
       for (int it = 0; it < nkb - 1; ++it) {
         lds_barrier<4>();
         SB();
 #pragma unroll
-        for (int j = 0; j < 4; ++j) LX(j, it + 2, it & 1);
+        for (int j = 0; j < 4; ++j) LX(j, it + 2, xst(it));
 #pragma unroll
         for (int j = 0; j < 4; ++j) LW(j, it + 3, w_ld);
         w_ld = w_rd;
@@ -392,13 +421,15 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       lds_barrier();  // the others' barrier in front of the write-out
       return;
     }
-    // ---- prologue: block 0 into stage 0, block 1 into stage 1, steps 0..2 of block 0.  Block 0 of every item but a
-    // workgroup's first was requested before the previous item's write-out.
-    if (first_item) {
+    // ---- prologue: blocks 0 and 1 into their stages, steps 0..2 of block 0.  Activation block 0 and weight blocks 0
+    // and 1 of every item but a workgroup's first were requested by the item before.
+    if (!pref) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+      for (int j = 0; j < 4; ++j) LX(j, 0, xst(0));
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+      for (int j = 0; j < 4; ++j) LW(j, 0, wst(0));
+#pragma unroll
+      for (int j = 0; j < 4; ++j) LW(j, 1, wst(1));
     }
     if (MODE == kModeBlock) { sc[0] = p.sx[sxo0]; sc[1] = p.sx[sxo1]; const float sb = swp[0]; sc[0] *= sb; sc[1] *= sb; }
     auto exponents = [&](uint32_t w0, uint32_t w1, float sb, int kb_abs) {  // -> sq, sqw for K block kb_abs
@@ -419,44 +450,44 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     }
     SB();
 #pragma unroll
-    for (int j = 0; j < 4; ++j) LX(j, 1, 1);
+    for (int j = 0; j < 4; ++j) LX(j, 1, xst(1));
 #pragma unroll
-    for (int j = 0; j < 4; ++j) LW(j, 1, 1);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) LW(j, 2, 2);
-    RX(0, 0, smem + kXBase); RX(1, 0, smem + kXBase); RW(0, smem, 0);
-    RX(0, 1, smem + kXBase); RX(1, 1, smem + kXBase); RW(1, smem, 0);
+    for (int j = 0; j < 4; ++j) LW(j, 2, wst(2));
+    const uint8_t* const stW0 = smem + wst(0) * kWStage;
+    const uint8_t* const stX0 = smem + kXBase + xst(0) * kXStage;
+    RX(0, 0, stX0); RX(1, 0, stX0); RW(0, stW0, 0);
+    RX(0, 1, stX0); RX(1, 1, stX0); RW(1, stW0, 0);
     SB();
     // steps 0..2 of block 0
     M(0, 0, 0); SB();
     M(1, 0, 0); SB();
-    RW(0, smem, 1); SB();
+    RW(0, stW0, 1); SB();
     M(0, 1, 0); SB();
     M(1, 1, 0); SB();
-    RW(1, smem, 1); SB();
+    RW(1, stW0, 1); SB();
     F(acc[0][0], tq[0], sc[0]); SB();
     M(0, 0, 1); SB();
     F(acc[0][1], tq[1], sc[1]); SB();
     M(1, 0, 1); SB();
-    RW(0, smem, 2); SB();
+    RW(0, stW0, 2); SB();
     M(0, 1, 1); SB();
     M(1, 1, 1); SB();
-    RW(1, smem, 2); SB();
+    RW(1, stW0, 2); SB();
     F(acc[1][0], tq[0], sc[0]); SB();
     M(0, 0, 2); SB();
     F(acc[1][1], tq[1], sc[1]); SB();
     M(1, 0, 2); SB();
-    RW(0, smem, 3); SB();
+    RW(0, stW0, 3); SB();
     M(0, 1, 2); SB();
     M(1, 1, 2); SB();
-    RW(1, smem, 3); SB();
+    RW(1, stW0, 3); SB();
     // pending: F(acc[2][0], tq[0], sc[0]), F(acc[2][1], tq[1], sc[1])
 
-    int w_ld = 0, w_rd = 1;  // weight stages: the one block it left (refilled with block it+3), the one of block it+1
+    int w_ld = wst(0), w_rd = wst(1);  // weight stages: the one block it left (refilled with block it+3), the one of block it+1
     for (int it = 0; it < nkb - 1; ++it) {
       const uint8_t* stW = smem + w_rd * kWStage;                     // block it+1
-      const uint8_t* stX = smem + kXBase + ((it + 1) & 1) * kXStage;
-      const int xl = it & 1;                                          // activation stage block it left
+      const uint8_t* stX = smem + kXBase + xst(it + 1) * kXStage;
+      const int xl = xst(it);                                         // activation stage block it left
       lds_barrier<4>();  // block it+1 has landed; the weights of block it+2 may still be on their way
       SB();
       // ---- step 3 of block it; every operand register is refilled from block it+1 after its last use
@@ -525,21 +556,25 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
 
     // Finished tiles leave through LDS so that every store instruction writes whole 256-byte row segments
     // (the accumulator layout alone gives 8 bytes per row per lane: 32 partial lines per instruction).
-    // Each wave re-lays its own 64 x 128 block out, 32 rows at a time, in a private 8 KB slot of weight stages 1 and
-    // 2, 16-byte chunks XOR-swizzled by the row so that both the 8-byte writes and the 16-byte reads spread over all
-    // banks; weight stage 0 and activation stage 0 meanwhile receive the first K block of the next item.
+    // Each wave re-lays its own 64 x 128 block out, 32 rows at a time, in a private 8 KB slot of the weight or the
+    // activation stage of the item's last block, 16-byte chunks XOR-swizzled by the row so that both the 8-byte writes
+    // and the 16-byte reads spread over all banks; the other stages meanwhile receive the first blocks of the next item.
     const bool wide = !is_split && (p.ldc & 7) == 0 && (reinterpret_cast<uintptr_t>(p.C) & 15) == 0;
-    wait_vm0();     // the loads past the last K block still target the stages: drain them before the stages are reused
-    lds_barrier();  // every wave has taken its last operands out of the stages, and every stale load has landed
-    Item next;
-    const bool has_next = next_item(next);
-    if (has_next) {
-      tile_rsrcs(next.t, next.half, next.is_half, next.is_split ? next.split * p.kb_per_split : 0);
+    // every wave has taken its last operands out of the stages.  The requests still in flight (the next item's first
+    // blocks, or requests past the last block that move nothing) point at the stages AFTER the last block's, never at
+    // the two the write-out uses.
+    lds_barrier();
+    const int ews = wst(nkb - 1), exs = xst(nkb - 1);  // the stages of the item's last block: free from here on
+    if (has_next && !stream) {
+      // an item of one or two K blocks has no trips to spare for it: the next item's first blocks are requested here
       SB();
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LX(j, 0, 0);
+      for (int j = 0; j < 4; ++j) buf_load16_to_lds(rXn, voX[j & 1] + (soX + j * stepX), 0, smem + kXBase + xst(nkb) * kXStage + w * 4096 + j * 1024);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LW(j, 0, 0);
+      for (int j = 0; j < 4; ++j) buf_load16_to_lds(rWn, voW[j & 1] + (soW + j * stepW), 0, smem + wst(nkb) * kWStage + w * 4096 + j * 1024);
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        buf_load16_to_lds(rWn, voW[j & 1] + (soW + j * stepW + (uint32_t)kTileK), 0, smem + wst(nkb + 1) * kWStage + w * 4096 + j * 1024);
       SB();
     }
 
@@ -570,7 +605,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
     };
 
     if (wide) {
-      uint8_t* ep = smem + kWStage + w * 8192;  // 32 rows x 256 B per pass
+      uint8_t* ep = smem + (w < 4 ? ews * kWStage + w * 8192 : kXBase + exs * kXStage + (w - 4) * 8192);  // 32 rows x 256 B per pass
 #pragma unroll
       for (int ms = 0; ms < 2; ++ms) {
         const int mrow = slot_at(wm * 64 + ms * 32 + lr);
@@ -617,9 +652,14 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
         }
       }
     }
-    if (!has_next) return;
+    if (!has_next) {
+      wait_vm0();  // requests that moved nothing still point at the stages: let them retire before the LDS goes back
+      return;
+    }
     item = next;
-    first_item = false;
+    pref = true;
+    gw0 = wst(nkb);
+    gx0 = xst(nkb);
   }
 }
 
