@@ -37,6 +37,16 @@ void fp8k_tune_force_gemm_plan(int kind, int splits);
 int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream);
 
 /*
+ * Measurement aid (no counterpart in the reference): the same read stream in the shape a GEMM fetches a weight that was
+ * NOT re-ordered after loading: the byte matrix [rows, pitch] at `src` is read as tiles of 256 rows, one K block (256
+ * pieces of 128 bytes, `pitch` bytes apart) per 32 KB stage, each workgroup walking the K blocks of its
+ * rows / 256 / CUs tiles.  Timed against fp8k_tune_stream_read on the same buffer it shows what a pre-shuffled
+ * (tile-contiguous) copy of the weights could gain on this machine.  pitch a multiple of 128; rows are rounded down to
+ * whole tiles per CU.
+ */
+int fp8k_tune_stream_read_tiles(const void* src, int64_t rows, int64_t pitch, void* stream);
+
+/*
  * Measurement aid (no counterpart in the reference): fp8k_tune_stream_read with a write-out inside the stream.  After
  * every stages_per_tile stages of 32 KB ("a weight tile") each of the workgroup's 8 wavefronts stores stores_per_wave
  * times 1 KB (16 bytes a lane) to a place of its own in dst: 8 KB x stores_per_wave per tile and workgroup, the shape of

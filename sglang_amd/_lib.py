@@ -69,6 +69,7 @@ SIGNATURES = {
     "fp8k_scaled_mm_workspace_bytes": (_c_i64, [_c_i64, _c_i64, _c_i64]),
     "fp8k_tune_force_gemm_plan": (None, [_c_int, _c_int]),
     "fp8k_tune_stream_read": (_c_int, [_c_ptr, _c_i64, _c_ptr]),
+    "fp8k_tune_stream_read_tiles": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr]),
     "fp8k_tune_stream_read_write": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr]),
     "fp8k_tune_mfma_peak": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
     "fp8k_moe_align_block_size": (

@@ -32,6 +32,49 @@ __global__ __launch_bounds__(512, 1) void stream_read_kernel(const uint8_t* __re
 }
 }  // namespace fp8k
 
+namespace fp8k {
+// The same stream in the shape a GEMM fetches an un-shuffled weight: a stage is one K block of a 256-row tile - 256
+// pieces of 128 bytes, `pitch` bytes apart - and a workgroup walks the K blocks of its tiles.  Wave w loads rows
+// w * 32 .. w * 32 + 31 of the tile, 8 rows (1 KB) per instruction, as the tile kernels do.
+__global__ __launch_bounds__(512, 1) void stream_read_tiles_kernel(const uint8_t* __restrict__ src, int64_t pitch, int kblocks,
+                                                                   int tiles_per_wg) {
+  __shared__ __attribute__((aligned(1024))) uint8_t stage[2 * 32768];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int trips = tiles_per_wg * kblocks;
+  const uint32_t vo = (uint32_t)((lane >> 3) * pitch + (lane & 7) * 16);
+  auto issue = [&](int t) {
+    const int tile = blockIdx.x * tiles_per_wg + t / kblocks, kb = t % kblocks;
+    // one descriptor per tile and K block: a tile of 256 rows may span more than a descriptor's 4 GB
+    const rsrc_t r = make_rsrc(src + ((int64_t)tile * 256 + w * 32) * pitch + (int64_t)kb * 128, (uint32_t)(31 * pitch + 128));
+#pragma unroll
+    for (int q = 0; q < 4; ++q) buf_load16_to_lds(r, vo + (uint32_t)(q * 8 * pitch), 0, stage + (t & 1) * 32768 + (w * 4 + q) * 1024);
+  };
+  issue(0);
+  if (trips > 1) issue(1);
+  for (int t = 0; t < trips; ++t) {
+    if (t + 1 < trips) lds_barrier<4>();
+    else lds_barrier<0>();
+    if (t + 2 < trips) issue(t + 2);
+  }
+  wait_vm0();
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_stream_read_tiles(const void* src, int64_t rows, int64_t pitch, void* stream) {
+  clear_error();
+  const char* op = "tune_stream_read_tiles";
+  FP8K_REQUIRE(src && aligned(src, 16), "%s: src must be a 16-byte aligned device pointer", op);
+  FP8K_REQUIRE(rows >= 0 && pitch >= 128 && pitch % 128 == 0 && pitch < (1LL << 23), "%s: pitch must be a multiple of 128 below 8 MiB", op);
+  const int ncu = num_cu();
+  const int64_t tiles_per_wg = rows / 256 / ncu;
+  if (tiles_per_wg == 0) return FP8K_OK;
+  FP8K_REQUIRE(tiles_per_wg * (pitch / 128) < (1LL << 30), "%s: too many stages per workgroup", op);
+  hipLaunchKernelGGL(stream_read_tiles_kernel, dim3((unsigned)ncu), dim3(512), 0, (hipStream_t)stream, (const uint8_t*)src, pitch,
+                     (int)(pitch / 128), (int)tiles_per_wg);
+  return check_launch(op);
+}
+
 extern "C" int fp8k_tune_stream_read(const void* src, int64_t bytes, void* stream) {
   clear_error();
   FP8K_REQUIRE(bytes >= 0 && bytes < (1LL << 40), "tune_stream_read: bad size");

@@ -36,6 +36,14 @@ def _rel_err(c, ref):
     return float(np.abs(c.astype(np.float64) - ref.astype(np.float64)).max() / max(np.abs(ref).max(), 1e-30))
 
 
+def _elem_rel_err(c, ref):
+    """Largest element-wise relative error over the elements that are not tiny (|ref| above 1 % of the largest): the strict
+    reading of "maximum relative error"; for a bf16 output it is bounded below by the output rounding, 2^-8."""
+    c, ref = c.astype(np.float64), ref.astype(np.float64)
+    big = np.abs(ref) > 1e-2 * np.abs(ref).max()
+    return float((np.abs(c - ref)[big] / np.abs(ref)[big]).max()) if big.any() else 0.0
+
+
 def _sample(rng, M, N):
     rows = np.unique(np.concatenate([[0, M - 1, min(M - 1, 127), min(M - 1, 128), min(M - 1, 255), min(M - 1, 256)],
                                      rng.integers(0, M, 6)]))
@@ -84,6 +92,7 @@ def test_block_gemm_deepseek_v3_every_config_point(dev, N, K, M):
         ref += (a[:, sl] @ b[:, sl].T) * xs[rows, kb][:, None] * ws_cols[:, kb][None, :]
     got = C[torch.from_numpy(rows).to(dev)][:, torch.from_numpy(cols).to(dev)].float().cpu().numpy()
     assert _rel_err(got, ref) <= REL_TOL, _rel_err(got, ref)
+    assert _elem_rel_err(got, ref) <= REL_TOL, _elem_rel_err(got, ref)
 
     # row-major scales (the Triton-side layout) take the same kernels after a scale copy: same bits
     C_row = w8a8_block_fp8_matmul(A, B, As_row, Bs, [128, 128], torch.bfloat16)
@@ -119,6 +128,7 @@ def test_scaled_mm_llama3_every_config_point(dev, N, K, M):
     ref = O.fp8_scaled_mm(aq[rows], wq[cols], sa[rows], sb[cols], "f32", bias[cols])
     assert _rel_err(C0[ti][:, tj].float().cpu().numpy(), ref0) <= REL_TOL
     assert _rel_err(C[ti][:, tj].float().cpu().numpy(), ref) <= REL_TOL
+    assert _elem_rel_err(C0[ti][:, tj].float().cpu().numpy(), ref0) <= REL_TOL
     # float32 bias of the same values: the same bits (the bias is added in float32 either way)
     assert torch.equal(fp8_scaled_mm(A, B, tsa, tsb, torch.bfloat16, tbias.float()), C)
     # power-of-two scale factors pass through exactly on the whole un-biased output

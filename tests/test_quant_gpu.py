@@ -59,19 +59,30 @@ def test_group_quant_sweep_4096(dev, seed, layout):
     _check(x, dev, 128, layout)
 
 
-def test_group_quant_16384_every_layout(dev):
-    """The largest size of the bandwidth sweep (bf16 [16384, 7168]) in all four scale layouts.  At this size the
-    expected bytes and scales come from the C restatement of the oracle (OpenMP), which tests/test_oracle.py holds
-    bit for bit against the numpy one."""
+@pytest.mark.parametrize("layout", [(False, False, False), (True, False, False), (True, True, True)])
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4])
+@pytest.mark.parametrize("M", [1, 64, 512])
+def test_group_quant_sweep_small_sizes_every_seed(dev, M, seed, layout):
+    """The bandwidth sweep's sizes below 4096 rows with each of its five seeds and three scale layouts (row-major
+    float, column-major float, packed UE8M0)."""
+    _check(O.make_activation(M, 7168, seed=seed), dev, 128, layout)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3, 4])
+def test_group_quant_16384_every_layout(dev, seed):
+    """The largest size of the bandwidth sweep (bf16 [16384, 7168]) with each of its five seeds, in all four scale
+    layouts.  At this size the expected bytes and scales come from the C restatement of the oracle (OpenMP), which
+    tests/test_oracle.py holds bit for bit against the numpy one."""
     from oracle import c_oracle
 
     M, K, G = 16384, 7168, 56
-    x = O.make_activation(M, K, seed=0)
+    x = O.make_activation(M, K, seed=seed)
     lib = c_oracle.load()
     eps = float(O.clamp_eps(1e-10, "bf16"))
+    refs = {ue: c_oracle.group_quant_bf16(lib, O.bf16_bits(x), 128, eps, ue) for ue in (False, True)}
     for layout in _layouts():
         cm, al, ue = layout
-        q_ref, s_ref = c_oracle.group_quant_bf16(lib, O.bf16_bits(x), 128, eps, ue)
+        q_ref, s_ref = refs[ue]
         q, s = _run_group_quant(x, dev, 128, layout)
         assert torch.equal(q.view(torch.uint8).cpu(), torch.from_numpy(q_ref)), layout
         if ue:
