@@ -644,9 +644,11 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     uint8_t* const ep = smem + (w < 4 ? ews * WBYTES + w * 8192 : XBASE + exs * XBYTES + (w - 4) * 8192);
 #pragma unroll
     for (int ph = 0; ph < 2; ++ph) {
+      if (ph * 2 >= nact) break;  // the wave's remaining slot groups are all padding (real slots come first): nothing to store
 #pragma unroll
       for (int mh = 0; mh < 2; ++mh) {
         const int ms = ph * 2 + mh;
+        if (ms >= nact) continue;
         const int row = mh * 32 + lr_e;  // inside the pass's 64 slots
         const int oslot = oslots[ms];
         const bool ok = oslot < nrows;
@@ -677,6 +679,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
         __builtin_amdgcn_wave_barrier();  // one wave's LDS accesses complete in order: no wait needed
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
+          if (ph * 2 + (i >> 2) >= nact) continue;
           const int row = i * 8 + er;
           const int s = srow[ph * 8 + i];
           const int n = en0 + wn * 64 + (ec << 3);
