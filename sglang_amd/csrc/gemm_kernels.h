@@ -490,6 +490,11 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       const int xl = xst(it);                                         // activation stage block it left
       lds_barrier<4>();  // block it+1 has landed; the weights of block it+2 may still be on their way
       SB();
+      // Two waves share a SIMD's matrix pipe.  Left to the arbiter, one of them is served first whenever both are ready,
+      // runs ahead and then sits at the barrier while the other works through most of its block alone - and one wave
+      // alone cannot keep the pipe busy (its products wait for their own scale FMAs).  The issue priority therefore falls
+      // with a wave's progress through the trip: whoever is behind goes first, and the two stay interleaved.
+      __builtin_amdgcn_s_setprio(3);
       // ---- step 3 of block it; every operand register is refilled from block it+1 after its last use
       F(acc[2][0], tq[0], sc[0]); SB();
       M(0, 0, 3); SB();
@@ -501,6 +506,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       RX(0, 1, stX); SB();
       M(1, 1, 3); SB();
       RX(1, 1, stX); RW(1, stW, 0); SB();
+      __builtin_amdgcn_s_setprio(2);
       if (MODE == kModeBlock) { scn[0] = s0n * sbn; scn[1] = s1n * sbn; }
       // ---- step 0 of block it+1; the pending products still belong to block it
       F(acc[3][0], tq[0], sc[0]); SB();
@@ -524,6 +530,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       M(0, 1, 0); SB();
       M(1, 1, 0); SB();
       RW(1, stW, 1); LW(2, it + 3, w_ld); LW(3, it + 3, w_ld); SB();
+      __builtin_amdgcn_s_setprio(1);
       // ---- steps 1 and 2 of block it+1
       F(acc[0][0], tq[0], sc[0]); SB();
       M(0, 0, 1); SB();
@@ -533,6 +540,7 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       M(0, 1, 1); SB();
       M(1, 1, 1); SB();
       RW(1, stW, 2); SB();
+      __builtin_amdgcn_s_setprio(0);
       F(acc[1][0], tq[0], sc[0]); SB();
       M(0, 0, 2); SB();
       F(acc[1][1], tq[1], sc[1]); SB();
