@@ -501,13 +501,16 @@ def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, num_fused_shared
 # --------------------------------------------------------------------------
 
 
-def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scaling_factor=1.0, block=(128, 128)):
+def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scaling_factor=1.0, block=(128, 128),
+                        apply_router_weight_on_input=False):
     """Reference: fused_experts_impl, python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:498-639
     (sequence) and torch_w8a8_block_fp8_moe, python/sglang/test/test_block_fp8.py:418-447 (math).
 
     x bf16 values [T,H]; w13q uint8 [E,2I,H]; w2q uint8 [E,H,I]; scales per 128x128 block.
     quant(x) -> GEMM1 -> silu_and_mul -> quant -> GEMM2 * topk_weight (f32, then bf16) ->
     sum over k in f32 * routed_scaling_factor -> bf16.
+    apply_router_weight_on_input (fused_moe.py:533,597; the kernel multiplies the float accumulator before the output
+    cast, fused_moe_triton_kernels.py MUL_ROUTED_WEIGHT): the weight multiplies the result of GEMM 1 instead.
     """
     T, H = x.shape
     E, I2, _ = w13q.shape
@@ -518,11 +521,15 @@ def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scalin
         t_idx, k_idx = np.nonzero(topk_ids == e)
         if t_idx.size == 0:
             continue
-        h1 = w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "bf16")
+        wk = topk_w[t_idx, k_idx][:, None].astype(np.float32)
+        if apply_router_weight_on_input:
+            h1 = to_bf16((w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "f32") * wk).astype(np.float32))
+        else:
+            h1 = w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "bf16")
         act = silu_and_mul(h1)
         aq, as_ = per_token_group_quant_fp8(act, block[1])
         h2 = w8a8_block_fp8_matmul(aq, w2q[e], as_, w2s[e], block, "f32")
-        inter[t_idx, k_idx] = to_bf16((h2 * topk_w[t_idx, k_idx][:, None].astype(np.float32)).astype(np.float32))
+        inter[t_idx, k_idx] = to_bf16(h2 if apply_router_weight_on_input else (h2 * wk).astype(np.float32))
     return moe_sum_reduce(inter, routed_scaling_factor)
 
 

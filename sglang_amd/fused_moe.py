@@ -172,8 +172,8 @@ def fused_experts_impl(
         raise RuntimeError("fused_experts_impl: only use_fp8_w8a8=True with block_shape=[128, 128] is built on this path")
     if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None:
         raise RuntimeError("fused_experts_impl: only the gated silu activation is built on this path")
-    if apply_router_weight_on_input or b1 is not None or b2 is not None or a1_scale is not None or a2_scale is not None:
-        raise RuntimeError("fused_experts_impl: router weight on input, biases and static activation scales are not built")
+    if b1 is not None or b2 is not None or a1_scale is not None or a2_scale is not None:
+        raise RuntimeError("fused_experts_impl: biases and static activation scales are not built on this path")
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
@@ -216,7 +216,9 @@ def fused_experts_impl(
         ic3 = out_hidden_states[begin:end] if no_combine else cache3[:tokens]
 
         sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(curr_ids, config["BLOCK_SIZE_M"], E)
-        if gemm1_fuses_activation(config, N):
+        # apply_router_weight_on_input (fused_moe.py:533,597 of the reference): the routed weight multiplies the result of
+        # GEMM 1 instead of GEMM 2; the fused write-out has no such factor, so that form keeps the three steps
+        if gemm1_fuses_activation(config, N) and not apply_router_weight_on_input:
             slots = tokens * topk
             a1_q, a1_s = sglang_per_token_group_quant_fp8(curr, block_shape[1])
             a1_s = _ops.moe_sort_scales(a1_s, sorted_token_ids, num_tokens_post_padded, topk, slots)
@@ -231,7 +233,7 @@ def fused_experts_impl(
             continue
         invoke_fused_moe_kernel(
             curr, w1, None, ic1, None, w1_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
-            num_tokens_post_padded, False, topk, config, use_fp8_w8a8=True, block_shape=block_shape,
+            num_tokens_post_padded, apply_router_weight_on_input, topk, config, use_fp8_w8a8=True, block_shape=block_shape,
         )
         # silu_and_mul fused into the requantisation (same bytes as silu_and_mul + group quant, one pass less
         # over the [tokens*topk, N] intermediate)
@@ -239,7 +241,7 @@ def fused_experts_impl(
                                                       fuse_silu_and_mul=True)
         invoke_fused_moe_kernel(
             a2_q, w2, None, ic3, a2_s, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
-            num_tokens_post_padded, True, 1, config, use_fp8_w8a8=True, block_shape=block_shape,
+            num_tokens_post_padded, not apply_router_weight_on_input, 1, config, use_fp8_w8a8=True, block_shape=block_shape,
         )
         if not no_combine:
             _ops.moe_sum_reduce(ic3, out_hidden_states[begin:end], routed_scaling_factor)

@@ -399,6 +399,26 @@ def test_fused_experts_vs_oracle(dev, T, E, H, I, topk, grouped):
     assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.02
 
 
+@pytest.mark.parametrize("T,E,H,I", [(40, 8, 512, 256), (1100, 4, 256, 128)])
+def test_fused_experts_router_weight_on_input(dev, T, E, H, I):
+    """apply_router_weight_on_input (one expert per token, as the reference requires): the routed weight multiplies
+    the result of GEMM 1; 1100 tokens on 4 experts take 256-slot blocks, where the default form would fuse GEMM 1's
+    write-out and this one keeps the three steps."""
+    from sglang_amd.fused_moe import fused_experts_impl
+
+    rng = np.random.default_rng(T)
+    x, w13q, w13s, w2q, w2s, tw, ids = _moe_problem(rng, T, E, H, I, 1, False)
+    tw = rng.uniform(0.2, 1.0, tw.shape).astype(np.float32)
+    ref = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0, apply_router_weight_on_input=True)
+    out = fused_experts_impl(
+        bf16_tensor(x, dev), fp8_tensor(w13q, dev), fp8_tensor(w2q, dev), torch.from_numpy(tw).to(dev),
+        torch.from_numpy(ids).to(dev), use_fp8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev),
+        w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], apply_router_weight_on_input=True,
+    )
+    torch.cuda.synchronize()
+    assert _rel_err(out.float().cpu().numpy(), ref) <= REL_TOL
+
+
 def test_fused_experts_with_absent_experts_and_no_combine(dev):
     """ids == -1 (expert on another rank) contribute zero; no_combine returns the per-slot rows."""
     from sglang_amd.fused_moe import fused_experts_impl

@@ -471,30 +471,41 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf):
     ids[rng.random(ids.shape) < 0.1] = -1          # experts on another rank contribute nothing
     tw = rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32)
     got = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf)
+    got_in = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, apply_router_weight_on_input=True)
 
     xt = torch.from_numpy(x).bfloat16()
     xq, xs = _t_group_quant(xt)
-    per_slot = torch.zeros((T, topk, H), dtype=torch.bfloat16)
     t_ids, t_w = torch.from_numpy(ids), torch.from_numpy(tw)
-    for e in range(E):
-        tok, slot = torch.nonzero(t_ids == e, as_tuple=True)
-        if tok.numel() == 0:
-            continue
-        W1, S1 = torch.from_numpy(w13q[e]).view(torch.float8_e4m3fn), torch.from_numpy(w13s[e])
-        W2, S2 = torch.from_numpy(w2q[e]).view(torch.float8_e4m3fn), torch.from_numpy(w2s[e])
-        h1 = _t_block_matmul_f64(xq[tok].float(), xs[tok], W1, S1).to(torch.float32).bfloat16()
-        act = torch.nn.functional.silu(h1[:, :I].float()).bfloat16() * h1[:, I:]
-        aq, a_s = _t_group_quant(act)
-        h2 = _t_block_matmul_f64(aq.float(), a_s, W2, S2).to(torch.float32)
-        per_slot[tok, slot] = (h2 * t_w[tok, slot].unsqueeze(1)).bfloat16()
-    acc = torch.zeros((T, H), dtype=torch.float32)
-    for k in range(topk):
-        acc = acc + per_slot[:, k].float()
-    ref = (acc * rsf).bfloat16().float().numpy()
 
+    def torch_pipeline(weight_on_input):
+        per_slot = torch.zeros((T, topk, H), dtype=torch.bfloat16)
+        for e in range(E):
+            tok, slot = torch.nonzero(t_ids == e, as_tuple=True)
+            if tok.numel() == 0:
+                continue
+            W1, S1 = torch.from_numpy(w13q[e]).view(torch.float8_e4m3fn), torch.from_numpy(w13s[e])
+            W2, S2 = torch.from_numpy(w2q[e]).view(torch.float8_e4m3fn), torch.from_numpy(w2s[e])
+            wk = t_w[tok, slot].unsqueeze(1)
+            h1 = _t_block_matmul_f64(xq[tok].float(), xs[tok], W1, S1).to(torch.float32)
+            h1 = (h1 * wk if weight_on_input else h1).bfloat16()
+            act = torch.nn.functional.silu(h1[:, :I].float()).bfloat16() * h1[:, I:]
+            aq, a_s = _t_group_quant(act)
+            h2 = _t_block_matmul_f64(aq.float(), a_s, W2, S2).to(torch.float32)
+            per_slot[tok, slot] = (h2 if weight_on_input else h2 * wk).bfloat16()
+        acc = torch.zeros((T, H), dtype=torch.float32)
+        for k in range(topk):
+            acc = acc + per_slot[:, k].float()
+        return (acc * rsf).bfloat16().float().numpy()
+
+    ref = torch_pipeline(False)
     assert got.shape == ref.shape == (T, H)
     assert (got == ref).mean() > 0.99, (got == ref).mean()
     assert np.abs(got - ref).max() <= 2.0**-6 * np.abs(ref).max()
+    # the routed weight on the result of GEMM 1 instead (fused_moe.py:533,597): another function of the same inputs
+    ref_in = torch_pipeline(True)
+    assert (got_in == ref_in).mean() > 0.99, (got_in == ref_in).mean()
+    assert np.abs(got_in - ref_in).max() <= 2.0**-6 * np.abs(ref_in).max()
+    assert not np.allclose(got_in, got, rtol=1e-2)
     # rows whose every expert is absent are exactly zero
     dead = (ids == -1).all(axis=1)
     assert (got[dead] == 0).all()
