@@ -120,6 +120,13 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
 #pragma unroll
     for (int q = 0; q < LW; ++q) buf_load16_to_lds(rX, voX[q] + ko, 0, base + q * 1024);
   };
+  // the same, one wave load at a time (q = 0 .. LW-1)
+  auto issue_w1 = [&](int q, const rsrc_t& r, int kblk, int stage) {
+    buf_load16_to_lds(r, voW[q & 1] + ((uint32_t)kblk * kTileK + (q >> 1) * w16), wsoff, smem + stage * WBYTES + w * (LW * 1024) + q * 1024);
+  };
+  auto issue_x1 = [&](int q, int kblk, int stage) {
+    buf_load16_to_lds(rX, voX[q] + (uint32_t)kblk * kTileK, 0, smem + XBASE + stage * XBYTES + w * (LW * 1024) + q * 1024);
+  };
   auto weights_of = [&](const MoeItem& it) -> rsrc_t {
     if (it.mb < 0) return make_rsrc(p.W, 0u);  // no item: every load is out of range and moves nothing
     const uint8_t* Wb = p.W + (int64_t)it.expert * p.w_expert_stride;
@@ -459,6 +466,140 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       if (it < nkb) trip(it);
       if constexpr (NA > 0) deferred(no{}, smem, smem);
     };
+    // The float-scale loop of the sorted forms, software-pipelined like the dense 256x256 tile kernel's with the roles
+    // of weights and activations swapped: the wave keeps the four weight fragments of a K block and walks its slot groups,
+    // one step (four MFMAs: n half 0 / 1 on K half 0, then on K half 1) per group.  The products of a step gather in
+    // tq[n half] and are folded into the accumulator with the block's scale behind the first MFMAs of the NEXT step, the
+    // activation fragments are refilled with the next group's behind their last use, and the step of a block's LAST group
+    // runs behind the next barrier, where every weight fragment is refilled from the new block right behind the MFMA that
+    // used it last.  The matrix core then has work across the barrier, and the operand fetches of the eight waves no
+    // longer come as one burst behind it.  Every wave issues the same loads at the same places whatever its group count.
+    auto run_piped = [&](auto na) {
+      constexpr int NA = decltype(na)::value;
+      constexpr int L = NA > 0 ? NA - 1 : 0, L2 = NA > 1 ? NA - 2 : 0;
+      using yes = std::integral_constant<bool, true>;
+      using no = std::integral_constant<bool, false>;
+      v8i wf[NS][2], xa, xb;
+      v16f tq[2], z;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { z[r] = 0.f; tq[0][r] = 0.f; tq[1][r] = 0.f; }
+      float sc[MS] = {0.f, 0.f, 0.f, 0.f};  // activation x weight scale of the block whose products are being formed
+      float sd0 = 0.f, sd1 = 0.f;          // ... of groups NA-2 and NA-1 of the block before: their products are folded after the barrier
+      // The eight stage loads of a trip (1 KB each) pass through the CU's address unit at 64 bytes a clock, all eight
+      // waves' at once: issued in one run behind the barrier they hold every wave for several hundred cycles (the later
+      // waves of the queue for more than a thousand) before its first MFMA.  A wave with groups to work on therefore
+      // spreads them over the step that follows the barrier, two behind each MFMA.
+      int ld_it = 0;
+      auto ld = [&](int i) {  // stage load i of trip ld_it: activations of block ld_it+1 (0..3), weights of block ld_it+2 (4..7)
+        if (i < 4) {
+          issue_x1(i, ld_it + 1, (gx0 + ld_it + 1) & 1);
+        } else {
+          const int k2 = ld_it + 2;
+          const bool nx = k2 >= nkb;
+          issue_w1(i - 4, nx ? rWn : rW, nx ? k2 - nkb : k2, (gw0 + k2) % WST);
+        }
+      };
+      auto open = [&](int it, auto all_loads) {
+        lds_barrier<LW>();  // everything but the wave's loads of weight block it+1 has landed
+        SB();
+        sd0 = sc[L2];
+        sd1 = sc[L];
+#pragma unroll
+        for (int ms = 0; ms < MS; ++ms) sc[ms] = sxn[ms] * sbn;
+        load_sx(it + 1);
+        load_sb(sbn, it + 1);
+        SB();  // scales, then activations, then weights
+        ld_it = it;
+        if constexpr (decltype(all_loads)::value) {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) ld(i);
+        }
+        SB();
+      };
+      auto fold = [&](auto ns_c, auto pg_c, float s) {
+        constexpr int NS_ = decltype(ns_c)::value, PG = decltype(pg_c)::value;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[NS_][PG][r] = __builtin_fmaf(tq[NS_][r], s, acc[NS_][PG][r]);
+      };
+      using n0_t = std::integral_constant<int, 0>;
+      using n1_t = std::integral_constant<int, 1>;
+      // One step.  PEND: the products of the step before (slot group PG, scale ps) are folded first.  FILL 0: the
+      // activation fragments of the group at nx_ follow; 1: those and the weight fragments of the block at nw_; 2: nothing.
+      auto step = [&](auto pend_c, auto pg_c, float ps, auto fill_c, const uint8_t* nw_, const uint8_t* nx_) {
+        constexpr bool PEND = decltype(pend_c)::value;
+        constexpr int FILL = decltype(fill_c)::value;
+        constexpr bool LOADS = FILL == 1;  // the step behind a barrier carries the trip's stage loads
+        const uint8_t* w0 = nw_ + (wn * 64) * kTileK;
+        const uint8_t* w1 = nw_ + (wn * 64 + 32) * kTileK;
+        if constexpr (PEND) { fold(n0_t{}, pg_c, ps); SB(); }
+        tq[0] = mfma_32x32x64(wf[0][0], xa, z); SB();
+        if constexpr (FILL == 1) { wf[0][0] = frag(w0, 0); SB(); }
+        if constexpr (LOADS) { ld(0); ld(1); SB(); }
+        if constexpr (PEND) { fold(n1_t{}, pg_c, ps); SB(); }
+        tq[1] = mfma_32x32x64(wf[1][0], xa, z); SB();
+        if constexpr (FILL != 2) xa = frag(nx_, 0);
+        if constexpr (FILL == 1) wf[1][0] = frag(w1, 0);
+        if constexpr (LOADS) { ld(2); ld(3); }
+        SB();
+        tq[0] = mfma_32x32x64(wf[0][1], xb, tq[0]); SB();
+        if constexpr (FILL == 1) { wf[0][1] = frag(w0, 1); SB(); }
+        if constexpr (LOADS) { ld(4); ld(5); SB(); }
+        tq[1] = mfma_32x32x64(wf[1][1], xb, tq[1]); SB();
+        if constexpr (FILL != 2) xb = frag(nx_, 1);
+        if constexpr (FILL == 1) wf[1][1] = frag(w1, 1);
+        if constexpr (LOADS) { ld(6); ld(7); }
+        SB();
+      };
+      using fill_x = std::integral_constant<int, 0>;
+      using fill_all = std::integral_constant<int, 1>;
+      using fill_none = std::integral_constant<int, 2>;
+      // groups 0 .. NA-2 of the block whose fragments sit in wf / xa / xb; FIRST: nothing is pending in front of group 0
+      auto groups = [&](auto first_c, const uint8_t* sx_) {
+        constexpr bool FIRST = decltype(first_c)::value;
+        if constexpr (NA >= 2) {
+          const uint8_t* g1 = sx_ + ((1 * 2 + wm) * 32) * kTileK;
+          if constexpr (FIRST) step(no{}, std::integral_constant<int, 0>{}, 0.f, fill_x{}, smem, g1);
+          else step(yes{}, std::integral_constant<int, L>{}, sd1, fill_x{}, smem, g1);
+        }
+        if constexpr (NA >= 3) step(yes{}, std::integral_constant<int, 0>{}, sc[0], fill_x{}, smem, sx_ + ((2 * 2 + wm) * 32) * kTileK);
+        if constexpr (NA >= 4) step(yes{}, std::integral_constant<int, 1>{}, sc[1], fill_x{}, smem, sx_ + ((3 * 2 + wm) * 32) * kTileK);
+      };
+      open(0, yes{});
+      if constexpr (NA > 0) {
+        const uint8_t* sw_ = smem + (gw0 % WST) * WBYTES;
+        const uint8_t* sx_ = smem + XBASE + (gx0 & 1) * XBYTES;
+#pragma unroll
+        for (int ns = 0; ns < NS; ++ns) {
+          wf[ns][0] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 0);
+          wf[ns][1] = frag(sw_ + (wn * 64 + ns * 32) * kTileK, 1);
+        }
+        xa = frag(sx_ + (wm * 32) * kTileK, 0);
+        xb = frag(sx_ + (wm * 32) * kTileK, 1);
+        SB();
+        groups(yes{}, sx_);
+      }
+      for (int it = 1; it < nkb; ++it) {
+        open(it, std::integral_constant<bool, NA == 0>{});
+        if constexpr (NA > 0) {
+          const uint8_t* sw_ = smem + ((gw0 + it) % WST) * WBYTES;
+          const uint8_t* sx_ = smem + XBASE + ((gx0 + it) & 1) * XBYTES;
+          // the last group of block it-1; the group before it (if the wave has two) is still pending
+          if constexpr (NA >= 2) step(yes{}, std::integral_constant<int, L2>{}, sd0, fill_all{}, sw_, sx_ + (wm * 32) * kTileK);
+          else step(no{}, std::integral_constant<int, 0>{}, 0.f, fill_all{}, sw_, sx_ + (wm * 32) * kTileK);
+          if constexpr (NA == 1) {  // a single group: its products are folded on the spot (the next step comes two barriers later)
+            fold(n0_t{}, std::integral_constant<int, 0>{}, sd1); fold(n1_t{}, std::integral_constant<int, 0>{}, sd1);
+            SB();
+          }
+          groups(no{}, sx_);
+        }
+      }
+      if constexpr (NA > 0) {
+        if constexpr (NA >= 2) step(yes{}, std::integral_constant<int, L2>{}, sc[L2], fill_none{}, smem, smem);
+        else step(no{}, std::integral_constant<int, 0>{}, 0.f, fill_none{}, smem, smem);
+        fold(n0_t{}, std::integral_constant<int, L>{}, sc[L]);
+        fold(n1_t{}, std::integral_constant<int, L>{}, sc[L]);
+      }
+    };
     // one copy of the loop per group count keeps every copy straight-line
     if constexpr (SCALED) {
       switch (nact) {  // wave-uniform
@@ -467,6 +608,14 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
         case 2: run_scaled(std::integral_constant<int, 2>{}); break;
         case 1: run_scaled(std::integral_constant<int, 1>{}); break;
         default: run_scaled(std::integral_constant<int, 0>{}); break;
+      }
+    } else if constexpr (SORTED && !PAIRS) {
+      switch (nact) {  // wave-uniform
+        case 4: run_piped(std::integral_constant<int, 4>{}); break;
+        case 3: run_piped(std::integral_constant<int, 3>{}); break;
+        case 2: run_piped(std::integral_constant<int, 2>{}); break;
+        case 1: run_piped(std::integral_constant<int, 1>{}); break;
+        default: run_piped(std::integral_constant<int, 0>{}); break;
       }
     } else {
       switch (nact) {  // wave-uniform
