@@ -547,16 +547,19 @@ def gemm_lines(torch, dev, shapes, data="random"):
 
     lines = ["| M | N | K | us | TFLOP/s | % of 5 PFLOP/s | GB/s (algorithmic) |", "|---|---|---|---|---|---|---|"]
     for (M, N, K) in shapes:
-        nbuf = 3
-        ws = [_block_quant_weight(torch, N, K, s, dev) for s in range(nbuf)]
-        qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s, dev), 128, column_major_scales=True)
+        # enough weights in rotation that none is still in the 256 MB memory-side cache when its turn comes again
+        nbuf = max(3, min(64, int(600e6 // (N * K)) + 1))
+        ws = [_block_quant_weight(torch, N, K, s % 3, dev) if s < 3 else None for s in range(nbuf)]
+        for s in range(3, nbuf):
+            ws[s] = (ws[s % 3][0].clone(), ws[s % 3][1].clone())
+        qs = [sglang_per_token_group_quant_fp8(_activation(torch, M, K, s % 3, dev), 128, column_major_scales=True)
               for s in range(nbuf)]
         if data == "zeros":
             for q, sc in ws + qs:
                 q.view(torch.uint8).zero_()
                 sc.fill_(1.0)
         us = _time_graph(torch, lambda i: w8a8_block_fp8_matmul(qs[i % nbuf][0], ws[i % nbuf][0], qs[i % nbuf][1],
-                                                                ws[i % nbuf][1], [128, 128], torch.bfloat16), 20)
+                                                                ws[i % nbuf][1], [128, 128], torch.bfloat16), max(20, nbuf))
         tf = 2.0 * M * N * K / us / 1e6
         lines.append("| %d | %d | %d | %.1f | %.1f | %.1f | %.0f |" % (M, N, K, us, tf, tf / PEAK_FP8_TFLOPS * 100,
                                                                       gemm_bytes(M, N, K) / us / 1e3))
@@ -733,6 +736,9 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 256 MiB read + 256 MiB write elementwise kernel (reference point for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--no-ceilings", action="store_true",
+                    help="skip the machine-ceiling legs (stream read, bare MFMA loop, headline launch on all-zero data): "
+                         "for counter runs, whose per-kernel averages should cover the random-data launches only")
     ap.add_argument("--moe", type=str, default=None,
                     help="only time the fused MoE layer at these token counts (comma separated) and print its table")
     ap.add_argument("--gemm", type=str, default=None,
@@ -740,6 +746,9 @@ def main() -> int:
     ap.add_argument("--gemm-data", choices=("random", "zeros"), default="random",
                     help="operands of the --gemm runs: synthetic random data (default) or all zeros (same work, no "
                          "toggling in the matrix cores: shows what the power management takes)")
+    ap.add_argument("--gemm-plan", type=str, default=None,
+                    help="kernel family of the --gemm runs as KIND or KIND:SPLITS (fp8k_tune_force_gemm_plan; e.g. 3 = the "
+                         "direct kernel with float partials, 5 = the direct kernel that cuts K across a workgroup's waves)")
     ap.add_argument("--grouped", type=str, default=None,
                     help="only time the masked grouped GEMM (groups x rows x N x K, comma separated) with float and "
                          "with packed UE8M0 scales")
@@ -767,6 +776,11 @@ def main() -> int:
         return 0
     if args.gemm:
         shapes = [tuple(int(v) for v in t.split("x")) for t in args.gemm.split(",")]
+        if args.gemm_plan:
+            from sglang_amd._lib import lib
+
+            kind, _, splits = args.gemm_plan.partition(":")
+            lib.fp8k_tune_force_gemm_plan(int(kind), int(splits or 0))
         print("\n".join(gemm_lines(torch, dev, shapes, args.gemm_data)))
         return 0
     if args.grouped:
@@ -845,9 +859,9 @@ def main() -> int:
             "avg_launch_us": round(q_us, 2),
             "other_layouts_GBps": {k: round(v[1], 1) for k, v in quant.items()},
         },
-        "hbm_stream_read_GBps": round(hbm_stream_read_gbs(torch, dev), 1),
-        "mfma_ceiling_TFLOPs": mfma_ceiling_tflops(torch, dev),
-        "headline_zero_data_us": round(headline_zero_data_us(torch, dev), 2),
+        "hbm_stream_read_GBps": None if args.no_ceilings else round(hbm_stream_read_gbs(torch, dev), 1),
+        "mfma_ceiling_TFLOPs": None if args.no_ceilings else mfma_ceiling_tflops(torch, dev),
+        "headline_zero_data_us": None if args.no_ceilings else round(headline_zero_data_us(torch, dev), 2),
         "cpu_baseline": cpu,
     }
     print(json.dumps(out))
