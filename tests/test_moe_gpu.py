@@ -288,6 +288,27 @@ def test_grouped_gemm_256_slot_blocks_every_group_count(dev):
         if rows.size:
             ref = O.w8a8_block_fp8_matmul(xq[rows], wq[e], xs[rows], ws[e], out_dtype="f32", acc=np.float64)
             assert _rel_err(got[rows], ref) <= REL_TOL, "expert %d with %d slots" % (e, rows.size)
+    # the same through the form with scales in sorted-slot order (its K loop is the software-pipelined one, one copy per
+    # group count), at one, two and three K blocks: the same arithmetic in the same order, so the same bits
+    from sglang_amd.sgl_kernel import moe_sort_scales
+
+    for kb in (3, 2, 1):
+        Kc = kb * 128
+        A = fp8_tensor(np.ascontiguousarray(xq[:, :Kc]), dev)
+        B = fp8_tensor(np.ascontiguousarray(wq[:, :, :Kc]), dev)
+        As = torch.from_numpy(np.ascontiguousarray(xs[:, :kb])).to(dev)
+        Bs = torch.from_numpy(np.ascontiguousarray(ws[:, :, :kb])).to(dev)
+        outs = []
+        for sort in (False, True):
+            Ck = torch.full((T, N), float("nan"), dtype=torch.bfloat16, device=dev)
+            sc = moe_sort_scales(As, sorted_ids, npad, 1, T) if sort else As
+            moe_block_gemm(A, B, Ck, sc, Bs, torch.ones((T, 1), device=dev), sorted_ids, expert_ids, npad, False, 1, block, T,
+                           scales_sorted=sort)
+            torch.cuda.synchronize()
+            outs.append(Ck)
+        assert torch.equal(outs[0], outs[1]), "K = %d" % Kc
+        if kb == 3:
+            assert torch.equal(outs[0], C)
 
 
 def test_grouped_gemm_random_routings_exact(dev):
