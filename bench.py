@@ -273,19 +273,57 @@ def mfma_ceiling_tflops(torch, dev, iters=40000, runs=3):
     sink = torch.empty(ncu * 512, dtype=torch.float32, device=dev)
     out = {}
     for name, ops in (("random", wq.view(torch.uint8)), ("zeros", torch.zeros_like(wq.view(torch.uint8)))):
-        flops = ctypes.c_int64(0)
-        best = float("inf")
-        for r in range(runs + 1):
-            a, b = _events(torch, 2)
-            a.record()
+        out[name] = _mfma_probe(torch, dev, ops, sink, 0, iters, runs)
+    return out
+
+
+def _mfma_probe(torch, dev, ops, sink, form, iters, runs):
+    """TFLOP/s of one form of the MFMA probes (0: fp8k_tune_mfma_peak, 1..4: fp8k_tune_mfma_loop), best of `runs`."""
+    import ctypes
+
+    from sglang_amd._lib import check, lib, stream_ptr
+
+    flops = ctypes.c_int64(0)
+    best = float("inf")
+    for r in range(runs + 1):
+        a, b = _events(torch, 2)
+        a.record()
+        if form == 0:
             check(lib.fp8k_tune_mfma_peak(ops.data_ptr(), ops.numel(), iters, sink.data_ptr(), sink.numel(),
                                           ctypes.byref(flops), stream_ptr(dev)))
-            b.record()
-            torch.cuda.synchronize()
-            if r:
-                best = min(best, a.elapsed_time(b))
-        out[name] = round(flops.value / best / 1e9, 1)
-    return out
+        else:
+            check(lib.fp8k_tune_mfma_loop(ops.data_ptr(), ops.numel(), iters // 2, form, sink.data_ptr(), sink.numel(),
+                                          ctypes.byref(flops), stream_ptr(dev)))
+        b.record()
+        torch.cuda.synchronize()
+        if r:
+            best = min(best, a.elapsed_time(b))
+    return round(flops.value / best / 1e9, 1)
+
+
+MFMA_LOOP_FORMS = ("bare MFMA loop", "+ block-scaled product form (16 scale FMAs per two MFMAs)",
+                   "+ operand fragments refilled from LDS", "+ one workgroup barrier per K block",
+                   "+ eight 1 KB stage loads per wave and K block")
+
+
+def mfma_loop_lines(torch, dev, iters=40000, runs=3):
+    """The tile kernel's K loop built up from the bare MFMA loop one ingredient at a time (fp8k_tune_mfma_loop), on
+    quantised-weight bytes and on zeros: what each ingredient costs the matrix cores on this machine."""
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    wq, _ = _block_quant_weight(torch, 4096, 4096, 0, dev)
+    sink = torch.empty(ncu * 512, dtype=torch.float32, device=dev)
+    rnd, zer = wq.view(torch.uint8), torch.zeros_like(wq.view(torch.uint8))
+    lines = ["| form | TFLOP/s on quantised-weight bytes | of 5 PFLOP/s | TFLOP/s on zeros | of 5 PFLOP/s |", "|---|---|---|---|---|"]
+    for form, name in enumerate(MFMA_LOOP_FORMS):
+        a = _mfma_probe(torch, dev, rnd, sink, form, iters, runs)
+        b = _mfma_probe(torch, dev, zer, sink, form, iters, runs)
+        lines.append("| %d: %s | %.0f | %.2f | %.0f | %.2f |" % (form, name, a, a / PEAK_FP8_TFLOPS, b, b / PEAK_FP8_TFLOPS))
+    # the stage loads above walk 16 MiB (more than one XCD's 4 MB L2: most come from the memory-side cache); the same with
+    # a 2 MiB range, every load an L2 hit
+    a = _mfma_probe(torch, dev, rnd[:2 << 20], sink, 4, iters, runs)
+    b = _mfma_probe(torch, dev, zer[:2 << 20], sink, 4, iters, runs)
+    lines.append("| 4 with every stage load an L2 hit | %.0f | %.2f | %.0f | %.2f |" % (a, a / PEAK_FP8_TFLOPS, b, b / PEAK_FP8_TFLOPS))
+    return lines
 
 
 def headline_zero_data_us(torch, dev):
@@ -755,6 +793,8 @@ def main() -> int:
     ap.add_argument("--stream-read", action="store_true", help="only measure the HBM read rate of the LDS-staged load path")
     ap.add_argument("--mfma-ceiling", action="store_true",
                     help="only measure the bare matrix-core rate on random and on all-zero FP8 operands")
+    ap.add_argument("--mfma-loop", action="store_true",
+                    help="only measure the tile kernel's K loop built up from the bare MFMA loop one ingredient at a time")
     ap.add_argument("--stream-mix", action="store_true",
                     help="only measure what small write-outs inside the read stream cost (read stream with stores, fill, copy)")
     args = ap.parse_args()
@@ -789,6 +829,9 @@ def main() -> int:
         return 0
     if args.stream_mix:
         print("\n".join(stream_mix_lines(torch, dev)))
+        return 0
+    if args.mfma_loop:
+        print("\n".join(mfma_loop_lines(torch, dev)))
         return 0
     if args.mfma_ceiling:
         c = mfma_ceiling_tflops(torch, dev)

@@ -69,6 +69,20 @@ int fp8k_tune_stream_read_write(const void* src, int64_t bytes, void* dst, int64
 int fp8k_tune_mfma_peak(const void* operands, int64_t bytes, int64_t iters, float* sink, int64_t sink_floats, int64_t* flops,
                         void* stream);
 
+/*
+ * Measurement aid (no counterpart in the reference): the K loop of the 256x256 block-scaled tile kernel built up from the
+ * bare MFMA loop of fp8k_tune_mfma_peak one ingredient at a time, on operands that never change, in the tile kernel's
+ * instruction order (16 MFMAs per wave and K block, 8 waves per CU).  form 1: the block-scaled product form (two MFMAs
+ * into a short-lived accumulator, 16 scale FMAs fold it into the long-lived one); form 2: + the operand fragments
+ * refilled from LDS behind their last use; form 3: + one LDS-only workgroup barrier per K block; form 4: + the eight
+ * 1 KB global -> LDS stage loads per wave and K block (from the first 16 MiB of `operands`, cache-resident) and the
+ * partial wait for them at the barrier.  `iters` K blocks; *flops receives the matrix FLOPs of the launch.  Timed by the
+ * caller, the steps down from form to form are what each ingredient costs the matrix cores.
+ * operands 32-byte aligned, bytes >= 1 MiB; sink: CUs x 512 floats.
+ */
+int fp8k_tune_mfma_loop(const void* operands, int64_t bytes, int64_t iters, int form, float* sink, int64_t sink_floats,
+                        int64_t* flops, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

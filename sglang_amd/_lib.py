@@ -72,6 +72,7 @@ SIGNATURES = {
     "fp8k_tune_stream_read_tiles": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr]),
     "fp8k_tune_stream_read_write": (_c_int, [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_i64, _c_i64, _c_ptr]),
     "fp8k_tune_mfma_peak": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
+    "fp8k_tune_mfma_loop": (_c_int, [_c_ptr, _c_i64, _c_i64, _c_int, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
     "fp8k_moe_align_block_size": (
         _c_int,
         [_c_ptr, _c_int, _c_i64, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr, _c_int, _c_ptr],

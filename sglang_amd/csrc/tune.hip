@@ -184,6 +184,163 @@ __global__ __launch_bounds__(512, 1) void mfma_peak_kernel(const uint8_t* __rest
 }
 }  // namespace fp8k
 
+namespace fp8k {
+// The K loop of the 256x256 block-scaled tile kernel built up from the bare MFMA loop, one ingredient at a time, on
+// operands that never change (LDS filled once, the stage loads fetch a small cache-resident range), so that what each
+// ingredient costs the matrix cores can be read off:
+//   FORM 1  the block-scaled product form: two MFMAs into a short-lived accumulator, folded into the long-lived one by 16
+//           scale FMAs placed behind the first MFMAs of the next product (8 products = 16 MFMAs per K block, as a wave of
+//           the tile kernel has them)
+//   FORM 2  + the operand fragments refilled from LDS behind their last use (24 ds_read_b128 per wave and K block)
+//   FORM 3  + one LDS-only workgroup barrier per K block
+//   FORM 4  + the eight 1 KB stage loads per wave and K block (global -> LDS) and the partial vmcnt wait at the barrier
+// The instruction order is the tile kernel's (steps 3, 0, 1, 2 of its loop).
+template <int FORM>
+__global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __restrict__ operands, int64_t bytes, int iters,
+                                                           float* __restrict__ sink) {
+  __shared__ __attribute__((aligned(1024))) uint8_t smem[5 * 32768];
+  const int lane = threadIdx.x & 63;
+  const int w = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int wn = w & 1, wm = w >> 1;
+  const uint32_t span = (uint32_t)std::min<int64_t>(bytes, 1 << 24) & ~65535u;  // the range the stage loads walk
+  const rsrc_t r = make_rsrc(operands, span);
+  for (int st = 0; st < 5; ++st)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      buf_load16_to_lds(r, (uint32_t)(((blockIdx.x * 5 + st) * 32768 + (w * 4 + q) * 1024 + lane * 16) % span), 0,
+                        smem + st * 32768 + (w * 4 + q) * 1024);
+  wait_vm0();
+  __syncthreads();
+  // a fragment = 64 lanes x 32 bytes, kept as two conflict-free 1 KB halves; a weight stage holds 16 of them, an
+  // activation stage 16
+  auto frag = [&](const uint8_t* base) -> v8i {
+    const v4i lo = *reinterpret_cast<const v4i*>(base + lane * 16);
+    const v4i hi = *reinterpret_cast<const v4i*>(base + 1024 + lane * 16);
+    v8i f;
+    f[0] = lo[0]; f[1] = lo[1]; f[2] = lo[2]; f[3] = lo[3];
+    f[4] = hi[0]; f[5] = hi[1]; f[6] = hi[2]; f[7] = hi[3];
+    return f;
+  };
+  v8i X[2][2], W[2];
+  v16f acc[4][2], tq[2], z;
+#pragma unroll
+  for (int q = 0; q < 16; ++q) { z[q] = 0.f; tq[0][q] = 0.f; tq[1][q] = 0.f; }
+#pragma unroll
+  for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) acc[ns][ms][q] = 0.f;
+  float sc[2] = {1.0f + lane * 1e-9f, 1.0f - lane * 1e-9f};
+  W[0] = frag(smem + (wn * 8) * 2048); W[1] = frag(smem + (wn * 8 + 1) * 2048);
+#pragma unroll
+  for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) X[ms][ks] = frag(smem + 3 * 32768 + (wm * 4 + ms * 2 + ks) * 2048);
+  // without the refills the operands would be loop constants, and the products with them: the register is passed through
+  // an empty asm statement instead, which the compiler cannot see through
+  auto RW = [&](int ks, const uint8_t* st, int ns) {
+    if (FORM >= 2) {
+      W[ks] = frag(st + (wn * 8 + ns * 2 + ks) * 2048);
+    } else {
+      int t = W[ks][0];
+      asm volatile("" : "+v"(t));
+      W[ks][0] = t;
+    }
+  };
+  auto RX = [&](int ms, int ks, const uint8_t* st) { if (FORM >= 2) X[ms][ks] = frag(st + (wm * 4 + ms * 2 + ks) * 2048); };
+  auto M = [&](int ms, int ks) {
+    if (ks == 0) tq[ms] = mfma_32x32x64(W[0], X[ms][0], z);
+    else tq[ms] = mfma_32x32x64(W[1], X[ms][1], tq[ms]);
+  };
+  auto F = [&](v16f& a, const v16f& t, float sv) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) a[q] = __builtin_fmaf(t[q], sv, a[q]);
+  };
+  int w_ld = 0, w_rd = 1;
+  for (int it = 0; it < iters; ++it) {
+    const uint8_t* stW = smem + w_rd * 32768;
+    const uint8_t* stX = smem + 3 * 32768 + ((it + 1) & 1) * 32768;
+    uint8_t* const ldX = smem + 3 * 32768 + (it & 1) * 32768 + w * 4096;
+    uint8_t* const ldW = smem + w_ld * 32768 + w * 4096;
+    const uint32_t go = (uint32_t)(((blockIdx.x * 3 + it) * 65536) % span) + w * 4096 + lane * 16;
+    auto LX = [&](int j) { if (FORM >= 4) buf_load16_to_lds(r, go + j * 1024, 0, ldX + j * 1024); };
+    auto LW = [&](int j) { if (FORM >= 4) buf_load16_to_lds(r, go + 32768 + j * 1024, 0, ldW + j * 1024); };
+    if (FORM >= 4) lds_barrier<4>();
+    else if (FORM == 3) lds_barrier();
+    SB();
+    F(acc[2][0], tq[0], sc[0]); SB();
+    M(0, 0); SB();
+    RX(0, 0, stX); LX(0); LX(1); SB();
+    F(acc[2][1], tq[1], sc[1]); SB();
+    M(1, 0); SB();
+    RX(1, 0, stX); RW(0, stW, 0); LX(2); LX(3); SB();
+    M(0, 1); SB();
+    RX(0, 1, stX); SB();
+    M(1, 1); SB();
+    RX(1, 1, stX); RW(1, stW, 0); SB();
+    F(acc[3][0], tq[0], sc[0]); SB();
+    M(0, 0); SB();
+    F(acc[3][1], tq[1], sc[1]); SB();
+    M(1, 0); SB();
+    RW(0, stW, 1); LW(0); LW(1); SB();
+    M(0, 1); SB();
+    M(1, 1); SB();
+    RW(1, stW, 1); LW(2); LW(3); SB();
+    F(acc[0][0], tq[0], sc[0]); SB();
+    M(0, 0); SB();
+    F(acc[0][1], tq[1], sc[1]); SB();
+    M(1, 0); SB();
+    RW(0, stW, 2); SB();
+    M(0, 1); SB();
+    M(1, 1); SB();
+    RW(1, stW, 2); SB();
+    F(acc[1][0], tq[0], sc[0]); SB();
+    M(0, 0); SB();
+    F(acc[1][1], tq[1], sc[1]); SB();
+    M(1, 0); SB();
+    RW(0, stW, 3); SB();
+    M(0, 1); SB();
+    M(1, 1); SB();
+    RW(1, stW, 3); SB();
+    w_ld = w_rd;
+    w_rd = w_rd == 2 ? 0 : w_rd + 1;
+  }
+  wait_vm0();
+  float sum = tq[0][0] + tq[1][0];
+#pragma unroll
+  for (int ns = 0; ns < 4; ++ns)
+#pragma unroll
+    for (int ms = 0; ms < 2; ++ms)
+#pragma unroll
+      for (int q = 0; q < 16; ++q) sum += acc[ns][ms][q];
+  sink[(int64_t)blockIdx.x * 512 + threadIdx.x] = sum;
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_tune_mfma_loop(const void* operands, int64_t bytes, int64_t iters, int form, float* sink,
+                                   int64_t sink_floats, int64_t* flops, void* stream) {
+  clear_error();
+  const char* op = "tune_mfma_loop";
+  FP8K_REQUIRE(operands && aligned(operands, 32), "%s: operands must be a 32-byte aligned device pointer", op);
+  FP8K_REQUIRE(bytes >= (1 << 20) && bytes < (1LL << 40), "%s: at least 1 MiB of operand bytes is needed", op);
+  FP8K_REQUIRE(iters >= 1 && iters <= (1 << 24), "%s: iters must be in [1, 2^24]", op);
+  FP8K_REQUIRE(form >= 1 && form <= 4, "%s: form must be 1..4", op);
+  const int ncu = num_cu();
+  FP8K_REQUIRE(sink && sink_floats >= (int64_t)ncu * 512, "%s: sink must hold %lld floats", op, (long long)ncu * 512);
+  if (flops) *flops = (int64_t)ncu * 8 * iters * 16 * (2LL * 32 * 32 * 64);
+  const dim3 grid((unsigned)ncu), block(512);
+  hipStream_t st = (hipStream_t)stream;
+  const uint8_t* o = (const uint8_t*)operands;
+  switch (form) {
+    case 1: hipLaunchKernelGGL(mfma_loop_kernel<1>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    case 2: hipLaunchKernelGGL(mfma_loop_kernel<2>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    case 3: hipLaunchKernelGGL(mfma_loop_kernel<3>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    default: hipLaunchKernelGGL(mfma_loop_kernel<4>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+  }
+  return check_launch(op);
+}
+
 extern "C" int fp8k_tune_mfma_peak(const void* operands, int64_t bytes, int64_t iters, float* sink, int64_t sink_floats,
                                    int64_t* flops, void* stream) {
   clear_error();

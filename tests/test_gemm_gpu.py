@@ -446,3 +446,45 @@ def test_stream_read_write_probe_writes_its_pattern_and_checks_its_arguments(dev
     assert (got[written // 4:] == -1).all()
     rc = lib.fp8k_tune_stream_read_write(src.data_ptr(), src.numel(), dst.data_ptr(), written - 1, spt, spw, stream_ptr(dev))
     assert rc != 0 and b"dst holds" in lib.fp8k_last_error()
+
+
+def test_mfma_probes_compute_what_they_claim_and_check_their_arguments(dev):
+    """The measurement aids fp8k_tune_mfma_peak / fp8k_tune_mfma_loop: on operand bytes 0x38 (1.0 in e4m3) every one of the
+    bare loop's 8 x 16 accumulator values per lane is 64 x iters, on all-zero bytes every form sums to zero; the FLOP
+    counts they report are those of their MFMAs; a form outside 1..4 is refused."""
+    import ctypes
+
+    from sglang_amd._lib import lib, stream_ptr
+
+    ncu = torch.cuda.get_device_properties(dev).multi_processor_count
+    sink = torch.full((ncu * 512,), float("nan"), dtype=torch.float32, device=dev)
+    ones = torch.full((1 << 20,), 0x38, dtype=torch.uint8, device=dev)
+    zeros = torch.zeros(1 << 20, dtype=torch.uint8, device=dev)
+    flops = ctypes.c_int64(0)
+    iters = 4
+    rc = lib.fp8k_tune_mfma_peak(ones.data_ptr(), ones.numel(), iters, sink.data_ptr(), sink.numel(), ctypes.byref(flops),
+                                 stream_ptr(dev))
+    assert rc == 0, lib.fp8k_last_error()
+    torch.cuda.synchronize()
+    assert flops.value == ncu * 8 * iters * 8 * 2 * 32 * 32 * 64
+    assert (sink == 128 * 64.0 * iters).all()
+    for form in (1, 2, 3, 4):
+        sink.fill_(float("nan"))
+        rc = lib.fp8k_tune_mfma_loop(zeros.data_ptr(), zeros.numel(), iters, form, sink.data_ptr(), sink.numel(),
+                                     ctypes.byref(flops), stream_ptr(dev))
+        assert rc == 0, lib.fp8k_last_error()
+        torch.cuda.synchronize()
+        assert flops.value == ncu * 8 * iters * 16 * 2 * 32 * 32 * 64
+        assert (sink == 0).all(), "form %d" % form
+    # with ones the block-scaled forms fold 64-sums with scales within 1e-7 of one: 8 accumulators x 16 values per lane,
+    # `iters` K blocks each (the products of the last block's final step are still pending in the short-lived pair)
+    rc = lib.fp8k_tune_mfma_loop(ones.data_ptr(), ones.numel(), iters, 2, sink.data_ptr(), sink.numel(), ctypes.byref(flops),
+                                 stream_ptr(dev))
+    assert rc == 0, lib.fp8k_last_error()
+    torch.cuda.synchronize()
+    got = sink.cpu().numpy()
+    assert np.isfinite(got).all() and (got > 0).all()
+    assert np.allclose(got, got[0], rtol=1e-5)
+    rc = lib.fp8k_tune_mfma_loop(zeros.data_ptr(), zeros.numel(), iters, 5, sink.data_ptr(), sink.numel(), ctypes.byref(flops),
+                                 stream_ptr(dev))
+    assert rc != 0 and b"form" in lib.fp8k_last_error()
