@@ -303,7 +303,8 @@ def _mfma_probe(torch, dev, ops, sink, form, iters, runs):
 
 MFMA_LOOP_FORMS = ("bare MFMA loop", "+ block-scaled product form (16 scale FMAs per two MFMAs)",
                    "+ operand fragments refilled from LDS", "+ one workgroup barrier per K block",
-                   "+ eight 1 KB stage loads per wave and K block")
+                   "+ eight 1 KB stage loads per wave and K block",
+                   "the complete loop without the scale FMAs (products accumulate in place)")
 
 
 def mfma_loop_lines(torch, dev, iters=40000, runs=3):

@@ -194,6 +194,8 @@ namespace fp8k {
 //   FORM 2  + the operand fragments refilled from LDS behind their last use (24 ds_read_b128 per wave and K block)
 //   FORM 3  + one LDS-only workgroup barrier per K block
 //   FORM 4  + the eight 1 KB stage loads per wave and K block (global -> LDS) and the partial vmcnt wait at the barrier
+//   FORM 5  form 4 without the scale FMAs: the products accumulate in place, as in the row-scaled and the
+//           hardware-scaled modes of the tile kernel
 // The instruction order is the tile kernel's (steps 3, 0, 1, 2 of its loop).
 template <int FORM>
 __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __restrict__ operands, int64_t bytes, int iters,
@@ -249,11 +251,15 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     }
   };
   auto RX = [&](int ms, int ks, const uint8_t* st) { if (FORM >= 2) X[ms][ks] = frag(st + (wm * 4 + ms * 2 + ks) * 2048); };
+  constexpr bool kFold = FORM != 5;
+  int step_ns = 0;  // the accumulator row the in-place form is working on (a constant after unrolling)
   auto M = [&](int ms, int ks) {
-    if (ks == 0) tq[ms] = mfma_32x32x64(W[0], X[ms][0], z);
+    if (!kFold) acc[step_ns][ms] = mfma_32x32x64(W[ks], X[ms][ks], acc[step_ns][ms]);
+    else if (ks == 0) tq[ms] = mfma_32x32x64(W[0], X[ms][0], z);
     else tq[ms] = mfma_32x32x64(W[1], X[ms][1], tq[ms]);
   };
   auto F = [&](v16f& a, const v16f& t, float sv) {
+    if (!kFold) return;
 #pragma unroll
     for (int q = 0; q < 16; ++q) a[q] = __builtin_fmaf(t[q], sv, a[q]);
   };
@@ -269,6 +275,7 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     if (FORM >= 4) lds_barrier<4>();
     else if (FORM == 3) lds_barrier();
     SB();
+    step_ns = 3;
     F(acc[2][0], tq[0], sc[0]); SB();
     M(0, 0); SB();
     RX(0, 0, stX); LX(0); LX(1); SB();
@@ -279,6 +286,7 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     RX(0, 1, stX); SB();
     M(1, 1); SB();
     RX(1, 1, stX); RW(1, stW, 0); SB();
+    step_ns = 0;
     F(acc[3][0], tq[0], sc[0]); SB();
     M(0, 0); SB();
     F(acc[3][1], tq[1], sc[1]); SB();
@@ -287,6 +295,7 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     M(0, 1); SB();
     M(1, 1); SB();
     RW(1, stW, 1); LW(2); LW(3); SB();
+    step_ns = 1;
     F(acc[0][0], tq[0], sc[0]); SB();
     M(0, 0); SB();
     F(acc[0][1], tq[1], sc[1]); SB();
@@ -295,6 +304,7 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     M(0, 1); SB();
     M(1, 1); SB();
     RW(1, stW, 2); SB();
+    step_ns = 2;
     F(acc[1][0], tq[0], sc[0]); SB();
     M(0, 0); SB();
     F(acc[1][1], tq[1], sc[1]); SB();
@@ -325,7 +335,7 @@ extern "C" int fp8k_tune_mfma_loop(const void* operands, int64_t bytes, int64_t 
   FP8K_REQUIRE(operands && aligned(operands, 32), "%s: operands must be a 32-byte aligned device pointer", op);
   FP8K_REQUIRE(bytes >= (1 << 20) && bytes < (1LL << 40), "%s: at least 1 MiB of operand bytes is needed", op);
   FP8K_REQUIRE(iters >= 1 && iters <= (1 << 24), "%s: iters must be in [1, 2^24]", op);
-  FP8K_REQUIRE(form >= 1 && form <= 4, "%s: form must be 1..4", op);
+  FP8K_REQUIRE(form >= 1 && form <= 5, "%s: form must be 1..5", op);
   const int ncu = num_cu();
   FP8K_REQUIRE(sink && sink_floats >= (int64_t)ncu * 512, "%s: sink must hold %lld floats", op, (long long)ncu * 512);
   if (flops) *flops = (int64_t)ncu * 8 * iters * 16 * (2LL * 32 * 32 * 64);
@@ -336,7 +346,8 @@ extern "C" int fp8k_tune_mfma_loop(const void* operands, int64_t bytes, int64_t 
     case 1: hipLaunchKernelGGL(mfma_loop_kernel<1>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
     case 2: hipLaunchKernelGGL(mfma_loop_kernel<2>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
     case 3: hipLaunchKernelGGL(mfma_loop_kernel<3>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
-    default: hipLaunchKernelGGL(mfma_loop_kernel<4>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    case 4: hipLaunchKernelGGL(mfma_loop_kernel<4>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    default: hipLaunchKernelGGL(mfma_loop_kernel<5>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
   }
   return check_launch(op);
 }
