@@ -47,19 +47,18 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     """Rows per block of the grouped GEMM (the reference's BLOCK_SIZE_M, fused_moe_triton_config.py).
 
     Measured on MI355X with 256 experts, top-8 and near-balanced routing: while the layer streams every expert's
-    weights for a handful of rows each, the register-streaming kernel with 16- or 32-row blocks wins; from about
-    16 rows per expert the LDS-staged streaming kernel with 64- and then 128-row blocks; from about 100 rows per
-    expert the 256-row kernel, which puts both 128-row halves of an expert on one pass over its weights.
+    weights for a handful of rows each, the register-streaming kernel with 16- or 32-row blocks wins (up to about 22
+    rows per expert: 1.95 ms against 2.02 ms at 512 tokens); from there on the 256-row kernel, which walks its items
+    with the weight stream running on across them, skips the slot groups that are padding and forms the activation and
+    the requantisation in the write-out of GEMM 1 (2.06 ms against 2.13 ms with 64-row blocks at 768 tokens, 2.21
+    against 2.29 with 128-row blocks at 1536, 2.48 against 2.65 at 3072).  The 64- and 128-row forms of the streaming
+    kernel remain for callers that pass their own BLOCK_SIZE_M.
     """
     per_expert = (M * topk + E - 1) // max(E, 1)
     if per_expert <= 4:
         bm = 16
     elif per_expert <= 22:
         bm = 32
-    elif per_expert <= 48:
-        bm = 64
-    elif per_expert <= 96:
-        bm = 128
     else:
         bm = 256
     return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}

@@ -756,8 +756,8 @@ def apply_shuffle_mul_sum(input: torch.Tensor, output: torch.Tensor, permutation
 
 
 def _expert_major_block_m(rows: int, num_experts: int) -> int:
-    """Slots per block of the grouped GEMM from the mean rows per expert; the thresholds are the measured ones of
-    fused_moe.get_default_config."""
+    """Slots per block of the grouped GEMM op from the mean rows per expert (the op hands the kernel per-row scales,
+    for which the 64- and 128-row streaming forms were measured ahead of the 256-row one up to about 96 rows)."""
     per_expert = (rows + num_experts - 1) // max(num_experts, 1)
     for limit, bm in ((4, 16), (22, 32), (48, 64), (96, 128)):
         if per_expert <= limit:

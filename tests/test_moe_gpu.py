@@ -537,15 +537,20 @@ def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
         assert torch.equal(out_p, out[perm])
 
 
-@pytest.mark.parametrize("T,block", [(1024, 64), (2048, 128)])
-def test_fused_experts_deepseek_dims_other_block_sizes(dev, deepseek_experts, T, block):
-    """The 64- and 128-slot grouped streaming kernels at the full expert dimensions (the default choice takes them
-    between 1024 and 3072 tokens): a sample of tokens against the oracle."""
-    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl, get_default_config
+@pytest.mark.parametrize("T,block", [(1024, 64), (2048, 128), (1024, 256)])
+def test_fused_experts_deepseek_dims_other_block_sizes(dev, deepseek_experts, T, block, monkeypatch):
+    """The 64- and 128-slot grouped streaming kernels at the full expert dimensions (a caller's own BLOCK_SIZE_M; the
+    default choice goes from 32-slot blocks straight to 256-slot ones, which 1024 tokens take half empty): a sample of
+    tokens against the oracle."""
+    import sglang_amd.fused_moe as fm
+    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl
 
     d = deepseek_experts
     E, H, topk = d["E"], d["H"], 8
-    assert get_default_config(T, E, topk)["BLOCK_SIZE_M"] == block
+    if block == 256:
+        assert fm.get_default_config(T, E, topk)["BLOCK_SIZE_M"] == 256
+    else:
+        monkeypatch.setattr(fm, "get_default_config", lambda M_, E_, k_: {"BLOCK_SIZE_M": block, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128})
     x = O.make_activation(T, H, T)
     logits = torch.randn((T, E), generator=d["gen"], device=dev)
     xt = bf16_tensor(x, dev)
