@@ -105,6 +105,11 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
   // The stages are two rings that run on across the items of a walk: block k of an item sits in weight stage
   // (gw0 + k) % 3 and activation stage (gx0 + k) & 1, the next item's block 0 in the stage after its last block.
   int gw0 = 0, gx0 = 0;
+  // Whether any of the wave's four activation loads of the item in work covers a real slot (real slots come first in a
+  // block).  A load of padding rows moves nothing and still takes its turn in the CU's address unit, so a wave whose rows
+  // are all padding runs a copy of the K loop without activation loads; the rows it leaves as they are belong to padding
+  // slots, whose products are never stored and reach no other slot's result.
+  bool xreal = true;
   // FUSE: the waves that load tile rows 128..255 (w >= 4) take them from the up rows, I - 128 rows further on
   const int half_n = p.N >> 1;
   const uint32_t wsoff = (FUSE && w >= 4) ? (uint32_t)((int64_t)(half_n - 128) * p.ldw) : 0u;
@@ -179,6 +184,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       const int sd = sid[q];
       voX[q] = sd < nrows ? (uint32_t)((int64_t)(sd / p.top_k) * p.ldx + c * 16) : 0xF0000000u;  // padding reads zeros
     }
+    xreal = __builtin_amdgcn_ballot_w64(sid[0] < nrows) != 0;  // the first row of the wave's first group: a prefix
     issue_x(0, gx0);
   };
   start_item(item, true);
@@ -474,8 +480,9 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
     // runs behind the next barrier, where every weight fragment is refilled from the new block right behind the MFMA that
     // used it last.  The matrix core then has work across the barrier, and the operand fetches of the eight waves no
     // longer come as one burst behind it.  Every wave issues the same loads at the same places whatever its group count.
-    auto run_piped = [&](auto na) {
+    auto run_piped = [&](auto na, auto xl) {
       constexpr int NA = decltype(na)::value;
+      constexpr bool XL = decltype(xl)::value;  // the wave's activation loads carry real slots
       constexpr int L = NA > 0 ? NA - 1 : 0, L2 = NA > 1 ? NA - 2 : 0;
       using yes = std::integral_constant<bool, true>;
       using no = std::integral_constant<bool, false>;
@@ -492,7 +499,7 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
       int ld_it = 0;
       auto ld = [&](int i) {  // stage load i of trip ld_it: activations of block ld_it+1 (0..3), weights of block ld_it+2 (4..7)
         if (i < 4) {
-          issue_x1(i, ld_it + 1, (gx0 + ld_it + 1) & 1);
+          if constexpr (XL) issue_x1(i, ld_it + 1, (gx0 + ld_it + 1) & 1);
         } else {
           const int k2 = ld_it + 2;
           const bool nx = k2 >= nkb;
@@ -610,12 +617,24 @@ __global__ __launch_bounds__(512, 1) void moe_stream256_kernel(const GemmArgs p)
         default: run_scaled(std::integral_constant<int, 0>{}); break;
       }
     } else if constexpr (SORTED && !PAIRS) {
-      switch (nact) {  // wave-uniform
-        case 4: run_piped(std::integral_constant<int, 4>{}); break;
-        case 3: run_piped(std::integral_constant<int, 3>{}); break;
-        case 2: run_piped(std::integral_constant<int, 2>{}); break;
-        case 1: run_piped(std::integral_constant<int, 1>{}); break;
-        default: run_piped(std::integral_constant<int, 0>{}); break;
+      using with_x = std::integral_constant<bool, true>;
+      using without_x = std::integral_constant<bool, false>;
+      if (xreal) {
+        switch (nact) {  // wave-uniform
+          case 4: run_piped(std::integral_constant<int, 4>{}, with_x{}); break;
+          case 3: run_piped(std::integral_constant<int, 3>{}, with_x{}); break;
+          case 2: run_piped(std::integral_constant<int, 2>{}, with_x{}); break;
+          case 1: run_piped(std::integral_constant<int, 1>{}, with_x{}); break;
+          default: run_piped(std::integral_constant<int, 0>{}, with_x{}); break;
+        }
+      } else {
+        switch (nact) {
+          case 4: run_piped(std::integral_constant<int, 4>{}, without_x{}); break;
+          case 3: run_piped(std::integral_constant<int, 3>{}, without_x{}); break;
+          case 2: run_piped(std::integral_constant<int, 2>{}, without_x{}); break;
+          case 1: run_piped(std::integral_constant<int, 1>{}, without_x{}); break;
+          default: run_piped(std::integral_constant<int, 0>{}, without_x{}); break;
+        }
       }
     } else {
       switch (nact) {  // wave-uniform
