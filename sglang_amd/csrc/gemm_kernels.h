@@ -389,12 +389,10 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       return;
     }
     if (is_half && wm >= 2) {
-      // half tile (always a workgroup's last item): the waves of the upper 128 rows issue their share of the loads
-      // (their activation rows are out of range and arrive as zeros) and keep the barriers, with the same order and
-      // counts of loads as the others
+      // half tile (always a workgroup's last item): the waves of the upper 128 rows issue their share of the weight loads
+      // and keep the barriers.  Their activation rows are out of range: those loads would move nothing and still take
+      // their turn in the CU's address unit, so they are not issued (nobody reads those rows of the stage)
       if (!pref) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) LX(j, 0, xst(0));
 #pragma unroll
         for (int j = 0; j < 4; ++j) LW(j, 0, wst(0));
 #pragma unroll
@@ -403,15 +401,11 @@ __global__ __launch_bounds__(512, 1) void gemm_tile256_kernel(const GemmArgs p) 
       wait_vm0();
       __syncthreads();
 #pragma unroll
-      for (int j = 0; j < 4; ++j) LX(j, 1, xst(1));
-#pragma unroll
       for (int j = 0; j < 4; ++j) LW(j, 2, wst(2));
       int w_ld = wst(0), w_rd = wst(1);
       for (int it = 0; it < nkb - 1; ++it) {
         lds_barrier<4>();
         SB();
-#pragma unroll
-        for (int j = 0; j < 4; ++j) LX(j, it + 2, xst(it));
 #pragma unroll
         for (int j = 0; j < 4; ++j) LW(j, it + 3, w_ld);
         w_ld = w_rd;
