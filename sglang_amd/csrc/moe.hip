@@ -836,9 +836,17 @@ __global__ __launch_bounds__(kAlignThreads) void moe_prepare_kernel(const int32_
   const int tid = threadIdx.x;
   for (int e = tid; e < E; e += kAlignThreads) counts[e] = 0;
   __syncthreads();
-  for (int i = tid; i < numel; i += kAlignThreads) {
-    const int e = ids[i];
-    if (e >= 0 && e < E) atomicAdd(&counts[e], 1);
+  // eight ids per lane and trip: eight loads in flight instead of one load latency per id
+  for (int i0 = tid; i0 < numel; i0 += 8 * kAlignThreads) {
+    int e8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kAlignThreads;
+      e8[u] = i < numel ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (e8[u] >= 0 && e8[u] < E) atomicAdd(&counts[e8[u]], 1);
   }
   __syncthreads();
   if (tid < 64) {
@@ -867,12 +875,127 @@ __global__ __launch_bounds__(kAlignThreads) void moe_prepare_kernel(const int32_
     ps2[e * 3] = counts[e]; ps2[e * 3 + 1] = k; ps2[e * 3 + 2] = n;
   }
   __syncthreads();
-  for (int i = tid; i < numel; i += kAlignThreads) {
-    const int e = ids[i];
-    if (e >= 0 && e < E) {
-      const int row = atomicAdd(&cursor[e], 1);
-      in_perm[row] = i / topk;
-      out_perm[i] = row;
+  for (int i0 = tid; i0 < numel; i0 += 8 * kAlignThreads) {
+    int e8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kAlignThreads;
+      e8[u] = i < numel ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = e8[u], i = i0 + u * kAlignThreads;
+      if (e >= 0 && e < E) {
+        const int row = atomicAdd(&cursor[e], 1);
+        in_perm[row] = i / topk;
+        out_perm[i] = row;
+      }
+    }
+  }
+}
+
+// Many ids (more than kAlignFusedMax): the same in four launches over workgroups that take kAlignChunk ids each, with the
+// caller's outputs as the only memory.  The row counts are summed up in problem_sizes1[e, 0] (zeroed first), one
+// workgroup turns them into offsets and sizes, and the placing workgroups reserve their share of an expert's rows with one
+// global atomic on the cell AFTER the expert's own in expert_offsets: that cell starts at the expert's first row and,
+// once every row of the expert is handed out, holds the first row of the next expert - its final value.
+__global__ __launch_bounds__(kAlignThreads) void moe_prepare_count_kernel(const int32_t* __restrict__ ids, int numel, int E,
+                                                                          int32_t* __restrict__ ps1) {
+  __shared__ int32_t counts[kAlignMaxBuckets];
+  for (int e = threadIdx.x; e < E; e += kAlignThreads) counts[e] = 0;
+  __syncthreads();
+  const int first = blockIdx.x * kAlignChunk, last = min(numel, first + kAlignChunk);
+  for (int i0 = first + threadIdx.x; i0 < last; i0 += 8 * kAlignThreads) {
+    int e8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kAlignThreads;
+      e8[u] = i < last ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (e8[u] >= 0 && e8[u] < E) atomicAdd(&counts[e8[u]], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kAlignThreads)
+    if (counts[e]) atomicAdd(&ps1[e * 3], counts[e]);
+}
+__global__ __launch_bounds__(kAlignThreads) void moe_prepare_scan_kernel(int E, int n, int k, int32_t* __restrict__ offsets,
+                                                                         int32_t* __restrict__ bs_offsets,
+                                                                         int32_t* __restrict__ ps1, int32_t* __restrict__ ps2) {
+  __shared__ int32_t counts[kAlignMaxBuckets];
+  __shared__ int32_t start[kAlignMaxBuckets];
+  __shared__ int32_t rounded[kAlignMaxBuckets];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += kAlignThreads) counts[e] = ps1[e * 3];
+  __syncthreads();
+  if (tid < 64) {
+    const int per = (E + 63) / 64;
+    const int e0 = tid * per, e1 = min(E, e0 + per);
+    int sum = 0, rsum = 0;
+    for (int e = e0; e < e1; ++e) { sum += counts[e]; rsum += (counts[e] + 127) / 128 * 128; }
+    int incl = sum, rincl = rsum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int v = __shfl_up(incl, off), rv = __shfl_up(rincl, off);
+      if (tid >= off) { incl += v; rincl += rv; }
+    }
+    int run = incl - sum, rrun = rincl - rsum;
+    for (int e = e0; e < e1; ++e) {
+      start[e] = run; rounded[e] = rrun;
+      run += counts[e]; rrun += (counts[e] + 127) / 128 * 128;
+    }
+    if (tid == 63 && bs_offsets) bs_offsets[E] = rincl;
+  }
+  __syncthreads();
+  if (tid == 0) offsets[0] = 0;
+  for (int e = tid; e < E; e += kAlignThreads) {
+    offsets[e + 1] = start[e];  // the cursor of expert e; its final value is the start of expert e + 1
+    if (bs_offsets) bs_offsets[e] = rounded[e];
+    ps1[e * 3 + 1] = 2 * n; ps1[e * 3 + 2] = k;
+    ps2[e * 3] = counts[e]; ps2[e * 3 + 1] = k; ps2[e * 3 + 2] = n;
+  }
+}
+__global__ __launch_bounds__(kAlignThreads) void moe_prepare_place_kernel(const int32_t* __restrict__ ids, int numel, int topk,
+                                                                          int E, int32_t* __restrict__ offsets,
+                                                                          int32_t* __restrict__ in_perm,
+                                                                          int32_t* __restrict__ out_perm) {
+  __shared__ int32_t cursor[kAlignMaxBuckets];
+  for (int e = threadIdx.x; e < E; e += kAlignThreads) cursor[e] = 0;
+  __syncthreads();
+  const int first = blockIdx.x * kAlignChunk, last = min(numel, first + kAlignChunk);
+  for (int i0 = first + threadIdx.x; i0 < last; i0 += 8 * kAlignThreads) {
+    int e8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kAlignThreads;
+      e8[u] = i < last ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u)
+      if (e8[u] >= 0 && e8[u] < E) atomicAdd(&cursor[e8[u]], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < E; e += kAlignThreads) {
+    const int c = cursor[e];
+    cursor[e] = c ? atomicAdd(&offsets[e + 1], c) : 0;  // from here on the workgroup's next free row of expert e
+  }
+  __syncthreads();
+  for (int i0 = first + threadIdx.x; i0 < last; i0 += 8 * kAlignThreads) {
+    int e8[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kAlignThreads;
+      e8[u] = i < last ? ids[i] : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = e8[u], i = i0 + u * kAlignThreads;
+      if (e >= 0 && e < E) {
+        const int row = atomicAdd(&cursor[e], 1);
+        in_perm[row] = i / topk;
+        out_perm[i] = row;
+      }
     }
   }
 }
@@ -930,6 +1053,7 @@ __global__ __launch_bounds__(256) void shuffle_mul_sum_kernel(const void* __rest
 // With slot_expert / slot_row given (the routed expert of every (token, k) slot and the expert-major row that
 // moe_prepare_kernel gave it) the table holds the SLOT at the position of its row, padded with num_slots: the grouped
 // GEMM then gathers token slot / top_k straight from the un-shuffled activations and writes its rows in slot order.
+template <bool SCATTER>
 __global__ __launch_bounds__(kAlignThreads) void moe_offset_blocks_kernel(const int32_t* __restrict__ starts,
                                                                           const int32_t* __restrict__ sizes, int E, int rows,
                                                                           int block, int32_t* __restrict__ sorted,
@@ -938,13 +1062,20 @@ __global__ __launch_bounds__(kAlignThreads) void moe_offset_blocks_kernel(const 
                                                                           const int32_t* __restrict__ slot_expert,
                                                                           const int32_t* __restrict__ slot_row,
                                                                           int num_slots) {
+  // Every workgroup scans the experts' block counts for itself (a few hundred values) and then takes its share of the
+  // work.  SCATTER = false: the blocks - the expert of each and its entries (rows, or with slot_row given the padding
+  // value num_slots in every entry); SCATTER = true, a second launch behind the first: the slots, each to the position of
+  // its row, so that a position no slot claims keeps the padding value.
   __shared__ int32_t first_block[kAlignMaxBuckets + 1];
+  __shared__ int32_t lstart[kAlignMaxBuckets], lsize[kAlignMaxBuckets];  // the experts' first rows and row counts
   const int tid = threadIdx.x;
+  for (int e = tid; e < E; e += kAlignThreads) { lstart[e] = starts[e]; lsize[e] = max(sizes[e * 3], 0); }
+  __syncthreads();
   if (tid < 64) {
     const int per = (E + 63) / 64;
     const int e0 = tid * per, e1 = min(E, e0 + per);
     int sum = 0;
-    for (int e = e0; e < e1; ++e) sum += (max(sizes[e * 3], 0) + block - 1) / block;
+    for (int e = e0; e < e1; ++e) sum += (lsize[e] + block - 1) / block;
     int incl = sum;
 #pragma unroll
     for (int off = 1; off < 64; off <<= 1) {
@@ -954,46 +1085,51 @@ __global__ __launch_bounds__(kAlignThreads) void moe_offset_blocks_kernel(const 
     int run = incl - sum;
     for (int e = e0; e < e1; ++e) {
       first_block[e] = run;
-      run += (max(sizes[e * 3], 0) + block - 1) / block;
+      run += (lsize[e] + block - 1) / block;
     }
     if (tid == 63) first_block[E] = incl;
   }
   __syncthreads();
   const int nblocks = min(first_block[E], max_blocks);
-  if (tid == 0) post_pad[0] = nblocks * block;
-  for (int b = tid; b < nblocks; b += kAlignThreads) {
-    int lo = 0, hi = E;  // first expert with first_block[e + 1] > b
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (first_block[mid + 1] <= b) lo = mid + 1;
-      else hi = mid;
-    }
-    expert_ids[b] = lo;
-  }
-  __syncthreads();
   const int total = nblocks * block;
-  for (int i = tid; i < total; i += kAlignThreads) {
-    const int b = i / block;
-    int lo = 0, hi = E;
-    while (lo < hi) {
-      const int mid = (lo + hi) >> 1;
-      if (first_block[mid + 1] <= b) lo = mid + 1;
-      else hi = mid;
+  if (!SCATTER) {
+    if (blockIdx.x == 0 && tid == 0) post_pad[0] = nblocks * block;
+    // one wavefront per block: its expert by a search that is uniform across the wave, then the block's entries with
+    // consecutive lanes on consecutive entries (a search per entry cost 60 us at 190 000 entries)
+    const int waves = kAlignThreads / 64, wave = blockIdx.x * waves + (tid >> 6), ln = tid & 63;
+    for (int b = wave; b < nblocks; b += gridDim.x * waves) {
+      int lo = 0, hi = E;  // first expert with first_block[e + 1] > b
+      while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (first_block[mid + 1] <= b) lo = mid + 1;
+        else hi = mid;
+      }
+      if (ln == 0) expert_ids[b] = lo;
+      const int base = (b - first_block[lo]) * block, st = lstart[lo], sz = lsize[lo];
+      for (int j = ln; j < block; j += 64) {
+        const int within = base + j, row = st + within;
+        sorted[b * block + j] = slot_row ? num_slots : ((within < sz && row >= 0 && row < rows) ? row : rows);
+      }
     }
-    const int within = i - first_block[lo] * block;
-    const int row = starts[lo] + within;
-    if (slot_row) sorted[i] = num_slots;
-    else sorted[i] = (within < sizes[lo * 3] && row >= 0 && row < rows) ? row : rows;
+    return;
   }
-  if (!slot_row) return;
-  __syncthreads();  // the padding values are in place before any slot lands on one of them
-  for (int i = tid; i < num_slots; i += kAlignThreads) {
-    const int e = slot_expert[i];
-    if (e < 0 || e >= E) continue;
-    const int within = slot_row[i] - starts[e];
-    if (within < 0 || within >= sizes[e * 3]) continue;
-    const int64_t pos = (int64_t)first_block[e] * block + within;
-    if (pos < total) sorted[pos] = i;
+  for (int i0 = blockIdx.x * 8 * kAlignThreads + tid; i0 < num_slots; i0 += gridDim.x * 8 * kAlignThreads) {
+    int e8[8], r8[8];  // eight loads of each table in flight
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int i = i0 + u * kAlignThreads;
+      e8[u] = i < num_slots ? slot_expert[i] : -1;
+      r8[u] = i < num_slots ? slot_row[i] : 0;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int e = e8[u];
+      if (e < 0 || e >= E) continue;
+      const int within = r8[u] - lstart[e];
+      if (within < 0 || within >= lsize[e]) continue;
+      const int64_t pos = (int64_t)first_block[e] * block + within;
+      if (pos < total) sorted[pos] = i0 + u * kAlignThreads;
+    }
   }
 }
 
@@ -1013,9 +1149,21 @@ extern "C" int fp8k_moe_prepare_input(const int32_t* topk_ids, int64_t numel, in
   FP8K_REQUIRE(n >= 0 && k >= 0 && 2 * n <= 0x7fffffffLL && k <= 0x7fffffffLL, "%s: bad n / k", op);
   FP8K_REQUIRE(expert_offsets && problem_sizes1 && problem_sizes2, "%s: null output pointer", op);
   FP8K_REQUIRE(numel == 0 || (topk_ids && input_permutation && output_permutation), "%s: null pointer", op);
-  hipLaunchKernelGGL(moe_prepare_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, topk_ids, (int)numel,
-                     (int)topk, (int)num_experts, (int)n, (int)k, expert_offsets, blockscale_offsets, problem_sizes1,
-                     problem_sizes2, input_permutation, output_permutation);
+  hipStream_t st = (hipStream_t)stream;
+  if (numel <= kAlignFusedMax) {
+    hipLaunchKernelGGL(moe_prepare_kernel, dim3(1), dim3(kAlignThreads), 0, st, topk_ids, (int)numel, (int)topk,
+                       (int)num_experts, (int)n, (int)k, expert_offsets, blockscale_offsets, problem_sizes1, problem_sizes2,
+                       input_permutation, output_permutation);
+    return check_launch(op);
+  }
+  const int E = (int)num_experts;
+  const unsigned chunks = (unsigned)((numel + kAlignChunk - 1) / kAlignChunk);
+  hipLaunchKernelGGL(zero_ints_kernel, dim3((3 * E + 255) / 256), dim3(256), 0, st, problem_sizes1, 3 * E);
+  hipLaunchKernelGGL(moe_prepare_count_kernel, dim3(chunks), dim3(kAlignThreads), 0, st, topk_ids, (int)numel, E, problem_sizes1);
+  hipLaunchKernelGGL(moe_prepare_scan_kernel, dim3(1), dim3(kAlignThreads), 0, st, E, (int)n, (int)k, expert_offsets,
+                     blockscale_offsets, problem_sizes1, problem_sizes2);
+  hipLaunchKernelGGL(moe_prepare_place_kernel, dim3(chunks), dim3(kAlignThreads), 0, st, topk_ids, (int)numel, (int)topk, E,
+                     expert_offsets, input_permutation, output_permutation);
   return check_launch(op);
 }
 
@@ -1078,7 +1226,9 @@ extern "C" int fp8k_moe_blocks_from_offsets(const int32_t* expert_starts, const 
                "%s: block table too small (%lld slots, %lld blocks; %lld slots may be needed)", op, (long long)sorted_capacity,
                (long long)expert_capacity, (long long)(worst / block_m * block_m));
   const int64_t max_blocks = sorted_capacity / block_m < expert_capacity ? sorted_capacity / block_m : expert_capacity;
-  hipLaunchKernelGGL(moe_offset_blocks_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, expert_starts,
+  const int64_t worst_blocks = std::min<int64_t>(worst / block_m, max_blocks);
+  const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(64, (worst_blocks + 63) / 64));
+  hipLaunchKernelGGL(moe_offset_blocks_kernel<false>, dim3(grid), dim3(kAlignThreads), 0, (hipStream_t)stream, expert_starts,
                      problem_sizes, (int)num_experts, (int)rows, (int)block_m, sorted_token_ids, expert_ids,
                      num_tokens_post_pad, (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks),
                      (const int32_t*)nullptr, (const int32_t*)nullptr, 0);
@@ -1104,9 +1254,19 @@ extern "C" int fp8k_moe_slot_blocks_from_offsets(const int32_t* expert_starts, c
                (long long)expert_capacity, (long long)(worst / block_m * block_m));
   const int64_t max_blocks = sorted_capacity / block_m < expert_capacity ? sorted_capacity / block_m : expert_capacity;
   // slot_rows of an empty problem is never read: any non-null pointer keeps the kernel on its slot path
-  hipLaunchKernelGGL(moe_offset_blocks_kernel, dim3(1), dim3(kAlignThreads), 0, (hipStream_t)stream, expert_starts,
-                     problem_sizes, (int)num_experts, (int)num_slots, (int)block_m, sorted_token_ids, expert_ids,
-                     num_tokens_post_pad, (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks), topk_ids,
-                     slot_rows ? slot_rows : expert_starts, (int)num_slots);
+  const int64_t worst_blocks = std::min<int64_t>(worst / block_m, max_blocks);
+  const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(64, (worst_blocks + 63) / 64));
+  const int mb = (int)(max_blocks > 0x7fffffffLL ? 0x7fffffffLL : max_blocks);
+  const int32_t* rows_map = slot_rows ? slot_rows : expert_starts;
+  hipStream_t st = (hipStream_t)stream;
+  hipLaunchKernelGGL(moe_offset_blocks_kernel<false>, dim3(grid), dim3(kAlignThreads), 0, st, expert_starts, problem_sizes,
+                     (int)num_experts, (int)num_slots, (int)block_m, sorted_token_ids, expert_ids, num_tokens_post_pad, mb,
+                     topk_ids, rows_map, (int)num_slots);
+  if (num_slots > 0) {  // behind the first launch: a slot lands on the padding value of its position
+    const unsigned sgrid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(64, (num_slots + 8 * kAlignThreads - 1) / (8 * kAlignThreads)));
+    hipLaunchKernelGGL(moe_offset_blocks_kernel<true>, dim3(sgrid), dim3(kAlignThreads), 0, st, expert_starts, problem_sizes,
+                       (int)num_experts, (int)num_slots, (int)block_m, sorted_token_ids, expert_ids, num_tokens_post_pad, mb,
+                       topk_ids, rows_map, (int)num_slots);
+  }
   return check_launch(op);
 }
