@@ -327,6 +327,19 @@ int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, const float* As
                                    void* stream);
 
 /*
+ * No counterpart in the reference (its grouped kernel reads the table of moe_align_block_size as it is): deals the slots
+ * of every expert out evenly over the blocks the expert already has.  moe_align_block_size fills all blocks of an expert
+ * but the last (600 slots: 256, 256, 88); the workgroups that take those blocks against one weight tile share the tile in
+ * L2 only while they keep pace, which blocks of 200, 200, 200 do and blocks of 256 and 88 do not.  sorted_out (a buffer
+ * of its own, sorted_capacity entries) receives the table; expert_ids and num_tokens_post_padded stay as they are; real
+ * slots still come first in every block; entries behind the blocks in use get the padding value num_valid_tokens.
+ * num_experts: the experts of the aligner call (ids 0 .. num_experts-1; blocks of expert id -1 are dealt out the same way).
+ */
+int fp8k_moe_balance_blocks(const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                            const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t block_m,
+                            int64_t num_valid_tokens, int64_t num_experts, int32_t* sorted_out, void* stream);
+
+/*
  * Activation scales in the order of sorted_token_ids (no counterpart in the reference, whose Triton kernel gathers
  * them per K block): out[kb * sorted_capacity + i] = As[sorted_token_ids[i] / top_k, kb] for i below
  * num_tokens_post_padded[0], 0 for padding entries.  Passing `out` to fp8k_moe_block_gemm with as_stride_m = 1,

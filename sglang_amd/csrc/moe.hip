@@ -325,6 +325,78 @@ __global__ __launch_bounds__(256) void moe_sort_scales_kernel(const float* __res
 }
 }  // namespace fp8k
 
+namespace fp8k {
+// moe_align_block_size fills every block of an expert but its last one, so an expert with 600 slots gets blocks of 256,
+// 256 and 88.  The workgroups of the grouped GEMM that take those blocks against the same weight tile are dispatched
+// together and share the tile in their XCD's L2 only while they keep pace - and a block of 88 slots runs away from one of
+// 256.  This kernel deals an expert's slots out evenly over the blocks it already has (200 / 200 / 200): slot number r of
+// the expert goes to block r mod nb, position r / nb.  Real slots still come first in every block, the block table
+// (expert_ids, the padded length) is unchanged, and which slot meets which row of a block is as unspecified as before.
+// Every workgroup finds the experts' first blocks, block counts and slot counts for itself; then one wavefront per block.
+__global__ __launch_bounds__(kAlignThreads) void moe_balance_blocks_kernel(const int32_t* __restrict__ sorted_in,
+                                                                           const int32_t* __restrict__ expert_ids,
+                                                                           const int32_t* __restrict__ post_pad, int capacity,
+                                                                           int block, int pad_value, int buckets,
+                                                                           int32_t* __restrict__ sorted_out) {
+  __shared__ int32_t first[kAlignMaxBuckets + 1], nblk[kAlignMaxBuckets + 1], creal[kAlignMaxBuckets + 1];
+  const int tid = threadIdx.x, wave = tid >> 6, ln = tid & 63, waves = kAlignThreads / 64;
+  const int nblocks = min(post_pad[0], capacity) / block;
+  for (int e = tid; e < buckets; e += kAlignThreads) { first[e] = 0x7fffffff; nblk[e] = 0; creal[e] = 0; }
+  __syncthreads();
+  for (int b = tid; b < nblocks; b += kAlignThreads) {
+    const int e = expert_ids[b] + 1;  // bucket 0: blocks of ids that belong to no expert of this rank
+    if (e >= 0 && e < buckets) { atomicMin(&first[e], b); atomicAdd(&nblk[e], 1); }
+  }
+  __syncthreads();
+  for (int e = tid; e < buckets; e += kAlignThreads) {  // slots of the expert = full blocks + the real entries of its last block
+    if (nblk[e] == 0) continue;
+    const int32_t* last = sorted_in + (int64_t)(first[e] + nblk[e] - 1) * block;
+    int lo = 0, hi = block;  // first padding entry of the last block (real slots come first)
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (last[mid] < pad_value) lo = mid + 1;
+      else hi = mid;
+    }
+    creal[e] = (nblk[e] - 1) * block + lo;
+  }
+  __syncthreads();
+  for (int b = blockIdx.x * waves + wave; b < nblocks; b += gridDim.x * waves) {
+    const int e = expert_ids[b] + 1;
+    if (e < 0 || e >= buckets) {  // not a bucket of this table: the block is copied as it is
+      for (int p = ln; p < block; p += 64) sorted_out[b * block + p] = sorted_in[b * block + p];
+      continue;
+    }
+    const int f = first[e], nb = nblk[e], c = creal[e], j = b - f;
+    for (int p = ln; p < block; p += 64) {
+      const int r = p * nb + j;
+      sorted_out[b * block + p] = r < c ? sorted_in[(f + r / block) * block + r % block] : pad_value;
+    }
+  }
+  // behind the blocks in use the table keeps the padding value
+  for (int i = nblocks * block + blockIdx.x * kAlignThreads + tid; i < capacity; i += gridDim.x * kAlignThreads) sorted_out[i] = pad_value;
+}
+}  // namespace fp8k
+
+extern "C" int fp8k_moe_balance_blocks(const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                       const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t block_m,
+                                       int64_t num_valid_tokens, int64_t num_experts, int32_t* sorted_out, void* stream) {
+  clear_error();
+  const char* op = "moe_balance_blocks";
+  FP8K_REQUIRE(sorted_capacity >= 0 && sorted_capacity < 0x7fffffffLL && block_m >= 1 && block_m <= 1024, "%s: bad shape", op);
+  FP8K_REQUIRE(num_valid_tokens >= 0 && num_valid_tokens < 0x7fffffffLL, "%s: bad slot count", op);
+  FP8K_REQUIRE(num_experts >= 1 && num_experts < kAlignMaxBuckets, "%s: num_experts must be in [1, %d) (got %lld)", op,
+               kAlignMaxBuckets, (long long)num_experts);
+  if (sorted_capacity == 0) return FP8K_OK;
+  FP8K_REQUIRE(sorted_token_ids && expert_ids && num_tokens_post_padded && sorted_out, "%s: null pointer", op);
+  FP8K_REQUIRE(sorted_out != sorted_token_ids, "%s: the balanced table needs a buffer of its own", op);
+  const int64_t blocks = sorted_capacity / block_m;
+  const unsigned grid = (unsigned)std::max<int64_t>(1, std::min<int64_t>(32, (blocks + 15) / 16));
+  hipLaunchKernelGGL(moe_balance_blocks_kernel, dim3(grid), dim3(kAlignThreads), 0, (hipStream_t)stream, sorted_token_ids,
+                     expert_ids, num_tokens_post_padded, (int)sorted_capacity, (int)block_m, (int)num_valid_tokens,
+                     (int)num_experts + 1, sorted_out);
+  return check_launch(op);
+}
+
 extern "C" int fp8k_moe_sort_scales(const float* As, float* out, const int32_t* sorted_token_ids,
                                     const int32_t* num_tokens_post_padded, int64_t sorted_capacity, int64_t k_blocks,
                                     int64_t top_k, int64_t num_valid_tokens, int64_t as_stride_m, int64_t as_stride_k,

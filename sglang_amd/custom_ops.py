@@ -124,6 +124,10 @@ def _sort_scales_fake(A_scale, sorted_token_ids, num_tokens_post_padded, top_k, 
 
 _register("moe_sort_scales(Tensor A_scale, Tensor sorted_token_ids, Tensor num_tokens_post_padded, int top_k, "
           "int num_valid_tokens) -> Tensor", _k.moe_sort_scales, _sort_scales_fake)
+_register("moe_balance_blocks(Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, int block_m, "
+          "int num_valid_tokens, int num_experts) -> Tensor", _k.moe_balance_blocks,
+          lambda sorted_token_ids, expert_ids, num_tokens_post_padded, block_m, num_valid_tokens, num_experts:
+          torch.empty_like(sorted_token_ids))
 _register(
     "moe_block_gemm(Tensor A, Tensor B, Tensor(a!) C, Tensor A_scale, Tensor B_scale, Tensor? topk_weights, "
     "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, bool mul_routed_weight, int top_k, "
@@ -250,6 +254,11 @@ def moe_sum_reduce(input_tensor, output_tensor, routed_scaling_factor: float = 0
 
 def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: int, num_valid_tokens: int) -> torch.Tensor:
     return _ops.moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k, num_valid_tokens)
+
+
+def moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded, block_m: int, num_valid_tokens: int,
+                       num_experts: int) -> torch.Tensor:
+    return _ops.moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded, block_m, num_valid_tokens, num_experts)
 
 
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,

@@ -64,6 +64,13 @@ def get_default_config(M: int, E: int, topk: int) -> Dict[str, int]:
     return {"BLOCK_SIZE_M": bm, "BLOCK_SIZE_N": 256, "BLOCK_SIZE_K": 128}
 
 
+def blocks_want_balancing(config: Dict[str, int], slots: int, num_experts: int) -> bool:
+    """Whether the layer deals every expert's slots out evenly over its blocks (moe_balance_blocks) before the grouped
+    GEMMs: with 256-slot blocks and, on average, more than 192 slots per expert most experts have two and more blocks,
+    whose workgroups share the expert's weight tiles in L2 only while the blocks take the same time."""
+    return int(config["BLOCK_SIZE_M"]) == 256 and slots > 192 * num_experts
+
+
 # block sizes from which the activation scales are first gathered into the order of sorted_token_ids
 SORT_SCALES_MIN_BLOCK = 64
 
@@ -215,6 +222,9 @@ def fused_experts_impl(
         ic3 = out_hidden_states[begin:end] if no_combine else cache3[:tokens]
 
         sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(curr_ids, config["BLOCK_SIZE_M"], E)
+        if blocks_want_balancing(config, tokens * topk, E):
+            sorted_token_ids = _ops.moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded,
+                                                       config["BLOCK_SIZE_M"], tokens * topk, E)
         # apply_router_weight_on_input (fused_moe.py:533,597 of the reference): the routed weight multiplies the result of
         # GEMM 1 instead of GEMM 2; the fused write-out has no such factor, so that form keeps the three steps
         if gemm1_fuses_activation(config, N) and not apply_router_weight_on_input:

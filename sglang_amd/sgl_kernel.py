@@ -632,6 +632,25 @@ def moe_sort_scales(A_scale, sorted_token_ids, num_tokens_post_padded, top_k: in
     return out.t()
 
 
+def moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded, block_m: int, num_valid_tokens: int,
+                       num_experts: int) -> torch.Tensor:
+    """The table of moe_align_block_size with every expert's slots dealt out evenly over the blocks the expert already has
+    (include/fp8k.h: fp8k_moe_balance_blocks); returns the new sorted_token_ids, expert_ids and num_tokens_post_padded
+    stay valid.  For the grouped GEMM with several blocks per expert: blocks of one expert then take the same time and
+    share their weight tiles in L2."""
+    require_cuda(sorted_token_ids, expert_ids, num_tokens_post_padded)
+    for t, name in ((sorted_token_ids, "sorted_token_ids"), (expert_ids, "expert_ids"), (num_tokens_post_padded, "num_tokens_post_padded")):
+        if t.dtype != torch.int32 or not t.is_contiguous():
+            raise RuntimeError("moe_balance_blocks: %s must be contiguous int32" % name)
+    cap = sorted_token_ids.numel()
+    if expert_ids.numel() * block_m < cap - cap % block_m:
+        raise RuntimeError("moe_balance_blocks: expert_ids is shorter than the block table")
+    out = torch.empty_like(sorted_token_ids)
+    check(lib.fp8k_moe_balance_blocks(sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(), cap,
+                                      block_m, num_valid_tokens, num_experts, out.data_ptr(), stream_ptr(out.device)))
+    return out
+
+
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                    mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int,
                    scales_sorted: bool = False, pow2_scales: bool = False) -> None:

@@ -712,3 +712,54 @@ def test_gemm1_with_fused_activation_quant_is_the_three_step_sequence(dev, T, E,
     finally:
         fm.get_default_config = old
     assert torch.equal(fused, plain)
+
+
+@pytest.mark.parametrize("T,E,topk,block", [(700, 4, 2, 256), (2100, 8, 3, 256), (300, 16, 4, 64), (16384, 256, 8, 256), (5, 8, 2, 16)])
+def test_moe_balance_blocks_deals_every_experts_slots_out_evenly(dev, T, E, topk, block):
+    """moe_balance_blocks: the same blocks per expert and the same slots per expert (as sets), every block of an expert
+    holding floor or ceil of slots / blocks of them, real slots first in every block, padding value elsewhere; the
+    grouped GEMM on the balanced table gives the same rows as on the aligner's."""
+    from sglang_amd.fused_moe import moe_align_block_size
+    from sglang_amd.sgl_kernel import moe_balance_blocks, moe_block_gemm, moe_sort_scales
+
+    rng = np.random.default_rng(T + E)
+    ids = _random_ids(rng, T, E, topk, 0.1 if T > 5 else 0.0)
+    numel = ids.size
+    sorted_ids, expert_ids, npad = moe_align_block_size(torch.from_numpy(ids).to(dev), block, E)
+    bal = moe_balance_blocks(sorted_ids, expert_ids, npad, block, numel, E)
+    torch.cuda.synchronize()
+    used = int(npad.item())
+    a, b, eid = sorted_ids.cpu().numpy(), bal.cpu().numpy(), expert_ids.cpu().numpy()[: used // block]
+    assert (b[used:] == numel).all()
+    flat = ids.reshape(-1)
+    for e in np.unique(eid):
+        blocks = np.nonzero(eid == e)[0]
+        assert np.array_equal(blocks, np.arange(blocks[0], blocks[0] + blocks.size))
+        seg_a = a[blocks[0] * block:(blocks[-1] + 1) * block]
+        seg_b = b[blocks[0] * block:(blocks[-1] + 1) * block].reshape(blocks.size, block)
+        real_a = seg_a[seg_a < numel]
+        assert np.array_equal(np.sort(seg_b[seg_b < numel]), np.sort(real_a))
+        if e >= 0:
+            assert np.array_equal(np.sort(real_a), np.nonzero(flat == e)[0])
+        per_block = (seg_b < numel).sum(axis=1)
+        assert per_block.max() - per_block.min() <= 1 and per_block.sum() == real_a.size
+        for row, n_real in zip(seg_b, per_block):
+            assert (row[:n_real] < numel).all() and (row[n_real:] == numel).all()
+    if block < 64:
+        return
+    # the grouped GEMM does not care which table it walks
+    N, K = 256, 256
+    wq, ws = _expert_weights(rng, E, N, K)
+    xq = O.f32_to_e4m3fn(np.clip(rng.standard_normal((T, K)).astype(np.float32) * 100, -448, 448))
+    xs = (rng.uniform(0.5, 2.0, (T, K // 128)) * 1e-2).astype(np.float32)
+    A, B = fp8_tensor(xq, dev), fp8_tensor(wq, dev)
+    As, Bs = torch.from_numpy(xs).to(dev), torch.from_numpy(ws).to(dev)
+    outs = []
+    for table in (sorted_ids, bal):
+        C = torch.zeros((numel, N), dtype=torch.bfloat16, device=dev)
+        sc = moe_sort_scales(As, table, npad, topk, numel)
+        moe_block_gemm(A, B, C, sc, Bs, torch.ones((T, topk), device=dev), table, expert_ids, npad, False, topk, block, numel,
+                       scales_sorted=True)
+        torch.cuda.synchronize()
+        outs.append(C)
+    assert torch.equal(outs[0], outs[1])
