@@ -216,8 +216,10 @@ int fp8k_moe_align_block_size(const void* topk_ids, int ids_are_int64, int64_t n
  * rows); As float (as_stride_m, as_stride_k); Bs float [E, ceil(N/128), K/128] (bs_stride_e, bs_stride_n,
  * bs_stride_k); C [num_valid_tokens, N] of out_dtype (ldc).  block_m in {16,32,64,128,256} is the block size
  * moe_align_block_size was called with; sorted_capacity = length of sorted_token_ids.  K % 128 == 0, N % 8 == 0.
- * as_sorted != 0 (block_m >= 64): As holds one row per position of sorted_token_ids instead of one per token
- * (see fp8k_moe_sort_scales).
+ * as_sorted bit 0 (block_m >= 64): As holds one row per position of sorted_token_ids instead of one per token
+ * (see fp8k_moe_sort_scales).  as_sorted bit 1 (value 2 or 3; a hint, the result does not depend on it): the table went
+ * through fp8k_moe_balance_blocks, so the blocks of an expert are equally full - the 256-slot kernel then runs as one
+ * walking workgroup per CU at every size instead of only up to 192 slots per expert.
  */
 int fp8k_moe_block_gemm(const void* A, const void* B, const float* As, const float* Bs, void* C,
                         const int32_t* sorted_token_ids, const int32_t* expert_ids,
@@ -316,7 +318,8 @@ int fp8k_moe_slot_blocks_from_offsets(const int32_t* expert_starts, const int32_
  * K blocks.  q_out e4m3fn [slots, I] (ldq bytes between rows, row = token slot); qs_out float, the scale of
  * activation column block g of the slot at position i of sorted_token_ids at qs_out[g * qs_stride_g + i] (0 for
  * padding) - the layout fp8k_moe_block_gemm takes with as_sorted = 1.  act_dtype: the 16-bit type whose roundings
- * the write-out reproduces (the dtype the layer runs in).  eps as for fp8k_group_quant.
+ * the write-out reproduces (the dtype the layer runs in).  eps as for fp8k_group_quant.  balanced != 0: the hint of
+ * fp8k_moe_block_gemm's as_sorted bit 1 (the table went through fp8k_moe_balance_blocks).
  */
 int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, const float* As_sorted, const float* Bs, void* q_out,
                                    float* qs_out, const int32_t* sorted_token_ids, const int32_t* expert_ids,
@@ -324,7 +327,7 @@ int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, const float* As
                                    int64_t top_k, int64_t num_experts, int64_t N, int64_t K, int64_t lda, int64_t as_stride_k,
                                    int64_t b_stride_e, int64_t ldb, int64_t bs_stride_e, int64_t bs_stride_n,
                                    int64_t bs_stride_k, int64_t ldq, int64_t qs_stride_g, float eps, int act_dtype,
-                                   void* stream);
+                                   int balanced, void* stream);
 
 /*
  * No counterpart in the reference (its grouped kernel reads the table of moe_align_block_size as it is): deals the slots

@@ -13,7 +13,7 @@ import torch
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "csrc", "libfp8k.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 F32, F16, BF16 = 0, 1, 2
 SCALE_F32, SCALE_UE8M0_PACKED, SCALE_UE8M0_F32 = 0, 1, 2
@@ -51,7 +51,7 @@ SIGNATURES = {
     "fp8k_apply_shuffle_mul_sum": (_c_int, [_c_ptr] * 4 + [_c_i64] * 4 + [_c_int, _c_ptr]),
     "fp8k_moe_blocks_from_offsets": (_c_int, [_c_ptr] * 2 + [_c_i64] * 3 + [_c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
     "fp8k_moe_slot_blocks_from_offsets": (_c_int, [_c_ptr] * 2 + [_c_i64, _c_ptr, _c_ptr, _c_i64, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_i64, _c_ptr, _c_ptr]),
-    "fp8k_moe_block_gemm_silu_quant": (_c_int, [_c_ptr] * 9 + [_c_i64] * 15 + [_c_f32, _c_int, _c_ptr]),
+    "fp8k_moe_block_gemm_silu_quant": (_c_int, [_c_ptr] * 9 + [_c_i64] * 15 + [_c_f32, _c_int, _c_int, _c_ptr]),
     "fp8k_block_gemm": (
         _c_int,
         [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i64] * 10 + [_c_int, _c_ptr, _c_i64, _c_ptr],

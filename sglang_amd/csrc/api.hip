@@ -40,4 +40,4 @@ int num_cu() {
 }  // namespace fp8k
 
 extern "C" const char* fp8k_last_error(void) { return fp8k::g_err; }
-extern "C" int fp8k_abi_version(void) { return 2; }
+extern "C" int fp8k_abi_version(void) { return 3; }

@@ -415,6 +415,12 @@ extern "C" int fp8k_moe_sort_scales(const float* As, float* out, const int32_t* 
   return check_launch(op);
 }
 
+// whether the 256-slot grouped kernel runs as one walking workgroup per CU (the walk hands the weight stream on two K
+// blocks ahead, so K must have them)
+static bool moe256_walks(int64_t num_valid_tokens, int64_t num_experts, int64_t K, bool balanced) {
+  return (balanced || num_valid_tokens <= num_experts * 192) && K >= 2 * kTileK;
+}
+
 static int moe_block_gemm_impl(const void* A, const void* B, const float* As, const float* Bs, void* C,
                                const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                const int32_t* num_tokens_post_padded, const float* topk_weights,
@@ -457,6 +463,8 @@ static int moe_block_gemm_impl(const void* A, const void* B, const float* As, co
   a.m_blocks = (int)(sorted_capacity / block_m);
   a.block_m = (int)block_m;
   a.w_expert_stride = b_stride_e; a.sw_expert_stride = bs_stride_e;
+  const bool balanced = (as_sorted & 2) != 0;  // the table went through fp8k_moe_balance_blocks
+  as_sorted &= 1;
   a.sx_sorted = as_sorted ? 1 : 0;
   FP8K_REQUIRE(!as_sorted || block_m >= 64, "%s: scales in sorted order are taken with block_m >= 64", op);
   const bool direct = block_m <= 32;  // few rows per expert: weights go straight to registers, 128-row tiles
@@ -485,8 +493,10 @@ static int moe_block_gemm_impl(const void* A, const void* B, const float* As, co
     // workgroup per CU (a multiple of 8: one share per XCD), which requests an item's first blocks in front of the
     // previous item's write-out (M = 4096 tokens, top-8 of 256 experts: both GEMMs 4 % faster).  With several blocks per
     // expert, some of them nearly empty, the item times differ and a fixed share per CU loses more than the overlap
-    // gains (M = 16384: 6 % slower): one workgroup per item, handed out by the dispatcher as CUs fall free.
-    const bool walk = num_valid_tokens <= num_experts * 192 && K >= 2 * kTileK;  // the walk hands the stream on two K blocks ahead
+    // gains (M = 16384: 6 % slower): one workgroup per item, handed out by the dispatcher as CUs fall free - unless the
+    // caller says that the blocks of an expert are equally full (moe_balance_blocks): then the walk is ahead at every
+    // size (16384 tokens: 2 %).
+    const bool walk = moe256_walks(num_valid_tokens, num_experts, K, balanced);
     const int64_t nwg = walk ? std::min<int64_t>(per_xcd * 8 * a.tiles_n, std::max(8, num_cu() / 8 * 8)) : per_xcd * 8 * a.tiles_n;
     // row-major activation scales (what fused_experts_impl produces for 256-slot blocks) take the form that fetches
     // two K blocks per load
@@ -550,7 +560,7 @@ extern "C" int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, cons
                                               int64_t num_valid_tokens, int64_t top_k, int64_t num_experts, int64_t N,
                                               int64_t K, int64_t lda, int64_t as_stride_k, int64_t b_stride_e, int64_t ldb,
                                               int64_t bs_stride_e, int64_t bs_stride_n, int64_t bs_stride_k, int64_t ldq,
-                                              int64_t qs_stride_g, float eps, int act_dtype, void* stream) {
+                                              int64_t qs_stride_g, float eps, int act_dtype, int balanced, void* stream) {
   clear_error();
   const char* op = "moe_block_gemm_silu_quant";
   constexpr int64_t block_m = 256;
@@ -598,7 +608,7 @@ extern "C" int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, cons
     memcpy(&a.q_eps, &u, 4);
   }
   const int64_t per_xcd = (a.m_blocks + 7) / 8;
-  const bool walk = num_valid_tokens <= num_experts * 192 && K >= 2 * kTileK;
+  const bool walk = moe256_walks(num_valid_tokens, num_experts, K, balanced != 0);
   const int64_t nwg = walk ? std::min<int64_t>(per_xcd * 8 * a.tiles_n, std::max(8, num_cu() / 8 * 8)) : per_xcd * 8 * a.tiles_n;
   FP8K_REQUIRE(nwg < 0x7fffffffLL, "%s: grid too large", op);
   hipStream_t st = (hipStream_t)stream;

@@ -131,7 +131,7 @@ _register("moe_balance_blocks(Tensor sorted_token_ids, Tensor expert_ids, Tensor
 _register(
     "moe_block_gemm(Tensor A, Tensor B, Tensor(a!) C, Tensor A_scale, Tensor B_scale, Tensor? topk_weights, "
     "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, bool mul_routed_weight, int top_k, "
-    "int block_m, int num_valid_tokens, bool scales_sorted=False, bool pow2_scales=False) -> ()",
+    "int block_m, int num_valid_tokens, bool scales_sorted=False, bool pow2_scales=False, bool balanced=False) -> ()",
     _k.moe_block_gemm, _none,
 )
 
@@ -139,7 +139,7 @@ _register(
 _register(
     "moe_block_gemm_silu_quant(Tensor A, Tensor B, Tensor A_scale_sorted, Tensor B_scale, Tensor(a!) out_q, Tensor(b!) out_s, "
     "Tensor sorted_token_ids, Tensor expert_ids, Tensor num_tokens_post_padded, int top_k, int num_valid_tokens, "
-    "ScalarType act_dtype, float eps=1e-10) -> ()",
+    "ScalarType act_dtype, float eps=1e-10, bool balanced=False) -> ()",
     _k.moe_block_gemm_silu_quant, _none,
 )
 
@@ -263,15 +263,16 @@ def moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded, blo
 
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                    mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int, scales_sorted: bool = False,
-                   pow2_scales: bool = False) -> None:
+                   pow2_scales: bool = False, balanced: bool = False) -> None:
     _ops.moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                        mul_routed_weight, top_k, block_m, num_valid_tokens, scales_sorted, pow2_scales)
+                        mul_routed_weight, top_k, block_m, num_valid_tokens, scales_sorted, pow2_scales, balanced)
 
 
 def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,
-                              num_tokens_post_padded, top_k: int, num_valid_tokens: int, act_dtype, eps: float = 1e-10) -> None:
+                              num_tokens_post_padded, top_k: int, num_valid_tokens: int, act_dtype, eps: float = 1e-10,
+                              balanced: bool = False) -> None:
     _ops.moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,
-                                   num_tokens_post_padded, top_k, num_valid_tokens, act_dtype, float(eps))
+                                   num_tokens_post_padded, top_k, num_valid_tokens, act_dtype, float(eps), balanced)
 
 
 def moe_fused_gate(input_tensor, bias, num_expert_group, topk_group, topk, num_fused_shared_experts=0,

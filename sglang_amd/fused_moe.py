@@ -222,7 +222,8 @@ def fused_experts_impl(
         ic3 = out_hidden_states[begin:end] if no_combine else cache3[:tokens]
 
         sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(curr_ids, config["BLOCK_SIZE_M"], E)
-        if blocks_want_balancing(config, tokens * topk, E):
+        balanced = blocks_want_balancing(config, tokens * topk, E)
+        if balanced:
             sorted_token_ids = _ops.moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded,
                                                        config["BLOCK_SIZE_M"], tokens * topk, E)
         # apply_router_weight_on_input (fused_moe.py:533,597 of the reference): the routed weight multiplies the result of
@@ -234,9 +235,9 @@ def fused_experts_impl(
             a2_q = torch.empty((slots, N // 2), device=dev, dtype=torch.float8_e4m3fn)
             a2_s = torch.empty((N // 256, sorted_token_ids.numel()), device=dev, dtype=torch.float32).t()
             _ops.moe_block_gemm_silu_quant(a1_q, w1, a1_s, w1_scale, a2_q, a2_s, sorted_token_ids, expert_ids,
-                                           num_tokens_post_padded, topk, slots, dt)
+                                           num_tokens_post_padded, topk, slots, dt, balanced=balanced)
             _ops.moe_block_gemm(a2_q, w2, ic3, a2_s, w2_scale, curr_w, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                                True, 1, 256, slots, scales_sorted=True)
+                                True, 1, 256, slots, scales_sorted=True, balanced=balanced)
             if not no_combine:
                 _ops.moe_sum_reduce(ic3, out_hidden_states[begin:end], routed_scaling_factor)
             continue

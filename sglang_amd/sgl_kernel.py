@@ -653,13 +653,14 @@ def moe_balance_blocks(sorted_token_ids, expert_ids, num_tokens_post_padded, blo
 
 def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded,
                    mul_routed_weight: bool, top_k: int, block_m: int, num_valid_tokens: int,
-                   scales_sorted: bool = False, pow2_scales: bool = False) -> None:
+                   scales_sorted: bool = False, pow2_scales: bool = False, balanced: bool = False) -> None:
     """Grouped block-FP8 GEMM behind invoke_fused_moe_kernel (see include/fp8k.h: fp8k_moe_block_gemm).
     A e4m3fn [rows, K]; B e4m3fn [E, N, K]; A_scale float32 [rows, K/128] (scales_sorted: one row per entry of
     sorted_token_ids, from moe_sort_scales); B_scale float32 [E, N/128, K/128];
     C [num_valid_tokens, N] (any leading shape, flattened) bf16/fp16, written in place.
     pow2_scales: the caller vouches that every scale is a power of two (UE8M0); 256-slot blocks with sorted scales
-    then let the matrix cores apply the scales (fp8k_moe_block_gemm_ue8m0)."""
+    then let the matrix cores apply the scales (fp8k_moe_block_gemm_ue8m0).
+    balanced: sorted_token_ids went through moe_balance_blocks (a hint for the 256-slot kernel's schedule)."""
     require_cuda(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, expert_ids, num_tokens_post_padded)
     if A.dtype != FP8_DTYPE or B.dtype != FP8_DTYPE:
         raise RuntimeError("moe_block_gemm: A and B must be Float8_e4m3fn")
@@ -694,7 +695,7 @@ def moe_block_gemm(A, B, C, A_scale, B_scale, topk_weights, sorted_token_ids, ex
             topk_weights.data_ptr() if mul_routed_weight else None, sorted_token_ids.numel(), block_m,
             num_valid_tokens, top_k, E, N, K, A.stride(0), A_scale.stride(0), A_scale.stride(1), B.stride(0),
             B.stride(1), B_scale.stride(0), B_scale.stride(1), B_scale.stride(2), C2.stride(0), _out_code(C.dtype),
-            1 if scales_sorted else 0, stream_ptr(A.device),
+            (1 if scales_sorted else 0) | (2 if balanced else 0), stream_ptr(A.device),
         )
     )
 
@@ -854,7 +855,7 @@ def moe_slot_blocks(topk_ids: torch.Tensor, expert_offsets: torch.Tensor, proble
 
 def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorted_token_ids, expert_ids,
                               num_tokens_post_padded, top_k: int, num_valid_tokens: int, act_dtype: torch.dtype,
-                              eps: float = 1e-10) -> None:
+                              eps: float = 1e-10, balanced: bool = False) -> None:
     """Grouped GEMM 1 of the fused MoE layer (256-slot blocks) with silu_and_mul and the group requantisation inside its
     write-out (include/fp8k.h: fp8k_moe_block_gemm_silu_quant).  A e4m3fn [rows, K]; B e4m3fn [E, 2 I, K] (gate rows,
     then up rows); A_scale_sorted float32 [len(sorted_token_ids), K/128] as moe_sort_scales returns it; B_scale float32
@@ -893,7 +894,7 @@ def moe_block_gemm_silu_quant(A, B, A_scale_sorted, B_scale, out_q, out_s, sorte
         sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(), cap, num_valid_tokens, top_k, E,
         N, K, A.stride(0), A_scale_sorted.stride(1) if kb > 1 else cap, B.stride(0), B.stride(1), B_scale.stride(0),
         B_scale.stride(1), B_scale.stride(2), out_q.stride(0), out_s.stride(1) if I // 128 > 1 else cap, float(eps),
-        dtype_code(act_dtype), stream_ptr(A.device)))
+        dtype_code(act_dtype), 1 if balanced else 0, stream_ptr(A.device)))
 
 
 def moe_fused_gate(
