@@ -178,14 +178,19 @@ def test_graph_capture_split_k_gemm_survives_workspace_growth(dev):
         torch.cuda.synchronize()
 
 
-def test_graph_capture_fused_moe_layer(dev):
+@pytest.mark.parametrize("T,E,topk", [(96, 16, 4), (900, 4, 4)])
+def test_graph_capture_fused_moe_layer(dev, monkeypatch, T, E, topk):
     """quant + grouped GEMMs + fused silu/requant + top-k sum of fused_experts_impl, and the dense linear, in one graph;
-    three replays with eager launches between them, each compared with the eager result."""
+    three replays with eager launches between them, each compared with the eager result.  The second case has 900 slots
+    per expert: several 256-slot blocks each, dealt out evenly (moe_balance_blocks) and walked; its result is also held
+    bit for bit against the layer on the aligner's own table."""
+    import sglang_amd.fused_moe as fm
     from sglang_amd.fp8_utils import w8a8_block_fp8_linear
-    from sglang_amd.fused_moe import fused_experts_impl
+    from sglang_amd.fused_moe import blocks_want_balancing, fused_experts_impl, get_default_config
 
     rng = np.random.default_rng(7)
-    T, E, H, I, topk = 96, 16, 1024, 512, 4
+    H, I = 1024, 512
+    assert blocks_want_balancing(get_default_config(T, E, topk), T * topk, E) == (T == 900)
     x = O.make_activation(T, H, 7)
     w13q = np.empty((E, 2 * I, H), np.uint8); w13s = np.empty((E, 2 * I // 128, H // 128), np.float32)
     w2q = np.empty((E, H, I), np.uint8); w2s = np.empty((E, H // 128, I // 128), np.float32)
@@ -208,7 +213,18 @@ def test_graph_capture_fused_moe_layer(dev):
     eager_h, eager_y = layer()
     torch.cuda.synchronize()
     ref = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 2.5)
-    assert _rel_err(eager_h.float().cpu().numpy(), ref) <= REL_TOL
+    # The 900-token input holds a row with an outlier (largest entry 280 times the row's median).  In the oracle itself a
+    # 0.2 % change of that row's GEMM 1 result moves some thirty fp8 codes and a few scales of the second quantisation per
+    # expert and the expert's output by up to 1.7 % of its largest value, so last-bit differences in the 16-bit GEMM 1
+    # result show: the row's sums over four experts differ from the oracle's by up to 1.13e-2 of the output's largest
+    # value, the same on every table form and block size (measured); all but one other row stay within 5e-3.
+    assert _rel_err(eager_h.float().cpu().numpy(), ref) <= (2 * REL_TOL if T == 900 else REL_TOL)
+    if T == 900:
+        with monkeypatch.context() as m:
+            m.setattr(fm, "blocks_want_balancing", lambda *a, **k: False)
+            plain_h = fused_experts_impl(*args, **kw)
+        torch.cuda.synchronize()
+        assert torch.equal(plain_h, eager_h)
 
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
