@@ -365,6 +365,17 @@ int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t
                       void* stream);
 
 /*
+ * out[r, c] = gelu(x[r, c]) * x[r, d + c] for c < d with the erf form of gelu, x * 0.5 * (1 + erf(x / sqrt 2)), in
+ * float32; roundings, shapes and alignment as fp8k_silu_and_mul.
+ * Replaces torch.ops.sgl_kernel.gelu_and_mul
+ *   (sgl-kernel/python/sgl_kernel/elementwise.py:202-214, sgl-kernel/csrc/elementwise/activation.cu:62-67,129-149);
+ *   the activation="gelu" branch of fused_experts_impl calls it
+ *   (python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:561-565).
+ */
+int fp8k_gelu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
+                      void* stream);
+
+/*
  * out[t, :] = scale * sum_k x[t, k, :], float32 accumulation in ascending k, one rounding.
  * Replaces torch.ops.sgl_kernel.moe_sum_reduce
  *   (sgl-kernel/python/sgl_kernel/moe.py:83-92, sgl-kernel/csrc/moe/moe_sum_reduce.cu:56-113,227-).

@@ -398,6 +398,21 @@ def silu_and_mul(x):
     return to_bf16((silu * u).astype(np.float32))
 
 
+def gelu_and_mul(x):
+    """Reference: sgl-kernel/csrc/elementwise/activation.cu:62-67,129-149 (bf16: v * (0.5 * (1 + erf(v / sqrt 2))) in
+    f32 operation by operation, round to bf16, multiply, round to bf16).  x float32-of-bf16 [..., 2d] -> [..., d].
+    erf is taken in float64 and rounded once (a correctly rounded erff; device libraries are within a few ulp of it)."""
+    from scipy.special import erf
+
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    d = x.shape[-1] // 2
+    g, u = x[..., :d], x[..., d:]
+    t = (g * np.float32(0.70710678118654752440)).astype(np.float32)
+    cdf = (np.float32(0.5) * (np.float32(1) + erf(t.astype(np.float64)).astype(np.float32))).astype(np.float32)
+    gelu = to_bf16((g * cdf).astype(np.float32))
+    return to_bf16((gelu * u).astype(np.float32))
+
+
 def silu_mul_per_token_group_quant_fp8(x, group_size=128, eps=1e-10, scale_ue8m0=False):
     """Reference: sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:336-341 (FUSE_SILU_AND_MUL: the value that
     is quantised is T(T(silu(gate))) * up in the input type T) - i.e. silu_and_mul followed by the group quant.
@@ -502,13 +517,13 @@ def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, num_fused_shared
 
 
 def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scaling_factor=1.0, block=(128, 128),
-                        apply_router_weight_on_input=False):
+                        apply_router_weight_on_input=False, activation="silu"):
     """Reference: fused_experts_impl, python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:498-639
     (sequence) and torch_w8a8_block_fp8_moe, python/sglang/test/test_block_fp8.py:418-447 (math).
 
     x bf16 values [T,H]; w13q uint8 [E,2I,H]; w2q uint8 [E,H,I]; scales per 128x128 block.
-    quant(x) -> GEMM1 -> silu_and_mul -> quant -> GEMM2 * topk_weight (f32, then bf16) ->
-    sum over k in f32 * routed_scaling_factor -> bf16.
+    quant(x) -> GEMM1 -> silu_and_mul (gelu_and_mul with activation="gelu", fused_moe.py:547-565) -> quant ->
+    GEMM2 * topk_weight (f32, then bf16) -> sum over k in f32 * routed_scaling_factor -> bf16.
     apply_router_weight_on_input (fused_moe.py:533,597; the kernel multiplies the float accumulator before the output
     cast, fused_moe_triton_kernels.py MUL_ROUTED_WEIGHT): the weight multiplies the result of GEMM 1 instead.
     """
@@ -526,7 +541,7 @@ def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scalin
             h1 = to_bf16((w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "f32") * wk).astype(np.float32))
         else:
             h1 = w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "bf16")
-        act = silu_and_mul(h1)
+        act = {"silu": silu_and_mul, "gelu": gelu_and_mul}[activation](h1)
         aq, as_ = per_token_group_quant_fp8(act, block[1])
         h2 = w8a8_block_fp8_matmul(aq, w2q[e], as_, w2s[e], block, "f32")
         inter[t_idx, k_idx] = to_bf16(h2 if apply_router_weight_on_input else (h2 * wk).astype(np.float32))

@@ -119,6 +119,10 @@ __device__ __forceinline__ float silu_f32(float v) {
   return v * (__builtin_amdgcn_rcpf((1.0f + e) * 0x1p-32f) * 0x1p-32f);
 }
 
+// gelu in float32, the reference's expression term for term: v * (0.5 * (1 + erf(v / sqrt 2)))
+// (sgl-kernel/csrc/elementwise/activation.cu:62-67), erf from the device math library
+__device__ __forceinline__ float gelu_f32(float v) { return v * (0.5f * (1.0f + erff(v * 0.70710678118654752440f))); }
+
 template <int DT>
 __device__ __forceinline__ float round_to(float v) {
   if (DT == FP8K_BF16) return __uint_as_float(f32_to_bf16_bits(v) << 16);

@@ -164,7 +164,7 @@ __global__ __launch_bounds__(kAlignThreads) void moe_align_kernel(const IdT* __r
 }
 
 // ------------------------------------------------------------------------------------------------
-// silu_and_mul: out[r, c] = T( T(silu_f32(x[r, c])) * x[r, d + c] ), T = bf16 / f16 (two roundings, as
+// silu_and_mul / gelu_and_mul: out[r, c] = T( T(act(x[r, c])) * x[r, d + c] ), T = bf16 / f16 (two roundings, as
 // the reference kernel computes Activation(x) * y on 16-bit values); float32 input has one rounding.
 // One lane handles 8 columns: two 16-byte loads, one 16-byte store.
 // ------------------------------------------------------------------------------------------------
@@ -202,9 +202,9 @@ __device__ __forceinline__ void store8(void* base, int64_t elem, const float (&a
   }
 }
 
-template <int DT>
-__global__ __launch_bounds__(256) void silu_and_mul_kernel(const void* __restrict__ x, void* __restrict__ out,
-                                                           int64_t rows, int d, int64_t ldx, int64_t ldo) {
+template <int DT, bool GELU>
+__global__ __launch_bounds__(256) void act_and_mul_kernel(const void* __restrict__ x, void* __restrict__ out,
+                                                          int64_t rows, int d, int64_t ldx, int64_t ldo) {
   const int chunks = d / 8;
   const int64_t total = rows * chunks;
   const int64_t stride = (int64_t)gridDim.x * 256;
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(const void* __restric
     load8<DT>(x, r * ldx + c, g);
     load8<DT>(x, r * ldx + d + c, u);
 #pragma unroll
-    for (int k = 0; k < 8; ++k) o[k] = round_to<DT>(silu_f32(g[k])) * u[k];
+    for (int k = 0; k < 8; ++k) o[k] = round_to<DT>(GELU ? gelu_f32(g[k]) : silu_f32(g[k])) * u[k];
     store8<DT>(out, r * ldo + c, o);
   }
 }
@@ -617,24 +617,35 @@ extern "C" int fp8k_moe_block_gemm_silu_quant(const void* A, const void* B, cons
   return check_launch(op);
 }
 
-extern "C" int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
-                                 void* stream) {
+template <bool GELU>
+static int act_and_mul_impl(const char* op, const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
+                            void* stream) {
   clear_error();
-  FP8K_REQUIRE(rows >= 0 && d >= 0, "silu_and_mul: negative shape");
-  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "silu_and_mul: bad dtype %d", dtype);
-  FP8K_REQUIRE(d % 8 == 0 && d <= 0x7fffffffLL, "silu_and_mul: the output width (%lld) must be a multiple of 8", (long long)d);
-  FP8K_REQUIRE(ldx >= 2 * d && ldo >= d && ldx % 8 == 0 && ldo % 8 == 0, "silu_and_mul: bad row strides");
+  FP8K_REQUIRE(rows >= 0 && d >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "%s: bad dtype %d", op, dtype);
+  FP8K_REQUIRE(d % 8 == 0 && d <= 0x7fffffffLL, "%s: the output width (%lld) must be a multiple of 8", op, (long long)d);
+  FP8K_REQUIRE(ldx >= 2 * d && ldo >= d && ldx % 8 == 0 && ldo % 8 == 0, "%s: bad row strides", op);
   if (rows == 0 || d == 0) return FP8K_OK;
-  FP8K_REQUIRE(x && out, "silu_and_mul: null pointer");
-  FP8K_REQUIRE(aligned(x, 16) && aligned(out, 16), "silu_and_mul: The pointers must be multiple of 16 bytes.");
+  FP8K_REQUIRE(x && out, "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(x, 16) && aligned(out, 16), "%s: The pointers must be multiple of 16 bytes.", op);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid(stream_grid(rows * (d / 8))), block(256);
   switch (dtype) {
-    case FP8K_BF16: hipLaunchKernelGGL(silu_and_mul_kernel<FP8K_BF16>, grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
-    case FP8K_F16: hipLaunchKernelGGL(silu_and_mul_kernel<FP8K_F16>, grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
-    default: hipLaunchKernelGGL(silu_and_mul_kernel<FP8K_F32>, grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
+    case FP8K_BF16: hipLaunchKernelGGL((act_and_mul_kernel<FP8K_BF16, GELU>), grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
+    case FP8K_F16: hipLaunchKernelGGL((act_and_mul_kernel<FP8K_F16, GELU>), grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
+    default: hipLaunchKernelGGL((act_and_mul_kernel<FP8K_F32, GELU>), grid, block, 0, st, x, out, rows, (int)d, ldx, ldo); break;
   }
-  return check_launch("silu_and_mul");
+  return check_launch(op);
+}
+
+extern "C" int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
+                                 void* stream) {
+  return act_and_mul_impl<false>("silu_and_mul", x, out, rows, d, ldx, ldo, dtype, stream);
+}
+
+extern "C" int fp8k_gelu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
+                                 void* stream) {
+  return act_and_mul_impl<true>("gelu_and_mul", x, out, rows, d, ldx, ldo, dtype, stream);
 }
 
 static int moe_sum_impl(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,

@@ -115,6 +115,13 @@ def _silu_and_mul_impl(input, out) -> None:
 
 
 _register("silu_and_mul(Tensor input, Tensor(a!) out) -> ()", _silu_and_mul_impl, _none)
+
+
+def _gelu_and_mul_impl(input, out) -> None:
+    _k.gelu_and_mul(input, out)
+
+
+_register("gelu_and_mul(Tensor input, Tensor(a!) out) -> ()", _gelu_and_mul_impl, _none)
 _register("moe_sum_reduce(Tensor input, Tensor(a!) output, float routed_scaling_factor) -> ()", _k.moe_sum_reduce, _none)
 
 
@@ -245,6 +252,13 @@ def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
     if out is None:
         out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
     _ops.silu_and_mul(input, out)
+    return out
+
+
+def gelu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if out is None:
+        out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
+    _ops.gelu_and_mul(input, out)
     return out
 
 

@@ -8,6 +8,7 @@ fused_moe.py:498-639 of the reference:
     times the routed weight) -> sum over top-k (times routed_scaling_factor)
 
 silu_and_mul and the second quant are one kernel; with 256-slot blocks they run inside the write-out of the first GEMM.
+activation="gelu" runs gelu_and_mul and the quant as two kernels at every block size.
 
 Every stage is a call into libfp8k.so; intermediates are torch tensors on the current stream.
 """
@@ -176,10 +177,17 @@ def fused_experts_impl(
     (-1 = expert on another rank, contributes zero)."""
     if not use_fp8_w8a8 or block_shape is None:
         raise RuntimeError("fused_experts_impl: only use_fp8_w8a8=True with block_shape=[128, 128] is built on this path")
-    if activation != "silu" or not is_gated or gemm1_alpha is not None or gemm1_limit is not None:
-        raise RuntimeError("fused_experts_impl: only the gated silu activation is built on this path")
-    if b1 is not None or b2 is not None or a1_scale is not None or a2_scale is not None:
-        raise RuntimeError("fused_experts_impl: biases and static activation scales are not built on this path")
+    if activation not in ("silu", "gelu") or not is_gated:
+        raise RuntimeError("fused_experts_impl: only the gated silu and gelu activations are built on this path")
+    if activation == "gelu":
+        assert gemm1_alpha is None, "gemm1_alpha is not supported for gelu"
+        assert gemm1_limit is None, "gemm1_limit is not supported for gelu"
+    if gemm1_alpha is not None or gemm1_limit is not None:
+        raise RuntimeError("fused_experts_impl: swiglu with alpha and limit is not built on this path")
+    if b1 is not None or b2 is not None:
+        raise RuntimeError("fused_experts_impl: biases are not built on this path")
+    # a1_scale / a2_scale: with a block_shape the reference quantises the activations per token group whatever scale
+    # it is handed (fused_moe_triton_kernels.py:619-637 overwrites A_scale), so they have no effect here either
     assert hidden_states.shape[1] == w1.shape[2], "Hidden size mismatch"
     assert topk_weights.shape == topk_ids.shape, "topk shape mismatch"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
@@ -228,7 +236,7 @@ def fused_experts_impl(
                                                        config["BLOCK_SIZE_M"], tokens * topk, E)
         # apply_router_weight_on_input (fused_moe.py:533,597 of the reference): the routed weight multiplies the result of
         # GEMM 1 instead of GEMM 2; the fused write-out has no such factor, so that form keeps the three steps
-        if gemm1_fuses_activation(config, N) and not apply_router_weight_on_input:
+        if gemm1_fuses_activation(config, N) and not apply_router_weight_on_input and activation == "silu":
             slots = tokens * topk
             a1_q, a1_s = sglang_per_token_group_quant_fp8(curr, block_shape[1])
             a1_s = _ops.moe_sort_scales(a1_s, sorted_token_ids, num_tokens_post_padded, topk, slots)
@@ -245,10 +253,16 @@ def fused_experts_impl(
             curr, w1, None, ic1, None, w1_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
             num_tokens_post_padded, apply_router_weight_on_input, topk, config, use_fp8_w8a8=True, block_shape=block_shape,
         )
-        # silu_and_mul fused into the requantisation (same bytes as silu_and_mul + group quant, one pass less
-        # over the [tokens*topk, N] intermediate)
-        a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] < 64,
-                                                      fuse_silu_and_mul=True)
+        if activation == "gelu":
+            # fused_moe.py:561-565 of the reference: gelu_and_mul, then the group quant at the head of GEMM 2
+            ic2 = torch.empty((tokens * topk, N // 2), device=dev, dtype=dt)
+            _ops.gelu_and_mul(ic1, ic2)
+            a2_q, a2_s = sglang_per_token_group_quant_fp8(ic2, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] < 64)
+        else:
+            # silu_and_mul fused into the requantisation (same bytes as silu_and_mul + group quant, one pass less
+            # over the [tokens*topk, N] intermediate)
+            a2_q, a2_s = sglang_per_token_group_quant_fp8(ic1, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] < 64,
+                                                          fuse_silu_and_mul=True)
         invoke_fused_moe_kernel(
             a2_q, w2, None, ic3, a2_s, w2_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
             num_tokens_post_padded, not apply_router_weight_on_input, 1, config, use_fp8_w8a8=True, block_shape=block_shape,

@@ -557,8 +557,7 @@ def moe_align_block_size(
     )
 
 
-def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """Reference: sgl-kernel/python/sgl_kernel/elementwise.py:172-184."""
+def _act_and_mul(name: str, fn, input: torch.Tensor, out: Optional[torch.Tensor]) -> torch.Tensor:
     if input.shape[-1] * input.dtype.itemsize % 16 != 0:
         raise ValueError("The pointers must be multiple of 16 bytes.")
     if out is not None:
@@ -569,14 +568,23 @@ def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
         out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
     require_cuda(input, out)
     if out.dtype != input.dtype:
-        raise RuntimeError("silu_and_mul: out must have the dtype of input")
+        raise RuntimeError("%s: out must have the dtype of input" % name)
     if not (input.is_contiguous() and out.is_contiguous()):
-        raise RuntimeError("silu_and_mul: input and out must be contiguous")
+        raise RuntimeError("%s: input and out must be contiguous" % name)
     d = out.shape[-1]
     rows = out.numel() // d if d else 0
-    check(lib.fp8k_silu_and_mul(input.data_ptr(), out.data_ptr(), rows, d, 2 * d, d, dtype_code(input.dtype),
-                                stream_ptr(input.device)))
+    check(fn(input.data_ptr(), out.data_ptr(), rows, d, 2 * d, d, dtype_code(input.dtype), stream_ptr(input.device)))
     return out
+
+
+def silu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Reference: sgl-kernel/python/sgl_kernel/elementwise.py:172-184."""
+    return _act_and_mul("silu_and_mul", lib.fp8k_silu_and_mul, input, out)
+
+
+def gelu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Reference: sgl-kernel/python/sgl_kernel/elementwise.py:202-214 (the erf form of gelu)."""
+    return _act_and_mul("gelu_and_mul", lib.fp8k_gelu_and_mul, input, out)
 
 
 def moe_sum_reduce(input_tensor: torch.Tensor, output_tensor: torch.Tensor, routed_scaling_factor: float = 0) -> None:

@@ -145,6 +145,58 @@ def test_silu_and_mul_other_dtypes_and_errors(dev):
     assert silu_and_mul(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16)).shape == (0, 32)
 
 
+@pytest.mark.parametrize("rows,d", [(1, 2048), (37, 256), (32768, 2048)])
+def test_gelu_and_mul(dev, rows, d):
+    """gelu_and_mul (erf form) against the oracle and against the library routine on the device.  The device erf and a
+    correctly rounded one differ by a few float32 ulp: that can move a result across a bf16 tie (one bf16 ulp, carried
+    through the product: 2^-6 relative), and for gates below -3 it is magnified by the cancellation in 1 + erf - an
+    absolute error of a few 2^-24 in a sum of 1e-3 and less, |gate up| 2^-20 in the result."""
+    from sglang_amd.sgl_kernel import gelu_and_mul
+
+    rng = np.random.default_rng(rows)
+    x = O.to_bf16(rng.standard_normal((rows, 2 * d)).astype(np.float32) * 3)
+    out = gelu_and_mul(bf16_tensor(x, dev))
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    ref = O.gelu_and_mul(x)
+    gate, up = x[:, :d], x[:, d:]
+    tol = np.abs(ref) * 2.0**-6 + np.abs(gate * up) * 2.0**-20 + 1e-30
+    assert (np.abs(got - ref) <= tol).all()
+    assert (got != ref)[gate > -3].mean() < 2e-3
+    xt = bf16_tensor(x, dev)
+    lib_ref = (torch.nn.functional.gelu(xt[:, :d].float()).to(torch.bfloat16) * xt[:, d:]).float().cpu().numpy()
+    assert (np.abs(got - lib_ref) <= np.abs(lib_ref) * 2.0**-6 + np.abs(gate * up) * 2.0**-20 + 1e-30).all()
+    # not the other activations
+    assert not np.allclose(got, O.silu_and_mul(x), rtol=2e-2)
+
+
+def test_gelu_and_mul_other_dtypes_and_errors(dev):
+    from sglang_amd.sgl_kernel import gelu_and_mul
+
+    x = torch.randn(9, 64, device=dev)
+    ref = torch.nn.functional.gelu(x[:, :32]) * x[:, 32:]
+    torch.testing.assert_close(gelu_and_mul(x), ref, rtol=1e-5, atol=1e-6)
+    xh = x.half()
+    refh = torch.nn.functional.gelu(xh[:, :32].float()).half() * xh[:, 32:]
+    torch.testing.assert_close(gelu_and_mul(xh), refh, rtol=2e-3, atol=1e-6)
+    out = torch.empty(9, 32, device=dev)
+    assert gelu_and_mul(x, out) is out
+    torch.testing.assert_close(out, ref, rtol=1e-5, atol=1e-6)
+    # the ends of the range: v for large v (no overflow in v * (0.5 * (1 + erf))), -0 for large negative v, NaN kept
+    edge = torch.tensor([0.0, -0.0, 1e-30, -1e-30, 6.0, -6.0, 20.0, -20.0, 1e4, -1e4, 3e38, -3e38, float("inf"), float("nan"),
+                         1.0, -1.0], device=dev)
+    xe = torch.cat([edge, torch.ones_like(edge)]).reshape(1, -1)
+    got = gelu_and_mul(xe)[0]
+    want = torch.tensor([0.0, -0.0, 5e-31, -5e-31, 6.0, -0.0, 20.0, -0.0, 1e4, -0.0, 3e38, -0.0, float("inf"), float("nan"),
+                         0.8413447, -0.1586553], device=dev)
+    torch.testing.assert_close(got, want, rtol=1e-5, atol=1e-8, equal_nan=True)
+    with pytest.raises(ValueError, match="multiple of 16 bytes"):
+        gelu_and_mul(torch.zeros(3, 12, device=dev, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="dtype of input"):
+        gelu_and_mul(torch.zeros(3, 16, device=dev, dtype=torch.bfloat16), torch.zeros(3, 8, device=dev))
+    assert gelu_and_mul(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16)).shape == (0, 32)
+
+
 @pytest.mark.parametrize("T,topk,H,scale", [(1, 8, 7168, 2.5), (19, 8, 128, 1.0), (4096, 8, 7168, 2.5), (5, 1, 64, 0.5)])
 def test_moe_sum_reduce_exact(dev, T, topk, H, scale):
     from sglang_amd.sgl_kernel import moe_sum_reduce
@@ -438,6 +490,38 @@ def test_fused_experts_router_weight_on_input(dev, T, E, H, I):
     )
     torch.cuda.synchronize()
     assert _rel_err(out.float().cpu().numpy(), ref) <= REL_TOL
+
+
+@pytest.mark.parametrize("T,E,H,I,topk", [(40, 8, 512, 256, 2), (1100, 4, 256, 128, 2), (300, 32, 1024, 512, 8)])
+def test_fused_experts_gelu_and_ignored_activation_scales(dev, T, E, H, I, topk):
+    """activation="gelu" (fused_moe.py:561-565 of the reference) at block sizes 16, 256 (where silu would take the fused
+    write-out of GEMM 1) and 32; a1_scale / a2_scale change nothing on the block-quantised path, as in the reference
+    (fused_moe_triton_kernels.py:619-637 replaces the scale it is handed by the per-token-group one)."""
+    from sglang_amd.fused_moe import fused_experts_impl
+
+    rng = np.random.default_rng(T + E)
+    x, w13q, w13s, w2q, w2s, tw, ids = _moe_problem(rng, T, E, H, I, topk, False)
+    ref = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 2.5, activation="gelu")
+    args = (bf16_tensor(x, dev), fp8_tensor(w13q, dev), fp8_tensor(w2q, dev), torch.from_numpy(tw).to(dev),
+            torch.from_numpy(ids).to(dev))
+    kw = dict(use_fp8_w8a8=True, w1_scale=torch.from_numpy(w13s).to(dev), w2_scale=torch.from_numpy(w2s).to(dev),
+              block_shape=[128, 128], routed_scaling_factor=2.5)
+    out = fused_experts_impl(*args, activation="gelu", **kw)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert _rel_err(got, ref) <= REL_TOL
+    assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.02
+    silu = fused_experts_impl(*args, **kw)
+    assert _rel_err(silu.float().cpu().numpy(), ref) > 3 * REL_TOL      # the two activations are told apart
+    one = torch.full((1,), 0.37, device=dev)
+    assert torch.equal(fused_experts_impl(*args, activation="gelu", a1_scale=one, a2_scale=one, **kw), out)
+    assert torch.equal(fused_experts_impl(*args, a1_scale=one, a2_scale=one, **kw), silu)
+    with pytest.raises(AssertionError, match="gemm1_alpha is not supported for gelu"):
+        fused_experts_impl(*args, activation="gelu", gemm1_alpha=1.7, gemm1_limit=7.0, **kw)
+    with pytest.raises(RuntimeError, match="alpha and limit"):
+        fused_experts_impl(*args, gemm1_alpha=1.7, gemm1_limit=7.0, **kw)
+    with pytest.raises(RuntimeError, match="gated silu and gelu"):
+        fused_experts_impl(*args, activation="relu2", is_gated=False, **kw)
 
 
 def test_fused_experts_with_absent_experts_and_no_combine(dev):

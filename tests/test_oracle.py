@@ -324,6 +324,52 @@ def test_silu_and_mul_and_sum_reduce_against_torch_bf16():
     assert np.array_equal(O.moe_sum_reduce(y, 2.5), ref2)
 
 
+def test_gelu_and_mul_against_torch_and_the_identities_of_the_erf_form():
+    """gelu_and_mul on every finite bf16 gate value: against torch's library gelu (erf form) with the same two roundings
+    and against what the definition fixes: gelu(v) - gelu(-v) = v (the two normal probabilities sum to one), gelu(v) = v
+    for v >= 6 and -0 <= gelu(v) for v <= -6 in bf16, gelu(0) = 0.  The tanh approximation and x * sigmoid(1.702 x),
+    the forms a mistaken restatement would take, fail the first check.
+    Where the two may differ: torch's float32 erf and a correctly rounded one can differ in the last float32 bit, which
+    shows where the product sits on a bf16 tie and, magnified, in 1 + erf for v < -4 (the sum cancels: an error of
+    2^-24 in it is |v| 2^-25 in a result of 1e-5 and less); above 1.7e38 torch's order of the products overflows where
+    the reference's, v * (0.5 * (1 + erf)), does not (activation.cu:66)."""
+    bits = np.arange(1 << 16, dtype=np.uint32)
+    g = (bits << 16).view(np.float32)
+    g = g[np.isfinite(g)]
+    one = np.ones_like(g)
+    got = O.gelu_and_mul(np.stack([g, one], axis=-1).reshape(-1, 2))[:, 0]
+    ref = torch.nn.functional.gelu(torch.from_numpy(g)).bfloat16().float().numpy()
+    huge = np.abs(g) > 1.7e38
+    assert np.array_equal(got[huge & (g > 0)], g[huge & (g > 0)]) and (got[huge & (g < 0)] == 0).all()
+    got, ref, g = got[~huge], ref[~huge], g[~huge]
+    assert (got == ref).mean() > 0.9995, (got == ref).mean()
+    assert (np.abs(got - ref) <= np.maximum(np.abs(ref) * 2.0**-7, np.abs(g) * 2.0**-22)).all()
+    tanh_form = torch.nn.functional.gelu(torch.from_numpy(g), approximate="tanh").bfloat16().float().numpy()
+    quick = (torch.from_numpy(g) * torch.sigmoid(1.702 * torch.from_numpy(g))).bfloat16().float().numpy()
+    mid = (np.abs(g) > 0.25) & (np.abs(g) < 3)     # beyond, every form is v / 2, v or next to 0 in bf16
+    assert (got[mid] == ref[mid]).all()
+    assert (got[mid] == tanh_form[mid]).mean() < 0.9 and (got[mid] == quick[mid]).mean() < 0.5
+    big = g >= 6
+    assert np.array_equal(got[big], g[big])
+    assert (got[g <= -6] <= 0).all() and (got[g <= -6] > -1e-7).all()
+    assert got[g == 0].tolist() == [0.0, 0.0]
+    # gelu(v) - gelu(-v) = v: both sides in bf16, so within an ulp of each term
+    pos = g[(g > 2.0**-100) & (g < 6)]
+    both = O.gelu_and_mul(np.stack([np.concatenate([pos, -pos]), np.ones(2 * pos.size, np.float32)], axis=-1))[:, 0]
+    diff = both[: pos.size] - both[pos.size:]
+    assert (np.abs(diff - pos) <= 2.0**-7 * pos).all()
+    # the second factor and its rounding
+    rng = np.random.default_rng(12)
+    x = O.to_bf16(rng.standard_normal((37, 512)).astype(np.float32) * 3)
+    xt = torch.from_numpy(x).bfloat16()
+    ref2 = (torch.nn.functional.gelu(xt[..., :256].float()).to(torch.bfloat16) * xt[..., 256:]).float().numpy()
+    got2 = O.gelu_and_mul(x)
+    gate, up = x[:, :256], x[:, 256:]
+    assert np.array_equal(got2[gate > -3], ref2[gate > -3])
+    assert (np.abs(got2 - ref2) <= 2.0**-6 * np.abs(ref2) + np.abs(gate * up) * 2.0**-21).all()
+    assert not np.allclose(got2, O.silu_and_mul(x), rtol=2e-2)
+
+
 def test_grouped_topk_properties():
     """python/sglang/srt/layers/moe/topk.py:665-738 with the DeepSeek-V3 tuple (256 experts, 8 groups, top-4 groups, top-8)."""
     rng = np.random.default_rng(11)
@@ -452,8 +498,9 @@ def test_block_fp8_linear_bias_branch_and_nd_input():
     assert np.abs(y - plain.reshape(12, 256)).max() <= 2.0**-7 * np.abs(y).max()
 
 
-@pytest.mark.parametrize("T,E,H,I,topk,rsf", [(20, 4, 256, 128, 2, 2.5), (33, 8, 384, 256, 3, 1.0)])
-def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf):
+@pytest.mark.parametrize("T,E,H,I,topk,rsf,activation", [(20, 4, 256, 128, 2, 2.5, "silu"), (33, 8, 384, 256, 3, 1.0, "silu"),
+                                                         (20, 4, 256, 128, 2, 2.5, "gelu")])
+def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf, activation):
     """fused_moe_block_fp8 against the same layer spelled with torch library ops, expert by expert as
     torch_w8a8_block_fp8_moe does (python/sglang/test/test_block_fp8.py:418-447), with the roundings of the fused
     path (fused_moe.py:498-639): GEMM1 -> bf16, silu -> bf16 -> times up -> bf16, requant, GEMM2 times the routed
@@ -470,8 +517,10 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf):
     ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
     ids[rng.random(ids.shape) < 0.1] = -1          # experts on another rank contribute nothing
     tw = rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32)
-    got = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf)
-    got_in = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, apply_router_weight_on_input=True)
+    got = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, activation=activation)
+    got_in = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, apply_router_weight_on_input=True,
+                                   activation=activation)
+    act_fn = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu}[activation]
 
     xt = torch.from_numpy(x).bfloat16()
     xq, xs = _t_group_quant(xt)
@@ -488,7 +537,7 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf):
             wk = t_w[tok, slot].unsqueeze(1)
             h1 = _t_block_matmul_f64(xq[tok].float(), xs[tok], W1, S1).to(torch.float32)
             h1 = (h1 * wk if weight_on_input else h1).bfloat16()
-            act = torch.nn.functional.silu(h1[:, :I].float()).bfloat16() * h1[:, I:]
+            act = act_fn(h1[:, :I].float()).bfloat16() * h1[:, I:]
             aq, a_s = _t_group_quant(act)
             h2 = _t_block_matmul_f64(aq.float(), a_s, W2, S2).to(torch.float32)
             per_slot[tok, slot] = (h2 if weight_on_input else h2 * wk).bfloat16()
@@ -510,9 +559,13 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf):
     dead = (ids == -1).all(axis=1)
     assert (got[dead] == 0).all()
     # what a plausible mistake would change: no routed weight, weight applied after the sum, no scaling factor
-    assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, np.ones_like(tw), ids, rsf), rtol=1e-2)
+    assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, np.ones_like(tw), ids, rsf,
+                                                      activation=activation), rtol=1e-2)
     if rsf != 1.0:
-        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0), rtol=1e-2)
+        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0, activation=activation),
+                               rtol=1e-2)
+    if activation != "silu":
+        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf), rtol=1e-2)
 
 
 def _t_fused_gate_bf16(x, bias, G, topk_group, topk):
