@@ -29,6 +29,9 @@ typedef enum {
 
 typedef enum { FP8K_F32 = 0, FP8K_F16 = 1, FP8K_BF16 = 2 } fp8k_dtype;
 
+/* activation of fp8k_activation */
+typedef enum { FP8K_ACT_SILU = 0, FP8K_ACT_GELU = 1, FP8K_ACT_RELU2 = 2 } fp8k_activation_kind;
+
 typedef enum {
   FP8K_SCALE_F32 = 0,         /* one float per group, addressed by (stride_m, stride_g) */
   FP8K_SCALE_UE8M0_PACKED = 1, /* int32 words, 4 exponent bytes each, word (g/4) byte (g%4) */
@@ -374,6 +377,17 @@ int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t
  */
 int fp8k_gelu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
                       void* stream);
+
+/*
+ * out[r, c] = act(x[r, c]) for c < d: the activation of experts without a gate projection, in float32 with one rounding
+ * to the element type.  kind: FP8K_ACT_SILU, FP8K_ACT_GELU (erf form), FP8K_ACT_RELU2 (relu(x)^2).
+ * Replaces the tensor-library calls of the ungated branch of fused_experts_impl - F.silu, F.gelu and
+ * torch.square(F.relu(.)) on the [tokens * topk, N] result of the first grouped GEMM
+ *   (python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:566-572).
+ * x [rows, d] (ldx elements between rows), out [rows, d] (ldo); d % 8 == 0; 16-byte aligned pointers.
+ */
+int fp8k_activation(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int kind, int dtype,
+                    void* stream);
 
 /*
  * out[t, :] = scale * sum_k x[t, k, :], float32 accumulation in ascending k, one rounding.

@@ -413,6 +413,28 @@ def gelu_and_mul(x):
     return to_bf16((gelu * u).astype(np.float32))
 
 
+def activation_only(x, kind):
+    """Reference: the ungated branch of fused_experts_impl, fused_moe.py:566-572 - F.silu, F.gelu (erf form),
+    torch.square(F.relu(.)) on a 16-bit tensor: the function in float32, one rounding to bf16.
+    x float32-of-bf16 -> same shape."""
+    from scipy.special import erf
+
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    if kind == "silu":
+        with np.errstate(over="ignore"):
+            y = x / (np.float32(1) + np.exp(-x).astype(np.float32))
+    elif kind == "gelu":
+        t = (x * np.float32(0.70710678118654752440)).astype(np.float32)
+        y = x * (np.float32(0.5) * (np.float32(1) + erf(t.astype(np.float64)).astype(np.float32))).astype(np.float32)
+    elif kind == "relu2":
+        r = np.maximum(x, np.float32(0))
+        with np.errstate(over="ignore"):
+            y = r * r
+    else:
+        raise ValueError(kind)
+    return to_bf16(y.astype(np.float32))
+
+
 def silu_mul_per_token_group_quant_fp8(x, group_size=128, eps=1e-10, scale_ue8m0=False):
     """Reference: sgl-kernel/csrc/gemm/per_token_group_quant_8bit_v2.cu:336-341 (FUSE_SILU_AND_MUL: the value that
     is quantised is T(T(silu(gate))) * up in the input type T) - i.e. silu_and_mul followed by the group quant.
@@ -517,12 +539,13 @@ def moe_fused_gate(x, bias, num_expert_group, topk_group, topk, num_fused_shared
 
 
 def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scaling_factor=1.0, block=(128, 128),
-                        apply_router_weight_on_input=False, activation="silu"):
+                        apply_router_weight_on_input=False, activation="silu", is_gated=True):
     """Reference: fused_experts_impl, python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:498-639
     (sequence) and torch_w8a8_block_fp8_moe, python/sglang/test/test_block_fp8.py:418-447 (math).
 
     x bf16 values [T,H]; w13q uint8 [E,2I,H]; w2q uint8 [E,H,I]; scales per 128x128 block.
-    quant(x) -> GEMM1 -> silu_and_mul (gelu_and_mul with activation="gelu", fused_moe.py:547-565) -> quant ->
+    quant(x) -> GEMM1 -> silu_and_mul (gelu_and_mul with activation="gelu", fused_moe.py:547-565; with is_gated=False
+    w13q is [E,I,H] and the activation - silu, gelu or relu2 - keeps the width, :566-572) -> quant ->
     GEMM2 * topk_weight (f32, then bf16) -> sum over k in f32 * routed_scaling_factor -> bf16.
     apply_router_weight_on_input (fused_moe.py:533,597; the kernel multiplies the float accumulator before the output
     cast, fused_moe_triton_kernels.py MUL_ROUTED_WEIGHT): the weight multiplies the result of GEMM 1 instead.
@@ -541,7 +564,7 @@ def fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, topk_w, topk_ids, routed_scalin
             h1 = to_bf16((w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "f32") * wk).astype(np.float32))
         else:
             h1 = w8a8_block_fp8_matmul(xq[t_idx], w13q[e], xs[t_idx], w13s[e], block, "bf16")
-        act = {"silu": silu_and_mul, "gelu": gelu_and_mul}[activation](h1)
+        act = {"silu": silu_and_mul, "gelu": gelu_and_mul}[activation](h1) if is_gated else activation_only(h1, activation)
         aq, as_ = per_token_group_quant_fp8(act, block[1])
         h2 = w8a8_block_fp8_matmul(aq, w2q[e], as_, w2s[e], block, "f32")
         inter[t_idx, k_idx] = to_bf16(h2 if apply_router_weight_on_input else (h2 * wk).astype(np.float32))

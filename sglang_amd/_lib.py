@@ -83,6 +83,7 @@ SIGNATURES = {
     "fp8k_moe_sort_scales": (_c_int, [_c_ptr] * 4 + [_c_i64] * 6 + [_c_ptr]),
     "fp8k_silu_and_mul": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr]),
     "fp8k_gelu_and_mul": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_ptr]),
+    "fp8k_activation": (_c_int, [_c_ptr, _c_ptr, _c_i64, _c_i64, _c_i64, _c_i64, _c_int, _c_int, _c_ptr]),
     "fp8k_moe_sum_reduce": (_c_int, [_c_ptr, _c_ptr] + [_c_i64] * 6 + [_c_f32, _c_int, _c_ptr]),
     "fp8k_moe_sum": (_c_int, [_c_ptr, _c_ptr] + [_c_i64] * 6 + [_c_int, _c_ptr]),
     "fp8k_moe_fused_gate": (

@@ -220,6 +220,29 @@ __global__ __launch_bounds__(256) void act_and_mul_kernel(const void* __restrict
   }
 }
 
+// activation without the second factor (the ungated experts of fused_experts_impl): out[r, c] = T(act(x[r, c])) with
+// act = silu, gelu (erf form) or relu(x)^2 in float32 and one rounding, as the tensor library's 16-bit ops round
+template <int DT, int KIND>
+__global__ __launch_bounds__(256) void act_only_kernel(const void* __restrict__ x, void* __restrict__ out, int64_t rows,
+                                                       int d, int64_t ldx, int64_t ldo) {
+  const int chunks = d / 8;
+  const int64_t total = rows * chunks;
+  const int64_t stride = (int64_t)gridDim.x * 256;
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / chunks;
+    const int c = (int)(i - r * chunks) * 8;
+    float g[8], o[8];
+    load8<DT>(x, r * ldx + c, g);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (KIND == FP8K_ACT_SILU) o[k] = silu_f32(g[k]);
+      else if (KIND == FP8K_ACT_GELU) o[k] = gelu_f32(g[k]);
+      else { const float t = g[k] > 0.f ? g[k] : (g[k] == g[k] ? 0.f : g[k]); o[k] = t * t; }  // NaN stays NaN, as relu keeps it
+    }
+    store8<DT>(out, r * ldo + c, o);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------
 // moe_sum_reduce: out[t, :] = T( scale * sum_k float(x[t, k, :]) ), k ascending, float32 accumulate
 // ------------------------------------------------------------------------------------------------
@@ -646,6 +669,37 @@ extern "C" int fp8k_silu_and_mul(const void* x, void* out, int64_t rows, int64_t
 extern "C" int fp8k_gelu_and_mul(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int dtype,
                                  void* stream) {
   return act_and_mul_impl<true>("gelu_and_mul", x, out, rows, d, ldx, ldo, dtype, stream);
+}
+
+template <int KIND>
+static void launch_act_only(dim3 grid, hipStream_t st, const void* x, void* out, int64_t rows, int d, int64_t ldx, int64_t ldo,
+                            int dtype) {
+  const dim3 block(256);
+  switch (dtype) {
+    case FP8K_BF16: hipLaunchKernelGGL((act_only_kernel<FP8K_BF16, KIND>), grid, block, 0, st, x, out, rows, d, ldx, ldo); break;
+    case FP8K_F16: hipLaunchKernelGGL((act_only_kernel<FP8K_F16, KIND>), grid, block, 0, st, x, out, rows, d, ldx, ldo); break;
+    default: hipLaunchKernelGGL((act_only_kernel<FP8K_F32, KIND>), grid, block, 0, st, x, out, rows, d, ldx, ldo); break;
+  }
+}
+
+extern "C" int fp8k_activation(const void* x, void* out, int64_t rows, int64_t d, int64_t ldx, int64_t ldo, int kind, int dtype,
+                               void* stream) {
+  clear_error();
+  const char* op = "activation";
+  FP8K_REQUIRE(rows >= 0 && d >= 0, "%s: negative shape", op);
+  FP8K_REQUIRE(kind == FP8K_ACT_SILU || kind == FP8K_ACT_GELU || kind == FP8K_ACT_RELU2, "%s: bad kind %d", op, kind);
+  FP8K_REQUIRE(dtype == FP8K_F32 || dtype == FP8K_F16 || dtype == FP8K_BF16, "%s: bad dtype %d", op, dtype);
+  FP8K_REQUIRE(d % 8 == 0 && d <= 0x7fffffffLL, "%s: the width (%lld) must be a multiple of 8", op, (long long)d);
+  FP8K_REQUIRE(ldx >= d && ldo >= d && ldx % 8 == 0 && ldo % 8 == 0, "%s: bad row strides", op);
+  if (rows == 0 || d == 0) return FP8K_OK;
+  FP8K_REQUIRE(x && out, "%s: null pointer", op);
+  FP8K_REQUIRE(aligned(x, 16) && aligned(out, 16), "%s: the pointers must be 16-byte aligned", op);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid(stream_grid(rows * (d / 8)));
+  if (kind == FP8K_ACT_SILU) launch_act_only<FP8K_ACT_SILU>(grid, st, x, out, rows, (int)d, ldx, ldo, dtype);
+  else if (kind == FP8K_ACT_GELU) launch_act_only<FP8K_ACT_GELU>(grid, st, x, out, rows, (int)d, ldx, ldo, dtype);
+  else launch_act_only<FP8K_ACT_RELU2>(grid, st, x, out, rows, (int)d, ldx, ldo, dtype);
+  return check_launch(op);
 }
 
 static int moe_sum_impl(const void* x, void* out, int64_t tokens, int64_t topk, int64_t hidden, int64_t stride_token,

@@ -122,6 +122,13 @@ def _gelu_and_mul_impl(input, out) -> None:
 
 
 _register("gelu_and_mul(Tensor input, Tensor(a!) out) -> ()", _gelu_and_mul_impl, _none)
+
+
+def _activation_impl(input, out, kind) -> None:
+    _k.activation(input, kind, out)
+
+
+_register("activation(Tensor input, Tensor(a!) out, str kind) -> ()", _activation_impl, _none)
 _register("moe_sum_reduce(Tensor input, Tensor(a!) output, float routed_scaling_factor) -> ()", _k.moe_sum_reduce, _none)
 
 
@@ -259,6 +266,13 @@ def gelu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
     if out is None:
         out = torch.empty(input.shape[:-1] + (input.shape[-1] // 2,), device=input.device, dtype=input.dtype)
     _ops.gelu_and_mul(input, out)
+    return out
+
+
+def activation(input: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    if out is None:
+        out = torch.empty_like(input)
+    _ops.activation(input, out, kind)
     return out
 
 

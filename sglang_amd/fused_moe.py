@@ -8,7 +8,8 @@ fused_moe.py:498-639 of the reference:
     times the routed weight) -> sum over top-k (times routed_scaling_factor)
 
 silu_and_mul and the second quant are one kernel; with 256-slot blocks they run inside the write-out of the first GEMM.
-activation="gelu" runs gelu_and_mul and the quant as two kernels at every block size.
+activation="gelu" runs gelu_and_mul and the quant as two kernels at every block size; experts without a gate projection
+(is_gated=False: silu, gelu, relu2) run the activation kernel and the quant.
 
 Every stage is a call into libfp8k.so; intermediates are torch tensors on the current stream.
 """
@@ -177,8 +178,8 @@ def fused_experts_impl(
     (-1 = expert on another rank, contributes zero)."""
     if not use_fp8_w8a8 or block_shape is None:
         raise RuntimeError("fused_experts_impl: only use_fp8_w8a8=True with block_shape=[128, 128] is built on this path")
-    if activation not in ("silu", "gelu") or not is_gated:
-        raise RuntimeError("fused_experts_impl: only the gated silu and gelu activations are built on this path")
+    if not ((is_gated and activation in ("silu", "gelu")) or (not is_gated and activation in ("silu", "gelu", "relu2"))):
+        raise ValueError(f"Unsupported activation: {activation=}, with {is_gated=}")
     if activation == "gelu":
         assert gemm1_alpha is None, "gemm1_alpha is not supported for gelu"
         assert gemm1_limit is None, "gemm1_limit is not supported for gelu"
@@ -236,7 +237,7 @@ def fused_experts_impl(
                                                        config["BLOCK_SIZE_M"], tokens * topk, E)
         # apply_router_weight_on_input (fused_moe.py:533,597 of the reference): the routed weight multiplies the result of
         # GEMM 1 instead of GEMM 2; the fused write-out has no such factor, so that form keeps the three steps
-        if gemm1_fuses_activation(config, N) and not apply_router_weight_on_input and activation == "silu":
+        if gemm1_fuses_activation(config, N) and not apply_router_weight_on_input and activation == "silu" and is_gated:
             slots = tokens * topk
             a1_q, a1_s = sglang_per_token_group_quant_fp8(curr, block_shape[1])
             a1_s = _ops.moe_sort_scales(a1_s, sorted_token_ids, num_tokens_post_padded, topk, slots)
@@ -253,7 +254,11 @@ def fused_experts_impl(
             curr, w1, None, ic1, None, w1_scale, None, curr_w, curr_ids, sorted_token_ids, expert_ids,
             num_tokens_post_padded, apply_router_weight_on_input, topk, config, use_fp8_w8a8=True, block_shape=block_shape,
         )
-        if activation == "gelu":
+        if not is_gated:
+            # fused_moe.py:566-572 of the reference: w1 is [E, N, H] without a gate half, the activation keeps the width
+            ic2 = _ops.activation(ic1, activation)
+            a2_q, a2_s = sglang_per_token_group_quant_fp8(ic2, block_shape[1], column_major_scales=config["BLOCK_SIZE_M"] < 64)
+        elif activation == "gelu":
             # fused_moe.py:561-565 of the reference: gelu_and_mul, then the group quant at the head of GEMM 2
             ic2 = torch.empty((tokens * topk, N // 2), device=dev, dtype=dt)
             _ops.gelu_and_mul(ic1, ic2)

@@ -587,6 +587,30 @@ def gelu_and_mul(input: torch.Tensor, out: Optional[torch.Tensor] = None) -> tor
     return _act_and_mul("gelu_and_mul", lib.fp8k_gelu_and_mul, input, out)
 
 
+ACTIVATION_KINDS = {"silu": 0, "gelu": 1, "relu2": 2}
+
+
+def activation(input: torch.Tensor, kind: str, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """out = act(input) elementwise: the activation of experts without a gate projection - F.silu, F.gelu (erf form) and
+    torch.square(F.relu(.)) in the reference (python/sglang/srt/layers/moe/fused_moe_triton/fused_moe.py:566-572)."""
+    if kind not in ACTIVATION_KINDS:
+        raise ValueError(f"Unsupported activation: {kind=}")
+    if input.shape[-1] * input.dtype.itemsize % 16 != 0:
+        raise ValueError("The pointers must be multiple of 16 bytes.")
+    if out is None:
+        out = torch.empty_like(input)
+    require_cuda(input, out)
+    if out.shape != input.shape or out.dtype != input.dtype:
+        raise RuntimeError("activation: out must have the shape and dtype of input")
+    if not (input.is_contiguous() and out.is_contiguous()):
+        raise RuntimeError("activation: input and out must be contiguous")
+    d = input.shape[-1]
+    rows = input.numel() // d if d else 0
+    check(lib.fp8k_activation(input.data_ptr(), out.data_ptr(), rows, d, d, d, ACTIVATION_KINDS[kind], dtype_code(input.dtype),
+                              stream_ptr(input.device)))
+    return out
+
+
 def moe_sum_reduce(input_tensor: torch.Tensor, output_tensor: torch.Tensor, routed_scaling_factor: float = 0) -> None:
     """Reference: sgl-kernel/python/sgl_kernel/moe.py:83-92; csrc/moe/moe_sum_reduce.cu:227-.
     input [tokens, topk, hidden] (hidden contiguous), output [tokens, hidden]."""

@@ -197,6 +197,54 @@ def test_gelu_and_mul_other_dtypes_and_errors(dev):
     assert gelu_and_mul(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16)).shape == (0, 32)
 
 
+@pytest.mark.parametrize("kind", ["silu", "gelu", "relu2"])
+def test_activation_without_gate(dev, kind):
+    """The activation of ungated experts against the oracle (bounds as for the gated kernels: one bf16 ulp where a
+    float32 result sits on a tie, and for gelu the cancellation in 1 + erf below -3) and against the tensor library's
+    op on the device; relu2 is exact."""
+    from sglang_amd.sgl_kernel import activation
+
+    rng = np.random.default_rng(len(kind))
+    x = O.to_bf16(rng.standard_normal((300, 512)).astype(np.float32) * 3)
+    xt = bf16_tensor(x, dev)
+    out = activation(xt, kind)
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    ref = O.activation_only(x, kind)
+    lib_ref = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu,
+               "relu2": lambda t: torch.square(torch.relu(t))}[kind](xt).float().cpu().numpy()
+    if kind == "relu2":
+        assert np.array_equal(got, ref) and np.array_equal(got, lib_ref)
+    else:
+        tol = np.abs(ref) * 2.0**-7 + (np.abs(x) * 2.0**-20 if kind == "gelu" else 0) + 1e-30
+        assert (np.abs(got - ref) <= tol).all() and (np.abs(got - lib_ref) <= tol).all()
+        assert (got != ref)[x > -3].mean() < 2e-3
+    # float32 and float16, an output tensor, the edges, the errors
+    xf = torch.randn(9, 64, device=dev)
+    want = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu2": lambda t: torch.square(torch.relu(t))}[kind]
+    torch.testing.assert_close(activation(xf, kind), want(xf), rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(activation(xf.half(), kind), want(xf.half().float()).half(), rtol=2e-3, atol=1e-6)
+    o = torch.empty_like(xf)
+    assert activation(xf, kind, o) is o
+    edge = torch.tensor([0.0, -0.0, 1e-30, -1e-30, 30.0, -30.0, 3e38, -3e38, float("inf"), float("-inf"), float("nan"), 1.0,
+                         -1.0, 0.5, -0.5, 100.0], device=dev).reshape(1, -1)
+    e = activation(edge, kind)[0]
+    if kind == "relu2":
+        torch.testing.assert_close(e, torch.square(torch.relu(edge[0])), rtol=0, atol=0, equal_nan=True)
+    elif kind == "silu":
+        torch.testing.assert_close(e, edge[0] / (1.0 + torch.exp(-edge[0])), rtol=1e-5, atol=1e-37, equal_nan=True)
+    else:
+        assert e[4] == 30.0 and e[5] == 0.0 and e[6] == 3e38 and e[7] == 0.0 and e[8] == float("inf") and torch.isnan(e[10])
+        torch.testing.assert_close(e[11:15], torch.tensor([0.8413447, -0.1586553, 0.3457312, -0.1542688], device=dev), rtol=1e-5, atol=1e-8)
+    with pytest.raises(ValueError, match="Unsupported activation"):
+        activation(xf, "tanh")
+    with pytest.raises(ValueError, match="multiple of 16 bytes"):
+        activation(torch.zeros(3, 12, device=dev, dtype=torch.bfloat16), kind)
+    with pytest.raises(RuntimeError, match="shape and dtype"):
+        activation(xf, kind, torch.empty(9, 32, device=dev))
+    assert activation(torch.zeros(0, 64, device=dev, dtype=torch.bfloat16), kind).shape == (0, 64)
+
+
 @pytest.mark.parametrize("T,topk,H,scale", [(1, 8, 7168, 2.5), (19, 8, 128, 1.0), (4096, 8, 7168, 2.5), (5, 1, 64, 0.5)])
 def test_moe_sum_reduce_exact(dev, T, topk, H, scale):
     from sglang_amd.sgl_kernel import moe_sum_reduce
@@ -520,8 +568,37 @@ def test_fused_experts_gelu_and_ignored_activation_scales(dev, T, E, H, I, topk)
         fused_experts_impl(*args, activation="gelu", gemm1_alpha=1.7, gemm1_limit=7.0, **kw)
     with pytest.raises(RuntimeError, match="alpha and limit"):
         fused_experts_impl(*args, gemm1_alpha=1.7, gemm1_limit=7.0, **kw)
-    with pytest.raises(RuntimeError, match="gated silu and gelu"):
-        fused_experts_impl(*args, activation="relu2", is_gated=False, **kw)
+    with pytest.raises(ValueError, match="Unsupported activation"):
+        fused_experts_impl(*args, activation="relu2", is_gated=True, **kw)
+    with pytest.raises(ValueError, match="Unsupported activation"):
+        fused_experts_impl(*args, activation="swish", **kw)
+
+
+@pytest.mark.parametrize("T,E,H,I,topk", [(40, 8, 512, 256, 2), (1100, 4, 256, 128, 2)])
+@pytest.mark.parametrize("kind", ["silu", "gelu", "relu2"])
+def test_fused_experts_without_gate(dev, T, E, H, I, topk, kind):
+    """is_gated=False (fused_moe.py:566-572 of the reference): w1 is [E, I, H], the activation keeps the width; block
+    sizes 16 and 256 (where the gated silu form would take the fused write-out of GEMM 1)."""
+    from sglang_amd.fused_moe import fused_experts_impl
+
+    rng = np.random.default_rng(T + E)
+    x, w13q, w13s, w2q, w2s, tw, ids = _moe_problem(rng, T, E, H, I, topk, False)
+    w1q, w1s = w13q[:, :I].copy(), w13s[:, : I // 128].copy()          # an [E, I, H] projection
+    ref = O.fused_moe_block_fp8(x, w1q, w1s, w2q, w2s, tw, ids, 1.5, activation=kind, is_gated=False)
+    out = fused_experts_impl(
+        bf16_tensor(x, dev), fp8_tensor(w1q, dev), fp8_tensor(w2q, dev), torch.from_numpy(tw).to(dev),
+        torch.from_numpy(ids).to(dev), use_fp8_w8a8=True, w1_scale=torch.from_numpy(w1s).to(dev),
+        w2_scale=torch.from_numpy(w2s).to(dev), block_shape=[128, 128], routed_scaling_factor=1.5, activation=kind,
+        is_gated=False,
+    )
+    torch.cuda.synchronize()
+    got = out.float().cpu().numpy()
+    assert out.shape == (T, H)
+    assert _rel_err(got, ref) <= REL_TOL
+    assert np.abs(got - ref).mean() / np.abs(ref).mean() < 0.02
+    others = [k for k in ("silu", "gelu", "relu2") if k != kind]
+    for k in others:
+        assert _rel_err(got, O.fused_moe_block_fp8(x, w1q, w1s, w2q, w2s, tw, ids, 1.5, activation=k, is_gated=False)) > 2 * REL_TOL
 
 
 def test_fused_experts_with_absent_experts_and_no_combine(dev):

@@ -370,6 +370,34 @@ def test_gelu_and_mul_against_torch_and_the_identities_of_the_erf_form():
     assert not np.allclose(got2, O.silu_and_mul(x), rtol=2e-2)
 
 
+def test_activation_only_against_torch_on_every_bf16_value():
+    """activation_only (the ungated experts' activation) against the tensor library's own ops on bf16 tensors, every finite
+    bf16 value: silu and relu2 bit for bit; gelu as in the gated test (last-bit differences of erf show on bf16 ties and,
+    magnified by the cancellation in 1 + erf, below -3; above 1.7e38 torch's product order overflows)."""
+    bits = np.arange(1 << 16, dtype=np.uint32)
+    g = (bits << 16).view(np.float32)
+    g = g[np.isfinite(g)]
+    t = torch.from_numpy(g).bfloat16()
+    silu = torch.nn.functional.silu(t).float().numpy()
+    assert np.array_equal(O.activation_only(g, "silu"), silu)
+    relu2 = torch.square(torch.nn.functional.relu(t)).float().numpy()
+    got = O.activation_only(g, "relu2")
+    assert np.array_equal(got, relu2) and (got[g < 0] == 0).all() and np.isinf(got[g > 2e19]).all()
+    gelu = torch.nn.functional.gelu(t).float().numpy()
+    got = O.activation_only(g, "gelu")
+    ok = (np.abs(g) < 1.7e38) & ((np.abs(g) > 2.0**-100) | (g == 0))   # torch's bf16 kernel flushes subnormal results
+    assert np.array_equal(got[ok & (g > -3)], gelu[ok & (g > -3)])
+    tiny = (np.abs(g) <= 2.0**-100) & (g != 0)
+    assert np.array_equal(got[tiny], O.to_bf16((g[tiny] * np.float32(0.5)).astype(np.float32)))   # gelu(v) = v / 2 there
+    assert (np.abs(got[ok] - gelu[ok]) <= np.maximum(np.abs(gelu[ok]) * 2.0**-7, np.abs(g[ok]) * 2.0**-22)).all()
+    # the gated forms with a second factor of one are the same functions
+    one = np.ones_like(g)
+    assert np.array_equal(O.silu_and_mul(np.stack([g, one], -1))[:, 0], O.activation_only(g, "silu"))
+    assert np.array_equal(O.gelu_and_mul(np.stack([g, one], -1))[:, 0], O.activation_only(g, "gelu"))
+    with pytest.raises(ValueError):
+        O.activation_only(g, "tanh")
+
+
 def test_grouped_topk_properties():
     """python/sglang/srt/layers/moe/topk.py:665-738 with the DeepSeek-V3 tuple (256 experts, 8 groups, top-4 groups, top-8)."""
     rng = np.random.default_rng(11)
@@ -499,7 +527,7 @@ def test_block_fp8_linear_bias_branch_and_nd_input():
 
 
 @pytest.mark.parametrize("T,E,H,I,topk,rsf,activation", [(20, 4, 256, 128, 2, 2.5, "silu"), (33, 8, 384, 256, 3, 1.0, "silu"),
-                                                         (20, 4, 256, 128, 2, 2.5, "gelu")])
+                                                         (20, 4, 256, 128, 2, 2.5, "gelu"), (20, 4, 256, 128, 2, 2.5, "relu2")])
 def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf, activation):
     """fused_moe_block_fp8 against the same layer spelled with torch library ops, expert by expert as
     torch_w8a8_block_fp8_moe does (python/sglang/test/test_block_fp8.py:418-447), with the roundings of the fused
@@ -509,18 +537,20 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf, a
     of a bf16 tie may round the other way; everything else must agree bit for bit."""
     rng = np.random.default_rng(T + E)
     x = O.make_activation(T, H, T)
-    w13q = np.empty((E, 2 * I, H), np.uint8); w13s = np.empty((E, 2 * I // 128, H // 128), np.float32)
+    gated = activation != "relu2"     # relu2: experts without a gate projection (fused_moe.py:566-572), w13 is [E, I, H]
+    n1 = 2 * I if gated else I
+    kw = dict(activation=activation, is_gated=gated)
+    w13q = np.empty((E, n1, H), np.uint8); w13s = np.empty((E, n1 // 128, H // 128), np.float32)
     w2q = np.empty((E, H, I), np.uint8); w2s = np.empty((E, H // 128, I // 128), np.float32)
     for e in range(E):
-        w13q[e], w13s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((2 * I, H)).astype(np.float32) * 0.05))
+        w13q[e], w13s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((n1, H)).astype(np.float32) * 0.05))
         w2q[e], w2s[e] = O.block_quant_weight(O.to_bf16(rng.standard_normal((H, I)).astype(np.float32) * 0.05))
     ids = np.stack([rng.permutation(E)[:topk] for _ in range(T)]).astype(np.int32)
     ids[rng.random(ids.shape) < 0.1] = -1          # experts on another rank contribute nothing
     tw = rng.uniform(0.1, 1.0, (T, topk)).astype(np.float32)
-    got = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, activation=activation)
-    got_in = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, apply_router_weight_on_input=True,
-                                   activation=activation)
-    act_fn = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu}[activation]
+    got = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, **kw)
+    got_in = O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, apply_router_weight_on_input=True, **kw)
+    act_fn = {"silu": torch.nn.functional.silu, "gelu": torch.nn.functional.gelu, "relu2": None}[activation]
 
     xt = torch.from_numpy(x).bfloat16()
     xq, xs = _t_group_quant(xt)
@@ -537,7 +567,7 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf, a
             wk = t_w[tok, slot].unsqueeze(1)
             h1 = _t_block_matmul_f64(xq[tok].float(), xs[tok], W1, S1).to(torch.float32)
             h1 = (h1 * wk if weight_on_input else h1).bfloat16()
-            act = act_fn(h1[:, :I].float()).bfloat16() * h1[:, I:]
+            act = act_fn(h1[:, :I].float()).bfloat16() * h1[:, I:] if gated else torch.square(torch.relu(h1))
             aq, a_s = _t_group_quant(act)
             h2 = _t_block_matmul_f64(aq.float(), a_s, W2, S2).to(torch.float32)
             per_slot[tok, slot] = (h2 if weight_on_input else h2 * wk).bfloat16()
@@ -559,13 +589,12 @@ def test_fused_moe_composite_against_torch_ops_pipeline(T, E, H, I, topk, rsf, a
     dead = (ids == -1).all(axis=1)
     assert (got[dead] == 0).all()
     # what a plausible mistake would change: no routed weight, weight applied after the sum, no scaling factor
-    assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, np.ones_like(tw), ids, rsf,
-                                                      activation=activation), rtol=1e-2)
+    assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, np.ones_like(tw), ids, rsf, **kw), rtol=1e-2)
     if rsf != 1.0:
-        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0, activation=activation),
-                               rtol=1e-2)
+        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, 1.0, **kw), rtol=1e-2)
     if activation != "silu":
-        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf), rtol=1e-2)
+        other = dict(kw, activation="silu")
+        assert not np.allclose(got, O.fused_moe_block_fp8(x, w13q, w13s, w2q, w2s, tw, ids, rsf, **other), rtol=1e-2)
 
 
 def _t_fused_gate_bf16(x, bias, G, topk_group, topk):
