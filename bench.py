@@ -304,7 +304,8 @@ def _mfma_probe(torch, dev, ops, sink, form, iters, runs):
 MFMA_LOOP_FORMS = ("bare MFMA loop", "+ block-scaled product form (16 scale FMAs per two MFMAs)",
                    "+ operand fragments refilled from LDS", "+ one workgroup barrier per K block",
                    "+ eight 1 KB stage loads per wave and K block",
-                   "the complete loop without the scale FMAs (products accumulate in place)")
+                   "the complete loop without the scale FMAs (products accumulate in place)",
+                   "the same with 16 multiplies per tile and K block (accumulators rescaled between K blocks)")
 
 
 def mfma_loop_lines(torch, dev, iters=40000, runs=3):

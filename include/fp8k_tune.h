@@ -77,7 +77,8 @@ int fp8k_tune_mfma_peak(const void* operands, int64_t bytes, int64_t iters, floa
  * refilled from LDS behind their last use; form 3: + one LDS-only workgroup barrier per K block; form 4: + the eight
  * 1 KB global -> LDS stage loads per wave and K block (from the first 16 MiB of `operands`, cache-resident) and the
  * partial wait for them at the barrier; form 5: form 4 without the scale FMAs (the products accumulate in place, as in the
- * row-scaled and hardware-scaled modes).  `iters` K blocks; *flops receives the matrix FLOPs of the launch.  Timed by the
+ * row-scaled and hardware-scaled modes); form 6: form 5 with 16 multiplies per 32x32 tile and K block in the place of
+ * the FMAs (a loop that accumulates in place and rescales the accumulators between K blocks).  `iters` K blocks; *flops receives the matrix FLOPs of the launch.  Timed by the
  * caller, the steps down from form to form are what each ingredient costs the matrix cores.
  * operands 32-byte aligned, bytes >= 1 MiB; sink: CUs x 512 floats.
  */

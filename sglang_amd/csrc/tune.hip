@@ -196,6 +196,8 @@ namespace fp8k {
 //   FORM 4  + the eight 1 KB stage loads per wave and K block (global -> LDS) and the partial vmcnt wait at the barrier
 //   FORM 5  form 4 without the scale FMAs: the products accumulate in place, as in the row-scaled and the
 //           hardware-scaled modes of the tile kernel
+//   FORM 6  form 5 with 16 multiplies per 32x32 tile and K block in the place of the FMAs: what a loop would issue that
+//           accumulates in place and multiplies the accumulators by the ratio of two consecutive blocks' scales
 // The instruction order is the tile kernel's (steps 3, 0, 1, 2 of its loop).
 template <int FORM>
 __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __restrict__ operands, int64_t bytes, int iters,
@@ -251,7 +253,7 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     }
   };
   auto RX = [&](int ms, int ks, const uint8_t* st) { if (FORM >= 2) X[ms][ks] = frag(st + (wm * 4 + ms * 2 + ks) * 2048); };
-  constexpr bool kFold = FORM != 5;
+  constexpr bool kFold = FORM != 5 && FORM != 6;
   int step_ns = 0;  // the accumulator row the in-place form is working on (a constant after unrolling)
   auto M = [&](int ms, int ks) {
     if (!kFold) acc[step_ns][ms] = mfma_32x32x64(W[ks], X[ms][ks], acc[step_ns][ms]);
@@ -259,6 +261,11 @@ __global__ __launch_bounds__(512, 1) void mfma_loop_kernel(const uint8_t* __rest
     else tq[ms] = mfma_32x32x64(W[1], X[ms][1], tq[ms]);
   };
   auto F = [&](v16f& a, const v16f& t, float sv) {
+    if (FORM == 6) {
+#pragma unroll
+      for (int q = 0; q < 16; ++q) a[q] = a[q] * sv;
+      return;
+    }
     if (!kFold) return;
 #pragma unroll
     for (int q = 0; q < 16; ++q) a[q] = __builtin_fmaf(t[q], sv, a[q]);
@@ -335,7 +342,7 @@ extern "C" int fp8k_tune_mfma_loop(const void* operands, int64_t bytes, int64_t 
   FP8K_REQUIRE(operands && aligned(operands, 32), "%s: operands must be a 32-byte aligned device pointer", op);
   FP8K_REQUIRE(bytes >= (1 << 20) && bytes < (1LL << 40), "%s: at least 1 MiB of operand bytes is needed", op);
   FP8K_REQUIRE(iters >= 1 && iters <= (1 << 24), "%s: iters must be in [1, 2^24]", op);
-  FP8K_REQUIRE(form >= 1 && form <= 5, "%s: form must be 1..5", op);
+  FP8K_REQUIRE(form >= 1 && form <= 6, "%s: form must be 1..6", op);
   const int ncu = num_cu();
   FP8K_REQUIRE(sink && sink_floats >= (int64_t)ncu * 512, "%s: sink must hold %lld floats", op, (long long)ncu * 512);
   if (flops) *flops = (int64_t)ncu * 8 * iters * 16 * (2LL * 32 * 32 * 64);
@@ -347,7 +354,8 @@ extern "C" int fp8k_tune_mfma_loop(const void* operands, int64_t bytes, int64_t 
     case 2: hipLaunchKernelGGL(mfma_loop_kernel<2>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
     case 3: hipLaunchKernelGGL(mfma_loop_kernel<3>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
     case 4: hipLaunchKernelGGL(mfma_loop_kernel<4>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
-    default: hipLaunchKernelGGL(mfma_loop_kernel<5>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    case 5: hipLaunchKernelGGL(mfma_loop_kernel<5>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
+    default: hipLaunchKernelGGL(mfma_loop_kernel<6>, grid, block, 0, st, o, bytes, (int)iters, sink); break;
   }
   return check_launch(op);
 }

@@ -451,7 +451,7 @@ def test_stream_read_write_probe_writes_its_pattern_and_checks_its_arguments(dev
 def test_mfma_probes_compute_what_they_claim_and_check_their_arguments(dev):
     """The measurement aids fp8k_tune_mfma_peak / fp8k_tune_mfma_loop: on operand bytes 0x38 (1.0 in e4m3) every one of the
     bare loop's 8 x 16 accumulator values per lane is 64 x iters, on all-zero bytes every form sums to zero; the FLOP
-    counts they report are those of their MFMAs; a form outside 1..5 is refused."""
+    counts they report are those of their MFMAs; a form outside 1..6 is refused."""
     import ctypes
 
     from sglang_amd._lib import lib, stream_ptr
@@ -468,7 +468,7 @@ def test_mfma_probes_compute_what_they_claim_and_check_their_arguments(dev):
     torch.cuda.synchronize()
     assert flops.value == ncu * 8 * iters * 8 * 2 * 32 * 32 * 64
     assert (sink == 128 * 64.0 * iters).all()
-    for form in (1, 2, 3, 4, 5):
+    for form in (1, 2, 3, 4, 5, 6):
         sink.fill_(float("nan"))
         rc = lib.fp8k_tune_mfma_loop(zeros.data_ptr(), zeros.numel(), iters, form, sink.data_ptr(), sink.numel(),
                                      ctypes.byref(flops), stream_ptr(dev))
@@ -485,6 +485,6 @@ def test_mfma_probes_compute_what_they_claim_and_check_their_arguments(dev):
     got = sink.cpu().numpy()
     assert np.isfinite(got).all() and (got > 0).all()
     assert np.allclose(got, got[0], rtol=1e-5)
-    rc = lib.fp8k_tune_mfma_loop(zeros.data_ptr(), zeros.numel(), iters, 6, sink.data_ptr(), sink.numel(), ctypes.byref(flops),
+    rc = lib.fp8k_tune_mfma_loop(zeros.data_ptr(), zeros.numel(), iters, 7, sink.data_ptr(), sink.numel(), ctypes.byref(flops),
                                  stream_ptr(dev))
     assert rc != 0 and b"form" in lib.fp8k_last_error()
