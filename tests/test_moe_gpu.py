@@ -656,21 +656,23 @@ def deepseek_experts(dev):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("T", [1, 3, 32, 256, 4096])
+@pytest.mark.parametrize("T", [1, 3, 32, 256, 4096, 16384])
 def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
     """The fused MoE layer at its full DeepSeek-V3 dimensions (256 experts, hidden 7168, intermediate 2048, top-8
-    grouped-sigmoid routing over 8 groups / 4 groups kept) for 1, 3, 32, 256 and 4096 tokens: these token counts
-    take the 16-, 32-, 64-slot and 256-slot grouped kernels in turn (asserted below).  A token's output depends on
+    grouped-sigmoid routing over 8 groups / 4 groups kept) for 1, 3, 32, 256, 4096 and 16384 tokens: these token counts
+    take the 16-, 32- and 256-slot grouped kernels in turn (asserted below), the last on a table that
+    moe_balance_blocks has dealt out evenly (several blocks per expert).  A token's output depends on
     nothing but its own row, its eight experts and its routed weights, so the oracle is evaluated on a sample of
     tokens (all of them up to 3 tokens) with only the experts those tokens hit copied back; the whole output must
     be finite, and permuting the tokens must permute the result (exactly where the kernel choice per expert is
     unchanged, which holds for a permutation: every expert keeps its slot count)."""
-    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl, get_default_config
+    from sglang_amd.fused_moe import biased_grouped_topk, blocks_want_balancing, fused_experts_impl, get_default_config
 
     d = deepseek_experts
     E, H, topk = d["E"], d["H"], 8
-    want_block = {1: 16, 3: 16, 32: 16, 256: 32, 4096: 256}[T]
+    want_block = {1: 16, 3: 16, 32: 16, 256: 32, 4096: 256, 16384: 256}[T]
     assert get_default_config(T, E, topk)["BLOCK_SIZE_M"] == want_block
+    assert blocks_want_balancing(get_default_config(T, E, topk), T * topk, E) == (T == 16384)
     x = O.make_activation(T, H, T)
     logits = torch.randn((T, E), generator=d["gen"], device=dev)
     xt = bf16_tensor(x, dev)
