@@ -700,6 +700,45 @@ def test_fused_experts_deepseek_dims(dev, deepseek_experts, T):
         assert torch.equal(out_p, out[perm])
 
 
+@pytest.mark.parametrize("T", [4096, 16384])
+def test_cutlass_fused_experts_deepseek_dims(dev, deepseek_experts, T):
+    """The expert-major layer (cutlass_fused_experts_fp8) at the full DeepSeek-V3 dimensions: 32768 and 131072 ids take
+    the multi-workgroup forms of prepare_moe_input and of the block table, GEMM 1 writes the requantised activation out
+    itself, and at 16384 tokens the table is dealt out evenly and walked.  Oracle (expert-major composite) on a sample of
+    tokens; the whole output against the slot-ordered layer of this library on the same inputs, as
+    python/sglang/test/test_cutlass_moe.py compares the two paths."""
+    from sglang_amd.cutlass_moe import cutlass_fused_experts_fp8
+    from sglang_amd.fused_moe import biased_grouped_topk, fused_experts_impl
+
+    d = deepseek_experts
+    E, H, I, topk = d["E"], d["H"], d["I"], 8
+    x = O.make_activation(T, H, T + 1)
+    logits = torch.randn((T, E), generator=d["gen"], device=dev)
+    xt = bf16_tensor(x, dev)
+    tw, ids = biased_grouped_topk(xt, logits, d["bias"], topk, True, 8, 4)
+    i64 = lambda: torch.empty((E,), device=dev, dtype=torch.int64)  # noqa: E731
+    out = cutlass_fused_experts_fp8(
+        xt, d["w1"].transpose(1, 2), d["w2"].transpose(1, 2), d["w1s"].transpose(1, 2), d["w2s"].transpose(1, 2), tw, ids,
+        torch.full((E,), H, device=dev, dtype=torch.int64), torch.full((E,), 2 * I, device=dev, dtype=torch.int64),
+        torch.full((E,), I, device=dev, dtype=torch.int64), torch.full((E,), H, device=dev, dtype=torch.int64),
+        torch.empty((1024,), device=dev, dtype=torch.uint8), i64(), i64(), i64(), i64(), i64(),
+        torch.empty((E + 1,), device=dev, dtype=torch.int32), torch.empty((E, 3), device=dev, dtype=torch.int32),
+        torch.empty((E, 3), device=dev, dtype=torch.int32), use_fp8_blockscale=True)
+    torch.cuda.synchronize()
+    assert out.shape == (T, H) and out.dtype == torch.bfloat16 and bool(torch.isfinite(out).all())
+    rng = np.random.default_rng(T)
+    sample = np.unique(np.concatenate([[0, T - 1], rng.integers(0, T, 4)]))
+    ref = O.cutlass_fused_experts_fp8(x[sample], _LazyExperts(d["w1"], True), _LazyExperts(d["w1s"], False),
+                                      _LazyExperts(d["w2"], True), _LazyExperts(d["w2s"], False),
+                                      tw.cpu().numpy()[sample], ids.cpu().numpy()[sample])
+    got = out[torch.from_numpy(sample).to(dev)].float().cpu().numpy()
+    assert _rel_err(got, ref) <= REL_TOL, _rel_err(got, ref)
+    slot_order = fused_experts_impl(xt, d["w1"], d["w2"], tw, ids, use_fp8_w8a8=True, w1_scale=d["w1s"], w2_scale=d["w2s"],
+                                    block_shape=[128, 128]).double()
+    o = out.double()
+    assert float(1 - 2 * (o * slot_order).sum() / ((o * o).sum() + (slot_order * slot_order).sum())) < 1e-3
+
+
 @pytest.mark.parametrize("T,block", [(1024, 64), (2048, 128), (1024, 256)])
 def test_fused_experts_deepseek_dims_other_block_sizes(dev, deepseek_experts, T, block, monkeypatch):
     """The 64- and 128-slot grouped streaming kernels at the full expert dimensions (a caller's own BLOCK_SIZE_M; the
